@@ -1,0 +1,167 @@
+/*
+ * clusten_hip.h — C ABI of libclusten_hip.so: the CLUSTEN neighbourhood-gather ops
+ * (QK, AV, WF; forward and backward) as hand-written gfx950 HIP kernels.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes, element strides, a dtype code and a HIP stream;
+ *   - enqueues its kernels on that stream and returns without synchronising;
+ *   - never allocates or frees memory (scratch comes in through a workspace argument);
+ *   - returns a clusten_status (0 = ok) instead of throwing;
+ *   - is re-entrant: the library keeps no mutable global state.
+ *
+ * The entry points stand in for the six functions the reference binds through pybind11
+ * (three extension modules, each exporting `forward` and `backward`):
+ *   clusten/src/clustenqk_cuda.cpp:25-51, clusten/src/clustenav_cuda.cpp:25-51,
+ *   clusten/src/clustenwf_cuda.cpp:25-51.
+ * Differences a caller must know:
+ *   - outputs are caller-allocated (the reference allocates them with torch::zeros);
+ *   - `key` is passed un-transposed, (B,H,N,C) — the reference's wrapper hands its kernel a
+ *     (B,H,C,N) copy (clusten/clusten.py:30), which is an implementation detail of that kernel;
+ *   - query / key / value may be strided views: element strides for the batch, head and token
+ *     axes are explicit arguments, the channel axis must have stride 1.  Passing the strides of a
+ *     (B,N,H,C)-stored tensor avoids the `.contiguous()` copies of clusten/clusten.py:23-24,49-50.
+ *
+ * Index convention: `nbhd_idx` is int64, contiguous, values in [0, N) — unchecked, as in the
+ * reference.  All tensors of one call live on the device that is current for `stream`.
+ */
+#ifndef CLUSTEN_HIP_H
+#define CLUSTEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CLUSTEN_ABI_VERSION 1
+
+/* Element type of every floating-point tensor of a call.  The reference dispatches
+ * double / float / half (AT_DISPATCH_FLOATING_TYPES_AND_HALF, clustenqk_cuda_kernel.cu:78);
+ * bfloat16 has no reference kernel and is checked against the gather oracle only. */
+typedef enum clusten_dtype {
+    CLUSTEN_F32 = 0,
+    CLUSTEN_F16 = 1,
+    CLUSTEN_BF16 = 2,
+    CLUSTEN_F64 = 3
+} clusten_dtype;
+
+typedef enum clusten_status {
+    CLUSTEN_OK = 0,
+    CLUSTEN_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    CLUSTEN_ERR_BAD_DTYPE = 2,      /* dtype code not in clusten_dtype */
+    CLUSTEN_ERR_BAD_DIMS = 3,       /* a size is <= 0, or N >= 2^31, or a per-batch slice >= 2^31 elements */
+    CLUSTEN_ERR_BAD_STRIDE = 4,     /* a stride is negative or makes rows overlap */
+    CLUSTEN_ERR_WORKSPACE = 5,      /* workspace missing or smaller than *_workspace_bytes() */
+    CLUSTEN_ERR_LAUNCH = 6,         /* hipGetLastError() reported a failure after a launch */
+    CLUSTEN_ERR_UNALIGNED = 7       /* clusten_copy_probe only: a pointer is not 16-byte aligned
+                                       (the gather ops route unaligned operands to element-wise kernels) */
+} clusten_status;
+
+/* Opaque stream handle: a hipStream_t.  NULL is the legacy default stream. */
+typedef void* clusten_stream;
+
+/* Shape of one QK / AV problem.
+ *   query/key/value : (B,H,N,C), element (b,h,n,c) at b*stride_b + h*stride_h + n*stride_n + c
+ *   nbhd_idx        : (B,N,M) int64 contiguous, shared by all heads
+ *   attn            : (B,H,N,M) contiguous */
+typedef struct clusten_attn_shape {
+    int32_t B, H, N, C, M;
+} clusten_attn_shape;
+
+/* Element strides of a (B,H,N,C) operand whose channel stride is 1. */
+typedef struct clusten_strides {
+    int64_t b, h, n;
+} clusten_strides;
+
+/* Shape of one WF problem.
+ *   weights  : (B,Nout,M,IC) contiguous
+ *   feat     : (B,N,C) contiguous
+ *   nbhd_idx : (B,Nout,M) int64 contiguous, values in [0,N)
+ *   feat_new : (B,Nout,IC,C) contiguous */
+typedef struct clusten_wf_shape {
+    int32_t B, N, Nout, C, M, IC;
+} clusten_wf_shape;
+
+/* ---- library ------------------------------------------------------------------------------ */
+
+/* CLUSTEN_ABI_VERSION the library was built with. */
+int clusten_abi_version(void);
+
+/* Static, NUL-terminated description of a status code. */
+const char* clusten_status_string(int status);
+
+/* ---- QK:  attn[b,h,i,j] = sum_c query[b,h,i,c] * key[b,h,nbhd_idx[b,i,j],c] ------------------- */
+
+/* Replaces clustenqk_cuda.forward (clusten/src/clustenqk_cuda.cpp:25-33, kernel
+ * clustenqk_cuda_kernel.cu:18-89).  `attn` need not be zeroed. */
+int clusten_qk_forward(const void* query, clusten_strides query_strides,
+                       const void* key, clusten_strides key_strides,
+                       const int64_t* nbhd_idx, void* attn,
+                       clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* Replaces clustenqk_cuda.backward (clustenqk_cuda.cpp:35-45, clustenqk_cuda_kernel.cu:91-178):
+ *   d_query[b,h,i,c] = sum_j key[b,h,idx[b,i,j],c] * d_attn[b,h,i,j]
+ *   d_key[b,h,n,c]   = sum_{(i,j): idx[b,i,j]=n} query[b,h,i,c] * d_attn[b,h,i,j]
+ * d_query, d_key are (B,H,N,C) contiguous, need not be zeroed.  For F16/BF16 the scatter is
+ * accumulated in fp32 in `workspace` (clusten_qk_backward_workspace_bytes) and rounded once. */
+size_t clusten_qk_backward_workspace_bytes(clusten_attn_shape shape, int dtype);
+int clusten_qk_backward(const void* d_attn,
+                        const void* query, clusten_strides query_strides,
+                        const void* key, clusten_strides key_strides,
+                        const int64_t* nbhd_idx, void* d_query, void* d_key,
+                        void* workspace, size_t workspace_bytes,
+                        clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* ---- AV:  feat[b,h,i,c] = sum_j attn[b,h,i,j] * value[b,h,nbhd_idx[b,i,j],c] ------------------ */
+
+/* Replaces clustenav_cuda.forward (clusten/src/clustenav_cuda.cpp:25-33, kernel
+ * clustenav_cuda_kernel.cu:18-90).  `feat` is written with the strides given (channel stride 1),
+ * so a caller can have it land directly in (B,N,H,C) storage. */
+int clusten_av_forward(const void* attn,
+                       const void* value, clusten_strides value_strides,
+                       const int64_t* nbhd_idx,
+                       void* feat, clusten_strides feat_strides,
+                       clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* Replaces clustenav_cuda.backward (clustenav_cuda.cpp:35-45, clustenav_cuda_kernel.cu:93-218):
+ *   d_attn[b,h,i,j]  = sum_c value[b,h,idx[b,i,j],c] * d_feat[b,h,i,c]
+ *   d_value[b,h,n,c] = sum_{(i,j): idx[b,i,j]=n} attn[b,h,i,j] * d_feat[b,h,i,c]
+ * d_attn (B,H,N,M) and d_value (B,H,N,C) are contiguous, need not be zeroed. */
+size_t clusten_av_backward_workspace_bytes(clusten_attn_shape shape, int dtype);
+int clusten_av_backward(const void* d_feat, clusten_strides d_feat_strides,
+                        const void* attn,
+                        const void* value, clusten_strides value_strides,
+                        const int64_t* nbhd_idx, void* d_attn, void* d_value,
+                        void* workspace, size_t workspace_bytes,
+                        clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* ---- WF:  feat_new[b,i,ic,c] = sum_j weights[b,i,j,ic] * feat[b,nbhd_idx[b,i,j],c] ------------ */
+
+/* Replaces clustenwf_cuda.forward (clusten/src/clustenwf_cuda.cpp:25-33, kernel
+ * clustenwf_cuda_kernel.cu:18-93). */
+int clusten_wf_forward(const void* weights, const void* feat, const int64_t* nbhd_idx,
+                       void* feat_new, clusten_wf_shape shape, int dtype, clusten_stream stream);
+
+/* Replaces clustenwf_cuda.backward (clustenwf_cuda.cpp:35-45, clustenwf_cuda_kernel.cu:96-229):
+ *   d_weights[b,i,j,ic] = sum_c feat[b,idx[b,i,j],c] * d_feat_new[b,i,ic,c]
+ *   d_feat[b,n,c]       = sum_{(i,j): idx[b,i,j]=n} sum_ic d_feat_new[b,i,ic,c] * weights[b,i,j,ic] */
+size_t clusten_wf_backward_workspace_bytes(clusten_wf_shape shape, int dtype);
+int clusten_wf_backward(const void* d_feat_new, const void* weights, const void* feat,
+                        const int64_t* nbhd_idx, void* d_weights, void* d_feat,
+                        void* workspace, size_t workspace_bytes,
+                        clusten_wf_shape shape, int dtype, clusten_stream stream);
+
+/* ---- measurement aid ------------------------------------------------------------------------ */
+
+/* Plain streaming copy of `bytes` bytes (multiple of 16, both pointers 16-byte aligned) with the
+ * same launch shape the gather kernels use.  It has no counterpart in the reference; it exists so
+ * that a profiler's HBM byte counters can be calibrated against a kernel of known traffic and so
+ * that a benchmark can print the copy bandwidth the device sustains next to the roofline figure. */
+int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CLUSTEN_HIP_H */

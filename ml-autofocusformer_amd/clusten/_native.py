@@ -1,0 +1,306 @@
+"""ctypes binding of libclusten_hip.so (C ABI in include/clusten_hip.h) for PyTorch-ROCm tensors.
+
+PyTorch is used for device memory and streams only: outputs and workspaces are allocated with
+`torch.empty` (stream-ordered caching allocator), kernels are enqueued on the tensor device's
+current stream, nothing synchronises.  There is no CPU path and no fallback: a missing library,
+a CPU tensor or a non-zero status raises RuntimeError.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "lib", "libclusten_hip.so"))
+
+ABI_VERSION = 1
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
+
+
+class AttnShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("B", "H", "N", "C", "M")]
+
+
+class Strides(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("b", "h", "n")]
+
+
+class WfShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("B", "N", "Nout", "C", "M", "IC")]
+
+
+_P = ctypes.c_void_p
+_PROTOTYPES = {
+    # name: (restype, argtypes)  — one entry per declaration in include/clusten_hip.h
+    "clusten_abi_version": (ctypes.c_int, []),
+    "clusten_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "clusten_qk_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_qk_backward_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
+    "clusten_qk_backward": (ctypes.c_int, [_P, _P, Strides, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape,
+                                           ctypes.c_int, _P]),
+    "clusten_av_forward": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
+    "clusten_av_backward_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
+    "clusten_av_backward": (ctypes.c_int, [_P, Strides, _P, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape,
+                                           ctypes.c_int, _P]),
+    "clusten_wf_forward": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
+    "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
+    "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
+    "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
+}
+
+EXPORTS = tuple(_PROTOTYPES)
+
+_lib = None
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load libclusten_hip.so once.  Raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                "Could not load the CLUSTEN HIP library (%s). Build it with `make -C ml-autofocusformer_amd/csrc` "
+                "(hipcc, gfx950); there is no CPU or PyTorch fallback." % _LIB_PATH)
+        try:
+            lib = ctypes.CDLL(_LIB_PATH)
+        except OSError as e:  # e.g. the HIP runtime is missing
+            raise RuntimeError("Could not load the CLUSTEN HIP library (%s): %s" % (_LIB_PATH, e)) from e
+        for name, (restype, argtypes) in _PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if lib.clusten_abi_version() != ABI_VERSION:
+            raise RuntimeError("libclusten_hip.so has ABI version %d, this binding expects %d" %
+                               (lib.clusten_abi_version(), ABI_VERSION))
+        _lib = lib
+    return _lib
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise RuntimeError("%s failed: %s (status %d)" % (what, load().clusten_status_string(status).decode(), status))
+
+
+def _dtype_code(t: torch.Tensor, name: str) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise RuntimeError("%s has unsupported dtype %s (float32, float16, bfloat16, float64)" % (name, t.dtype))
+
+
+def _require_cuda(name: str, t: torch.Tensor, device=None) -> None:
+    # same message as the reference's CHECK_CUDA (clusten/src/clustenqk_cuda.cpp:21)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if device is not None and t.device != device:
+        raise RuntimeError("%s is on %s, expected %s" % (name, t.device, device))
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """A (B,H,N,C) tensor the kernels can address: channel stride 1, rows that do not overlap.
+    Anything else (e.g. a transposed channel axis) is copied, as the reference always does
+    (clusten/clusten.py:23-24)."""
+    sb, sh, sn, sc = t.stride()
+    C = t.shape[3]
+    if (sc == 1 or C == 1) and sn >= C and sb >= 0 and sh >= 0:
+        return t
+    return t.contiguous()
+
+
+def _strides(t: torch.Tensor) -> Strides:
+    return Strides(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _ptr(t) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _idx(nbhd_idx: torch.Tensor, shape, device) -> torch.Tensor:
+    _require_cuda("nbhd_idx", nbhd_idx, device)
+    if nbhd_idx.dtype != torch.int64:
+        raise RuntimeError("nbhd_idx must be int64, got %s" % nbhd_idx.dtype)
+    if tuple(nbhd_idx.shape[:2]) != tuple(shape):
+        raise RuntimeError("nbhd_idx has shape %s, expected (%d, %d, m)" % (tuple(nbhd_idx.shape), shape[0], shape[1]))
+    return nbhd_idx.contiguous()
+
+
+def _attn_problem(a: torch.Tensor, rows: torch.Tensor, nbhd_idx: torch.Tensor, names):
+    """Common checks of (query,key) / (d_feat,value) pairs: returns device, dtype code, idx, shape."""
+    _require_cuda(names[0], a)
+    device = a.device
+    _require_cuda(names[1], rows, device)
+    if a.dim() != 4 or rows.dim() != 4 or nbhd_idx.dim() != 3:
+        raise RuntimeError("%s and %s must be (b,h,n,c) and nbhd_idx (b,n,m)" % names)
+    if a.shape != rows.shape:
+        raise RuntimeError("%s %s and %s %s must have the same shape" % (names[0], tuple(a.shape), names[1],
+                                                                         tuple(rows.shape)))
+    if a.dtype != rows.dtype:
+        raise RuntimeError("%s and %s must have the same dtype" % names)
+    B, H, N, C = a.shape
+    idx = _idx(nbhd_idx, (B, N), device)
+    return device, _dtype_code(a, names[0]), idx, AttnShape(B, H, N, C, idx.shape[2])
+
+
+def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
+    """attn (b,h,n,m) = query · key[nbhd_idx]; query/key (b,h,n,c) may be strided views."""
+    lib = load()
+    device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
+    query, key = _rows(query), _rows(key)
+    attn = torch.empty((shape.B, shape.H, shape.N, shape.M), dtype=query.dtype, device=device)
+    if attn.numel() == 0:
+        return attn
+    with torch.cuda.device(device):
+        _check(lib.clusten_qk_forward(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx), _ptr(attn),
+                                      shape, code, _stream(device)), "clusten_qk_forward")
+    return attn
+
+
+def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor):
+    """(d_query, d_key), both contiguous (b,h,n,c)."""
+    lib = load()
+    device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
+    _require_cuda("d_attn", d_attn, device)
+    if tuple(d_attn.shape) != (shape.B, shape.H, shape.N, shape.M) or d_attn.dtype != query.dtype:
+        raise RuntimeError("d_attn must be (b,h,n,m) with the dtype of query")
+    d_attn = d_attn.contiguous()
+    query, key = _rows(query), _rows(key)
+    d_query = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=query.dtype, device=device)
+    d_key = torch.empty_like(d_query)
+    if d_query.numel() == 0 or shape.M == 0:
+        return d_query.zero_(), d_key.zero_()
+    ws_bytes = lib.clusten_qk_backward_workspace_bytes(shape, code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    with torch.cuda.device(device):
+        _check(lib.clusten_qk_backward(_ptr(d_attn), _ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx),
+                                       _ptr(d_query), _ptr(d_key), _ptr(ws), ws_bytes, shape, code, _stream(device)),
+               "clusten_qk_backward")
+    return d_query, d_key
+
+
+def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, token_major: bool = False) -> torch.Tensor:
+    """feat (b,h,n,c) = attn · v[nbhd_idx].  With token_major=True the result is a (b,h,n,c) view of
+    (b,n,h,c) storage, so that `.permute(0,2,1,3).reshape(b,n,h*c)` needs no copy."""
+    lib = load()
+    _require_cuda("attn", attn)
+    device = attn.device
+    _require_cuda("v", v, device)
+    if attn.dim() != 4 or v.dim() != 4 or nbhd_idx.dim() != 3:
+        raise RuntimeError("attn must be (b,h,n,m), v (b,h,n,c) and nbhd_idx (b,n,m)")
+    if attn.shape[:3] != v.shape[:3] or attn.dtype != v.dtype:
+        raise RuntimeError("attn %s and v %s must agree in (b,h,n) and dtype" % (tuple(attn.shape), tuple(v.shape)))
+    B, H, N, C = v.shape
+    idx = _idx(nbhd_idx, (B, N), device)
+    if idx.shape[2] != attn.shape[3]:
+        raise RuntimeError("attn has %d slots per token, nbhd_idx %d" % (attn.shape[3], idx.shape[2]))
+    shape = AttnShape(B, H, N, C, idx.shape[2])
+    code = _dtype_code(attn, "attn")
+    attn, v = attn.contiguous(), _rows(v)
+    if token_major:
+        feat = torch.empty((B, N, H, C), dtype=attn.dtype, device=device).permute(0, 2, 1, 3)
+    else:
+        feat = torch.empty((B, H, N, C), dtype=attn.dtype, device=device)
+    if feat.numel() == 0:
+        return feat
+    if shape.M == 0:
+        return feat.zero_()
+    with torch.cuda.device(device):
+        _check(lib.clusten_av_forward(_ptr(attn), _ptr(v), _strides(v), _ptr(idx), _ptr(feat), _strides(feat), shape,
+                                      code, _stream(device)), "clusten_av_forward")
+    return feat
+
+
+def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor):
+    """(d_attn (b,h,n,m), d_v (b,h,n,c)), both contiguous."""
+    lib = load()
+    device, code, idx, shape = _attn_problem(d_feat, v, nbhd_idx, ("d_feat", "v"))
+    _require_cuda("attn", attn, device)
+    if tuple(attn.shape) != (shape.B, shape.H, shape.N, shape.M) or attn.dtype != v.dtype:
+        raise RuntimeError("attn must be (b,h,n,m) with the dtype of v")
+    attn = attn.contiguous()
+    d_feat, v = _rows(d_feat), _rows(v)
+    d_attn = torch.empty((shape.B, shape.H, shape.N, shape.M), dtype=attn.dtype, device=device)
+    d_v = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=attn.dtype, device=device)
+    if d_v.numel() == 0 or shape.M == 0:
+        return d_attn.zero_(), d_v.zero_()
+    ws_bytes = lib.clusten_av_backward_workspace_bytes(shape, code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    with torch.cuda.device(device):
+        _check(lib.clusten_av_backward(_ptr(d_feat), _strides(d_feat), _ptr(attn), _ptr(v), _strides(v), _ptr(idx),
+                                       _ptr(d_attn), _ptr(d_v), _ptr(ws), ws_bytes, shape, code, _stream(device)),
+               "clusten_av_backward")
+    return d_attn, d_v
+
+
+def _wf_problem(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor):
+    _require_cuda("weights", weights)
+    device = weights.device
+    _require_cuda("feat", feat, device)
+    if weights.dim() != 4 or feat.dim() != 3 or nbhd_idx.dim() != 3:
+        raise RuntimeError("weights must be (b,n_,m,ic), feat (b,n,c) and nbhd_idx (b,n_,m)")
+    if weights.shape[0] != feat.shape[0] or weights.dtype != feat.dtype:
+        raise RuntimeError("weights and feat must agree in batch size and dtype")
+    B, Nout, M, IC = weights.shape
+    N, C = feat.shape[1], feat.shape[2]
+    idx = _idx(nbhd_idx, (B, Nout), device)
+    if idx.shape[2] != M:
+        raise RuntimeError("weights has %d slots per token, nbhd_idx %d" % (M, idx.shape[2]))
+    return device, _dtype_code(weights, "weights"), idx, WfShape(B, N, Nout, C, M, IC)
+
+
+def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
+    """feat_new (b,n_,ic,c) = weightsᵀ · feat[nbhd_idx]."""
+    lib = load()
+    device, code, idx, shape = _wf_problem(weights, feat, nbhd_idx)
+    weights, feat = weights.contiguous(), feat.contiguous()
+    out = torch.empty((shape.B, shape.Nout, shape.IC, shape.C), dtype=weights.dtype, device=device)
+    if out.numel() == 0:
+        return out
+    if shape.M == 0 or shape.N == 0:
+        return out.zero_()
+    with torch.cuda.device(device):
+        _check(lib.clusten_wf_forward(_ptr(weights), _ptr(feat), _ptr(idx), _ptr(out), shape, code, _stream(device)),
+               "clusten_wf_forward")
+    return out
+
+
+def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor):
+    """(d_weights (b,n_,m,ic), d_feat (b,n,c)), both contiguous."""
+    lib = load()
+    device, code, idx, shape = _wf_problem(weights, feat, nbhd_idx)
+    _require_cuda("d_feat_new", d_feat_new, device)
+    if tuple(d_feat_new.shape) != (shape.B, shape.Nout, shape.IC, shape.C) or d_feat_new.dtype != weights.dtype:
+        raise RuntimeError("d_feat_new must be (b,n_,ic,c) with the dtype of weights")
+    d_feat_new, weights, feat = d_feat_new.contiguous(), weights.contiguous(), feat.contiguous()
+    d_weights = torch.empty_like(weights)
+    d_feat = torch.empty_like(feat)
+    if d_weights.numel() == 0 or d_feat.numel() == 0:
+        return d_weights.zero_(), d_feat.zero_()
+    ws_bytes = lib.clusten_wf_backward_workspace_bytes(shape, code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    with torch.cuda.device(device):
+        _check(lib.clusten_wf_backward(_ptr(d_feat_new), _ptr(weights), _ptr(feat), _ptr(idx), _ptr(d_weights),
+                                       _ptr(d_feat), _ptr(ws), ws_bytes, shape, code, _stream(device)),
+               "clusten_wf_backward")
+    return d_weights, d_feat
+
+
+def copy_probe(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst <- src with the library's streaming copy kernel (measurement aid)."""
+    lib = load()
+    _require_cuda("src", src)
+    _require_cuda("dst", dst, src.device)
+    nbytes = src.numel() * src.element_size()
+    if not (src.is_contiguous() and dst.is_contiguous()) or dst.numel() * dst.element_size() != nbytes:
+        raise RuntimeError("copy_probe needs contiguous tensors of equal byte size")
+    with torch.cuda.device(src.device):
+        _check(lib.clusten_copy_probe(_ptr(src), _ptr(dst), nbytes, _stream(src.device)), "clusten_copy_probe")

@@ -1,0 +1,142 @@
+// extern "C" surface of libclusten_hip.so (declared in include/clusten_hip.h): argument checks,
+// then the internal launch functions.  Nothing here allocates, frees or synchronises.
+#include "launch.hpp"
+
+using namespace clusten;
+
+namespace {
+
+inline hipStream_t as_stream(clusten_stream s) { return static_cast<hipStream_t>(s); }
+
+inline int check_attn_call(const clusten_attn_shape& s, int dtype) {
+    if (!dtype_ok(dtype)) return CLUSTEN_ERR_BAD_DTYPE;
+    return check_attn_shape(s);
+}
+
+inline clusten_strides contiguous_strides(const clusten_attn_shape& s) {
+    clusten_strides r;
+    r.n = s.C;
+    r.h = (int64_t)s.N * s.C;
+    r.b = (int64_t)s.H * s.N * s.C;
+    return r;
+}
+
+}  // namespace
+
+extern "C" {
+
+int clusten_abi_version(void) { return CLUSTEN_ABI_VERSION; }
+
+const char* clusten_status_string(int status) {
+    switch (status) {
+        case CLUSTEN_OK: return "ok";
+        case CLUSTEN_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case CLUSTEN_ERR_BAD_DTYPE: return "unknown dtype code";
+        case CLUSTEN_ERR_BAD_DIMS: return "a size is not positive or exceeds the 32-bit indexing limits";
+        case CLUSTEN_ERR_BAD_STRIDE: return "a stride is negative or rows overlap";
+        case CLUSTEN_ERR_WORKSPACE: return "workspace missing or too small";
+        case CLUSTEN_ERR_LAUNCH: return "kernel launch failed";
+        case CLUSTEN_ERR_UNALIGNED: return "pointer or stride is not aligned";
+        default: return "unknown status";
+    }
+}
+
+int clusten_qk_forward(const void* query, clusten_strides query_strides, const void* key, clusten_strides key_strides,
+                       const int64_t* nbhd_idx, void* attn, clusten_attn_shape shape, int dtype,
+                       clusten_stream stream) {
+    if (!query || !key || !nbhd_idx || !attn) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_gather_dot(query, query_strides, key, key_strides, nbhd_idx, attn, shape, dtype, as_stream(stream));
+}
+
+size_t clusten_qk_backward_workspace_bytes(clusten_attn_shape shape, int dtype) {
+    if (!dtype_ok(dtype) || check_attn_shape(shape) != CLUSTEN_OK) return 0;
+    return scatter_rows_workspace_bytes(shape, dtype);
+}
+
+int clusten_qk_backward(const void* d_attn, const void* query, clusten_strides query_strides, const void* key,
+                        clusten_strides key_strides, const int64_t* nbhd_idx, void* d_query, void* d_key,
+                        void* workspace, size_t workspace_bytes, clusten_attn_shape shape, int dtype,
+                        clusten_stream stream) {
+    if (!d_attn || !query || !key || !nbhd_idx || !d_query || !d_key) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    const size_t need = scatter_rows_workspace_bytes(shape, dtype);
+    if (need && (!workspace || workspace_bytes < need)) return CLUSTEN_ERR_WORKSPACE;
+    // d_query = gather_sum(d_attn, key)
+    int st = launch_gather_sum(d_attn, key, key_strides, nbhd_idx, d_query, contiguous_strides(shape), shape, dtype,
+                               as_stream(stream));
+    if (st != CLUSTEN_OK) return st;
+    // d_key = scatter_rows(d_attn, query)
+    return launch_scatter_rows(d_attn, query, query_strides, nbhd_idx, d_key, workspace, shape, dtype,
+                               as_stream(stream));
+}
+
+int clusten_av_forward(const void* attn, const void* value, clusten_strides value_strides, const int64_t* nbhd_idx,
+                       void* feat, clusten_strides feat_strides, clusten_attn_shape shape, int dtype,
+                       clusten_stream stream) {
+    if (!attn || !value || !nbhd_idx || !feat) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(value_strides, shape.C) || !strides_ok(feat_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_gather_sum(attn, value, value_strides, nbhd_idx, feat, feat_strides, shape, dtype,
+                             as_stream(stream));
+}
+
+size_t clusten_av_backward_workspace_bytes(clusten_attn_shape shape, int dtype) {
+    if (!dtype_ok(dtype) || check_attn_shape(shape) != CLUSTEN_OK) return 0;
+    return scatter_rows_workspace_bytes(shape, dtype);
+}
+
+int clusten_av_backward(const void* d_feat, clusten_strides d_feat_strides, const void* attn, const void* value,
+                        clusten_strides value_strides, const int64_t* nbhd_idx, void* d_attn, void* d_value,
+                        void* workspace, size_t workspace_bytes, clusten_attn_shape shape, int dtype,
+                        clusten_stream stream) {
+    if (!d_feat || !attn || !value || !nbhd_idx || !d_attn || !d_value) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(d_feat_strides, shape.C) || !strides_ok(value_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    const size_t need = scatter_rows_workspace_bytes(shape, dtype);
+    if (need && (!workspace || workspace_bytes < need)) return CLUSTEN_ERR_WORKSPACE;
+    // d_attn = gather_dot(d_feat, value)
+    int st = launch_gather_dot(d_feat, d_feat_strides, value, value_strides, nbhd_idx, d_attn, shape, dtype,
+                               as_stream(stream));
+    if (st != CLUSTEN_OK) return st;
+    // d_value = scatter_rows(attn, d_feat)
+    return launch_scatter_rows(attn, d_feat, d_feat_strides, nbhd_idx, d_value, workspace, shape, dtype,
+                               as_stream(stream));
+}
+
+int clusten_wf_forward(const void* weights, const void* feat, const int64_t* nbhd_idx, void* feat_new,
+                       clusten_wf_shape shape, int dtype, clusten_stream stream) {
+    if (!weights || !feat || !nbhd_idx || !feat_new) return CLUSTEN_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype)) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_wf_shape(shape)) return st;
+    return launch_wf_forward(weights, feat, nbhd_idx, feat_new, shape, dtype, as_stream(stream));
+}
+
+size_t clusten_wf_backward_workspace_bytes(clusten_wf_shape shape, int dtype) {
+    if (!dtype_ok(dtype) || check_wf_shape(shape) != CLUSTEN_OK) return 0;
+    return wf_dfeat_workspace_bytes(shape, dtype);
+}
+
+int clusten_wf_backward(const void* d_feat_new, const void* weights, const void* feat, const int64_t* nbhd_idx,
+                        void* d_weights, void* d_feat, void* workspace, size_t workspace_bytes, clusten_wf_shape shape,
+                        int dtype, clusten_stream stream) {
+    if (!d_feat_new || !weights || !feat || !nbhd_idx || !d_weights || !d_feat) return CLUSTEN_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype)) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_wf_shape(shape)) return st;
+    const size_t need = wf_dfeat_workspace_bytes(shape, dtype);
+    if (need && (!workspace || workspace_bytes < need)) return CLUSTEN_ERR_WORKSPACE;
+    int st = launch_wf_dweights(d_feat_new, feat, nbhd_idx, d_weights, shape, dtype, as_stream(stream));
+    if (st != CLUSTEN_OK) return st;
+    return launch_wf_dfeat(d_feat_new, weights, nbhd_idx, d_feat, workspace, shape, dtype, as_stream(stream));
+}
+
+int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream) {
+    if (!src || !dst) return CLUSTEN_ERR_NULL_POINTER;
+    if (bytes == 0 || bytes % 16 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(src) || !aligned16(dst)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_copy(src, dst, bytes, as_stream(stream));
+}
+
+}  // extern "C"

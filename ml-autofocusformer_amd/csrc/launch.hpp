@@ -1,0 +1,49 @@
+// Internal launch functions behind the C ABI.  Each one validates nothing: the extern "C" layer
+// has already checked pointers, sizes and strides.  All return a clusten_status.
+#pragma once
+
+#include "common.hpp"
+
+namespace clusten {
+
+// out[b,h,i,j] = sum_c a[b,h,i,c] * rows[b,h,idx[b,i,j],c]      (QK forward; AV's d_attn)
+//   a, rows : strided (B,H,N,C);  out : contiguous (B,H,N,M)
+int launch_gather_dot(const void* a, clusten_strides a_strides, const void* rows, clusten_strides rows_strides,
+                      const int64_t* idx, void* out, clusten_attn_shape s, int dtype, hipStream_t stream);
+
+// out[b,h,i,c] = sum_j p[b,h,i,j] * rows[b,h,idx[b,i,j],c]      (AV forward; QK's d_query)
+//   p : contiguous (B,H,N,M);  rows, out : strided (B,H,N,C)
+int launch_gather_sum(const void* p, const void* rows, clusten_strides rows_strides, const int64_t* idx, void* out,
+                      clusten_strides out_strides, clusten_attn_shape s, int dtype, hipStream_t stream);
+
+// out[b,h,idx[b,i,j],c] += p[b,h,i,j] * x[b,h,i,c]               (QK's d_key; AV's d_value)
+//   p : contiguous (B,H,N,M);  x : strided (B,H,N,C);  out : contiguous (B,H,N,C), zeroed here.
+//   For F16/BF16 the sum is built in fp32 in `workspace` and rounded once.
+size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype);
+int launch_scatter_rows(const void* p, const void* x, clusten_strides x_strides, const int64_t* idx, void* out,
+                        void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream);
+
+// out[b,i,ic,c] = sum_j w[b,i,j,ic] * feat[b,idx[b,i,j],c]      (WF forward)
+int launch_wf_forward(const void* w, const void* feat, const int64_t* idx, void* out, clusten_wf_shape s, int dtype,
+                      hipStream_t stream);
+
+// d_w[b,i,j,ic] = sum_c feat[b,idx[b,i,j],c] * d_out[b,i,ic,c]  (WF backward, weights)
+int launch_wf_dweights(const void* d_out, const void* feat, const int64_t* idx, void* d_w, clusten_wf_shape s,
+                       int dtype, hipStream_t stream);
+
+// d_feat[b,idx[b,i,j],c] += sum_ic d_out[b,i,ic,c] * w[b,i,j,ic]  (WF backward, features; zeroed here)
+size_t wf_dfeat_workspace_bytes(clusten_wf_shape s, int dtype);
+int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* d_feat, void* workspace,
+                    clusten_wf_shape s, int dtype, hipStream_t stream);
+
+// dst[0:bytes) = src[0:bytes), 16 bytes per lane per step.
+int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+
+// Fill `count` fp32 / fp64 words with zero (a kernel, so that callers may capture it in a HIP graph).
+int launch_zero_f32(float* dst, size_t count, hipStream_t stream);
+int launch_zero_f64(double* dst, size_t count, hipStream_t stream);
+
+// dst[i] = round(src[i]) for i < count, T in {F16, BF16}.
+int launch_round_from_f32(const float* src, void* dst, size_t count, int dtype, hipStream_t stream);
+
+}  // namespace clusten

@@ -1,0 +1,203 @@
+// scatter_rows: out[b,h,idx[b,i,j],c] += p[b,h,i,j] * x[b,h,i,c]
+//
+// This is the d_key half of the CLUSTEN QK backward (p = d_attn, x = query; reference kernel
+// clusten/src/clustenqk_cuda_kernel.cu:91-132, the fastAtomicAdd line) and the d_value kernel of
+// the AV backward (p = attn, x = d_feat; clusten/src/clustenav_cuda_kernel.cu:93-127).
+//
+// Work decomposition: as in gather_sum — one wave per tile of 8 consecutive tokens, lanes are 64
+// consecutive (head, channel) pairs, the p-rows are read through DPP row broadcasts.
+//
+//   shared-list path — all tokens of the tile carry the same list: the 8 products that go to one
+//     destination row are summed in registers and leave the wave as ONE fp32 atomic per (slot,
+//     channel): 8x fewer atomics than one per product, and each wave-wide atomic instruction adds
+//     to whole contiguous rows.
+//   per-token path — one atomic per product, for tiles whose lists differ.
+//
+// The destination is accumulated in fp32: directly in `out` for fp32, in a caller-provided fp32
+// workspace that is rounded once at the end for fp16/bf16.  fp64, head dims other than 16/32/64
+// and list lengths that are not a multiple of 4 take the element-per-thread kernel.
+// The order in which atomics from different waves arrive is not fixed, so the last bits of the
+// result can differ from run to run (as they do in the reference).
+#pragma once
+
+#include "dpp.hpp"
+#include "launch.hpp"
+
+namespace clusten {
+
+template <typename T, int C, int Q, bool GUARD>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void scatter_rows_tile_kernel(
+    const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out, int H,
+    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles) {
+    constexpr int HPW = kWave / C;
+    constexpr int SLOTS = 16 * Q;
+    static_assert(C == 16 || C == 32 || C == 64, "a row of 16 lanes must stay inside one head");
+    static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
+    typedef typename Quad<T>::raw QuadRaw;
+
+    const int tile = xcd_tile(blockIdx.x, total_tiles);
+    if (tile < 0) return;
+    const int b = tile / tiles_per_batch;
+    const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
+    const int nt = min(kTileTokens, N - i0);
+    const int lane = threadIdx.x;
+    const int c = lane % C;
+    const int rl = lane & 15;
+
+    const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
+    float* out_b = out + (int64_t)b * H * N * C;
+
+    for (int h0 = 0; h0 < H; h0 += HPW) {
+        const int h_raw = h0 + lane / C;
+        const bool head_ok = h_raw < H;
+        const int h = min(h_raw, H - 1);
+        const int lane_off = h * N * C + c;  // out is contiguous (B,H,N,C)
+        const T* p_head = p + (((int64_t)b * H + h) * N + i0) * M;
+        const T* x_lane = x + (int64_t)b * xs.b + (int64_t)h * xs.h + (int64_t)i0 * xs.n + c;
+
+        // x-rows of the tile; tokens past the end of a partial tile contribute nothing
+        float xv[kTileTokens];
+#pragma unroll
+        for (int t = 0; t < kTileTokens; ++t) {
+            const float v = to_acc(x_lane[(int64_t)min(t, nt - 1) * xs.n]);
+            xv[t] = (t < nt) ? v : 0.f;
+        }
+
+        for (int j0 = 0; j0 < M; j0 += kWave) {
+            const int mc = min(kWave, M - j0);
+            const int slot = min(lane, mc - 1);
+
+            int list[kTileTokens];
+            bool same = true;
+            {
+                int64_t wide[kTileTokens];
+#pragma unroll
+                for (int t = 0; t < kTileTokens; ++t) wide[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
+#pragma unroll
+                for (int t = 0; t < kTileTokens; ++t) {
+                    same = same && (wide[t] == wide[0]);
+                    list[t] = (int)wide[t];
+                }
+            }
+            const bool shared_list = __all(same ? 1 : 0) != 0;
+
+            float pv[kTileTokens][4];
+            {
+                const int q4 = min(4 * rl, mc - 4);
+                QuadRaw raw[kTileTokens];
+#pragma unroll
+                for (int t = 0; t < kTileTokens; ++t) {
+                    raw[t] = *reinterpret_cast<const QuadRaw*>(p_head + (int64_t)min(t, nt - 1) * M + j0 + q4);
+                }
+#pragma unroll
+                for (int t = 0; t < kTileTokens; ++t) {
+                    Quad<T>::unpack(raw[t], pv[t]);
+                    if (t >= nt) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) pv[t][e] = 0.f;
+                    }
+                }
+            }
+
+            if (shared_list) {
+                static_for<0, SLOTS>([&](auto ji) {
+                    constexpr int j = decltype(ji)::value;
+                    if (!GUARD || j < mc) {
+                        float sum = 0.f;
+                        fma4_rowlane<j / 4>(sum, pv[0][j % 4], pv[1][j % 4], pv[2][j % 4], pv[3][j % 4], xv[0], xv[1],
+                                            xv[2], xv[3]);
+                        fma4_rowlane<j / 4>(sum, pv[4][j % 4], pv[5][j % 4], pv[6][j % 4], pv[7][j % 4], xv[4], xv[5],
+                                            xv[6], xv[7]);
+                        const int row = __builtin_amdgcn_readlane(list[0], j);
+                        float* dst = out_b + (int64_t)row * C;
+                        if (head_ok) unsafeAtomicAdd(dst + lane_off, sum);
+                    }
+                });
+            } else {
+                static_for<0, kTileTokens>([&](auto ti) {
+                    constexpr int t = decltype(ti)::value;
+                    static_for<0, SLOTS>([&](auto ji) {
+                        constexpr int j = decltype(ji)::value;
+                        if (!GUARD || j < mc) {
+                            float prod = 0.f;
+                            fma1_rowlane<j / 4>(prod, pv[t][j % 4], xv[t]);
+                            const int row = __builtin_amdgcn_readlane(list[t], j);
+                            float* dst = out_b + (int64_t)row * C;
+                            if (head_ok && t < nt) unsafeAtomicAdd(dst + lane_off, prod);
+                        }
+                    });
+                });
+            }
+        }
+    }
+}
+
+// One thread per (b,h,i,c); loops over the list with one atomic per product.  Any dtype whose
+// accumulation type A has a hardware atomic add (float, double).
+template <typename T, typename A>
+__global__ __launch_bounds__(256) void scatter_rows_elem_kernel(const T* __restrict__ p, const T* __restrict__ x,
+                                                                const int64_t* __restrict__ idx, A* __restrict__ out,
+                                                                int B, int H, int N, int C, int M,
+                                                                clusten_strides xs) {
+    const int64_t total = (int64_t)B * H * N * C;
+    for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(o % C);
+        const int64_t q1 = o / C;
+        const int i = (int)(q1 % N);
+        const int64_t q2 = q1 / N;
+        const int h = (int)(q2 % H);
+        const int b = (int)(q2 / H);
+        const int64_t* list = idx + ((int64_t)b * N + i) * M;
+        const T* prow = p + (((int64_t)b * H + h) * N + i) * M;
+        const A xval = to_acc(x[b * xs.b + h * xs.h + i * xs.n + c]);
+        A* dst = out + ((int64_t)b * H + h) * N * C + c;
+        for (int j = 0; j < M; ++j) unsafeAtomicAdd(dst + list[j] * C, (A)to_acc(prow[j]) * xval);
+    }
+}
+
+template <typename T, int C, int Q, bool GUARD>
+int scatter_tile_q(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
+                   const clusten_attn_shape& s, hipStream_t stream) {
+    const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
+    const int total = s.B * tiles_per_batch;
+    hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+                       static_cast<const T*>(p), static_cast<const T*>(x), idx, out, s.H, s.N, s.M, xs,
+                       tiles_per_batch, total);
+    return launch_status();
+}
+
+template <typename T, int C>
+int scatter_tile(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
+                 const clusten_attn_shape& s, hipStream_t stream) {
+    if (s.M == 48) return scatter_tile_q<T, C, 3, false>(p, x, xs, idx, out, s, stream);
+    return scatter_tile_q<T, C, 4, true>(p, x, xs, idx, out, s, stream);
+}
+
+template <typename T, typename A>
+int scatter_elem(const void* p, const void* x, clusten_strides xs, const int64_t* idx, A* out,
+                 const clusten_attn_shape& s, hipStream_t stream) {
+    const int64_t total = (int64_t)s.B * s.H * s.N * s.C;
+    const int64_t want = (total + 255) / 256;
+    const int grid = (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
+    hipLaunchKernelGGL((scatter_rows_elem_kernel<T, A>), dim3(grid), dim3(256), 0, stream, static_cast<const T*>(p),
+                       static_cast<const T*>(x), idx, out, s.B, s.H, s.N, s.C, s.M, xs);
+    return launch_status();
+}
+
+// Accumulate into the zeroed fp32 buffer `acc32` (which is `out` itself for fp32 storage).
+template <typename T>
+int scatter_rows_typed(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* acc32,
+                       const clusten_attn_shape& s, hipStream_t stream) {
+    const bool quads_ok = s.M % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0;
+    if (quads_ok) {
+        switch (s.C) {
+            case 16: return scatter_tile<T, 16>(p, x, xs, idx, acc32, s, stream);
+            case 32: return scatter_tile<T, 32>(p, x, xs, idx, acc32, s, stream);
+            case 64: return scatter_tile<T, 64>(p, x, xs, idx, acc32, s, stream);
+            default: break;
+        }
+    }
+    return scatter_elem<T, float>(p, x, xs, idx, acc32, s, stream);
+}
+
+}  // namespace clusten

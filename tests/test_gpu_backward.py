@@ -1,0 +1,199 @@
+"""GPU parity of the backward kernels and of the drop-in autograd surface against autograd through
+the CPU gather oracle, with RANDOM upstream gradients (the reference's scripts use `.mean()`, whose
+constant gradient cannot detect a mis-indexed d_attn / d_feat).
+
+Bar: <= 1e-5 (fp32) for the gather-type gradients d_query, d_attn, d_weights; <= 1e-4 for the
+scatter-type gradients d_key, d_value, d_feat, whose fp32 atomics arrive in arbitrary order;
+<= 1e-2 for fp16/bf16.
+"""
+import pytest
+import torch
+
+import workloads as wl
+from clusten import CLUSTENAVFunction, CLUSTENQKFunction, CLUSTENWFFunction, _native
+from conftest import TOL, TOL_SCATTER_F32
+from oracle import clusten_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _scatter_tol(dtype):
+    return TOL_SCATTER_F32 if dtype == torch.float32 else TOL[dtype]
+
+
+def _ref(t):
+    return t.double() if t.dtype == torch.float64 else t.float()
+
+
+def _check_attn_backward(case, device, dtype):
+    g = torch.Generator().manual_seed(70)
+    q, k, v, idx = case.query.to(dtype), case.key.to(dtype), case.value.to(dtype), case.nbhd_idx
+    B, H, N, C = q.shape
+    M = idx.shape[-1]
+    d_attn = torch.randn(B, H, N, M, generator=g).to(dtype)
+    d_feat = torch.randn(B, H, N, C, generator=g).to(dtype)
+    p = torch.softmax(torch.randn(B, H, N, M, generator=g), dim=-1).to(dtype)
+
+    dq_ref, dk_ref = oracle.qk_gather_backward(_ref(d_attn), _ref(q), _ref(k), idx)
+    dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx.to(device))
+    assert dq.dtype == dtype and dk.dtype == dtype
+    assert oracle.rel_err(dq, dq_ref) <= TOL[dtype], "d_query %s" % case.name
+    assert oracle.rel_err(dk, dk_ref) <= _scatter_tol(dtype), "d_key %s" % case.name
+
+    da_ref, dv_ref = oracle.av_gather_backward(_ref(d_feat), _ref(p), _ref(v), idx)
+    da, dv = _native.av_backward(d_feat.to(device), p.to(device), v.to(device), idx.to(device))
+    assert oracle.rel_err(da, da_ref) <= TOL[dtype], "d_attn %s" % case.name
+    assert oracle.rel_err(dv, dv_ref) <= _scatter_tol(dtype), "d_value %s" % case.name
+
+
+def _check_wf_backward(case, device, dtype):
+    g = torch.Generator().manual_seed(71)
+    w, f, idx = case.weights.to(dtype), case.feat.to(dtype), case.nbhd_idx
+    B, Nout, M, IC = w.shape
+    C = f.shape[-1]
+    d_out = torch.randn(B, Nout, IC, C, generator=g).to(dtype)
+    dw_ref, df_ref = oracle.wf_gather_backward(_ref(d_out), _ref(w), _ref(f), idx)
+    dw, df = _native.wf_backward(d_out.to(device), w.to(device), f.to(device), idx.to(device))
+    assert dw.dtype == dtype and df.dtype == dtype and dw.shape == w.shape and df.shape == f.shape
+    assert oracle.rel_err(dw, dw_ref) <= TOL[dtype], "d_weights %s" % case.name
+    assert oracle.rel_err(df, df_ref) <= _scatter_tol(dtype), "d_feat %s" % case.name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_attn_backward_cluster_shared(device, dtype):
+    _check_attn_backward(wl.attn_case("shared", 72, B=2, H=2, N=200, C=32), device, dtype)
+
+
+@pytest.mark.parametrize("lists", ["random", "model"])
+def test_attn_backward_per_token_lists(device, lists):
+    _check_attn_backward(wl.attn_case(lists, 73, B=2, H=4, N=392, C=32, lists=lists), device, torch.float32)
+
+
+@pytest.mark.parametrize("c,h,m,n", [(16, 3, 48, 104), (64, 2, 48, 100), (24, 2, 48, 64), (32, 2, 20, 77),
+                                     (32, 5, 144, 160), (32, 2, 5, 40)])
+def test_attn_backward_shapes(device, c, h, m, n):
+    _check_attn_backward(wl.attn_case("shape", 74, B=2, H=h, N=n, C=c, M=m), device, torch.float32)
+
+
+def test_attn_backward_aff_base_384_shape_fp32(device):
+    # configuration 3's backward check at its real token count and head layout, batch reduced so the
+    # CPU autograd reference stays small
+    _check_attn_backward(wl.config3_attn(dtype=torch.float32, B=1), device, torch.float32)
+
+
+def test_scatter_integer_valued_data_is_bit_exact(device):
+    g = torch.Generator().manual_seed(75)
+    B, H, N, C, M = 2, 2, 136, 32, 48
+    q = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    k = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    d_attn = torch.randint(-4, 5, (B, H, N, M), generator=g).float()
+    for idx in (wl.windowed_cluster_lists(B, N, M, g), torch.randint(N, (B, N, M), generator=g)):
+        dq_ref, dk_ref = oracle.qk_gather_backward(d_attn, q, k, idx)
+        dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx.to(device))
+        assert torch.equal(dq.cpu(), dq_ref) and torch.equal(dk.cpu(), dk_ref)
+
+
+def test_scatter_conserves_mass_at_full_size(device):
+    """Configuration 3's backward shape at full size (B64 H4 N9216 C32, fp32): the sum of d_key over
+    destination rows equals the sum of all products whatever the indices are, and three batch
+    elements are compared with the oracle."""
+    case = wl.config3_attn(dtype=torch.float32, B=64)
+    d = case.to(device)
+    g = torch.Generator(device="cpu").manual_seed(76)
+    d_attn = torch.randn(64, 4, 9216, 48, generator=g).to(device)
+    dq, dk = _native.qk_backward(d_attn, d.query, d.key, d.nbhd_idx)
+    lhs = dk.double().sum(2)
+    rhs = (d_attn.double().sum(-1, keepdim=True) * d.query.double()).sum(2)
+    assert oracle.rel_err(lhs, rhs) <= 1e-6
+    for b in (0, 63):
+        dq_ref, dk_ref = oracle.qk_gather_backward(d_attn[b:b + 1].cpu(), case.query[b:b + 1], case.key[b:b + 1],
+                                                   case.nbhd_idx[b:b + 1])
+        assert oracle.rel_err(dq[b:b + 1], dq_ref) <= TOL[torch.float32]
+        assert oracle.rel_err(dk[b:b + 1], dk_ref) <= TOL_SCATTER_F32
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_wf_backward_dtypes(device, dtype):
+    _check_wf_backward(wl.wf_case("wf", 77, B=2, N=196, C=64, dtype=dtype), device, dtype)
+
+
+@pytest.mark.parametrize("c,ic,m", [(128, 4, 48), (256, 1, 48), (32, 4, 48), (96, 3, 20), (512, 4, 16)])
+def test_wf_backward_shapes(device, c, ic, m):
+    _check_wf_backward(wl.wf_case("wf", 78, B=2, N=196, C=c, IC=ic, M=m, Nout=40), device, torch.float32)
+
+
+def test_wf_backward_aff_base_384_shape(device):
+    _check_wf_backward(wl.config3_wf(dtype=torch.float32, B=1), device, torch.float32)
+
+
+# ---- the drop-in autograd surface ------------------------------------------------------------------------
+
+def test_autograd_functions_match_oracle_autograd(device):
+    """The three Functions used the way the model uses them: QK -> softmax -> AV, and WF, with a loss
+    that gives every output element its own random weight."""
+    g = torch.Generator().manual_seed(79)
+    case = wl.attn_case("auto", 79, B=2, H=2, N=200, C=32)
+    loss_w = torch.randn(2, 2, 200, 32, generator=g)
+
+    def run(qk, av, dev):
+        q = case.query.to(dev).requires_grad_(True)
+        k = case.key.to(dev).requires_grad_(True)
+        v = case.value.to(dev).requires_grad_(True)
+        idx = case.nbhd_idx.to(dev)
+        attn = torch.softmax(qk(q, k, idx), dim=-1)
+        feat = av(attn, v, idx)
+        (feat * loss_w.to(dev)).sum().backward()
+        return feat.detach(), q.grad, k.grad, v.grad
+
+    got = run(CLUSTENQKFunction.apply, CLUSTENAVFunction.apply, device)
+    ref = run(oracle.qk_gather, oracle.av_gather, "cpu")
+    for name, x, y, tol in zip(("feat", "d_query", "d_key", "d_value"), got, ref,
+                               (1e-5, 2e-5, TOL_SCATTER_F32, TOL_SCATTER_F32)):
+        assert oracle.rel_err(x, y) <= tol, name
+
+    wcase = wl.wf_case("auto_wf", 80, B=2, N=196, C=64)
+    wloss = torch.randn(2, 49, 4, 64, generator=g)
+
+    def run_wf(fn, dev):
+        w = wcase.weights.to(dev).requires_grad_(True)
+        f = wcase.feat.to(dev).requires_grad_(True)
+        out = fn(w, f, wcase.nbhd_idx.to(dev))
+        (out * wloss.to(dev)).sum().backward()
+        return out.detach(), w.grad, f.grad
+
+    got = run_wf(CLUSTENWFFunction.apply, device)
+    ref = run_wf(oracle.wf_gather, "cpu")
+    for name, x, y, tol in zip(("feat_new", "d_weights", "d_feat"), got, ref, (1e-5, 1e-5, TOL_SCATTER_F32)):
+        assert oracle.rel_err(x, y) <= tol, name
+
+
+def test_dtype_rules_of_the_reference_wrappers(device):
+    """Second operand is cast to the first operand's dtype; output has the first operand's dtype
+    (clusten/clusten.py:25-26,52-53,78-79) — the mixed dtypes fp16 autocast produces."""
+    case = wl.attn_case("mixed", 81, B=2, H=2, N=104, C=32).to(device)
+    attn16 = CLUSTENQKFunction.apply(case.query.half(), case.key, case.nbhd_idx)         # fp16 q, fp32 k
+    assert attn16.dtype == torch.float16
+    ref = oracle.qk_gather(case.query.half().float().cpu(), case.key.half().float().cpu(), case.nbhd_idx.cpu())
+    assert oracle.rel_err(attn16, ref) <= 1e-2
+    p = torch.softmax(attn16.float(), dim=-1)                                             # fp32 attn, fp16 v
+    feat = CLUSTENAVFunction.apply(p, case.value.half(), case.nbhd_idx)
+    assert feat.dtype == torch.float32
+    ref = oracle.av_gather(p.cpu(), case.value.half().float().cpu(), case.nbhd_idx.cpu())
+    assert oracle.rel_err(feat, ref) <= 1e-5
+    wcase = wl.wf_case("mixed_wf", 82, B=2, N=196, C=64).to(device)
+    out = CLUSTENWFFunction.apply(wcase.weights, wcase.feat.half(), wcase.nbhd_idx)      # fp32 w, fp16 feat
+    assert out.dtype == torch.float32
+    ref = oracle.wf_gather(wcase.weights.cpu(), wcase.feat.half().float().cpu(), wcase.nbhd_idx.cpu())
+    assert oracle.rel_err(out, ref) <= 1e-5
+
+
+def test_backward_returns_none_for_indices_and_accepts_noncontiguous_grads(device):
+    case = wl.attn_case("nc", 83, B=2, H=2, N=104, C=32).to(device)
+    q = case.query.clone().requires_grad_(True)
+    k = case.key.clone().requires_grad_(True)
+    attn = CLUSTENQKFunction.apply(q, k, case.nbhd_idx)
+    up = torch.randn(2, 2, 48, 104, device=device).transpose(2, 3)                        # non-contiguous upstream
+    attn.backward(up)
+    dq_ref, dk_ref = oracle.qk_gather_backward(up.cpu(), case.query.cpu(), case.key.cpu(), case.nbhd_idx.cpu())
+    assert oracle.rel_err(q.grad, dq_ref) <= 1e-5 and oracle.rel_err(k.grad, dk_ref) <= TOL_SCATTER_F32
+    assert not case.nbhd_idx.requires_grad

@@ -1,0 +1,248 @@
+"""GPU parity of the forward kernels against the CPU gather oracle, through the C ABI.
+
+Bar: bit-exact for index handling (integer-valued data), max|x-ref|/max|ref| <= 1e-5 for fp32,
+<= 1e-2 for fp16/bf16 (oracle evaluated in fp32 from the same rounded inputs), 1e-12 for fp64.
+"""
+import pytest
+import torch
+
+import workloads as wl
+from clusten import _native
+from conftest import TOL
+from oracle import clusten_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref_inputs(*tensors):
+    """The oracle sees the same rounded values, in fp32 (fp64 stays fp64)."""
+    return [t.double() if t.dtype == torch.float64 else t.float() for t in tensors]
+
+
+def _check_attn(case, device, dtype, check_av=True):
+    q, k, v, idx = case.query.to(dtype), case.key.to(dtype), case.value.to(dtype), case.nbhd_idx
+    qr, kr, vr = _ref_inputs(q, k, v)
+    attn_ref = oracle.qk_gather_chunked(qr, kr, idx)
+    attn = _native.qk_forward(q.to(device), k.to(device), idx.to(device))
+    assert attn.dtype == dtype and attn.shape == attn_ref.shape and attn.is_contiguous()
+    err = oracle.rel_err(attn, attn_ref)
+    assert err <= TOL[dtype], "QK %s %s rel err %.3g" % (case.name, dtype, err)
+    if check_av:
+        p = torch.softmax(attn_ref, dim=-1).to(dtype)
+        feat_ref = oracle.av_gather_chunked(_ref_inputs(p)[0], vr, idx)
+        feat = _native.av_forward(p.to(device), v.to(device), idx.to(device))
+        assert feat.dtype == dtype and feat.shape == feat_ref.shape and feat.is_contiguous()
+        err = oracle.rel_err(feat, feat_ref)
+        assert err <= TOL[dtype], "AV %s %s rel err %.3g" % (case.name, dtype, err)
+
+
+def _check_wf(case, device, dtype):
+    w, f, idx = case.weights.to(dtype), case.feat.to(dtype), case.nbhd_idx
+    wr, fr = _ref_inputs(w, f)
+    ref = oracle.wf_gather_chunked(wr, fr, idx)
+    out = _native.wf_forward(w.to(device), f.to(device), idx.to(device))
+    assert out.dtype == dtype and out.shape == ref.shape and out.is_contiguous()
+    err = oracle.rel_err(out, ref)
+    assert err <= TOL[dtype], "WF %s %s rel err %.3g" % (case.name, dtype, err)
+
+
+# ---- QK / AV -----------------------------------------------------------------------------------------
+
+def test_config0_fp32(device):
+    _check_attn(wl.config0(), device, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+def test_cluster_shared_lists_all_dtypes(device, dtype):
+    _check_attn(wl.attn_case("shared", 50, B=3, H=2, N=392, C=32), device, dtype)
+
+
+@pytest.mark.parametrize("lists", ["random", "model", "model_canonical"])
+def test_per_token_lists(device, lists):
+    # random lists hold duplicates, like the reference's own test scripts (torch.randint)
+    _check_attn(wl.attn_case(lists, 51, B=2, H=4, N=784 if lists != "random" else 196, C=32, lists=lists), device,
+                torch.float32)
+
+
+def test_reference_script_shape(device):
+    # clusten/test_qk_kernel.py:14-18 (b reduced from 256 so the CPU oracle stays fast)
+    _check_attn(wl.attn_case("refscript", 52, B=16, H=4, N=196, C=32, lists="random", scale_q=False), device,
+                torch.float32)
+
+
+@pytest.mark.parametrize("n", [49, 197, 8, 5])
+def test_partial_tiles(device, n):
+    m = min(48, n) if n >= 48 else 4
+    lists = "windowed" if n >= 48 else "random"
+    _check_attn(wl.attn_case("ragged", 53, B=2, H=2, N=n, C=32, M=m, lists=lists), device, torch.float32)
+
+
+@pytest.mark.parametrize("c", [16, 64, 24, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_head_dims(device, c, dtype):
+    # 16/32/64 take the tile kernels, anything else the element kernels
+    _check_attn(wl.attn_case("c%d" % c, 54, B=2, H=3, N=200, C=c), device, dtype)
+
+
+@pytest.mark.parametrize("m", [4, 16, 20, 32, 64, 144, 5])
+def test_list_lengths(device, m):
+    # 48 is the unguarded kernel; others are range-checked; 144 (the 384x384 models) spans three chunks;
+    # 5 is not a multiple of 4 (element kernel for AV)
+    _check_attn(wl.attn_case("m%d" % m, 55, B=2, H=2, N=320, C=32, M=m), device, torch.float32)
+
+
+@pytest.mark.parametrize("h", [1, 3, 5, 16])
+def test_head_counts(device, h):
+    _check_attn(wl.attn_case("h%d" % h, 56, B=2, H=h, N=104, C=32), device, torch.float32)
+
+
+def test_head_dim_16_with_odd_head_count(device):
+    _check_attn(wl.attn_case("c16h3", 57, B=2, H=3, N=104, C=16), device, torch.float32)
+
+
+def test_integer_valued_data_is_bit_exact(device):
+    # products and partial sums of small integers are exact in fp32, so any summation order gives the
+    # same bits: a wrong index, offset or stride cannot hide inside a tolerance
+    g = torch.Generator().manual_seed(58)
+    B, H, N, C, M = 3, 4, 136, 32, 48
+    q = torch.randint(-8, 9, (B, H, N, C), generator=g).float()
+    k = torch.randint(-8, 9, (B, H, N, C), generator=g).float()
+    v = torch.randint(-8, 9, (B, H, N, C), generator=g).float()
+    p = torch.randint(-4, 5, (B, H, N, M), generator=g).float()
+    for idx in (wl.windowed_cluster_lists(B, N, M, g), torch.randint(N, (B, N, M), generator=g)):
+        attn = _native.qk_forward(q.to(device), k.to(device), idx.to(device))
+        assert torch.equal(attn.cpu(), oracle.qk_gather(q, k, idx))
+        feat = _native.av_forward(p.to(device), v.to(device), idx.to(device))
+        assert torch.equal(feat.cpu(), oracle.av_gather(p, v, idx))
+
+
+def test_strided_views_are_read_in_place(device):
+    # the model hands over permuted views of (b,n,h,c) / (b,n,h,2,c) storage (aff_transformer.py:117-119)
+    g = torch.Generator().manual_seed(59)
+    B, H, N, C, M = 2, 4, 200, 32, 48
+    q_store = torch.randn(B, N, H, C, generator=g)
+    kv_store = torch.randn(B, N, H, 2, C, generator=g)
+    idx = wl.windowed_cluster_lists(B, N, M, g)
+    qd, kvd = q_store.to(device), kv_store.to(device)
+    q = qd.permute(0, 2, 1, 3)
+    kv = kvd.permute(3, 0, 2, 1, 4)
+    key, val = kv[0], kv[1]
+    assert not q.is_contiguous() and not key.is_contiguous()
+    attn = _native.qk_forward(q, key, idx.to(device))
+    attn_ref = oracle.qk_gather(q.cpu(), key.cpu(), idx)
+    assert oracle.rel_err(attn, attn_ref) <= TOL[torch.float32]
+    p = torch.softmax(attn_ref, dim=-1)
+    feat = _native.av_forward(p.to(device), val, idx.to(device))
+    assert oracle.rel_err(feat, oracle.av_gather(p, val.cpu(), idx)) <= TOL[torch.float32]
+    # token-major output: same values, storage laid out (b,n,h,c)
+    feat_tm = _native.av_forward(p.to(device), val, idx.to(device), token_major=True)
+    assert feat_tm.shape == feat.shape and feat_tm.permute(0, 2, 1, 3).is_contiguous()
+    assert torch.equal(feat_tm, feat)
+    # a transposed channel axis cannot be read in place and is copied
+    qt = torch.randn(B, H, C, N, generator=g).to(device).transpose(2, 3)
+    attn_t = _native.qk_forward(qt, key, idx.to(device))
+    assert oracle.rel_err(attn_t, oracle.qk_gather(qt.cpu(), key.cpu(), idx)) <= TOL[torch.float32]
+
+
+def test_unaligned_rows_take_the_element_kernels(device):
+    g = torch.Generator().manual_seed(60)
+    B, H, N, C, M = 2, 2, 64, 32, 48
+    store = torch.randn(B, H, N, C + 1, generator=g)          # row pitch 33 floats: rows are not 16-byte aligned
+    idx = wl.windowed_cluster_lists(B, N, M, g)
+    k = store.to(device)[..., 1:]
+    q = torch.randn(B, H, N, C, generator=g)
+    attn = _native.qk_forward(q.to(device), k, idx.to(device))
+    assert oracle.rel_err(attn, oracle.qk_gather(q, store[..., 1:], idx)) <= TOL[torch.float32]
+
+
+def test_aff_mini_stage1_shape_fp32_fp16(device):
+    # configuration 1 at a batch the CPU oracle handles in seconds
+    for dtype in (torch.float32, torch.float16):
+        _check_attn(wl.config1(dtype=dtype, B=4), device, dtype)
+
+
+@pytest.mark.parametrize("stage", [1, 2, 3, 4])
+def test_aff_tiny_stage_shapes(device, stage):
+    # configuration 2 (all four stages) at batch 4
+    _check_attn(wl.config2_attn(stage, B=4), device, torch.float32)
+
+
+def test_aff_base_384_shape_bf16(device):
+    _check_attn(wl.config3_attn(B=2), device, torch.bfloat16)
+
+
+def test_full_size_stage1_batch_slices_and_linearity(device):
+    """Configuration 2 stage 1 at its full batch of 128: three batch elements against the oracle, and
+    two properties that hold for every element: out(2a) == 2*out(a) bit for bit (scaling by a power of
+    two commutes with every rounding), and the batch elements are independent of each other."""
+    case = wl.config2_attn(1, B=128)
+    d = case.to(device)
+    attn = _native.qk_forward(d.query, d.key, d.nbhd_idx)
+    for b in (0, 63, 127):
+        ref = oracle.qk_gather(case.query[b:b + 1], case.key[b:b + 1], case.nbhd_idx[b:b + 1])
+        assert oracle.rel_err(attn[b:b + 1], ref) <= TOL[torch.float32]
+    assert torch.equal(_native.qk_forward(2 * d.query, d.key, d.nbhd_idx), 2 * attn)
+    sub = _native.qk_forward(d.query[100:104], d.key[100:104], d.nbhd_idx[100:104])
+    assert torch.equal(sub, attn[100:104])
+    p = torch.softmax(attn, dim=-1)
+    feat = _native.av_forward(p, d.value, d.nbhd_idx)
+    for b in (0, 63, 127):
+        ref = oracle.av_gather(p[b:b + 1].cpu(), case.value[b:b + 1], case.nbhd_idx[b:b + 1])
+        assert oracle.rel_err(feat[b:b + 1], ref) <= TOL[torch.float32]
+    assert torch.equal(_native.av_forward(p, 2 * d.value, d.nbhd_idx), 2 * feat)
+    # softmax rows sum to one, so every output lies inside the range of the gathered values
+    assert feat.abs().max() <= d.value.abs().max()
+
+
+# ---- WF ----------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("stage", [1, 2, 3, 4])
+@pytest.mark.parametrize("ic", [4, 1])
+def test_wf_aff_tiny_stages(device, stage, ic):
+    _check_wf(wl.config2_wf(stage, IC=ic, B=4), device, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("c", [64, 128, 256, 512])
+def test_wf_dtypes_and_channel_counts(device, dtype, c):
+    _check_wf(wl.wf_case("wf", 61, B=2, N=196, C=c, dtype=dtype), device, dtype)
+
+
+@pytest.mark.parametrize("c,ic,m", [(32, 4, 48), (96, 4, 48), (64, 3, 48), (64, 2, 48), (64, 4, 16), (64, 4, 144),
+                                    (128, 1, 20), (64, 1, 5)])
+def test_wf_other_shapes(device, c, ic, m):
+    # (32,4,48) is the reference script's shape family (test_wf_kernel.py:14-19) and AFF-Mini stage 1
+    _check_wf(wl.wf_case("wf", 62, B=2, N=196, C=c, IC=ic, M=m, Nout=64), device, torch.float32)
+
+
+def test_wf_integer_valued_data_is_bit_exact(device):
+    g = torch.Generator().manual_seed(63)
+    B, N, Nout, C, M, IC = 2, 196, 49, 128, 48, 4
+    w = torch.randint(-4, 5, (B, Nout, M, IC), generator=g).float()
+    f = torch.randint(-8, 9, (B, N, C), generator=g).float()
+    idx = torch.randint(N, (B, Nout, M), generator=g)
+    out = _native.wf_forward(w.to(device), f.to(device), idx.to(device))
+    assert torch.equal(out.cpu(), oracle.wf_gather(w, f, idx))
+
+
+def test_wf_aff_base_384_shape_bf16(device):
+    _check_wf(wl.config3_wf(B=2), device, torch.bfloat16)
+
+
+def test_wf_full_size_stage1(device):
+    case = wl.config2_wf(1, IC=4, B=128)
+    d = case.to(device)
+    out = _native.wf_forward(d.weights, d.feat, d.nbhd_idx)
+    for b in (0, 77, 127):
+        ref = oracle.wf_gather(case.weights[b:b + 1], case.feat[b:b + 1], case.nbhd_idx[b:b + 1])
+        assert oracle.rel_err(out[b:b + 1], ref) <= TOL[torch.float32]
+    assert torch.equal(_native.wf_forward(d.weights, 2 * d.feat, d.nbhd_idx), 2 * out)
+    # rows of the weights are non-negative and sum to one: outputs are convex combinations
+    assert out.abs().max() <= d.feat.abs().max() * (1 + 1e-6)
+
+
+def test_copy_probe(device):
+    src = torch.randn(1 << 20, device=device)
+    dst = torch.zeros_like(src)
+    _native.copy_probe(src, dst)
+    assert torch.equal(src, dst)

@@ -1,0 +1,79 @@
+"""The synthetic input generators produce what the benchmark configurations describe."""
+import torch
+
+import workloads as wl
+
+
+def test_windowed_lists_are_cluster_shared_distinct_and_local():
+    gen = wl.generator(0)
+    B, N, M = 3, 1024, 48
+    idx = wl.windowed_cluster_lists(B, N, M, gen)
+    assert idx.shape == (B, N, M) and idx.dtype == torch.int64
+    assert idx.min() >= 0 and idx.max() < N
+    g = idx.reshape(B, N // 8, 8, M)
+    assert (g == g[:, :, :1]).all()                                    # the 8 tokens of a cluster share the list
+    first = g[:, :, 0]
+    assert (first.sort(dim=-1).values.diff(dim=-1) > 0).all()          # 48 distinct indices
+    centre = (torch.arange(N // 8) * 8 + 4).reshape(1, -1, 1)
+    assert ((first - centre).abs() <= 256).all()                       # inside the +-256 window
+    assert not (first[0] == first[1]).all()                            # drawn independently per batch element
+
+
+def test_windowed_lists_small_and_ragged_n():
+    gen = wl.generator(1)
+    for N in (49, 196, 197):
+        idx = wl.windowed_cluster_lists(2, N, 48, gen)
+        assert idx.shape == (2, N, 48) and idx.min() >= 0 and idx.max() < N
+        assert (idx[:, :8] == idx[:, :1]).all()
+        assert (idx[:, 0].sort(dim=-1).values.diff(dim=-1) > 0).all()
+
+
+def test_generators_are_deterministic():
+    a = wl.config0()
+    b = wl.config0()
+    assert torch.equal(a.query, b.query) and torch.equal(a.nbhd_idx, b.nbhd_idx)
+    assert a.query.shape == (2, 2, 1024, 32) and a.nbhd_idx.shape == (2, 1024, 48)
+
+
+def test_knn_lists_are_the_nearest_neighbours():
+    gen = wl.generator(2)
+    B, N, Nout, M = 2, 64, 16, 8
+    state = gen.get_state()
+    idx = wl.knn_lists(B, N, Nout, M, gen)
+    gen.set_state(state)
+    pos = torch.rand(B, N, 2, generator=gen)
+    perm = torch.rand(B, N, generator=gen).argsort(dim=1)[:, :Nout]
+    for b in range(B):
+        for i in range(Nout):
+            d = ((pos[b] - pos[b, perm[b, i]]) ** 2).sum(-1)
+            assert set(idx[b, i].tolist()) == set(d.argsort()[:M].tolist())
+            assert idx[b, i, 0] == perm[b, i]                          # a centre is its own nearest token
+
+
+def test_wf_case_shapes_and_normalised_weights():
+    c = wl.config2_wf(3, IC=4, B=2)
+    assert c.weights.shape == (2, 49, 48, 4) and c.feat.shape == (2, 196, 256) and c.nbhd_idx.shape == (2, 49, 48)
+    assert (c.weights >= 0).all()
+    torch.testing.assert_close(c.weights.sum(dim=2), torch.ones(2, 49, 4))
+
+
+def test_model_like_lists_are_six_aligned_runs_of_eight():
+    idx = wl.model_like_lists(2, 784, wl.generator(3))
+    assert idx.shape == (2, 784, 48)
+    runs = idx.reshape(2, 784, 6, 8)
+    assert (runs[..., 0] % 8 == 0).all()
+    assert (runs == runs[..., :1] + torch.arange(8)).all()
+    tiles = idx.reshape(2, 98, 8, 48)
+    assert not (tiles == tiles[:, :, :1]).all(dim=-1).all(dim=-1).any()   # nearest-first order differs per token
+    canon = wl.model_like_lists(2, 784, wl.generator(3), canonical=True)
+    assert torch.equal(canon.sort(dim=-1).values, idx.sort(dim=-1).values)   # same sets, other order
+    assert (canon.reshape(2, 784, 6, 8)[..., 0].diff(dim=-1) > 0).all()      # cluster ids ascending
+
+
+def test_algorithmic_bytes_match_the_published_table():
+    # AFF-Tiny stage 1, fp32: QK = AV = 513.8 MB, WF IC4 = 321.1 MB, IC1 = 186.3 MB
+    assert round(wl.attn_bytes(128, 2, 3136, 32, 48, 4) / 1e6, 1) == 513.8
+    assert round(wl.wf_bytes(128, 3136, 784, 64, 48, 4, 4) / 1e6, 1) == 321.1
+    assert round(wl.wf_bytes(128, 3136, 784, 64, 48, 1, 4) / 1e6, 1) == 186.3
+    assert round(wl.attn_bytes(64, 4, 9216, 32, 48, 2) / 1e6, 1) == 755.0
+    assert wl.attn_flops(128, 2, 3136, 32, 48) == 2 * 128 * 2 * 3136 * 48 * 32
