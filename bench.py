@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the CLUSTEN hot path on one MI355X.
+
+A step is one pass of the forward hot path over one batch of synthetic input at the AFF-Tiny
+stage-1 shape (BASELINE.json configs[2], stage 1: B128, H2, N3136, head dim 32, 48 neighbours,
+fp32; WF 3136 -> 784 tokens, 64 channels, 4 inner channels): one QK launch, one AV launch, one WF
+launch through the C ABI, inputs resident in HBM.  `value` is the algorithmic bytes of the three ops
+(every input read once, every output written once, int64 neighbour lists) divided by the time of a
+step.  The `roofline` object prices the slowest of the three kernels against the 8 TB/s HBM peak
+from per-launch HIP-event timings taken inside the timed region; `cpu_baseline` is the PyTorch
+gather oracle timed on the host cores on a batch slice of the same workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
+
+`--full` adds the other stages and configurations to the JSON line under "other_configs".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "ml-autofocusformer_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+
+def _time_kernels(fns, steps, warmup):
+    """Run the launch closures `fns` back to back for warmup + steps steps on the current stream.
+    Returns (ms per step over the timed region, [average ms per launch of each closure])."""
+    import torch
+
+    for _ in range(warmup):
+        for fn in fns:
+            fn()
+    torch.cuda.synchronize()
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(fns) + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        marks[s][0].record()
+        for i, fn in enumerate(fns):
+            fn()
+            marks[s][i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    region_ms = marks[0][0].elapsed_time(marks[-1][-1])
+    per = [sum(marks[s][i].elapsed_time(marks[s][i + 1]) for s in range(steps)) / steps for i in range(len(fns))]
+    return region_ms / steps, per, wall_ms / steps
+
+
+def _cpu_baseline(attn_case, wf_case, full_bytes, full_batch, slice_b=4, reps=3):
+    """The gather oracle on the host cores, on a batch slice of the same inputs."""
+    import torch
+    from oracle import clusten_oracle as oracle
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q, k, v, idx = (t[:slice_b] for t in (attn_case.query, attn_case.key, attn_case.value, attn_case.nbhd_idx))
+    w, f, widx = (t[:slice_b] for t in (wf_case.weights, wf_case.feat, wf_case.nbhd_idx))
+    attn = torch.softmax(oracle.qk_gather(q, k, idx), dim=-1)   # warm-up, and the AV input
+    oracle.av_gather(attn, v, idx)
+    oracle.wf_gather(w, f, widx)
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        oracle.qk_gather(q, k, idx)
+        oracle.av_gather(attn, v, idx)
+        oracle.wf_gather(w, f, widx)
+        best = min(best, time.perf_counter() - t0)
+    slice_bytes = full_bytes * slice_b / full_batch
+    return {
+        "value": round(slice_bytes / best / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "PyTorch gather oracle, QK+AV+WF forward on a batch slice of %d of %d (same tensors), best of %d "
+                  "passes, %.2f s per pass; a baseline, not the target" % (slice_b, full_batch, reps, best),
+    }
+
+
+def _copy_bandwidth(nbytes=1 << 30, reps=20):
+    import torch
+    from clusten import _native
+
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        _native.copy_probe(src, dst)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        _native.copy_probe(src, dst)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2 * nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+
+def _bench_attn(case, steps, warmup, dtype=None):
+    import torch
+    import workloads as wl
+    from clusten import _native
+
+    d = case.to("cuda")
+    q, k, v = d.query, d.key, d.value
+    attn = torch.softmax(_native.qk_forward(q, k, d.nbhd_idx).float(), dim=-1).to(q.dtype)
+    B, H, N, C = q.shape
+    M = d.nbhd_idx.shape[-1]
+    nbytes = wl.attn_bytes(B, H, N, C, M, q.element_size())
+    _, per, _ = _time_kernels([lambda: _native.qk_forward(q, k, d.nbhd_idx),
+                               lambda: _native.av_forward(attn, v, d.nbhd_idx)], steps, warmup)
+    return {"shape": "B%d H%d N%d C%d M%d %s" % (B, H, N, C, M, str(q.dtype).replace("torch.", "")),
+            "qk_us": round(per[0] * 1e3, 1), "qk_GBps": round(nbytes / per[0] / 1e6, 1),
+            "av_us": round(per[1] * 1e3, 1), "av_GBps": round(nbytes / per[1] / 1e6, 1), "bytes_each": nbytes}
+
+
+def _bench_wf(case, steps, warmup):
+    import workloads as wl
+    from clusten import _native
+
+    d = case.to("cuda")
+    B, Nout, M, IC = d.weights.shape
+    N, C = d.feat.shape[1], d.feat.shape[2]
+    nbytes = wl.wf_bytes(B, N, Nout, C, M, IC, d.feat.element_size())
+    _, per, _ = _time_kernels([lambda: _native.wf_forward(d.weights, d.feat, d.nbhd_idx)], steps, warmup)
+    return {"shape": "B%d N%d->%d C%d M%d IC%d %s" % (B, N, Nout, C, M, IC, str(d.feat.dtype).replace("torch.", "")),
+            "wf_us": round(per[0] * 1e3, 1), "wf_GBps": round(nbytes / per[0] / 1e6, 1), "bytes": nbytes}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--full", action="store_true", help="also time the other stages and configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the hot path shards trivially over the batch axis and "
+                 "needs no exchange); --gpus %d is not supported, use --gpus 1." % args.gpus)
+
+    import torch
+    import workloads as wl
+    from clusten import _native
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the CLUSTEN kernels have no CPU path.")
+    _native.load()
+    torch.cuda.set_device(0)
+
+    B = 128
+    acase = wl.config2_attn(1, B=B)
+    wcase = wl.config2_wf(1, IC=4, B=B)
+    da, dw = acase.to("cuda"), wcase.to("cuda")
+    q, k, v, idx = da.query, da.key, da.value, da.nbhd_idx
+    attn = torch.softmax(_native.qk_forward(q, k, idx), dim=-1)
+    H, N, C, M = q.shape[1], q.shape[2], q.shape[3], idx.shape[2]
+    qk_bytes = wl.attn_bytes(B, H, N, C, M, 4)
+    wf_bytes = wl.wf_bytes(B, wcase.feat.shape[1], wcase.weights.shape[1], wcase.feat.shape[2], M, 4, 4)
+    total_bytes = 2 * qk_bytes + wf_bytes
+
+    fns = [lambda: _native.qk_forward(q, k, idx),
+           lambda: _native.av_forward(attn, v, idx),
+           lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
+    torch.cuda.synchronize()
+    ms_per_step, per, wall_ms = _time_kernels(fns, args.steps, args.warmup)
+    torch.cuda.synchronize()
+
+    names = ("gather_dot_tile_kernel (QK)", "gather_sum_tile_kernel (AV)", "wf_forward_row_kernel (WF)")
+    kbytes = (qk_bytes, qk_bytes, wf_bytes)
+    kernels = [{"kernel": n, "avg_us": round(t * 1e3, 2), "algorithmic_bytes": nb,
+                "achieved_GBps": round(nb / t / 1e6, 1), "frac_of_hbm_peak": round(nb / t / 1e6 / HBM_PEAK_GBPS, 4)}
+               for n, t, nb in zip(names, per, kbytes)]
+    dom = max(range(3), key=lambda i: per[i])
+    value = total_bytes / ms_per_step / 1e6
+    out = {
+        "metric": "CLUSTEN QK+AV+WF forward, algorithmic GB/s (AFF-Tiny stage-1 shape)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2] stage 1: QK+AV+WF(IC=4) forward, B128 H2 N3136 C32 M48 fp32, "
+                               "WF 3136->784 C64; cluster-shared windowed lists (QK/AV), 48-nearest lists (WF)",
+                   "global_batch": B, "algorithmic_bytes_per_step": total_bytes},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": kernels[dom]["frac_of_hbm_peak"], "traffic": None, "kernel": names[dom]},
+        "kernels": kernels,
+        "host_wall_ms_per_step": round(wall_ms, 4),
+        "copy_probe_GBps": round(_copy_bandwidth(), 1),
+    }
+    if args.full:
+        other = {}
+        for s in (2, 3, 4):
+            other["cfg2_s%d_attn" % s] = _bench_attn(wl.config2_attn(s, B=B), args.steps, args.warmup)
+            other["cfg2_s%d_wf_ic4" % s] = _bench_wf(wl.config2_wf(s, IC=4, B=B), args.steps, args.warmup)
+        other["cfg2_s1_wf_ic1"] = _bench_wf(wl.config2_wf(1, IC=1, B=B), args.steps, args.warmup)
+        other["cfg1_fp32"] = _bench_attn(wl.config1(torch.float32), args.steps, args.warmup)
+        other["cfg1_fp16"] = _bench_attn(wl.config1(torch.float16), args.steps, args.warmup)
+        other["cfg3_bf16_attn"] = _bench_attn(wl.config3_attn(), args.steps, args.warmup)
+        other["cfg3_bf16_wf_ic4"] = _bench_wf(wl.config3_wf(), args.steps, args.warmup)
+        other["cfg2_s1_model_like_lists"] = _bench_attn(
+            wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
+        out["other_configs"] = other
+    if not args.no_cpu:
+        out["cpu_baseline"] = _cpu_baseline(acase, wcase, total_bytes, B)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
