@@ -137,6 +137,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--full", action="store_true", help="also time the other stages and configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=("qk", "av", "wf", "copy"), default=None,
+                    help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the hot path shards trivially over the batch axis and "
@@ -166,6 +168,18 @@ def main():
            lambda: _native.av_forward(attn, v, idx),
            lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
     torch.cuda.synchronize()
+    if args.only:
+        if args.only == "copy":  # a plain copy of known traffic, to calibrate a profiler's byte counters
+            src = torch.empty(qk_bytes // 8, dtype=torch.float32, device="cuda").normal_()
+            dst = torch.empty_like(src)
+            one, nbytes = (lambda: _native.copy_probe(src, dst)), 2 * src.numel() * 4
+        else:
+            i = ("qk", "av", "wf").index(args.only)
+            one, nbytes = fns[i], (qk_bytes, qk_bytes, wf_bytes)[i]
+        _, per, _ = _time_kernels([one], args.steps, args.warmup)
+        print(json.dumps({"only": args.only, "launches": args.steps + args.warmup, "avg_us": round(per[0] * 1e3, 2),
+                          "algorithmic_bytes": nbytes, "achieved_GBps": round(nbytes / per[0] / 1e6, 1)}), flush=True)
+        return
     ms_per_step, per, wall_ms = _time_kernels(fns, args.steps, args.warmup)
     torch.cuda.synchronize()
 

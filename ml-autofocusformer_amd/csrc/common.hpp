@@ -180,10 +180,26 @@ struct VecIO {
 template <typename T>
 using Quad = VecIO<T, 4>;
 
+// ---- addressing ---------------------------------------------------------------------------------
+
+// Pin a wave-uniform pointer in scalar registers and hide how it was computed, so that
+// `base + (uint32_t)lane_offset` is selected as the scalar-base + 32-bit-vector-offset addressing
+// mode (one VGPR per access instead of a 64-bit VGPR pair and a 64-bit add).
+template <typename P>
+__device__ __forceinline__ P* uniform_base(P* p) {
+    asm volatile("" : "+s"(p));
+    return p;
+}
+
 // ---- workgroup id -> tile ----------------------------------------------------------------------
 
-// Workgroup `wg` of `total` runs on XCD wg % 8.  Give XCD x the contiguous tile range
-// [x*per, (x+1)*per): returns the tile index, or -1 for the padding workgroups of the last XCDs.
+// One short-lived one-wave workgroup per tile: on this device many small workgroups stream from HBM
+// faster than few persistent ones (a plain copy loses 15-20 % of its bandwidth as a grid-stride loop).
+//
+// Workgroup `wg` of the grid runs on XCD wg % 8.  XCD x is given the contiguous tile range
+// [x*per, (x+1)*per), so the waves that run at the same time on one XCD work on neighbouring tiles
+// and the rows they gather are in that XCD's private L2.  Returns the tile index, or -1 for the
+// padding workgroups of the last XCDs.
 __device__ __forceinline__ int xcd_tile(int wg, int total) {
     const int per = (total + kXcds - 1) / kXcds;
     const int tile = (wg % kXcds) * per + wg / kXcds;
@@ -218,9 +234,10 @@ inline bool rows_aligned16(const void* p, const clusten_strides& s, size_t elem)
     return aligned16(p) && (s.b * elem) % 16 == 0 && (s.h * elem) % 16 == 0 && (s.n * elem) % 16 == 0;
 }
 
-// True when every element offset inside one batch element of a strided (B,H,N,C) operand fits an int.
+// True when every byte offset inside one batch element of a strided (B,H,N,C) operand with 8-byte
+// elements at most fits an int, so that kernels may use 32-bit offsets from a per-batch base.
 inline bool slice_fits_int32(const clusten_strides& s, int H, int N, int C) {
-    return (int64_t)(H - 1) * s.h + (int64_t)(N - 1) * s.n + C < ((int64_t)1 << 31);
+    return ((int64_t)(H - 1) * s.h + (int64_t)(N - 1) * s.n + C) * 8 < ((int64_t)1 << 31);
 }
 
 inline int check_attn_shape(const clusten_attn_shape& s) {

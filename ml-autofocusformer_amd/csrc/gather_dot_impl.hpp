@@ -6,17 +6,33 @@
 //
 // Work decomposition.  One wave owns a tile of 8 consecutive tokens of one batch element and
 // walks all heads, so the int64 neighbour lists of the tile are read from HBM exactly once.
-// Lane j of the wave owns neighbour slot j (slots are taken 64 at a time when M > 64).
+// Per head the tile is a small matrix product  D[slot][token] = G[slot][c] * A^T[c][token]  with
+// G the gathered rows, and it runs on the matrix cores as fp32 MFMA 16x16x4 blocks.
+//
+// Data path per head:
+//   1. gather: `global_load_lds_dwordx4` moves the rows from HBM/L2 straight into LDS, 16 bytes per
+//      lane, consecutive lanes on consecutive pieces of one row (row-coalesced: a wave access covers
+//      64/pieces-per-row whole rows).  No VGPRs are held while the data travels, so the bytes a CU
+//      keeps in flight are bounded by its LDS, not by its register file.  The 8 a-rows of the tile
+//      take the same path.
+//   2. operands: lane (r = lane % 16, kq = lane / 16) reads the quarter [kq*C/4, (kq+1)*C/4) of row r
+//      of every 16-slot block from LDS with 16-byte reads: the registers it fills are the MFMA A
+//      operands (channel e of the quarter is the k-index kq of MFMA step e), and the same quarter of
+//      a-row r % 8 gives the B operands.  The piece index is XOR-swizzled with the row number on
+//      the way in so that these reads are free of bank conflicts.
+//   3. the D block leaves lane (r, kq) with slots 4*kq..4*kq+3 of token r.  The output of one
+//      (tile, head) is a single contiguous chunk of 8*M elements, so the blocks are laid out
+//      row-major in LDS and leave with full-width 16-byte stores (lists of up to 64 slots).
+// One short-lived one-wave workgroup per tile; the latency of its dependent chain (lists, rows,
+// product, store) is hidden by the ~20 other waves resident on the CU.
 //
 //   shared-list path — all tokens of the tile carry the same list (true for every tile of a
-//     cluster-ordered token sequence whose cluster shares its neighbourhood).  The M gathered rows
-//     are fetched once per head with row-coalesced 16-byte accesses (consecutive lanes cover one
-//     row, a wave access covers 64/pieces-per-row whole rows), turned through LDS so that lane j
-//     ends up with row j in registers, and reused for the 8 tokens: 8 FMAs per gathered element.
-//     The a-rows are wave-uniform and come in through the scalar data path.
-//   per-token path — any other tile: lane j gathers its own row for every token.  Exact for
-//     arbitrary indices (duplicates, any order), only slower.
+//     cluster-ordered token sequence whose cluster shares its neighbourhood): one gather and one
+//     set of MFMAs per head serve the 8 tokens.
+//   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
+//     token's column is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
 //
+// Storage types narrower than fp32 are widened in registers; all products and sums are fp32.
 // Rows whose start is not 16-byte aligned, head dims other than 16/32/64 and fp64 take the
 // element-per-thread kernel at the bottom of the file.
 //
@@ -24,29 +40,63 @@
 // so that the translation units build in parallel, gather_dot.hip holds the dtype dispatch.
 #pragma once
 
-#include "dpp.hpp"
 #include "launch.hpp"
 
 namespace clusten {
 
+typedef float F32x4 __attribute__((ext_vector_type(4)));
+
+// s_waitcnt immediate (gfx9 encoding) that waits until at most `vm` vector-memory operations are
+// outstanding and leaves the LDS/scalar and export counters alone.
+constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// Geometry of the staging buffer in LDS: rows of RB bytes, filled 1 KiB (one wave access) at a time.
+//   [0, G_BYTES)            gathered rows of one head (16*Q rows); reused to turn the D blocks into
+//                           the row-major output chunk once the operands are in registers
+//   [A_BASE, +2*A_SLOT)     a-rows of two heads (slot h % 2)
 template <typename T, int C, int Q>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void gather_dot_tile_kernel(const T* __restrict__ a, const T* __restrict__ rows,
+struct Staging {
+    static constexpr int RB = C * (int)sizeof(T);               // bytes per row
+    static constexpr int PPR = RB / 16;                         // 16-byte pieces per row
+    static constexpr int RPI = kWave / PPR;                     // rows per wave access
+    static constexpr int NI_G = (16 * Q + RPI - 1) / RPI;       // accesses for the gathered rows of a chunk
+    static constexpr int NI_A = (kTileTokens + RPI - 1) / RPI;  // accesses for the tile's a-rows
+    static constexpr int OUT_BYTES = kTileTokens * 16 * Q * (int)sizeof(T);  // one (tile, head) output chunk
+    static constexpr int G_BYTES = NI_G * 1024 > OUT_BYTES ? NI_G * 1024 : (OUT_BYTES + 1023) / 1024 * 1024;
+    static constexpr int A_BASE = G_BYTES;
+    static constexpr int A_SLOT_BYTES = NI_A * 1024;
+    static constexpr int BYTES = G_BYTES + 2 * A_SLOT_BYTES;
+    static constexpr int EL = C / 4;                            // channels per lane (a quarter row)
+    static constexpr int QB = RB / 4;                           // bytes per lane
+    static constexpr int UNIT = QB < 16 ? QB : 16;              // bytes per LDS read
+    static constexpr int NU = QB / UNIT;                        // LDS reads per quarter row
+    static constexpr int VEC = UNIT / (int)sizeof(T);           // elements per LDS read
+    static_assert(RB >= 32 && kWave % PPR == 0, "row size");
+
+    // XOR swizzle of the piece index: rows r, r+1, ... of a block land in different bank groups
+    static __device__ __forceinline__ int swz(int row) { return ((row & 7) ^ ((row >> 3) & 1)) & (PPR - 1); }
+};
+
+#define CLUSTEN_LDS_DMA16(gptr, lptr)                                                         \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr), \
+                                     (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+// FAST = the list has at most 64 slots and a multiple of 4 of them: one chunk, and every access to
+// an out row is a whole aligned 16-byte group.  Otherwise lists go 64 slots at a time and the last
+// group of a row may be stored element by element.
+template <typename T, int C, int Q, bool FAST>
+__global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restrict__ a, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H, int N, int M,
                                                                 clusten_strides as, clusten_strides rs,
                                                                 int tiles_per_batch, int total_tiles) {
-    constexpr int EPP = PieceOf<T>::kElems;          // elements per 16-byte piece
-    constexpr int PPR = C / EPP;                     // pieces per row
-    constexpr int RPP = kWave / PPR;                 // rows covered by one wave-wide access
-    constexpr int PITCH = PPR + 1;                   // LDS row pitch in pieces: the pad keeps row-per-lane reads conflict free
-    constexpr int NPASS = (16 * Q + RPP - 1) / RPP;  // wave-wide accesses that cover the 16*Q slots of a chunk
-    constexpr int NA = kTileTokens * C / (16 * EPP); // pieces per lane that hold the tile's a-rows (each row of 16 lanes holds all of them)
-    static_assert(C % EPP == 0 && kWave % PPR == 0, "unsupported head dim");
-    static_assert((kTileTokens * C) % (16 * EPP) == 0, "the a-tile must fill whole 16-lane rows");
+    typedef Staging<T, C, Q> S;
+    typedef VecIO<T, S::VEC> RunIO;
+    typedef VecIO<T, 4> OutIO;
+    static_assert(C % 16 == 0, "a lane holds a quarter of a row in whole 4-element groups");
     static_assert(Q >= 1 && Q <= 4, "a chunk holds 16, 32, 48 or 64 neighbour slots");
 
-    extern __shared__ Piece lds_rows[];  // [kWave][PITCH] pieces, then kWave ints
-    int* lds_idx = reinterpret_cast<int*>(lds_rows + kWave * PITCH);
+    __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
 
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
@@ -54,137 +104,182 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
     const int lane = threadIdx.x;
+    const int r = lane & 15;   // MFMA row of the A operand / column of the B operand
+    const int kq = lane >> 4;  // MFMA k index; also the quarter of the row this lane holds
+    // gather side: in access i this lane moves one piece of staging row i*RPI + lane/PPR
+    const int g_sub = lane / S::PPR;
+    const int g_pos = lane % S::PPR;
 
-    const T* a_tile = a + (int64_t)b * as.b + (int64_t)i0 * as.n;
-    const T* rows_b = rows + (int64_t)b * rs.b;
-    T* out_tile = out + ((int64_t)b * H * N + i0) * M;
+    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b);
+    const char* a_tile = reinterpret_cast<const char*>(a + (int64_t)b * as.b + (int64_t)i0 * as.n);
+    char* out_tile = reinterpret_cast<char*>(out + ((int64_t)b * H * N + i0) * M);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
+    const uint32_t row_pitch = (uint32_t)rs.n * sizeof(T);
 
-    const int piece = lane % PPR;  // row-coalesced fetch: lane covers piece `piece` of row pass*RPP + sub
-    const int sub = lane / PPR;
-
-    // a-tile: flat element f = t*C + c of the tile's 8 a-rows sits in piece f / (16*EPP) of row-lane
-    // (f / EPP) % 16, element f % EPP.  Tokens past the end of a partial tile repeat its last token.
-    int a_off[NA];  // element offsets inside one batch element fit 32 bits (checked on the host)
+    // a-rows of head h -> slot h % 2.  Staging row = token; tokens past the end of a partial tile
+    // repeat its last token.  They do not depend on the lists, so the first two heads are requested
+    // before the lists are even read.
+    uint32_t a_off[S::NI_A];
 #pragma unroll
-    for (int m = 0; m < NA; ++m) {
-        const int f0 = (16 * m + (lane & 15)) * EPP;
-        a_off[m] = min(f0 / C, nt - 1) * (int)as.n + f0 % C;
+    for (int i = 0; i < S::NI_A; ++i) {
+        const int srow = i * S::RPI + g_sub;
+        a_off[i] = (uint32_t)min(srow, nt - 1) * (uint32_t)as.n * sizeof(T) + (uint32_t)((g_pos ^ S::swz(srow)) * 16);
     }
-    auto load_a = [&](const T* a_head, Piece (&dst)[NA]) {
+    auto fetch_a = [&](int h) {
+        const char* a_bh = a_tile + (int64_t)h * as.h * sizeof(T);
 #pragma unroll
-        for (int m = 0; m < NA; ++m) dst[m] = *reinterpret_cast<const Piece*>(a_head + a_off[m]);
-    };
-    // acc[t] += sum_c a[t][c] * kr[c], the a operand read across the row of 16 lanes
-    auto dot_token = [&](auto ti, const Piece (&av)[NA], const float (&kr)[C], float& acc) {
-        constexpr int t = decltype(ti)::value;
-        float aflat[NA * EPP];
-#pragma unroll
-        for (int m = 0; m < NA; ++m) {
-#pragma unroll
-            for (int e = 0; e < EPP; ++e) aflat[m * EPP + e] = piece_get<T>(av[m], e);
+        for (int i = 0; i < S::NI_A; ++i) {
+            CLUSTEN_LDS_DMA16(a_bh + a_off[i], stage + S::A_BASE + (h & 1) * S::A_SLOT_BYTES + i * 1024);
         }
-        static_for<0, C / 4>([&](auto gi) {
-            constexpr int f = t * C + 4 * decltype(gi)::value;
-            constexpr int m = f / (16 * EPP);
-            constexpr int n = (f / EPP) % 16;
-            constexpr int e = f % EPP;
-            constexpr int c = 4 * decltype(gi)::value;
-            fma4_rowlane<n>(acc, aflat[m * EPP + e], aflat[m * EPP + e + 1], aflat[m * EPP + e + 2],
-                            aflat[m * EPP + e + 3], kr[c], kr[c + 1], kr[c + 2], kr[c + 3]);
-        });
     };
+    fetch_a(0);
+    if (H > 1) fetch_a(1);
 
-    for (int j0 = 0; j0 < M; j0 += kWave) {
+    // operand side: byte offsets of this lane's quarter rows inside the staging buffer
+    int lds_g[S::NU];  // row r of slot block 0; block blk is 16 rows further
+    int lds_a[S::NU];
+#pragma unroll
+    for (int u = 0; u < S::NU; ++u) {
+        const int byte = kq * S::QB + u * S::UNIT;  // offset inside the row
+        const int piece = byte / 16, within = byte % 16;
+        lds_g[u] = r * S::RB + ((piece ^ S::swz(r)) * 16) + within;  // swz(16*blk + r) == swz(r)
+        lds_a[u] = S::A_BASE + (r & 7) * S::RB + ((piece ^ S::swz(r & 7)) * 16) + within;
+    }
+
+    const bool vec_store = FAST || (M & 3) == 0;  // 16-byte accesses to out rows need aligned rows
+
+    for (int j0 = 0; j0 < (FAST ? 1 : M); j0 += kWave) {
         const int mc = min(kWave, M - j0);
-        const bool active = lane < mc;
-        const int slot = min(lane, mc - 1);  // lanes past the list repeat its last slot; only their store is masked
+        const int slot = min(lane, mc - 1);  // lanes past the list repeat its last slot
 
-        int64_t list[kTileTokens];
-#pragma unroll
-        for (int t = 0; t < kTileTokens; ++t) {
-            list[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
-        }
+        // the tile's lists: are they all the same?  (only the first is kept in registers)
+        int list0;
         bool same = true;
+        {
+            int64_t wide[kTileTokens];
 #pragma unroll
-        for (int t = 1; t < kTileTokens; ++t) same = same && (list[t] == list[0]);
+            for (int t = 0; t < kTileTokens; ++t) wide[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
+#pragma unroll
+            for (int t = 1; t < kTileTokens; ++t) same = same && (wide[t] == wide[0]);
+            list0 = (int)wide[0];
+        }
         const bool shared_list = __all(same ? 1 : 0) != 0;
 
-        if (shared_list) {
-            __syncthreads();  // the previous chunk's readers are done with the LDS
-            lds_idx[lane] = (int)list[0];
-            __syncthreads();
-            int src_off[NPASS];  // element offset of this lane's piece inside one (b,h) slice, per pass
+        // the list entry of staging row i*RPI + g_sub lives in the lane of that slot
+        int src_lane[S::NI_G];
 #pragma unroll
-            for (int pass = 0; pass < NPASS; ++pass) {
-                const int r = min(pass * RPP + sub, mc - 1);
-                src_off[pass] = lds_idx[r] * (int)rs.n + piece * EPP;
+        for (int i = 0; i < S::NI_G; ++i) src_lane[i] = min(i * S::RPI + g_sub, mc - 1);
+
+        // shared list: one pass that serves all tokens; otherwise one pass per token that keeps its column
+        const int passes = shared_list ? 1 : nt;
+        for (int pass = 0; pass < passes; ++pass) {
+            const int tok_lo = shared_list ? 0 : pass;
+            const int tok_hi = shared_list ? nt : pass + 1;
+            // this pass's list: token `pass` of the tile (re-read from L2 for the per-token passes)
+            const int mine = pass == 0 ? list0 : (int)idx_tile[(int64_t)pass * M + j0 + slot];
+            uint32_t g_off[S::NI_G];
+#pragma unroll
+            for (int i = 0; i < S::NI_G; ++i) {
+                const int srow = i * S::RPI + g_sub;
+                g_off[i] = (uint32_t)__shfl(mine, src_lane[i]) * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16);
             }
-            Piece stage[NPASS];
-            Piece a_stage[NA];
-#pragma unroll
-            for (int pass = 0; pass < NPASS; ++pass) {
-                stage[pass] = *reinterpret_cast<const Piece*>(rows_b + src_off[pass]);
-            }
-            load_a(a_tile, a_stage);
-            for (int h = 0; h < H; ++h) {
-#pragma unroll
-                for (int pass = 0; pass < NPASS; ++pass) {
-                    lds_rows[(pass * RPP + sub) * PITCH + piece] = stage[pass];
-                }
-                Piece a_cur[NA];
-#pragma unroll
-                for (int m = 0; m < NA; ++m) a_cur[m] = a_stage[m];
+            if (pass > 0 || j0 > 0) {  // the a-row slots hold the last heads of the previous pass
                 __syncthreads();
-                if (h + 1 < H) {  // the next head's rows travel while this head is computed
-                    const T* rows_next = rows_b + (int64_t)(h + 1) * rs.h;
-#pragma unroll
-                    for (int pass = 0; pass < NPASS; ++pass) {
-                        stage[pass] = *reinterpret_cast<const Piece*>(rows_next + src_off[pass]);
-                    }
-                    load_a(a_tile + (int64_t)(h + 1) * as.h, a_stage);
-                }
-                float kr[C];
-#pragma unroll
-                for (int p = 0; p < PPR; ++p) {
-                    const Piece pc = lds_rows[lane * PITCH + p];
-#pragma unroll
-                    for (int e = 0; e < EPP; ++e) kr[p * EPP + e] = piece_get<T>(pc, e);
-                }
-                __syncthreads();  // rows are in registers; the LDS may be refilled for the next head
-                float acc[kTileTokens];
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) acc[t] = 0.f;
-                static_for<0, kTileTokens>([&](auto ti) { dot_token(ti, a_cur, kr, acc[decltype(ti)::value]); });
-                T* out_head = out_tile + (int64_t)h * N * M + j0 + lane;
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) {
-                    if (active && t < nt) out_head[(int64_t)t * M] = from_acc<T>(acc[t]);
-                }
+                fetch_a(0);
+                if (H > 1) fetch_a(1);
             }
-        } else {
+
             for (int h = 0; h < H; ++h) {
-                const T* rows_bh = rows_b + (int64_t)h * rs.h;
-                Piece a_cur[NA];
-                load_a(a_tile + (int64_t)h * as.h, a_cur);
-                float acc[kTileTokens];
-                static_for<0, kTileTokens>([&](auto ti) {
-                    constexpr int t = decltype(ti)::value;
-                    const Piece* src = reinterpret_cast<const Piece*>(rows_bh + list[t] * rs.n);
-                    float kr[C];
+                // gather: rows of head h -> LDS (and the a-rows of head h when they were not prefetched)
+                const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
 #pragma unroll
-                    for (int p = 0; p < PPR; ++p) {
-                        const Piece pc = src[p];
+                for (int i = 0; i < S::NI_G; ++i) CLUSTEN_LDS_DMA16(rows_bh + g_off[i], stage + i * 1024);
+                if (h >= 2) fetch_a(h);
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                __syncthreads();
+
+                // operands: LDS -> registers
+                typename RunIO::raw g_raw[Q][S::NU];
+                typename RunIO::raw a_raw[S::NU];
 #pragma unroll
-                        for (int e = 0; e < EPP; ++e) kr[p * EPP + e] = piece_get<T>(pc, e);
+                for (int u = 0; u < S::NU; ++u) {
+#pragma unroll
+                    for (int blk = 0; blk < Q; ++blk) {
+                        g_raw[blk][u] =
+                            *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] + blk * 16 * S::RB);
                     }
-                    acc[t] = 0.f;
-                    dot_token(ti, a_cur, kr, acc[t]);
-                });
-                T* out_head = out_tile + (int64_t)h * N * M + j0 + lane;
+                    a_raw[u] =
+                        *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] + (h & 1) * S::A_SLOT_BYTES);
+                }
+                __syncthreads();  // operands are in registers: the staging buffer may be reused
+
+                float bop[S::EL];
 #pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) {
-                    if (active && t < nt) out_head[(int64_t)t * M] = from_acc<T>(acc[t]);
+                for (int u = 0; u < S::NU; ++u) {
+                    float x[S::VEC];
+                    RunIO::unpack(a_raw[u], x);
+#pragma unroll
+                    for (int e = 0; e < S::VEC; ++e) bop[u * S::VEC + e] = x[e];
+                }
+                F32x4 d[Q];
+#pragma unroll
+                for (int blk = 0; blk < Q; ++blk) {
+                    d[blk] = F32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int u = 0; u < S::NU; ++u) {
+                        float x[S::VEC];
+                        RunIO::unpack(g_raw[blk][u], x);
+#pragma unroll
+                        for (int e = 0; e < S::VEC; ++e) {
+                            d[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], bop[u * S::VEC + e], d[blk], 0, 0, 0);
+                        }
+                    }
+                }
+
+                // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of token r
+                char* out_h = out_tile + (int64_t)h * N * M * sizeof(T);
+                if (FAST && shared_list) {
+                    // the (tile, head) output is one contiguous chunk of nt*M elements: turn the D blocks
+                    // into it through LDS and write it with full-width 16-byte stores
+                    if (r < nt) {
+#pragma unroll
+                        for (int blk = 0; blk < Q; ++blk) {
+                            const int s0 = 16 * blk + 4 * kq;
+                            float v[4] = {d[blk][0], d[blk][1], d[blk][2], d[blk][3]};
+                            if (s0 < mc) {
+                                *reinterpret_cast<typename OutIO::raw*>(stage + (r * M + s0) * (int)sizeof(T)) =
+                                    OutIO::pack(v);
+                            }
+                        }
+                    }
+                    __syncthreads();
+                    const int chunk_bytes = nt * M * (int)sizeof(T);
+                    Piece o[(S::OUT_BYTES + 1023) / 1024];
+#pragma unroll
+                    for (int i = 0; i < (S::OUT_BYTES + 1023) / 1024; ++i) {
+                        o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
+                    }
+                    __syncthreads();  // the chunk is in registers: the next head's gather may overwrite it
+#pragma unroll
+                    for (int i = 0; i < (S::OUT_BYTES + 1023) / 1024; ++i) {
+                        const int off = i * 1024 + lane * 16;
+                        if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
+                    }
+                } else if (r >= tok_lo && r < tok_hi) {
+                    T* out_row = reinterpret_cast<T*>(out_h) + r * M + j0;
+#pragma unroll
+                    for (int blk = 0; blk < Q; ++blk) {
+                        const int s0 = 16 * blk + 4 * kq;
+                        float v[4] = {d[blk][0], d[blk][1], d[blk][2], d[blk][3]};
+                        if (FAST || vec_store) {
+                            if (s0 < mc) *reinterpret_cast<typename OutIO::raw*>(out_row + s0) = OutIO::pack(v);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                if (s0 + e < mc) out_row[s0 + e] = from_acc<T>(v[e]);
+                            }
+                        }
+                    }
                 }
             }
         }
@@ -214,25 +309,25 @@ __global__ __launch_bounds__(256) void gather_dot_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q>
+template <typename T, int C, int Q, bool FAST>
 int launch_tile_q(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
                   void* out, const clusten_attn_shape& s, hipStream_t stream) {
-    constexpr int PPR = C / PieceOf<T>::kElems;
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    const size_t lds = (size_t)kWave * (PPR + 1) * sizeof(Piece) + kWave * sizeof(int);
-    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q>), dim3(xcd_grid(total)), dim3(kWave), lds, stream,
+    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q, FAST>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
                        static_cast<const T*>(a), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, as, rs, tiles_per_batch, total);
     return launch_status();
 }
 
-// Lists of up to 48 slots (the model's neighbourhood size) are one chunk of 48; anything longer goes 64 slots at a time.
+// Lists of up to 48 slots (the neighbourhood size of every 224x224 model) are one chunk of three
+// slot blocks; anything longer goes 64 slots (four blocks) at a time.
 template <typename T, int C>
 int launch_tile(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
                 const clusten_attn_shape& s, hipStream_t stream) {
-    if (s.M <= 48) return launch_tile_q<T, C, 3>(a, as, rows, rs, idx, out, s, stream);
-    return launch_tile_q<T, C, 4>(a, as, rows, rs, idx, out, s, stream);
+    if (s.M % 4 == 0 && s.M <= 48) return launch_tile_q<T, C, 3, true>(a, as, rows, rs, idx, out, s, stream);
+    if (s.M % 4 == 0 && s.M <= 64) return launch_tile_q<T, C, 4, true>(a, as, rows, rs, idx, out, s, stream);
+    return launch_tile_q<T, C, 4, false>(a, as, rows, rs, idx, out, s, stream);
 }
 
 template <typename T>
@@ -247,9 +342,11 @@ int launch_elem(const void* a, clusten_strides as, const void* rows, clusten_str
 }
 
 template <typename T>
-int gather_dot_typed(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
-                 const clusten_attn_shape& s, hipStream_t stream) {
-    const bool vec_ok = rows_aligned16(rows, rs, sizeof(T)) && rows_aligned16(a, as, sizeof(T)) &&
+int gather_dot_typed(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
+                     void* out, const clusten_attn_shape& s, hipStream_t stream) {
+    // the lane runs are 8- or 16-byte accesses at multiples of a quarter row; out rows start 16-byte aligned
+    // when M is a multiple of 4 (checked in the kernel) and the base is aligned
+    const bool vec_ok = rows_aligned16(rows, rs, sizeof(T)) && rows_aligned16(a, as, sizeof(T)) && aligned16(out) &&
                         slice_fits_int32(rs, s.H, s.N, s.C) && slice_fits_int32(as, s.H, s.N, s.C);
     if (vec_ok) {
         switch (s.C) {
@@ -261,6 +358,5 @@ int gather_dot_typed(const void* a, clusten_strides as, const void* rows, cluste
     }
     return launch_elem<T>(a, as, rows, rs, idx, out, s, stream);
 }
-
 
 }  // namespace clusten

@@ -42,6 +42,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
+    {
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
@@ -135,6 +136,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             if (head_ok && t < nt) out_lane[(int64_t)t * os.n] = from_acc<T>(acc[t]);
         }
     }
+    }
 }
 
 // One thread per output element; any dtype, any head dim, any list length, any alignment.
@@ -165,7 +167,8 @@ int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, GUARD>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+    const int grid = xcd_grid(total);
+    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, rs, os, tiles_per_batch, total);
     return launch_status();

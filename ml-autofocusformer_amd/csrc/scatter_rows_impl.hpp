@@ -37,6 +37,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
+    {
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
@@ -130,6 +131,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             }
         }
     }
+    }
 }
 
 // One thread per (b,h,i,c); loops over the list with one atomic per product.  Any dtype whose
@@ -160,7 +162,8 @@ int scatter_tile_q(const void* p, const void* x, clusten_strides xs, const int64
                    const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+    const int grid = xcd_grid(total);
+    hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(x), idx, out, s.H, s.N, s.M, xs,
                        tiles_per_batch, total);
     return launch_status();

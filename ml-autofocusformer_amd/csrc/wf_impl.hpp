@@ -41,6 +41,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 
     const int token = xcd_tile(blockIdx.x, total_tokens);
     if (token < 0) return;
+    {
     const int b = token / Nout;
     const int lane = threadIdx.x;
     const int rl = lane & 15;
@@ -103,6 +104,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             *reinterpret_cast<VecRaw*>(out_tok + (int64_t)ic * C + c) = VecIO<T, VEC>::pack(acc[ic]);
         }
     }
+    }
 }
 
 // One thread per output element; any dtype and shape.
@@ -153,6 +155,7 @@ __global__ __launch_bounds__(256) void wf_dfeat_kernel(const T* __restrict__ d_o
                                                        int Nout, int C, int M, int IC, int total_tokens) {
     const int token = xcd_tile(blockIdx.x, total_tokens);
     if (token < 0) return;
+    {
     const int b = token / Nout;
     const int64_t* list = idx + (int64_t)token * M;
     const T* wtok = w + (int64_t)token * M * IC;
@@ -164,6 +167,7 @@ __global__ __launch_bounds__(256) void wf_dfeat_kernel(const T* __restrict__ d_o
             for (int ic = 0; ic < IC; ++ic) sum += (A)to_acc(gtok[(int64_t)ic * C + c]) * (A)to_acc(wtok[j * IC + ic]);
             unsafeAtomicAdd(dst_b + list[j] * C + c, sum);
         }
+    }
     }
 }
 
@@ -177,11 +181,13 @@ int wf_forward_row(const void* w, const void* feat, const int64_t* idx, void* ou
                    hipStream_t stream) {
     const int total = s.B * s.Nout;
     if (s.M == 48) {
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 3, false>), dim3(xcd_grid(total)), dim3(kWave), 0,
+        const int grid = xcd_grid(total);
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 3, false>), dim3(grid), dim3(kWave), 0,
                            stream, static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out),
                            s.N, s.Nout, s.C, s.M, total);
     } else {
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 4, true>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+        const int grid = xcd_grid(total);
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 4, true>), dim3(grid), dim3(kWave), 0, stream,
                            static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
                            s.Nout, s.C, s.M, total);
     }
