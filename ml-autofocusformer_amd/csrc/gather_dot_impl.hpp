@@ -41,14 +41,9 @@
 #pragma once
 
 #include "launch.hpp"
+#include "mfma.hpp"
 
 namespace clusten {
-
-typedef float F32x4 __attribute__((ext_vector_type(4)));
-
-// s_waitcnt immediate (gfx9 encoding) that waits until at most `vm` vector-memory operations are
-// outstanding and leaves the LDS/scalar and export counters alone.
-constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (15 << 8); }
 
 // Geometry of the staging buffer in LDS: rows of RB bytes, filled 1 KiB (one wave access) at a time.
 //   [0, G_BYTES)            gathered rows of one head (16*Q rows); reused to turn the D blocks into
@@ -76,10 +71,6 @@ struct Staging {
     // XOR swizzle of the piece index: rows r, r+1, ... of a block land in different bank groups
     static __device__ __forceinline__ int swz(int row) { return ((row & 7) ^ ((row >> 3) & 1)) & (PPR - 1); }
 };
-
-#define CLUSTEN_LDS_DMA16(gptr, lptr)                                                         \
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr), \
-                                     (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
 // FAST = the list has at most 64 slots and a multiple of 4 of them: one chunk, and every access to
 // an out row is a whole aligned 16-byte group.  Otherwise lists go 64 slots at a time and the last

@@ -4,138 +4,258 @@
 // clusten/src/clustenav_cuda_kernel.cu:18-50) and the d_query half of the QK backward
 // (p = d_attn, rows = key; clusten/src/clustenqk_cuda_kernel.cu:91-132, the dq_update sum).
 //
-// Work decomposition.  One wave owns a tile of 8 consecutive tokens of one batch element.  Its 64
-// lanes are 64 consecutive (head, channel) pairs, so with head dim 32 a wave covers two heads and
-// a gathered row is read as one contiguous run per head.  The tile's neighbour lists are read once.
-// The p-rows of the tile are loaded so that each row of 16 lanes holds 16 consecutive slots of its
-// own head; the FMAs read them through DPP row broadcasts (see dpp.hpp).
+// Work decomposition.  One wave owns a tile of 8 consecutive tokens of one batch element and
+// walks all heads, so the int64 neighbour lists of the tile are read from HBM exactly once.
+// Per head the tile is a small matrix product  D[token][c] = P[token][slot] * G[slot][c]  with G
+// the gathered rows; it runs on the matrix cores as fp32 MFMA 16x16x4 blocks (16 tokens of which
+// 8 are real x 16 channels, 4 slots per step).
 //
-//   shared-list path — all tokens of the tile carry the same list: every gathered element is
-//     loaded once and used for the 8 tokens (8 FMAs per load).
-//   per-token path — any other tile: one load per token and slot.
+// Data path per head:
+//   1. gather: `global_load_lds_dwordx4` moves the gathered rows straight into LDS, row-coalesced
+//      (consecutive lanes on consecutive 16-byte pieces of one row), and the tile's p-rows as well.
+//      The p pieces (4 slots of one token, 16 bytes) are laid out piece-transposed, [slot group][token],
+//      so that the 8 tokens' pieces of one slot group are contiguous.
+//   2. operands: lane (n = lane % 16, kq = lane / 16) is column n of the B operand and k-index kq.
+//      For MFMA step s it reads channels [n*C/16, (n+1)*C/16) of gathered row 4*s + kq (channel
+//      n*C/16 + e belongs to channel block e), and element kq of p piece (token n % 8, slot group s).
+//   3. the D blocks leave lane (n, mq = lane / 16) with tokens 4*mq..4*mq+3 of channels
+//      n*C/16 + e.  When the out rows of the tile are contiguous they are laid out row-major in
+//      LDS and leave with full-width 16-byte stores.
+// One short-lived one-wave workgroup per tile; the latency of its dependent chain (lists, rows,
+// product, store) is hidden by the other waves resident on the CU.
 //
-// Head dims other than 16/32/64, list lengths that are not a multiple of 4, unaligned p and fp64
-// take the element-per-thread kernel at the bottom of the file.
+//   shared-list path — all tokens of the tile carry the same list: one gather and one set of MFMAs
+//     per head serve the 8 tokens.
+//   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
+//     token's row is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
+//
+// Storage types narrower than fp32 are widened in registers; all products and sums are fp32.
+// Head dims other than 16/32/64, p rows that are not whole 16-byte pieces (M*sizeof(T) % 16 != 0),
+// rows whose start is not 16-byte aligned and fp64 take the element-per-thread kernel at the
+// bottom of the file.
 //
 // This header holds the templates; gather_sum_{f32,f16,bf16}.hip instantiate them per storage type
 // so that the translation units build in parallel, gather_sum.hip holds the dtype dispatch.
 #pragma once
 
-#include "dpp.hpp"
 #include "launch.hpp"
+#include "mfma.hpp"
 
 namespace clusten {
 
-// GUARD = false: the list has exactly 16*Q slots.  GUARD = true: any list length that is a
-// multiple of 4, taken 64 slots at a time (Q = 4) with every slot range-checked.
-template <typename T, int C, int Q, bool GUARD>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
+// Geometry of the gather_sum staging buffer in LDS.
+//   [0, G_BYTES)          gathered rows of one chunk (16*Q rows of RB bytes); reused to turn the D
+//                         blocks into the row-major output chunk
+//   [P_BASE, +2*P_SLOT)   p pieces of two heads (slot h % 2), piece-transposed: piece (slot group s,
+//                         token t) at (s*8 + t)*16
+template <typename T, int C, int Q>
+struct SumStaging {
+    static constexpr int RB = C * (int)sizeof(T);               // bytes per gathered row
+    static constexpr int PPR = RB / 16;                         // 16-byte pieces per row
+    static constexpr int RPI = kWave / PPR;                     // rows per wave access
+    static constexpr int NI_G = (16 * Q + RPI - 1) / RPI;       // accesses for the gathered rows of a chunk
+    static constexpr int G_BYTES = NI_G * 1024 > kTileTokens * RB ? NI_G * 1024 : kTileTokens * RB;
+    static constexpr int SPP = 16 / (int)sizeof(T);             // slots per p piece
+    static constexpr int STEPS_PER_PIECE = SPP / 4;             // MFMA steps (4 slots) per p piece
+    static constexpr int P_PIECES = 16 * Q / SPP * kTileTokens;  // p pieces of one (tile, head, chunk)
+    static constexpr int NI_P = (P_PIECES + kWave - 1) / kWave;  // accesses for them
+    static constexpr int P_BASE = G_BYTES;
+    static constexpr int P_SLOT_BYTES = NI_P * 1024;
+    static constexpr int BYTES = G_BYTES + 2 * P_SLOT_BYTES;
+    static constexpr int ECH = C / 16;                          // channels per lane = channel blocks
+    static constexpr int STEPS = 4 * Q;                         // MFMA steps per chunk
+    static_assert(RB >= 32 && kWave % PPR == 0, "row size");
+};
+
+// FAST = the list has at most 64 slots: one chunk, p-rows of two heads prefetched before the lists
+// are read.  Otherwise lists go 64 slots at a time and the D blocks accumulate over the chunks.
+template <typename T, int C, int Q, bool FAST>
+__global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H, int N, int M,
                                                                 clusten_strides rs, clusten_strides os,
                                                                 int tiles_per_batch, int total_tiles) {
-    constexpr int HPW = kWave / C;  // heads covered by the wave's 64 lanes
-    constexpr int SLOTS = 16 * Q;   // neighbour slots taken per chunk
-    static_assert(C == 16 || C == 32 || C == 64, "a row of 16 lanes must stay inside one head");
-    static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
-    typedef typename Quad<T>::raw QuadRaw;
+    typedef SumStaging<T, C, Q> S;
+    typedef VecIO<T, S::ECH> ChIO;   // the lane's channels of one gathered row
+    typedef VecIO<T, S::SPP> PieceIO;
+    static_assert(C == 16 || C == 32 || C == 64, "channel blocks of 16");
+    static_assert(FAST || Q == 4, "long lists are taken 64 slots at a time");
+
+    __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
 
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
-    {
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
     const int lane = threadIdx.x;
-    const int c = lane % C;
-    const int rl = lane & 15;  // lane inside its row of 16
+    const int n = lane & 15;   // MFMA column of the B operand / row (token) of the A operand
+    const int kq = lane >> 4;  // MFMA k index: slot 4*s + kq in step s; also the token group of the D rows
+    const int g_sub = lane / S::PPR;  // gather side: in access i this lane moves one piece of row i*RPI + g_sub
+    const int g_pos = lane % S::PPR;
 
-    const T* rows_b = rows + (int64_t)b * rs.b;
+    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
+    const uint32_t row_pitch = (uint32_t)rs.n * sizeof(T);
 
-    for (int h0 = 0; h0 < H; h0 += HPW) {
-        const int h_raw = h0 + lane / C;
-        const bool head_ok = h_raw < H;
-        const int h = min(h_raw, H - 1);  // lanes past the last head repeat it; only their store is masked
-        const int lane_off = h * (int)rs.h + c;
-        const T* p_head = p + (((int64_t)b * H + h) * N + i0) * M;
-
-        float acc[kTileTokens];
+    // p pieces of head h, chunk at slot j0 -> slot `ps` of the staging buffer.  Access i moves pieces
+    // 64*i + lane; piece q is slot group q / 8 of token q % 8 (tokens past the end of a partial tile
+    // repeat its last token, slot groups past the end of the list repeat its last group).
+    auto fetch_p = [&](int h, int j0, int mc, int ps) {
+        const char* p_head = reinterpret_cast<const char*>(p + (((int64_t)b * H + h) * N + i0) * M + j0);
 #pragma unroll
-        for (int t = 0; t < kTileTokens; ++t) acc[t] = 0.f;
-
-        for (int j0 = 0; j0 < M; j0 += kWave) {
-            const int mc = min(kWave, M - j0);
-            const int slot = min(lane, mc - 1);
-
-            int list[kTileTokens];
-            bool same = true;
-            {
-                int64_t wide[kTileTokens];
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) wide[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) {
-                    same = same && (wide[t] == wide[0]);
-                    list[t] = (int)wide[t];
-                }
-            }
-            const bool shared_list = __all(same ? 1 : 0) != 0;
-
-            // p-rows: row-lane n of every row of 16 holds slots 4n..4n+3 of the lane's head, per token
-            float pv[kTileTokens][4];
-            {
-                const int q4 = min(4 * rl, mc - 4);
-                QuadRaw raw[kTileTokens];
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) {
-                    raw[t] = *reinterpret_cast<const QuadRaw*>(p_head + (int64_t)min(t, nt - 1) * M + j0 + q4);
-                }
-#pragma unroll
-                for (int t = 0; t < kTileTokens; ++t) Quad<T>::unpack(raw[t], pv[t]);
-            }
-
-            if (shared_list) {
-                float val[SLOTS];
-                slot_pipeline<SLOTS, 16>(
-                    [&](auto ji) {
-                        constexpr int j = decltype(ji)::value;
-                        const int row = __builtin_amdgcn_readlane(list[0], min(j, mc - 1));
-                        const T* rowp = rows_b + (int64_t)row * rs.n;  // wave-uniform base, per-lane 32-bit offset
-                        val[j] = to_acc(rowp[lane_off]);
-                    },
-                    [&](auto ji) {
-                        constexpr int j = decltype(ji)::value;
-                        if (!GUARD || j < mc) {
-                            fma8_rowlane<j / 4>(acc, pv[0][j % 4], pv[1][j % 4], pv[2][j % 4], pv[3][j % 4],
-                                                pv[4][j % 4], pv[5][j % 4], pv[6][j % 4], pv[7][j % 4], val[j]);
-                        }
-                    });
-            } else {
-                static_for<0, kTileTokens>([&](auto ti) {
-                    constexpr int t = decltype(ti)::value;
-                    float val[SLOTS];
-                    slot_pipeline<SLOTS, 16>(
-                        [&](auto ji) {
-                            constexpr int j = decltype(ji)::value;
-                            const int row = __builtin_amdgcn_readlane(list[t], min(j, mc - 1));
-                            const T* rowp = rows_b + (int64_t)row * rs.n;
-                            val[j] = to_acc(rowp[lane_off]);
-                        },
-                        [&](auto ji) {
-                            constexpr int j = decltype(ji)::value;
-                            if (!GUARD || j < mc) fma1_rowlane<j / 4>(acc[t], pv[t][j % 4], val[j]);
-                        });
-                });
-            }
+        for (int i = 0; i < S::NI_P; ++i) {
+            const int q = i * kWave + lane;
+            const int grp = min(q / kTileTokens, mc / S::SPP - 1);
+            const int tok = min(q % kTileTokens, nt - 1);
+            CLUSTEN_LDS_DMA16(p_head + ((int64_t)tok * M + grp * S::SPP) * sizeof(T),
+                              stage + S::P_BASE + ps * S::P_SLOT_BYTES + i * 1024);
         }
+    };
+    if (FAST) {
+        fetch_p(0, 0, M, 0);
+        if (H > 1) fetch_p(1, 0, M, 1);
+    }
 
-        T* out_lane = out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n + c;
+    // Are all lists of the tile the same?  (over all chunks; the first list of each chunk stays in registers)
+    constexpr int MAXCH = FAST ? 1 : 4;  // chunks whose first list is kept in registers; longer lists re-read
+    int list0[MAXCH];
+    bool same = true;
+    for (int j0 = 0, ch = 0; j0 < M; j0 += kWave, ++ch) {
+        const int mc = min(kWave, M - j0);
+        const int slot = min(lane, mc - 1);  // lanes past the list repeat its last slot
+        int64_t wide[kTileTokens];
 #pragma unroll
-        for (int t = 0; t < kTileTokens; ++t) {
-            if (head_ok && t < nt) out_lane[(int64_t)t * os.n] = from_acc<T>(acc[t]);
+        for (int t = 0; t < kTileTokens; ++t) wide[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
+#pragma unroll
+        for (int t = 1; t < kTileTokens; ++t) same = same && (wide[t] == wide[0]);
+#pragma unroll
+        for (int k = 0; k < MAXCH; ++k) {
+            if (k == ch) list0[k] = (int)wide[0];
         }
     }
+    const bool shared_list = __all(same ? 1 : 0) != 0;
+
+    // operand side
+    const int lds_g = kq * S::RB + n * S::ECH * (int)sizeof(T);         // row kq of a step's 4 rows, the lane's channels
+    const int lds_p = (n & 7) * 16;                                     // the lane's token inside a slot group
+    // out: lane (n, kq) holds tokens 4*kq + i of channels n*ECH + e
+    const bool rows_contiguous = os.n == C;
+
+    // shared list: one pass that serves all tokens; otherwise one pass per token that keeps its row
+    const int passes = shared_list ? 1 : nt;
+    for (int pass = 0; pass < passes; ++pass) {
+        const int tok_lo = shared_list ? 0 : pass;
+        const int tok_hi = shared_list ? nt : pass + 1;
+        if (FAST && pass > 0) {  // the p slots hold the last heads of the previous pass
+            __syncthreads();
+            fetch_p(0, 0, M, 0);
+            if (H > 1) fetch_p(1, 0, M, 1);
+        }
+        for (int h = 0; h < H; ++h) {
+            const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+            F32x4 d[S::ECH];
+#pragma unroll
+            for (int e = 0; e < S::ECH; ++e) d[e] = F32x4{0.f, 0.f, 0.f, 0.f};
+
+            for (int j0 = 0, ch = 0; j0 < (FAST ? 1 : M); j0 += kWave, ++ch) {
+                const int mc = FAST ? M : min(kWave, M - j0);
+                const int slot = min(lane, mc - 1);
+                // this pass's list of the chunk
+                int mine;
+                if (pass == 0 && ch < MAXCH) {
+                    mine = list0[0];
+#pragma unroll
+                    for (int k = 1; k < MAXCH; ++k) mine = (k == ch) ? list0[k] : mine;
+                } else {
+                    mine = (int)idx_tile[(int64_t)pass * M + j0 + slot];
+                }
+                // gather: rows of this chunk -> LDS (and the p pieces when they were not prefetched)
+                if (!FAST) __syncthreads();  // the previous chunk's operand reads are complete
+#pragma unroll
+                for (int i = 0; i < S::NI_G; ++i) {
+                    const int srow = min(i * S::RPI + g_sub, mc - 1);
+                    const uint32_t off = (uint32_t)__shfl(mine, srow) * row_pitch + (uint32_t)(g_pos * 16);
+                    CLUSTEN_LDS_DMA16(rows_bh + off, stage + i * 1024);
+                }
+                const int ps = FAST ? (h & 1) : 0;
+                if (!FAST) {
+                    fetch_p(h, j0, mc, 0);
+                } else if (h >= 2) {
+                    fetch_p(h, 0, M, ps);
+                }
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                __syncthreads();
+
+                // steps: 4 slots each
+#pragma unroll
+                for (int sp = 0; sp < S::STEPS / S::STEPS_PER_PIECE; ++sp) {
+                    if (sp * S::SPP < mc) {  // wave-uniform: the list may end before the chunk does
+                        float pv[S::SPP];
+                        PieceIO::unpack(*reinterpret_cast<const typename PieceIO::raw*>(
+                                            stage + S::P_BASE + ps * S::P_SLOT_BYTES + sp * kTileTokens * 16 + lds_p),
+                                        pv);
+#pragma unroll
+                        for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
+                            const int s = sp * S::STEPS_PER_PIECE + ss;
+                            // element kq of the 4 slots of this step
+                            float aop = pv[4 * ss];
+#pragma unroll
+                            for (int k = 1; k < 4; ++k) aop = (kq == k) ? pv[4 * ss + k] : aop;
+                            float g[S::ECH];
+                            ChIO::unpack(*reinterpret_cast<const typename ChIO::raw*>(stage + 4 * s * S::RB + lds_g), g);
+#pragma unroll
+                            for (int e = 0; e < S::ECH; ++e) {
+                                d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(aop, g[e], d[e], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+
+            // store: lane (n, kq) holds tokens 4*kq + i, channels n*ECH + e
+            char* out_h = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
+            if (FAST && shared_list && rows_contiguous) {
+                __syncthreads();  // every operand read of this head is complete: reuse the row area
+                if (kq < 2) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float v[S::ECH];
+#pragma unroll
+                        for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
+                        *reinterpret_cast<typename ChIO::raw*>(stage + ((4 * kq + i) * C + n * S::ECH) * (int)sizeof(T)) =
+                            ChIO::pack(v);
+                    }
+                }
+                __syncthreads();
+                constexpr int NO = (kTileTokens * S::RB + 1023) / 1024;
+                Piece o[NO];
+#pragma unroll
+                for (int i = 0; i < NO; ++i) {
+                    o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
+                }
+                __syncthreads();  // the chunk is in registers: the next head's gather may overwrite it
+                const int chunk_bytes = nt * S::RB;
+#pragma unroll
+                for (int i = 0; i < NO; ++i) {
+                    const int off = i * 1024 + lane * 16;
+                    if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
+                }
+            } else {
+                if (FAST) __syncthreads();  // operand reads complete before the next head's gather
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int tok = 4 * kq + i;
+                    if (tok >= tok_lo && tok < tok_hi) {
+                        float v[S::ECH];
+#pragma unroll
+                        for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
+                        *reinterpret_cast<typename ChIO::raw*>(out_h + ((int64_t)tok * os.n + n * S::ECH) * sizeof(T)) =
+                            ChIO::pack(v);
+                    }
+                }
+            }
+        }
     }
 }
 
@@ -162,13 +282,13 @@ __global__ __launch_bounds__(256) void gather_sum_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q, bool GUARD>
+template <typename T, int C, int Q, bool FAST>
 int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int grid = xcd_grid(total);
-    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, rs, os, tiles_per_batch, total);
     return launch_status();
@@ -177,9 +297,10 @@ int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int
 template <typename T, int C>
 int launch_tile(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out, clusten_strides os,
                 const clusten_attn_shape& s, hipStream_t stream) {
-    // 48 slots is the neighbourhood size of every 224x224 model; it gets the unguarded kernel
-    if (s.M == 48) return launch_tile_q<T, C, 3, false>(p, rows, rs, idx, out, os, s, stream);
-    return launch_tile_q<T, C, 4, true>(p, rows, rs, idx, out, os, s, stream);
+    // lists of up to 48 slots (the neighbourhood size of every 224x224 model) are three slot blocks
+    if (s.M <= 48) return launch_tile_q<T, C, 3, true>(p, rows, rs, idx, out, os, s, stream);
+    if (s.M <= 64) return launch_tile_q<T, C, 4, true>(p, rows, rs, idx, out, os, s, stream);
+    return launch_tile_q<T, C, 4, false>(p, rows, rs, idx, out, os, s, stream);
 }
 
 template <typename T>
@@ -196,9 +317,10 @@ int launch_elem(const void* p, const void* rows, clusten_strides rs, const int64
 template <typename T>
 int gather_sum_typed(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out, clusten_strides os,
                  const clusten_attn_shape& s, hipStream_t stream) {
-    // the p quads are 4*sizeof(T)-byte accesses at slot offsets that are multiples of 4
-    const bool quads_ok = s.M % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0 &&
-                          slice_fits_int32(rs, s.H, s.N, s.C);
+    // p rows are whole 16-byte pieces; gathered rows and out rows are read / written in 16-byte (or, for the
+    // strided store, C/16-element) groups
+    const bool quads_ok = ((int64_t)s.M * sizeof(T)) % 16 == 0 && aligned16(p) && rows_aligned16(rows, rs, sizeof(T)) &&
+                          rows_aligned16(out, os, sizeof(T)) && slice_fits_int32(rs, s.H, s.N, s.C);
     if (quads_ok) {
         switch (s.C) {
             case 16: return launch_tile<T, 16>(p, rows, rs, idx, out, os, s, stream);
