@@ -112,6 +112,19 @@ __device__ __forceinline__ void fma_vec_rowlane(float (&acc)[VEC], float b, cons
     }
 }
 
+// Lane L of the caller's row of 16 lanes, in every lane of that row.
+template <int L>
+__device__ __forceinline__ int rowlane_bcast(int x) {
+    static_assert(L >= 0 && L < 16, "row lane");
+    int r;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mov_b32_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf"
+        : "=v"(r)
+        : "v"(x), "n"(L));
+    return r;
+}
+
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).
 template <int I>
 struct Index {

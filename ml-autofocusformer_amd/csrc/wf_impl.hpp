@@ -7,13 +7,15 @@
 //   d_feat    d_feat[b,idx[b,i,j],c] += sum_ic d_out[b,i,ic,c] * w[b,i,j,ic]
 //             (clustenwf_cuda_kernel.cu:96-135)
 //
-// Forward: one wave per output token.  The 64 lanes cover 64*VEC consecutive channels with one
-// VEC-element access each, so every gathered row is read as one contiguous run, once, for all IC
-// inner channels (the reference re-gathers it IC times).  The token's weights w[b,i,:,:] — M*IC
-// values shared by all lanes — are loaded so that each row of 16 lanes holds 64 consecutive values
-// per register and are read through DPP row broadcasts (see dpp.hpp).  The neighbour list is read
-// once per token.  Channel counts that are not a multiple of 64, inner channel counts other than
-// 1 and 4, and M*IC not a multiple of 4 take the element-per-thread kernel.
+// Forward.  A gathered feature row is C*sizeof(T) bytes; LPT = that / 16 lanes cover it with one
+// 16-byte access each, so a wave serves 64/LPT output tokens at once (4 tokens of 64 fp32 channels)
+// and every gather instruction moves whole rows, 1 KiB per wave access.  Each row is read once for
+// all IC inner channels (the reference re-gathers it IC times).  What the lanes of one token share —
+// the token's weights w[b,i,:,:] and its neighbour list — is held spread over the rows of 16 lanes
+// that belong to the token and read through DPP row broadcasts (see dpp.hpp): no LDS, no scalar
+// loads.  Rows wider than 64 lanes are taken in 1 KiB column blocks.
+// Rows that are not a multiple of 256 bytes, inner channel counts other than 1, 2 and 4, and M*IC
+// not a multiple of 4 take the element-per-thread kernel.
 //
 // Backward: plain kernels (one thread per d_w element; one wave-row per token for d_feat with one
 // fp32 atomic per (slot, channel)).
@@ -27,43 +29,56 @@
 
 namespace clusten {
 
-template <typename T, int VEC, int IC, int Q, bool GUARD>
+// LPT = lanes per token (16, 32 or 64).  GUARD = false: the list has exactly 16*Q slots;
+// GUARD = true: any length, taken 64 slots at a time (Q = 4) with every slot range-checked.
+template <typename T, int LPT, int IC, int Q, bool GUARD>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void wf_forward_row_kernel(
     const T* __restrict__ w, const T* __restrict__ feat, const int64_t* __restrict__ idx, T* __restrict__ out, int N,
-    int Nout, int C, int M, int total_tokens) {
+    int Nout, int C, int M, int total_tokens, int total_groups) {
+    constexpr int TPW = kWave / LPT;               // output tokens per wave
+    constexpr int VEC = 16 / (int)sizeof(T);       // channels per lane and column block
     constexpr int SLOTS = 16 * Q;
-    constexpr int NW = (SLOTS * IC + 63) / 64;  // registers that hold one chunk of the token's weights
+    constexpr int NW = (SLOTS * IC + 63) / 64;     // registers that hold one chunk of a token's weights
+    constexpr int NL = Q;                          // registers that hold one chunk of a token's list
+    constexpr int GS = 4;                          // gather accesses per pipeline group (two groups in flight)
+    static_assert(LPT == 16 || LPT == 32 || LPT == 64, "a row of 16 lanes must belong to one token");
     static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
     static_assert(IC == 1 || IC == 2 || IC == 4, "inner channels of one slot must stay inside one quad");
     typedef typename Quad<T>::raw QuadRaw;
-    typedef typename VecIO<T, VEC>::raw VecRaw;
-    constexpr int GS = VEC >= 4 ? 4 : 16 / VEC;  // slots per pipeline group: 16 registers of row data per group
 
-    const int token = xcd_tile(blockIdx.x, total_tokens);
-    if (token < 0) return;
-    {
-    const int b = token / Nout;
+    const int group = xcd_tile(blockIdx.x, total_groups);
+    if (group < 0) return;
     const int lane = threadIdx.x;
     const int rl = lane & 15;
+    // the lane's token (waves past the end repeat the last token; their stores are masked)
+    const int token_raw = group * TPW + lane / LPT;
+    const bool token_ok = token_raw < total_tokens;
+    const int token = min(token_raw, total_tokens - 1);
+    const int b = token / Nout;
+    const int col = (lane % LPT) * VEC;  // first channel of the lane inside a column block
 
     const int64_t* list_p = idx + (int64_t)token * M;
     const T* w_tok = w + (int64_t)token * M * IC;
-    const T* feat_b = feat + (int64_t)b * N * C;
+    const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
     T* out_tok = out + (int64_t)token * IC * C;
+    const uint32_t row_bytes = (uint32_t)C * sizeof(T);
 
-    for (int c0 = 0; c0 < C; c0 += kWave * VEC) {
-        const int c = c0 + lane * VEC;
+    for (int c0 = 0; c0 < C; c0 += LPT * VEC) {
         float acc[IC][VEC];
 #pragma unroll
         for (int ic = 0; ic < IC; ++ic) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[ic][v] = 0.f;
         }
+        const uint32_t lane_bytes = (uint32_t)(c0 + col) * sizeof(T);
 
         for (int j0 = 0; j0 < M; j0 += kWave) {
             const int mc = min(kWave, M - j0);
-            const int list = (int)list_p[j0 + min(lane, mc - 1)];
 
+            // list: slot 16*k + rl of the token in register k of its row(s) of 16 lanes
+            int lst[NL];
+#pragma unroll
+            for (int k = 0; k < NL; ++k) lst[k] = (int)list_p[j0 + min(16 * k + rl, mc - 1)];
             // weights: flat element f = j*IC + ic of the chunk sits in register f/64 of row-lane (f%64)/4, element f%4
             float wv[NW][4];
             {
@@ -77,13 +92,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                 for (int m = 0; m < NW; ++m) Quad<T>::unpack(raw[m], wv[m]);
             }
 
-            VecRaw fv[SLOTS];
+            Piece fv[SLOTS];
             slot_pipeline<SLOTS, GS>(
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
-                    const int row = __builtin_amdgcn_readlane(list, min(j, mc - 1));
-                    const T* rowp = feat_b + (int64_t)row * C;  // wave-uniform base, per-lane 32-bit offset
-                    fv[j] = *reinterpret_cast<const VecRaw*>(rowp + c);
+                    // row index of slot j: lane j % 16 of list register j / 16, broadcast inside each row of 16
+                    const int row = rowlane_bcast<j % 16>(lst[j / 16]);
+                    const uint32_t off = (uint32_t)((GUARD && j >= mc) ? 0 : row) * row_bytes + lane_bytes;
+                    fv[j] = *reinterpret_cast<const Piece*>(feat_b + off);
                 },
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
@@ -99,11 +115,12 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                 });
         }
 
+        if (token_ok) {
 #pragma unroll
-        for (int ic = 0; ic < IC; ++ic) {
-            *reinterpret_cast<VecRaw*>(out_tok + (int64_t)ic * C + c) = VecIO<T, VEC>::pack(acc[ic]);
+            for (int ic = 0; ic < IC; ++ic) {
+                *reinterpret_cast<Piece*>(out_tok + (int64_t)ic * C + c0 + col) = VecIO<T, VEC>::pack(acc[ic]);
+            }
         }
-    }
     }
 }
 
@@ -176,20 +193,19 @@ inline int elem_grid(int64_t total) {
     return (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
 }
 
-template <typename T, int VEC, int IC>
+template <typename T, int LPT, int IC>
 int wf_forward_row(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
     const int total = s.B * s.Nout;
+    const int groups = (total + kWave / LPT - 1) / (kWave / LPT);
     if (s.M == 48) {
-        const int grid = xcd_grid(total);
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 3, false>), dim3(grid), dim3(kWave), 0,
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, IC, 3, false>), dim3(xcd_grid(groups)), dim3(kWave), 0,
                            stream, static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out),
-                           s.N, s.Nout, s.C, s.M, total);
+                           s.N, s.Nout, s.C, s.M, total, groups);
     } else {
-        const int grid = xcd_grid(total);
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, VEC, IC, 4, true>), dim3(grid), dim3(kWave), 0, stream,
-                           static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
-                           s.Nout, s.C, s.M, total);
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, IC, 4, true>), dim3(xcd_grid(groups)), dim3(kWave), 0,
+                           stream, static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out),
+                           s.N, s.Nout, s.C, s.M, total, groups);
     }
     return launch_status();
 }
@@ -197,13 +213,11 @@ int wf_forward_row(const void* w, const void* feat, const int64_t* idx, void* ou
 template <typename T, int IC>
 int wf_forward_vec(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
-    // widest access of at most 16 bytes per lane that tiles the channel count
-    if constexpr (sizeof(T) == 2) {
-        if (s.C % (kWave * 8) == 0) return wf_forward_row<T, 8, IC>(w, feat, idx, out, s, stream);
-    }
-    if (s.C % (kWave * 4) == 0) return wf_forward_row<T, 4, IC>(w, feat, idx, out, s, stream);
-    if (s.C % (kWave * 2) == 0) return wf_forward_row<T, 2, IC>(w, feat, idx, out, s, stream);
-    return wf_forward_row<T, 1, IC>(w, feat, idx, out, s, stream);
+    // lanes per token: the widest of 64, 32, 16 whose 16-byte accesses tile the row
+    const int row_bytes = s.C * (int)sizeof(T);
+    if (row_bytes % 1024 == 0) return wf_forward_row<T, 64, IC>(w, feat, idx, out, s, stream);
+    if (row_bytes % 512 == 0) return wf_forward_row<T, 32, IC>(w, feat, idx, out, s, stream);
+    return wf_forward_row<T, 16, IC>(w, feat, idx, out, s, stream);
 }
 
 template <typename T>
@@ -219,10 +233,13 @@ int wf_forward_elem(const void* w, const void* feat, const int64_t* idx, void* o
 template <typename T>
 int wf_forward_typed(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                      hipStream_t stream) {
-    const bool rows_ok = s.C % kWave == 0 && aligned16(feat) && aligned16(out);
+    // whole 256-byte rows, and 32-bit byte offsets inside one batch element of feat
+    const bool rows_ok = (s.C * (int)sizeof(T)) % 256 == 0 && aligned16(feat) && aligned16(out) &&
+                         (int64_t)s.N * s.C * (int64_t)sizeof(T) < ((int64_t)1 << 31);
     const bool quads_ok = (s.M * s.IC) % 4 == 0 && (reinterpret_cast<uintptr_t>(w) % (4 * sizeof(T))) == 0;
     if (rows_ok && quads_ok) {
         if (s.IC == 4) return wf_forward_vec<T, 4>(w, feat, idx, out, s, stream);
+        if (s.IC == 2) return wf_forward_vec<T, 2>(w, feat, idx, out, s, stream);
         if (s.IC == 1) return wf_forward_vec<T, 1>(w, feat, idx, out, s, stream);
     }
     return wf_forward_elem<T>(w, feat, idx, out, s, stream);
