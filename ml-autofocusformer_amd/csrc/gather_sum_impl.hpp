@@ -69,7 +69,8 @@ struct SumStaging {
 
 // FAST = the list has at most 64 slots: one chunk, p-rows of two heads prefetched before the lists
 // are read.  Otherwise lists go 64 slots at a time and the D blocks accumulate over the chunks.
-template <typename T, int C, int Q, bool FAST>
+// EXACT = the list has exactly 16*Q slots (no slot of the chunk is missing).
+template <typename T, int C, int Q, bool FAST, bool EXACT>
 __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H, int N, int M,
@@ -187,26 +188,53 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 __syncthreads();
 
-                // steps: 4 slots each
+                // steps of 4 slots, taken one p piece at a time: all LDS reads of a batch of pieces are
+                // issued before its MFMAs so that their latency is paid once per batch, not once per step.
+                // No branches: when the list can end inside the chunk (!EXACT) the operands of the
+                // missing slots are replaced by zeros.
+                constexpr int NPIECE = S::STEPS / S::STEPS_PER_PIECE;
+                constexpr int BATCH = (4 / S::STEPS_PER_PIECE) < 1 ? 1 : (4 / S::STEPS_PER_PIECE);  // pieces per batch = 4 steps
+                const char* p_lds = stage + S::P_BASE + ps * S::P_SLOT_BYTES + lds_p;
 #pragma unroll
-                for (int sp = 0; sp < S::STEPS / S::STEPS_PER_PIECE; ++sp) {
-                    if (sp * S::SPP < mc) {  // wave-uniform: the list may end before the chunk does
-                        float pv[S::SPP];
-                        PieceIO::unpack(*reinterpret_cast<const typename PieceIO::raw*>(
-                                            stage + S::P_BASE + ps * S::P_SLOT_BYTES + sp * kTileTokens * 16 + lds_p),
-                                        pv);
+                for (int sb = 0; sb < NPIECE; sb += BATCH) {
+                    typename PieceIO::raw p_raw[BATCH];
+                    typename ChIO::raw g_raw[BATCH * S::STEPS_PER_PIECE];
 #pragma unroll
-                        for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
-                            const int s = sp * S::STEPS_PER_PIECE + ss;
-                            // element kq of the 4 slots of this step
-                            float aop = pv[4 * ss];
+                    for (int q = 0; q < BATCH; ++q) {
+                        if (sb + q < NPIECE) {
+                            p_raw[q] = *reinterpret_cast<const typename PieceIO::raw*>(p_lds + (sb + q) * kTileTokens * 16);
 #pragma unroll
-                            for (int k = 1; k < 4; ++k) aop = (kq == k) ? pv[4 * ss + k] : aop;
-                            float g[S::ECH];
-                            ChIO::unpack(*reinterpret_cast<const typename ChIO::raw*>(stage + 4 * s * S::RB + lds_g), g);
+                            for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
+                                const int s = (sb + q) * S::STEPS_PER_PIECE + ss;
+                                g_raw[q * S::STEPS_PER_PIECE + ss] =
+                                    *reinterpret_cast<const typename ChIO::raw*>(stage + 4 * s * S::RB + lds_g);
+                            }
+                        }
+                    }
 #pragma unroll
-                            for (int e = 0; e < S::ECH; ++e) {
-                                d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(aop, g[e], d[e], 0, 0, 0);
+                    for (int q = 0; q < BATCH; ++q) {
+                        if (sb + q < NPIECE) {
+                            float pv[S::SPP];
+                            PieceIO::unpack(p_raw[q], pv);
+#pragma unroll
+                            for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
+                                const int s = (sb + q) * S::STEPS_PER_PIECE + ss;
+                                // element kq of the 4 slots of this step
+                                float aop = pv[4 * ss];
+#pragma unroll
+                                for (int k = 1; k < 4; ++k) aop = (kq == k) ? pv[4 * ss + k] : aop;
+                                float g[S::ECH];
+                                ChIO::unpack(g_raw[q * S::STEPS_PER_PIECE + ss], g);
+                                if (!EXACT) {
+                                    const bool live = 4 * s < mc;  // mc is a multiple of 4: a step is whole or missing
+                                    aop = live ? aop : 0.f;
+#pragma unroll
+                                    for (int e = 0; e < S::ECH; ++e) g[e] = live ? g[e] : 0.f;
+                                }
+#pragma unroll
+                                for (int e = 0; e < S::ECH; ++e) {
+                                    d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(aop, g[e], d[e], 0, 0, 0);
+                                }
                             }
                         }
                     }
@@ -282,13 +310,13 @@ __global__ __launch_bounds__(256) void gather_sum_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q, bool FAST>
+template <typename T, int C, int Q, bool FAST, bool EXACT>
 int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int grid = xcd_grid(total);
-    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST>), dim3(grid), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, rs, os, tiles_per_batch, total);
     return launch_status();
@@ -297,10 +325,10 @@ int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int
 template <typename T, int C>
 int launch_tile(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out, clusten_strides os,
                 const clusten_attn_shape& s, hipStream_t stream) {
-    // lists of up to 48 slots (the neighbourhood size of every 224x224 model) are three slot blocks
-    if (s.M <= 48) return launch_tile_q<T, C, 3, true>(p, rows, rs, idx, out, os, s, stream);
-    if (s.M <= 64) return launch_tile_q<T, C, 4, true>(p, rows, rs, idx, out, os, s, stream);
-    return launch_tile_q<T, C, 4, false>(p, rows, rs, idx, out, os, s, stream);
+    // 48 slots is the neighbourhood size of every 224x224 model: three slot blocks, no range checks
+    if (s.M == 48) return launch_tile_q<T, C, 3, true, true>(p, rows, rs, idx, out, os, s, stream);
+    if (s.M <= 64) return launch_tile_q<T, C, 4, true, false>(p, rows, rs, idx, out, os, s, stream);
+    return launch_tile_q<T, C, 4, false, false>(p, rows, rs, idx, out, os, s, stream);
 }
 
 template <typename T>
