@@ -8,14 +8,23 @@
 //             (clustenwf_cuda_kernel.cu:96-135)
 //
 // Forward.  A gathered feature row is C*sizeof(T) bytes; LPT = that / 16 lanes cover it with one
-// 16-byte access each, so a wave serves 64/LPT output tokens at once (4 tokens of 64 fp32 channels)
-// and every gather instruction moves whole rows, 1 KiB per wave access.  Each row is read once for
-// all IC inner channels (the reference re-gathers it IC times).  What the lanes of one token share —
-// the token's weights w[b,i,:,:] and its neighbour list — is held spread over the rows of 16 lanes
-// that belong to the token and read through DPP row broadcasts (see dpp.hpp): no LDS, no scalar
-// loads.  Rows wider than 64 lanes are taken in 1 KiB column blocks.
-// Rows that are not a multiple of 256 bytes, inner channel counts other than 1, 2 and 4, and M*IC
-// not a multiple of 4 take the element-per-thread kernel.
+// 16-byte access each, so a wave serves 64/LPT consecutive output tokens at once (4 tokens of 64
+// fp32 channels) and every gather instruction moves whole rows, 1 KiB per wave access, straight
+// into registers.  Each row is read once for all IC inner channels (the reference re-gathers it
+// IC times).
+// The products run on the matrix cores as `v_mfma_f32_4x4x1_16b_f32`: 16 independent 4x4 blocks,
+// one slot (k = 1) per instruction.  Block l/4 takes, as its B row, element e of the 16-byte groups
+// that lanes 4*(l/4)..+3 hold (four channels of one token), and as its A column the token's four
+// weights w[slot][0..3]; its D block is out[ic][those channels].  One MFMA per element e does the
+// work of 4 VALU FMAs per lane at twice their rate, and leaves the accumulators exactly where a
+// 16-byte store per inner channel needs them.
+// The weights of the wave's tokens are one contiguous run of 64/LPT * M * IC elements; they go to
+// LDS with LDS-direct loads and every lane reads weight (token, slot, l % 4) back as its A operand.
+// The neighbour list of a token is spread over the rows of 16 lanes that belong to it and row
+// indices are fetched by DPP row broadcast (see dpp.hpp).  Rows wider than 64 lanes are taken in
+// 1 KiB column blocks.
+// Rows that are not a multiple of 256 bytes, more than 4 inner channels, and weight rows that are
+// not whole 16-byte pieces take the element-per-thread kernel.
 //
 // Backward: plain kernels (one thread per d_w element; one wave-row per token for d_feat with one
 // fp32 atomic per (slot, channel)).
@@ -26,50 +35,55 @@
 
 #include "dpp.hpp"
 #include "launch.hpp"
+#include "mfma.hpp"
 
 namespace clusten {
 
 // LPT = lanes per token (16, 32 or 64).  GUARD = false: the list has exactly 16*Q slots;
 // GUARD = true: any length, taken 64 slots at a time (Q = 4) with every slot range-checked.
-template <typename T, int LPT, int IC, int Q, bool GUARD>
+template <typename T, int LPT, int Q, bool GUARD>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void wf_forward_row_kernel(
     const T* __restrict__ w, const T* __restrict__ feat, const int64_t* __restrict__ idx, T* __restrict__ out, int N,
-    int Nout, int C, int M, int total_tokens, int total_groups) {
+    int Nout, int C, int M, int IC, int total_tokens, int total_groups) {
     constexpr int TPW = kWave / LPT;               // output tokens per wave
     constexpr int VEC = 16 / (int)sizeof(T);       // channels per lane and column block
     constexpr int SLOTS = 16 * Q;
-    constexpr int NW = (SLOTS * IC + 63) / 64;     // registers that hold one chunk of a token's weights
     constexpr int NL = Q;                          // registers that hold one chunk of a token's list
     constexpr int GS = 4;                          // gather accesses per pipeline group (two groups in flight)
+    constexpr int W_BYTES = TPW * SLOTS * 4 * (int)sizeof(T);  // weights of one chunk of the wave's tokens (IC <= 4)
+    constexpr int NI_W = (W_BYTES + 1023) / 1024;
     static_assert(LPT == 16 || LPT == 32 || LPT == 64, "a row of 16 lanes must belong to one token");
     static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
-    static_assert(IC == 1 || IC == 2 || IC == 4, "inner channels of one slot must stay inside one quad");
-    typedef typename Quad<T>::raw QuadRaw;
+
+    __shared__ __attribute__((aligned(1024))) char wbuf[NI_W * 1024];
 
     const int group = xcd_tile(blockIdx.x, total_groups);
     if (group < 0) return;
     const int lane = threadIdx.x;
     const int rl = lane & 15;
-    // the lane's token (waves past the end repeat the last token; their stores are masked)
-    const int token_raw = group * TPW + lane / LPT;
-    const bool token_ok = token_raw < total_tokens;
-    const int token = min(token_raw, total_tokens - 1);
+    // the lane's token (lanes past the last token repeat it; their stores are masked)
+    const int tl = lane / LPT;                            // token of the lane inside the wave
+    const int token0 = group * TPW;
+    const int ntok = min(TPW, total_tokens - token0);    // tokens of this wave
+    const bool token_ok = tl < ntok;
+    const int token = token0 + min(tl, ntok - 1);
     const int b = token / Nout;
     const int col = (lane % LPT) * VEC;  // first channel of the lane inside a column block
+    const int ic_lane = lane & 3;        // the row of the 4x4 blocks this lane feeds: inner channel
+    const bool ic_live = ic_lane < IC;
 
     const int64_t* list_p = idx + (int64_t)token * M;
-    const T* w_tok = w + (int64_t)token * M * IC;
     const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
     T* out_tok = out + (int64_t)token * IC * C;
     const uint32_t row_bytes = (uint32_t)C * sizeof(T);
+    // weights: the wave's tokens are consecutive, so their rows are one contiguous run
+    const char* w_wave = reinterpret_cast<const char*>(w + (int64_t)token0 * M * IC);
+    const int w_tok_bytes = M * IC * (int)sizeof(T);
 
     for (int c0 = 0; c0 < C; c0 += LPT * VEC) {
-        float acc[IC][VEC];
+        F32x4 acc[VEC];  // acc[e][ic] = out[ic][c0 + col + e]
 #pragma unroll
-        for (int ic = 0; ic < IC; ++ic) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) acc[ic][v] = 0.f;
-        }
+        for (int e = 0; e < VEC; ++e) acc[e] = F32x4{0.f, 0.f, 0.f, 0.f};
         const uint32_t lane_bytes = (uint32_t)(c0 + col) * sizeof(T);
 
         for (int j0 = 0; j0 < M; j0 += kWave) {
@@ -79,18 +93,31 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             int lst[NL];
 #pragma unroll
             for (int k = 0; k < NL; ++k) lst[k] = (int)list_p[j0 + min(16 * k + rl, mc - 1)];
-            // weights: flat element f = j*IC + ic of the chunk sits in register f/64 of row-lane (f%64)/4, element f%4
-            float wv[NW][4];
-            {
-                QuadRaw raw[NW];
+
+            // weights of this chunk -> LDS.  A single chunk (M <= 64) of all the wave's tokens is one
+            // contiguous run; otherwise each token's mc*IC elements are moved separately to t*mc*IC.
+            __syncthreads();  // the previous chunk's / column block's reads are complete
+            const int w_chunk_bytes = mc * IC * (int)sizeof(T);
+            if (mc == M) {
+                const int pieces = ntok * w_chunk_bytes / 16;
 #pragma unroll
-                for (int m = 0; m < NW; ++m) {
-                    const int f0 = min(64 * m + 4 * rl, mc * IC - 4);
-                    raw[m] = *reinterpret_cast<const QuadRaw*>(w_tok + (int64_t)j0 * IC + f0);
+                for (int i = 0; i < NI_W; ++i) {
+                    CLUSTEN_LDS_DMA16(w_wave + min(i * kWave + lane, pieces - 1) * 16, wbuf + i * 1024);
                 }
+            } else {
+                const int ppt = w_chunk_bytes / 16;  // pieces per token
 #pragma unroll
-                for (int m = 0; m < NW; ++m) Quad<T>::unpack(raw[m], wv[m]);
+                for (int i = 0; i < NI_W; ++i) {
+                    const int q = min(i * kWave + lane, ntok * ppt - 1);
+                    const int t = q / ppt, pc = q - t * ppt;
+                    CLUSTEN_LDS_DMA16(w_wave + (int64_t)t * w_tok_bytes + (int64_t)j0 * IC * sizeof(T) + pc * 16,
+                                      wbuf + i * 1024);
+                }
             }
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            __syncthreads();
+            // this lane's A operands: weight (its token, slot j, inner channel l % 4)
+            const char* w_lane = wbuf + min(tl, ntok - 1) * w_chunk_bytes + min(ic_lane, IC - 1) * (int)sizeof(T);
 
             Piece fv[SLOTS];
             slot_pipeline<SLOTS, GS>(
@@ -103,22 +130,28 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                 },
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
-                    if (!GUARD || j < mc) {
-                        float x[VEC];
-                        VecIO<T, VEC>::unpack(fv[j], x);
-                        static_for<0, IC>([&](auto ici) {
-                            constexpr int ic = decltype(ici)::value;
-                            constexpr int f = j * IC + ic;
-                            fma_vec_rowlane<(f % 64) / 4, VEC>(acc[ic], wv[f / 64][f % 4], x);
-                        });
+                    const bool live = ic_live && (!GUARD || j < mc);
+                    const int jj = GUARD ? min(j, mc - 1) : j;
+                    const float aop = live ? to_acc(*reinterpret_cast<const T*>(w_lane + jj * IC * (int)sizeof(T))) : 0.f;
+                    float x[VEC];
+                    VecIO<T, VEC>::unpack(fv[j], x);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float bop = (!GUARD || j < mc) ? x[e] : 0.f;
+                        acc[e] = __builtin_amdgcn_mfma_f32_4x4x1f32(aop, bop, acc[e], 0, 0, 0);
                     }
                 });
         }
 
         if (token_ok) {
 #pragma unroll
-            for (int ic = 0; ic < IC; ++ic) {
-                *reinterpret_cast<Piece*>(out_tok + (int64_t)ic * C + c0 + col) = VecIO<T, VEC>::pack(acc[ic]);
+            for (int ic = 0; ic < 4; ++ic) {
+                if (ic < IC) {
+                    float v[VEC];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) v[e] = acc[e][ic];
+                    *reinterpret_cast<Piece*>(out_tok + (int64_t)ic * C + c0 + col) = VecIO<T, VEC>::pack(v);
+                }
             }
         }
     }
@@ -193,31 +226,31 @@ inline int elem_grid(int64_t total) {
     return (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
 }
 
-template <typename T, int LPT, int IC>
+template <typename T, int LPT>
 int wf_forward_row(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
     const int total = s.B * s.Nout;
     const int groups = (total + kWave / LPT - 1) / (kWave / LPT);
-    if (s.M == 48) {
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, IC, 3, false>), dim3(xcd_grid(groups)), dim3(kWave), 0,
-                           stream, static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out),
-                           s.N, s.Nout, s.C, s.M, total, groups);
+    if (s.M == 48) {  // the neighbourhood size of every 224x224 model: no range checks
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 3, false>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
+                           static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
+                           s.Nout, s.C, s.M, s.IC, total, groups);
     } else {
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, IC, 4, true>), dim3(xcd_grid(groups)), dim3(kWave), 0,
-                           stream, static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out),
-                           s.N, s.Nout, s.C, s.M, total, groups);
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 4, true>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
+                           static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
+                           s.Nout, s.C, s.M, s.IC, total, groups);
     }
     return launch_status();
 }
 
-template <typename T, int IC>
+template <typename T>
 int wf_forward_vec(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
     // lanes per token: the widest of 64, 32, 16 whose 16-byte accesses tile the row
     const int row_bytes = s.C * (int)sizeof(T);
-    if (row_bytes % 1024 == 0) return wf_forward_row<T, 64, IC>(w, feat, idx, out, s, stream);
-    if (row_bytes % 512 == 0) return wf_forward_row<T, 32, IC>(w, feat, idx, out, s, stream);
-    return wf_forward_row<T, 16, IC>(w, feat, idx, out, s, stream);
+    if (row_bytes % 1024 == 0) return wf_forward_row<T, 64>(w, feat, idx, out, s, stream);
+    if (row_bytes % 512 == 0) return wf_forward_row<T, 32>(w, feat, idx, out, s, stream);
+    return wf_forward_row<T, 16>(w, feat, idx, out, s, stream);
 }
 
 template <typename T>
@@ -236,12 +269,10 @@ int wf_forward_typed(const void* w, const void* feat, const int64_t* idx, void* 
     // whole 256-byte rows, and 32-bit byte offsets inside one batch element of feat
     const bool rows_ok = (s.C * (int)sizeof(T)) % 256 == 0 && aligned16(feat) && aligned16(out) &&
                          (int64_t)s.N * s.C * (int64_t)sizeof(T) < ((int64_t)1 << 31);
-    const bool quads_ok = (s.M * s.IC) % 4 == 0 && (reinterpret_cast<uintptr_t>(w) % (4 * sizeof(T))) == 0;
-    if (rows_ok && quads_ok) {
-        if (s.IC == 4) return wf_forward_vec<T, 4>(w, feat, idx, out, s, stream);
-        if (s.IC == 2) return wf_forward_vec<T, 2>(w, feat, idx, out, s, stream);
-        if (s.IC == 1) return wf_forward_vec<T, 1>(w, feat, idx, out, s, stream);
-    }
+    // weight rows (and every 64-slot chunk of one) are whole 16-byte pieces; at most 4 inner channels
+    const bool w_ok = s.IC <= 4 && ((int64_t)s.M * s.IC * sizeof(T)) % 16 == 0 && aligned16(w) &&
+                      (s.M <= 64 || (64 * s.IC * (int)sizeof(T)) % 16 == 0);
+    if (rows_ok && w_ok) return wf_forward_vec<T>(w, feat, idx, out, s, stream);
     return wf_forward_elem<T>(w, feat, idx, out, s, stream);
 }
 
