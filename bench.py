@@ -145,6 +145,65 @@ def _bench_wf(case, steps, warmup):
             "wf_us": round(per[0] * 1e3, 1), "wf_GBps": round(nbytes / per[0] / 1e6, 1), "bytes": nbytes}
 
 
+def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
+    """Images/s of the AFF-Tiny classifier at 224x224 (random weights, N(0,1) images, fp16 autocast, eval mode),
+    timed like the reference's `throughput` (main.py:343-354: 50 untimed and 30 timed forwards), and the share
+    of one forward spent in each operator, measured in a separate pass with stream events around the calls."""
+    import torch
+    from types import SimpleNamespace
+    from aff import model as aff_model
+
+    torch.manual_seed(0)
+    spans = {}
+
+    def timed_call(name, fn):
+        def call(*a, **kw):
+            if not spans.get("on"):
+                return fn(*a, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn(*a, **kw)
+            e1.record()
+            spans.setdefault(name, []).append((e0, e1))
+            return out
+        return call
+
+    real = aff_model.default_ops()
+    ops = SimpleNamespace(qk=timed_call("qk", real.qk), av=timed_call("av", real.av), wf=timed_call("wf", real.wf))
+    net = aff_model.aff_tiny(ops=ops).cuda().eval()
+    for layer in net.layers:
+        layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)
+        if layer.downsample is not None:
+            layer.downsample.select = timed_call("merge_select", layer.downsample.select)
+    x = torch.randn(batch, 3, 224, 224, device="cuda")
+
+    def forward():
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+            return net(x)
+
+    for _ in range(warmup):
+        forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(timed):
+        forward()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+
+    spans["on"] = True
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    forward()
+    e1.record()
+    torch.cuda.synchronize()
+    total = e0.elapsed_time(e1)
+    share = {k: round(sum(a.elapsed_time(b) for a, b in v) / total, 4) for k, v in spans.items() if k != "on"}
+    share["everything_else"] = round(1.0 - sum(share.values()), 4)
+    return {"img_per_s": round(timed * batch / dt, 1), "ms_per_batch": round(dt / timed * 1e3, 2), "batch": batch,
+            "warmup": warmup, "timed": timed, "dtype": "fp16 autocast (QK fp16; AV, WF fp32)",
+            "share_of_forward": share}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -152,6 +211,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--full", action="store_true", help="also time the other stages and configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the AFF-Tiny images/s leg")
+    ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy"), default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
@@ -167,6 +228,9 @@ def main():
         sys.exit("bench.py needs a GPU: the CLUSTEN kernels have no CPU path.")
     _native.load()
     torch.cuda.set_device(0)
+    if args.e2e_only:
+        print(json.dumps({"aff_tiny_224": _aff_tiny_throughput()}), flush=True)
+        return
 
     B = 128
     acase = wl.config2_attn(1, B=B)
@@ -242,6 +306,8 @@ def main():
         other["cfg2_s1_model_like_lists"] = _bench_attn(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
         out["other_configs"] = other
+    if not args.no_e2e:
+        out["aff_tiny_224"] = _aff_tiny_throughput()
     if not args.no_cpu:
         out["cpu_baseline"] = _cpu_baseline(acase, wcase, total_bytes, B)
     print(json.dumps(out), flush=True)

@@ -1,0 +1,357 @@
+"""AutoFocusFormer classifier assembled around the CLUSTEN operators.
+
+This is the build's own counterpart of models/aff_transformer.py, kept to what drives the three operators and
+what an end-to-end images/s figure needs.  Parameter names and shapes equal the reference's, so a reference
+`state_dict` loads unchanged.  What each class must reproduce:
+
+  ClusterAttention  (aff_transformer.py:87-160)  q scaled by head_dim^-0.5 before QK; q/key/v handed to the
+                    operators as permuted views of the Linear outputs; position bias, padding mask (-100),
+                    blank token and softmax between QK and AV; dense branch when a stage attends globally.
+  ClusterMerging    (aff_transformer.py:276-365) merge centres = top scores of grid prior + alpha * learned
+                    score, reserve tokens on the coarse grid; weights (b, n', m, 4) = weight_net(table)[pe_idx] *
+                    learned score * mask; WF output (b, n', 4, c) flattened so that channel = ic * c + c'.
+  BasicLayer        (aff_transformer.py:441-507) balanced clusters, the nnc nearest clusters of every token, the
+                    neighbourhood list = members of those clusters, nearest cluster first.
+
+Differences from the reference, none of which change results: the relative-position table is a module buffer
+instead of a module-level global; the neighbourhoods of the first stage, whose tokens sit on the image grid,
+are computed once and reused (the reference caches the clustering but repeats the neighbour search); nearest
+neighbours use a sort of exact distances instead of an external library; the operators are reached through
+`self.ops`, so a test can run the very same modules on another implementation of the three functions.
+"""
+import math
+from types import SimpleNamespace
+
+import torch
+import torch.nn as nn
+
+from .points import knn, space_filling_cluster
+
+
+def default_ops():
+    """The three operators as the HIP library provides them."""
+    from clusten import CLUSTENAVFunction, CLUSTENQKFunction, CLUSTENWFFunction
+    return SimpleNamespace(qk=CLUSTENQKFunction.apply, av=CLUSTENAVFunction.apply, wf=CLUSTENWFFunction.apply)
+
+
+def relative_position_table(img_size):
+    """(table_width^2, 5) rows (dx, dy, distance, sin, cos) for every offset between two stride-4 tokens.
+
+    aff_transformer.py:14-33: offsets range over [-R, R] with R = img_size // 4 - 1; the row of offset (dx, dy)
+    is (dy + R) * (2R + 1) + (dx + R); the undefined angle at the origin is 0.
+    """
+    r = img_size // 4 - 1
+    axis = torch.arange(2 * r + 1).float() - r
+    dy, dx = torch.meshgrid(axis, axis, indexing="ij")
+    dist = (dx ** 2 + dy ** 2) ** 0.5
+    table = torch.stack([dx, dy, dist, dy / dist, dx / dist], dim=2)
+    table[~torch.isfinite(table)] = 0
+    return table.reshape(-1, 5), r
+
+
+class DropPath(nn.Module):
+    """Stochastic depth: drops the whole residual branch of a sample with probability p while training."""
+
+    def __init__(self, p):
+        super().__init__()
+        self.p = float(p)
+
+    def forward(self, x):
+        if not self.training or self.p == 0.0:
+            return x
+        keep = 1.0 - self.p
+        shape = (x.shape[0],) + (1,) * (x.dim() - 1)
+        return x * x.new_empty(shape).bernoulli_(keep).div_(keep)
+
+
+class Mlp(nn.Module):
+    def __init__(self, dim, hidden, drop=0.0):
+        super().__init__()
+        self.fc1 = nn.Linear(dim, hidden)
+        self.act = nn.GELU()
+        self.fc2 = nn.Linear(hidden, dim)
+        self.drop = nn.Dropout(drop)
+
+    def forward(self, x):
+        return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
+
+
+class ClusterAttention(nn.Module):
+    """Attention of every token over the members of its nearest clusters, plus one learned blank token."""
+
+    def __init__(self, dim, num_heads, attn_drop=0.0, proj_drop=0.0, ops=None):
+        super().__init__()
+        self.dim, self.num_heads = dim, num_heads
+        self.scale = (dim // num_heads) ** -0.5
+        self.q = nn.Linear(dim, dim)
+        self.kv = nn.Linear(dim, 2 * dim)
+        self.blank_k = nn.Parameter(torch.randn(dim))
+        self.blank_v = nn.Parameter(torch.randn(dim))
+        self.pos_embed = nn.Linear(5, num_heads)
+        self.attn_drop = nn.Dropout(attn_drop)
+        self.proj = nn.Linear(dim, dim)
+        self.proj_drop = nn.Dropout(proj_drop)
+        self.ops = ops
+
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table):
+        b, n, c = feat.shape
+        h = self.num_heads
+        ch = c // h
+        q = (self.q(feat) * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)        # (b,h,n,ch) view
+        kv = self.kv(feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
+        key, v = kv[0], kv[1]
+        if global_attn:
+            attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
+        else:
+            attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
+
+        bias = self.pos_embed(table)                                                     # (rows, h)
+        attn = attn + bias[pe_idx].permute(0, 3, 1, 2)
+        if cluster_mask is not None and not global_attn:
+            attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
+
+        blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)            # (b,h,n,1)
+        attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
+        attn = self.attn_drop(attn)
+        blank, attn = attn[..., -1:], attn[..., :-1]
+
+        out = attn @ v if global_attn else self.ops.av(attn, v, member_idx)              # (b,h,n,ch)
+        out = out + blank * self.blank_v.reshape(1, h, 1, ch)
+        out = out.permute(0, 2, 1, 3).reshape(b, n, c)
+        return self.proj_drop(self.proj(out))
+
+
+class ClusterTransformerBlock(nn.Module):
+    def __init__(self, dim, num_heads, mlp_ratio=2.0, drop=0.0, attn_drop=0.0, drop_path=0.0, layer_scale=0.0,
+                 ops=None):
+        super().__init__()
+        self.norm1 = nn.LayerNorm(dim)
+        self.attn = ClusterAttention(dim, num_heads, attn_drop=attn_drop, proj_drop=drop, ops=ops)
+        self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
+        self.norm2 = nn.LayerNorm(dim)
+        self.mlp = Mlp(dim, int(dim * mlp_ratio), drop=drop)
+        self.layer_scale = isinstance(layer_scale, (int, float)) and layer_scale > 0
+        if self.layer_scale:
+            self.gamma1 = nn.Parameter(layer_scale * torch.ones(dim))
+            self.gamma2 = nn.Parameter(layer_scale * torch.ones(dim))
+
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table):
+        a = self.attn(self.norm1(feat), member_idx, cluster_mask, pe_idx, global_attn, table)
+        feat = feat + self.drop_path(self.gamma1 * a if self.layer_scale else a)
+        f = self.mlp(self.norm2(feat))
+        return feat + self.drop_path(self.gamma2 * f if self.layer_scale else f)
+
+
+class ClusterMerging(nn.Module):
+    """Adaptive down-sampling: keeps ds_rate of the tokens and merges each one's neighbourhood into it."""
+
+    INNER = 4
+
+    def __init__(self, dim, out_dim, alpha=4.0, ds_rate=0.25, reserve_on=True, ops=None):
+        super().__init__()
+        self.alpha, self.ds_rate, self.reserve_on = alpha, ds_rate, reserve_on
+        self.weight_net = nn.Sequential(nn.Linear(5, self.INNER), nn.LayerNorm(self.INNER), nn.GELU())
+        self.norm = nn.LayerNorm(self.INNER * dim)
+        self.linear = nn.Linear(self.INNER * dim, out_dim)
+        self.ops = ops
+
+    def select(self, pos, learned_prob, stride, reserve_num):
+        """Indices (b, n') of the tokens kept as merge centres (aff_transformer.py:296-334)."""
+        b, n, _ = pos.shape
+        keep = int(n * self.ds_rate)
+        if stride == 2:                      # tokens still fill the grid: every other row and column
+            prior = ((pos % stride).sum(-1) == 0).float()
+        else:                                # adaptive grid: spacing from the distance to the nearest other token
+            _, dist = knn(pos, pos, 2, return_dist=True)
+            spacing = 2 ** (dist[:, :, 1].log2().ceil() + 1)
+            prior = ((pos.long() % spacing.unsqueeze(2).long()).sum(-1) == 0).float()
+        score = prior
+        if learned_prob is not None:
+            score = score + learned_prob.detach().view(b, n) * self.alpha
+        if not self.reserve_on:
+            return score.topk(keep, dim=1, sorted=False)[1]
+        reserved = ((pos % (stride * 2)).sum(-1) == 0)
+        score = score + reserved.float() * (-100)
+        sampled = score.topk(keep - reserve_num, dim=1, sorted=False)[1]
+        # the reserved tokens in ascending index order; there are exactly reserve_num of them per image
+        kept = reserved.to(torch.uint8).sort(dim=1, descending=True, stable=True)[1][:, :reserve_num]
+        return torch.cat([sampled, kept], dim=1)
+
+    def forward(self, pos, feat, member_idx, cluster_mask, learned_prob, stride, pe_idx, reserve_num, table):
+        b, n, c = feat.shape
+        m = member_idx.shape[-1]
+        centre = self.select(pos, learned_prob, stride, reserve_num)                     # (b, n')
+        n_out = centre.shape[1]
+        assert n_out == int(n * self.ds_rate), "number of merge centres"
+        pos = pos.gather(1, centre.unsqueeze(2).expand(-1, -1, pos.shape[2]))
+        rows = centre.unsqueeze(2).expand(-1, -1, m)
+        member_idx = member_idx.gather(1, rows)                                          # (b, n', m)
+        pe_idx = pe_idx.gather(1, rows)
+        weights = self.weight_net(table)[pe_idx]                                         # (b, n', m, 4)
+        if learned_prob is not None:
+            weights = weights * learned_prob.gather(1, member_idx.reshape(b, -1, 1)).reshape(b, n_out, m, 1)
+        if cluster_mask is not None:
+            weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
+        merged = self.ops.wf(weights, feat, member_idx).reshape(b, n_out, -1)            # channel = ic * c + c'
+        return pos, self.linear(self.norm(merged))
+
+
+class BasicLayer(nn.Module):
+    """One stage: neighbourhood lists, `depth` blocks over them, optional merging into the next stage."""
+
+    def __init__(self, dim, out_dim, cluster_size, nbhd_size, depth, num_heads, mlp_ratio, alpha=4.0, ds_rate=0.25,
+                 reserve_on=True, drop=0.0, attn_drop=0.0, drop_path=0.0, layer_scale=0.0, downsample=True,
+                 ops=None):
+        super().__init__()
+        assert cluster_size > 0
+        self.cluster_size, self.nbhd_size = cluster_size, nbhd_size
+        rates = drop_path if isinstance(drop_path, (list, tuple)) else [drop_path] * depth
+        self.blocks = nn.ModuleList([
+            ClusterTransformerBlock(dim, num_heads, mlp_ratio, drop, attn_drop, rates[i], layer_scale, ops=ops)
+            for i in range(depth)])
+        if downsample:
+            self.downsample = ClusterMerging(dim, out_dim, alpha, ds_rate, reserve_on, ops=ops)
+            self.prob_net = nn.Linear(dim, 1)
+        else:
+            self.downsample = None
+        self._grid_cache = {}
+
+    def neighbourhoods(self, pos, h, w, radius, table_width):
+        """(pos reordered, ranking or None, member_idx (b,n,nbhd), mask or None, pe_idx (b,n,nbhd)).
+
+        aff_transformer.py:454-487.  The list of token i holds the members of its nnc nearest clusters,
+        nearest cluster first; members of cluster g are tokens g*m .. g*m+m-1 of the reordered sequence.
+        """
+        b, n, d = pos.shape
+        m = self.cluster_size
+        k = int(math.ceil(n / float(m)))
+        nnc = min(int(round(self.nbhd_size / float(m))), k)
+        ranking = None
+        if k == n:
+            centres, members, mask = pos, torch.arange(n, device=pos.device).reshape(1, n, 1).expand(b, -1, -1), None
+        else:
+            pos, centres, members, mask, ranking = space_filling_cluster(pos, m, h, w)
+        nearest = knn(pos, centres, nnc)                                                  # (b, n, nnc)
+        pick = nearest.reshape(b, -1, 1).expand(-1, -1, m)
+        member_idx = members.gather(1, pick).reshape(b, n, nnc * m)
+        if mask is not None:
+            mask = mask.gather(1, pick).reshape(b, n, nnc * m)
+        nb_pos = pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, d)).reshape(b, n, nnc * m, d)
+        rel = nb_pos - (pos.unsqueeze(2) - radius)
+        pe_idx = (rel[..., 1] * table_width + rel[..., 0]).long()
+        return pos, ranking, member_idx, mask, pe_idx
+
+    def forward(self, pos, feat, h, w, on_grid, stride, table, radius):
+        b, n, d = pos.shape
+        table_width = 2 * radius + 1
+        global_attn = self.nbhd_size >= n
+        if global_attn:
+            member_idx = mask = None
+            rel = (pos[:, None, :, :] + radius) - pos[:, :, None, :]
+            pe_idx = (rel[..., 1] * table_width + rel[..., 0]).long()
+        else:
+            if on_grid:
+                # grid tokens are the same for every image: one image's lists serve the whole batch
+                key = (n, h, w, str(pos.device))
+                if key not in self._grid_cache:
+                    self._grid_cache[key] = self.neighbourhoods(pos[:1], h, w, radius, table_width)
+                pos1, ranking, member_idx, mask, pe_idx = self._grid_cache[key]
+                pos = pos1.expand(b, -1, -1)
+                member_idx = member_idx.expand(b, -1, -1).contiguous()
+                pe_idx = pe_idx.expand(b, -1, -1)
+                mask = None if mask is None else mask.expand(b, -1, -1)
+                if ranking is not None:
+                    feat = feat[:, ranking[0, :, 0]]
+            else:
+                pos, ranking, member_idx, mask, pe_idx = self.neighbourhoods(pos, h, w, radius, table_width)
+                if ranking is not None:
+                    feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
+
+        for blk in self.blocks:
+            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table)
+
+        if self.downsample is not None:
+            if global_attn:   # merging after a dense stage: every token is every token's neighbour
+                member_idx = torch.arange(n, device=feat.device).expand(b, n, n).contiguous()
+            learned_prob = self.prob_net(feat).sigmoid()
+            reserve_num = math.ceil(h / (stride * 2)) * math.ceil(w / (stride * 2))
+            pos, feat = self.downsample(pos, feat, member_idx, mask, learned_prob, stride, pe_idx, reserve_num, table)
+        return pos, feat
+
+
+class PatchEmbed(nn.Module):
+    """Two stride-2 3x3 convolutions (BatchNorm + GELU between them): one token per 4x4 pixels."""
+
+    def __init__(self, in_chans=3, embed_dim=32, patch_norm=True):
+        super().__init__()
+        self.proj1 = nn.Conv2d(in_chans, embed_dim // 2, kernel_size=3, stride=2, padding=1)
+        self.bn = nn.BatchNorm2d(embed_dim // 2)
+        self.act1 = nn.GELU()
+        self.proj2 = nn.Conv2d(embed_dim // 2, embed_dim, kernel_size=3, stride=2, padding=1)
+        self.norm = nn.LayerNorm(embed_dim) if patch_norm else None
+
+    def forward(self, x):
+        x = self.proj2(self.act1(self.bn(self.proj1(x))))
+        b, c, h, w = x.shape
+        x = x.flatten(2).transpose(1, 2)
+        if self.norm is not None:
+            x = self.norm(x)
+        ys, xs = torch.meshgrid(torch.arange(h, device=x.device), torch.arange(w, device=x.device), indexing="ij")
+        pos = torch.stack([xs, ys], dim=2).reshape(1, -1, 2).expand(b, -1, -1).to(x.dtype)
+        return pos, x, h, w
+
+
+class AutoFocusFormer(nn.Module):
+    """aff_transformer.py:560-670.  Defaults are the reference's; `aff_tiny()` gives configs/aff_tiny.yaml."""
+
+    def __init__(self, in_chans=3, num_classes=1000, embed_dim=(32, 128, 256, 512), cluster_size=8,
+                 nbhd_size=(48, 48, 48, 49), alpha=4.0, ds_rate=0.25, reserve_on=True, depths=(2, 2, 6, 2),
+                 num_heads=(3, 6, 12, 24), mlp_ratio=2.0, drop_rate=0.0, attn_drop_rate=0.0, drop_path_rate=0.1,
+                 patch_norm=True, layer_scale=0.0, img_size=224, ops=None):
+        super().__init__()
+        ops = ops if ops is not None else default_ops()
+        self.num_classes = num_classes
+        self.num_features = embed_dim[-1]
+        self.patch_embed = PatchEmbed(in_chans, embed_dim[0], patch_norm)
+        self.pos_drop = nn.Dropout(drop_rate)
+        table, self.radius = relative_position_table(img_size)
+        self.register_buffer("pre_table", table, persistent=False)
+        rates = [r.item() for r in torch.linspace(0, drop_path_rate, sum(depths))]
+        last = len(depths) - 1
+        self.layers = nn.ModuleList([
+            BasicLayer(embed_dim[i], embed_dim[i + 1] if i < last else None, cluster_size, nbhd_size[i], depths[i],
+                       num_heads[i], mlp_ratio, alpha, ds_rate, reserve_on, drop_rate, attn_drop_rate,
+                       rates[sum(depths[:i]):sum(depths[:i + 1])], layer_scale, downsample=i < last, ops=ops)
+            for i in range(len(depths))])
+        self.norm = nn.LayerNorm(self.num_features)
+        self.head = nn.Linear(self.num_features, num_classes) if num_classes > 0 else nn.Identity()
+        self.apply(self._init_weights)
+
+    @staticmethod
+    def _init_weights(mod):
+        if isinstance(mod, nn.Linear):
+            nn.init.trunc_normal_(mod.weight, std=0.02)
+            if mod.bias is not None:
+                nn.init.zeros_(mod.bias)
+        elif isinstance(mod, nn.LayerNorm):
+            nn.init.zeros_(mod.bias)
+            nn.init.ones_(mod.weight)
+
+    def forward_features(self, x):
+        pos, x, h, w = self.patch_embed(x)
+        x = self.pos_drop(x)
+        for i, layer in enumerate(self.layers):
+            pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=self.pre_table,
+                           radius=self.radius)
+        return self.norm(x).mean(1)
+
+    def forward(self, x):
+        return self.head(self.forward_features(x))
+
+
+def aff_tiny(**kw):
+    """configs/aff_tiny.yaml: depths 3/4/18/5, dims 64/128/256/512, heads 2/4/8/16, mlp ratio 3, 48 neighbours."""
+    cfg = dict(embed_dim=(64, 128, 256, 512), depths=(3, 4, 18, 5), num_heads=(2, 4, 8, 16), mlp_ratio=3.0,
+               cluster_size=8, nbhd_size=(48, 48, 48, 49), alpha=4.0, ds_rate=0.25, drop_path_rate=0.2)
+    cfg.update(kw)
+    return AutoFocusFormer(**cfg)

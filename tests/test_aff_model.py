@@ -1,0 +1,220 @@
+"""The callers of the operators (ClusterAttention, ClusterMerging, BasicLayer) and the classifier built from them.
+
+On the CPU the modules run on the oracle's gather expressions; on the GPU the same modules, same weights and
+same input run once on the HIP operators and once on the oracle, and the logits must agree.
+"""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from aff.model import (AutoFocusFormer, BasicLayer, ClusterAttention, ClusterMerging, aff_tiny,
+                       relative_position_table)
+from oracle import clusten_oracle as oracle
+
+
+def oracle_ops():
+    """The reference wrappers' dtype rule (second operand cast to the first's) around the gather expressions."""
+    return SimpleNamespace(
+        qk=lambda q, k, idx: oracle.qk_gather(q, k.to(q.dtype), idx),
+        av=lambda a, v, idx: oracle.av_gather(a, v.to(a.dtype), idx),
+        wf=lambda w, f, idx: oracle.wf_gather(w, f.to(w.dtype), idx))
+
+
+def small_model(ops, **kw):
+    cfg = dict(embed_dim=(32, 64, 128, 256), depths=(1, 2, 1, 1), num_heads=(2, 4, 8, 16), mlp_ratio=2.0,
+               num_classes=10, img_size=128, drop_path_rate=0.0, ops=ops)
+    cfg.update(kw)
+    torch.manual_seed(0)
+    return AutoFocusFormer(**cfg).eval()
+
+
+def test_relative_position_table_rows():
+    table, r = relative_position_table(224)
+    assert r == 55 and table.shape == (111 * 111, 5)
+    row = lambda dx, dy: table[(dy + r) * 111 + (dx + r)]
+    assert row(0, 0).tolist() == [0, 0, 0, 0, 0]
+    got = row(3, -4)
+    assert torch.allclose(got, torch.tensor([3.0, -4.0, 5.0, -0.8, 0.6]))
+    assert torch.isfinite(table).all()
+
+
+def test_parameter_names_follow_the_reference_layout():
+    names = set(small_model(oracle_ops()).state_dict().keys())
+    for key in ["patch_embed.proj1.weight", "patch_embed.bn.running_mean", "patch_embed.proj2.bias",
+                "patch_embed.norm.weight", "layers.0.blocks.0.norm1.weight", "layers.0.blocks.0.attn.q.weight",
+                "layers.0.blocks.0.attn.kv.bias", "layers.0.blocks.0.attn.blank_k", "layers.0.blocks.0.attn.blank_v",
+                "layers.0.blocks.0.attn.pos_embed.weight", "layers.0.blocks.0.attn.proj.weight",
+                "layers.0.blocks.0.mlp.fc1.weight", "layers.0.blocks.0.mlp.fc2.bias",
+                "layers.0.downsample.weight_net.0.weight", "layers.0.downsample.weight_net.1.bias",
+                "layers.0.downsample.norm.weight", "layers.0.downsample.linear.weight", "layers.0.prob_net.weight",
+                "layers.3.blocks.0.attn.q.weight", "norm.weight", "head.bias"]:
+        assert key in names, key
+    assert not any(k.startswith("layers.3.downsample") or "pre_table" in k for k in names)
+
+
+def test_classifier_runs_on_the_oracle_and_is_deterministic():
+    model = small_model(oracle_ops())
+    x = torch.randn(2, 3, 128, 128, generator=torch.Generator().manual_seed(1))
+    with torch.no_grad():
+        y1, y2 = model(x), model(x)
+    assert y1.shape == (2, 10) and torch.isfinite(y1).all()
+    assert torch.equal(y1, y2)
+    # images of a batch do not interact
+    with torch.no_grad():
+        y_first = model(x[:1])
+    assert torch.allclose(y_first, y1[:1], atol=1e-5)
+
+
+def test_classifier_trains_through_the_oracle():
+    model = small_model(oracle_ops()).train()
+    x = torch.randn(2, 3, 128, 128, generator=torch.Generator().manual_seed(2))
+    model(x).square().mean().backward()
+    missing = [n for n, p in model.named_parameters() if p.grad is None]
+    assert missing == []
+
+
+def _stage_inputs(b, side, c, gen):
+    ys, xs = torch.meshgrid(torch.arange(side), torch.arange(side), indexing="ij")
+    pos = torch.stack([xs, ys], 2).reshape(1, -1, 2).expand(b, -1, -1).float()
+    return pos, torch.randn(b, side * side, c, generator=gen)
+
+
+def test_neighbourhood_lists_are_runs_of_whole_clusters_nearest_first():
+    layer = BasicLayer(32, 64, 8, 48, 1, 2, 2.0, ops=oracle_ops())
+    pos, _ = _stage_inputs(2, 14, 32, torch.Generator().manual_seed(0))         # 196 tokens: 25 clusters, 4 pads
+    new_pos, ranking, member_idx, mask, pe_idx = layer.neighbourhoods(pos, 14, 14, 55, 111)
+    b, n, m = member_idx.shape
+    assert (n, m) == (196, 48) and mask is not None
+    runs = member_idx.reshape(b, n, 6, 8)
+    start = runs[..., 0]
+    full = mask.reshape(b, n, 6, 8).all(-1)
+    # a run is cluster g's members 8g..8g+7; in the padded last cluster the pad slots hold 0 and mask 0
+    assert torch.equal(runs[full], (start[full][:, None] + torch.arange(8)))
+    assert (start % 8 == 0).all()
+    padded = runs[~full]
+    assert padded.numel() > 0 and (padded[:, :4] == torch.arange(192, 196)).all() and (padded[:, 4:] == 0).all()
+    assert (mask.reshape(b, n, 6, 8)[~full][:, 4:] == 0).all()
+    # a token's first run is its own cluster or one at least as near
+    centres = new_pos.new_zeros(b, 25, 2)
+    for g in range(25):
+        centres[:, g] = new_pos[:, 8 * g:min(8 * g + 8, 196)].mean(1)
+    d_first = (new_pos - centres.gather(1, (start[..., 0] // 8)[..., None].expand(-1, -1, 2))).norm(dim=-1)
+    d_own = (new_pos - centres[:, torch.arange(196) // 8]).norm(dim=-1)
+    assert (d_first <= d_own + 1e-6).all()
+    # position-table index = (dy + R) * width + (dx + R) of neighbour minus token
+    nb = new_pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, 2)).reshape(b, n, m, 2)
+    rel = nb - new_pos[:, :, None]
+    assert torch.equal(pe_idx, ((rel[..., 1] + 55) * 111 + rel[..., 0] + 55).long())
+
+
+def test_attention_with_every_token_as_neighbour_equals_the_dense_branch():
+    torch.manual_seed(0)
+    attn = ClusterAttention(32, 2, ops=oracle_ops()).eval()
+    table, r = relative_position_table(64)
+    b, n = 2, 24
+    feat = torch.randn(b, n, 32)
+    pos = torch.stack([torch.randperm(225)[:n] for _ in range(b)])
+    pos = torch.stack([pos % 15, pos // 15], 2).float()
+    rel = (pos[:, None] + r) - pos[:, :, None]
+    pe_idx = (rel[..., 1] * (2 * r + 1) + rel[..., 0]).long()
+    member_idx = torch.arange(n).expand(b, n, n).contiguous()
+    with torch.no_grad():
+        local = attn(feat, member_idx, None, pe_idx, False, table)
+        dense = attn(feat, None, None, pe_idx, True, table)
+    assert torch.allclose(local, dense, atol=1e-5)
+    # masked neighbours get no weight: masking a column equals removing it
+    mask = torch.ones(b, n, n, dtype=torch.int64)
+    mask[:, :, -3:] = 0
+    with torch.no_grad():
+        masked = attn(feat, member_idx, mask, pe_idx, False, table)
+        dropped = attn(feat, member_idx[:, :, :-3].contiguous(), None, pe_idx[:, :, :-3], False, table)
+    assert torch.allclose(masked, dropped, atol=1e-5)
+
+
+def test_merging_keeps_a_quarter_with_reserved_tokens_last_and_orders_channels_ic_major():
+    torch.manual_seed(0)
+    ops = oracle_ops()
+    layer = BasicLayer(16, 32, 8, 48, 1, 2, 2.0, ops=ops).eval()
+    table, r = relative_position_table(64)
+    pos, feat = _stage_inputs(2, 16, 16, torch.Generator().manual_seed(4))
+    new_pos, ranking, member_idx, mask, pe_idx = layer.neighbourhoods(pos, 16, 16, r, 2 * r + 1)
+    feat = feat.gather(1, ranking.expand(-1, -1, 16))
+    merge = layer.downsample
+    prob = torch.rand(2, 256, 1)
+    centre = merge.select(new_pos, prob, 2, 16)
+    assert centre.shape == (2, 64)
+    for b in range(2):
+        assert len(set(centre[b].tolist())) == 64
+        kept = new_pos[b, centre[b, -16:]]
+        assert (kept % 4 == 0).all() and len({tuple(p.tolist()) for p in kept}) == 16
+        assert centre[b, -16:].tolist() == sorted(centre[b, -16:].tolist())
+        # the sampled ones are the best-scored unreserved tokens
+        score = ((new_pos[b] % 2).sum(-1) == 0).float() + 4.0 * prob[b, :, 0]
+        score[(new_pos[b] % 4).sum(-1) == 0] -= 100
+        assert set(centre[b, :48].tolist()) == set(score.topk(48)[1].tolist())
+    with torch.no_grad():
+        out_pos, out = merge(new_pos, feat, member_idx, mask, prob, 2, pe_idx, 16, table)
+        # the same merge spelled out: out[b,i, ic*c + ch] = sum_j w[b,i,j,ic] * feat[b, idx[b,i,j], ch]
+        rows = centre.unsqueeze(2).expand(-1, -1, 48)
+        idx = member_idx.gather(1, rows)
+        w = merge.weight_net(table)[pe_idx.gather(1, rows)] * prob.gather(1, idx.reshape(2, -1, 1)).reshape(2, 64, 48, 1)
+        g = feat.gather(1, idx.reshape(2, -1, 1).expand(-1, -1, 16)).reshape(2, 64, 48, 16)
+        flat = torch.einsum("bijk,bijc->bikc", w, g).reshape(2, 64, 64)
+        assert torch.allclose(out, merge.linear(merge.norm(flat)), atol=1e-5)
+    assert torch.equal(out_pos, new_pos.gather(1, centre.unsqueeze(2).expand(-1, -1, 2)))
+
+
+# ----------------------------------------------------------------------------------------------- GPU
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("amp", [False, True])
+def test_logits_equal_with_hip_operators_and_with_the_oracle(device, amp):
+    from aff.model import default_ops
+    hip = small_model(default_ops(), img_size=128, num_classes=16).to(device)
+    ref = small_model(oracle_ops(), img_size=128, num_classes=16).to(device)
+    ref.load_state_dict(hip.state_dict())
+    x = torch.randn(4, 3, 128, 128, generator=torch.Generator().manual_seed(7)).to(device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16, enabled=amp):
+        y_hip, y_ref = hip(x), ref(x)
+    assert torch.isfinite(y_hip).all()
+    tol = 2e-2 if amp else 1e-4
+    assert oracle.rel_err(y_hip.float(), y_ref.float()) < tol
+
+
+@pytest.mark.gpu
+def test_operator_dtypes_under_autocast(device):
+    """fp16 autocast hands QK fp16 operands and AV / WF fp32 first operands, as in the reference model."""
+    from aff.model import default_ops
+    seen = {}
+    real = default_ops()
+
+    def spy(name, fn):
+        def call(a, b, idx):
+            seen.setdefault(name, (a.dtype, b.dtype, a.is_contiguous(), b.is_contiguous()))
+            return fn(a, b, idx)
+        return call
+    ops = SimpleNamespace(qk=spy("qk", real.qk), av=spy("av", real.av), wf=spy("wf", real.wf))
+    model = small_model(ops, img_size=128).to(device)
+    x = torch.randn(2, 3, 128, 128, device=device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        model(x)
+    assert seen["qk"][:2] == (torch.float16, torch.float16)
+    assert seen["av"][:2] == (torch.float32, torch.float16)
+    assert seen["wf"][0] == torch.float32
+    # q, key and v reach the operators as permuted views, not copies
+    assert seen["qk"][2:] == (False, False) and seen["av"][3] is False
+
+
+@pytest.mark.gpu
+def test_aff_tiny_224_forward_and_gradients(device):
+    model = aff_tiny().to(device)
+    x = torch.randn(2, 3, 224, 224, device=device)
+    model.eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        y = model(x)
+    assert y.shape == (2, 1000) and torch.isfinite(y).all()
+    model.train()
+    model(x).square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
