@@ -49,7 +49,11 @@ namespace clusten {
 //   [0, G_BYTES)            gathered rows of one head (16*Q rows); reused to turn the D blocks into
 //                           the row-major output chunk once the operands are in registers
 //   [A_BASE, +2*A_SLOT)     a-rows of two heads (slot h % 2)
-template <typename T, int C, int Q>
+//   union path only (FAST kernels):
+//   [0, G_BYTES)            rows of 2*Q distinct runs per pass; reused for the score matrix of the pass
+//   [ULIST_BASE, +512)      row indices of up to U_MAX distinct runs, 8 per run
+//   [USLOT_BASE, +256)      distinct-run number of each of the tile's runs
+template <typename T, int C, int Q, bool UNION>
 struct Staging {
     static constexpr int RB = C * (int)sizeof(T);               // bytes per row
     static constexpr int PPR = RB / 16;                         // 16-byte pieces per row
@@ -57,10 +61,18 @@ struct Staging {
     static constexpr int NI_G = (16 * Q + RPI - 1) / RPI;       // accesses for the gathered rows of a chunk
     static constexpr int NI_A = (kTileTokens + RPI - 1) / RPI;  // accesses for the tile's a-rows
     static constexpr int OUT_BYTES = kTileTokens * 16 * Q * (int)sizeof(T);  // one (tile, head) output chunk
-    static constexpr int G_BYTES = NI_G * 1024 > OUT_BYTES ? NI_G * 1024 : (OUT_BYTES + 1023) / 1024 * 1024;
+    static constexpr int QU = Q;                                // slot blocks per pass of the union path
+    static constexpr int NI_U = NI_G;                           // accesses for the rows of a union pass
+    static constexpr int U_MAX = 16;                            // distinct runs the union path holds
+    static constexpr int SROW = 16 * QU + 4;                    // floats per token row of the score matrix
+    static constexpr int U_BYTES = UNION ? kTileTokens * SROW * 4 : 0;
+    static constexpr int G_PLAIN = NI_G * 1024 > OUT_BYTES ? NI_G * 1024 : (OUT_BYTES + 1023) / 1024 * 1024;
+    static constexpr int G_BYTES = G_PLAIN > U_BYTES ? G_PLAIN : (U_BYTES + 1023) / 1024 * 1024;
     static constexpr int A_BASE = G_BYTES;
     static constexpr int A_SLOT_BYTES = NI_A * 1024;
-    static constexpr int BYTES = G_BYTES + 2 * A_SLOT_BYTES;
+    static constexpr int ULIST_BASE = A_BASE + 2 * A_SLOT_BYTES;
+    static constexpr int USLOT_BASE = ULIST_BASE + (UNION ? U_MAX * 8 * 4 : 0);
+    static constexpr int BYTES = USLOT_BASE + (UNION ? kWave * 4 : 0);
     static constexpr int EL = C / 4;                            // channels per lane (a quarter row)
     static constexpr int QB = RB / 4;                           // bytes per lane
     static constexpr int UNIT = QB < 16 ? QB : 16;              // bytes per LDS read
@@ -81,7 +93,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                                                                 T* __restrict__ out, int H, int N, int M,
                                                                 clusten_strides as, clusten_strides rs,
                                                                 int tiles_per_batch, int total_tiles) {
-    typedef Staging<T, C, Q> S;
+    typedef Staging<T, C, Q, FAST> S;
     typedef VecIO<T, S::VEC> RunIO;
     typedef VecIO<T, 4> OutIO;
     static_assert(C % 16 == 0, "a lane holds a quarter of a row in whole 4-element groups");
@@ -155,6 +167,154 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
             list0 = (int)wide[0];
         }
         const bool shared_list = __all(same ? 1 : 0) != 0;
+
+        if constexpr (FAST) {
+            if (!shared_list && (M & 7) == 0) {
+                // ---- union path: lists made of runs of 8 slots, many of them common to several tokens ----
+                // (the neighbourhoods of a cluster-ordered sequence: a run is the 8 members of one cluster, and
+                // the tokens of a tile pick their clusters from the same dozen.)  Every distinct run is gathered
+                // and multiplied once per head; each token then picks its own slots from the score matrix.
+                constexpr int QU = S::QU;
+                constexpr int UROWS = 16 * QU;   // union rows per pass
+                const int R = M >> 3;             // runs per token
+                const int nruns = nt * R;         // <= 64: lane rho owns run rho = token * R + run
+                int v[8];
+                {
+                    const int64_t* p = idx_tile + (int64_t)min(lane, nruns - 1) * 8;  // the tile's lists are contiguous
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) v[t] = (int)p[t];
+                }
+                bool regular = true;  // 8 consecutive rows
+#pragma unroll
+                for (int t = 1; t < 8; ++t) regular = regular && (v[t] == v[0] + t);
+                const int key = regular ? v[0] : ~lane;  // other runs never merge
+
+                // number the distinct keys in order of first appearance
+                uint64_t remaining = nruns >= 64 ? ~0ull : ((1ull << nruns) - 1);
+                int uslot = 0, U = 0;
+                bool first = false;
+                while (remaining != 0 && U < S::U_MAX) {
+                    const int s = __builtin_ctzll(remaining);
+                    const int ks = __builtin_amdgcn_readlane(key, s);
+                    const bool hit = key == ks;
+                    const uint64_t match = __ballot(hit) & remaining;
+                    if (hit) uslot = U;
+                    first = first || lane == s;
+                    remaining &= ~match;
+                    ++U;
+                }
+                if (remaining == 0) {  // at most U_MAX distinct runs; tiles with more take the per-token passes
+                int* ulist = reinterpret_cast<int*>(stage + S::ULIST_BASE);
+                int* uslots = reinterpret_cast<int*>(stage + S::USLOT_BASE);
+                if (first) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) ulist[uslot * 8 + t] = v[t];
+                }
+                if (lane < nruns) uslots[lane] = uslot;
+                __syncthreads();
+
+                // this lane's share of the output chunk: groups of 4 consecutive elements (inside one run)
+                constexpr int NQD = (kTileTokens * 16 * Q / 4 + kWave - 1) / kWave;
+                int sidx[NQD], qtok[NQD];
+                bool qvalid[NQD];
+#pragma unroll
+                for (int k = 0; k < NQD; ++k) {
+                    const int e = 4 * (lane + kWave * k);
+                    qvalid[k] = e < nt * M;
+                    const int ec = qvalid[k] ? e : 0;
+                    const int i = ec / M, j = ec - i * M;
+                    qtok[k] = i;
+                    sidx[k] = uslots[i * R + (j >> 3)] * 8 + (j & 7);
+                }
+
+                const int total_rows = 8 * U;
+                for (int h = 0; h < H; ++h) {
+                    const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+                    F32x4 val[NQD];
+#pragma unroll
+                    for (int k = 0; k < NQD; ++k) val[k] = F32x4{0.f, 0.f, 0.f, 0.f};
+                    for (int base = 0; base < total_rows; base += UROWS) {
+                        const int rows_here = min(UROWS, total_rows - base);
+                        __syncthreads();  // the previous pass has picked its scores
+#pragma unroll
+                        for (int i = 0; i < S::NI_U; ++i) {
+                            if (i * S::RPI < rows_here) {
+                                const int srow = i * S::RPI + g_sub;
+                                const uint32_t urow = (uint32_t)ulist[min(base + srow, total_rows - 1)];
+                                CLUSTEN_LDS_DMA16(rows_bh + (urow * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
+                                                  stage + i * 1024);
+                            }
+                        }
+                        if (h >= 2 && base == 0) fetch_a(h);
+                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                        __syncthreads();
+
+                        typename RunIO::raw g_raw[QU][S::NU];
+                        typename RunIO::raw a_raw[S::NU];
+#pragma unroll
+                        for (int u = 0; u < S::NU; ++u) {
+#pragma unroll
+                            for (int blk = 0; blk < QU; ++blk) {
+                                if (blk * 16 < rows_here) {
+                                    g_raw[blk][u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] +
+                                                                                                  blk * 16 * S::RB);
+                                }
+                            }
+                            a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] +
+                                                                                     (h & 1) * S::A_SLOT_BYTES);
+                        }
+                        __syncthreads();  // operands are in registers: the rows make room for the scores
+
+                        float bop[S::EL];
+#pragma unroll
+                        for (int u = 0; u < S::NU; ++u) {
+                            float x[S::VEC];
+                            RunIO::unpack(a_raw[u], x);
+#pragma unroll
+                            for (int e = 0; e < S::VEC; ++e) bop[u * S::VEC + e] = x[e];
+                        }
+#pragma unroll
+                        for (int blk = 0; blk < QU; ++blk) {
+                            if (blk * 16 < rows_here) {
+                                F32x4 d = F32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                                for (int u = 0; u < S::NU; ++u) {
+                                    float x[S::VEC];
+                                    RunIO::unpack(g_raw[blk][u], x);
+#pragma unroll
+                                    for (int e = 0; e < S::VEC; ++e) {
+                                        d = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], bop[u * S::VEC + e], d, 0, 0, 0);
+                                    }
+                                }
+                                // lane (r, kq): union rows 16*blk + 4*kq .. +3 of token r
+                                if (r < kTileTokens) {
+                                    *reinterpret_cast<F32x4*>(stage + (r * S::SROW + 16 * blk + 4 * kq) * 4) = d;
+                                }
+                            }
+                        }
+                        __syncthreads();
+#pragma unroll
+                        for (int k = 0; k < NQD; ++k) {
+                            const int sl = sidx[k] - base;
+                            if (sl >= 0 && sl < UROWS) {
+                                val[k] = *reinterpret_cast<const F32x4*>(stage + (qtok[k] * S::SROW + sl) * 4);
+                            }
+                        }
+                    }
+                    char* out_h = out_tile + (int64_t)h * N * M * sizeof(T);
+#pragma unroll
+                    for (int k = 0; k < NQD; ++k) {
+                        if (qvalid[k]) {
+                            float o[4] = {val[k][0], val[k][1], val[k][2], val[k][3]};
+                            *reinterpret_cast<typename OutIO::raw*>(out_h + (lane + kWave * k) * 4 * (int)sizeof(T)) =
+                                OutIO::pack(o);
+                        }
+                    }
+                }
+                return;
+                }
+            }
+        }
 
         // the list entry of staging row i*RPI + g_sub lives in the lane of that slot
         int src_lane[S::NI_G];

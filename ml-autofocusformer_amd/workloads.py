@@ -125,6 +125,42 @@ class WfCase:
         return WfCase(self.name, self.weights.to(device), self.feat.to(device), self.nbhd_idx.to(device))
 
 
+def run_lists(B: int, N: int, M: int, gen, kind: str = "clusters", spread: int = 12) -> torch.Tensor:
+    """Lists made of runs of 8 slots, the shape the model's neighbourhoods have, with the irregularities real
+    sequences show.  Token i draws its M/8 runs from the `spread` clusters around its own.
+
+      clusters   every run is the 8 members 8g..8g+7 of a cluster, clusters distinct per token
+      unaligned  runs of 8 consecutive rows starting anywhere
+      padded     as clusters, but a last cluster of N % 8 (or 4) members whose other slots hold index 0
+      scattered  every token draws from the whole sequence: few runs are common to the tokens of a tile
+      repeated   as clusters, and every token's second run repeats its first
+    """
+    R = M // 8
+    assert M % 8 == 0 and N >= 8 * R
+    G = (N + 7) // 8 if kind == "padded" else N // 8   # clusters to draw from (whole ones unless padded)
+    own = (torch.arange(N) // 8).clamp(max=G - 1)
+    lo = (own - spread // 2).clamp(min=0, max=max(G - spread, 0))
+    width = min(spread, G) if kind != "scattered" else G
+    if kind == "scattered":
+        lo = torch.zeros_like(lo)
+    keys = torch.rand(B, N, width, generator=gen)
+    pick = keys.argsort(dim=2)[:, :, :R] + lo.view(1, N, 1)            # (B, N, R) distinct clusters
+    if kind == "repeated" and R > 1:
+        pick[:, :, 1] = pick[:, :, 0]
+    base = pick * 8
+    if kind == "unaligned":
+        base = (base + torch.randint(0, 8, base.shape, generator=gen)).clamp(max=N - 8)
+    idx = (base.unsqueeze(3) + torch.arange(8).view(1, 1, 1, 8)).reshape(B, N, M)
+    if kind == "padded":
+        tail = N % 8 if N % 8 else 4              # members of the short last cluster
+        last = (N - 1) // 8 * 8
+        run = torch.arange(last, last + 8)
+        run[tail:] = 0
+        hit = (idx.reshape(B, N, R, 8)[..., 0] == last)
+        idx = torch.where(hit.unsqueeze(3), run.view(1, 1, 1, 8), idx.reshape(B, N, R, 8)).reshape(B, N, M)
+    return idx.contiguous()
+
+
 def attn_case(name: str, config_id: int, B: int, H: int, N: int, C: int, M: int = NBHD, dtype=torch.float32,
               scale_q: bool = True, lists: str = "windowed") -> AttnCase:
     gen = generator(config_id)
@@ -141,6 +177,8 @@ def attn_case(name: str, config_id: int, B: int, H: int, N: int, C: int, M: int 
         idx = model_like_lists(B, N, gen, canonical=True)
     elif lists == "random":
         idx = torch.randint(N, (B, N, M), generator=gen)
+    elif lists.startswith("runs:"):
+        idx = run_lists(B, N, M, gen, kind=lists[5:])
     else:
         raise ValueError(lists)
     return AttnCase(name, q.to(dtype), k.to(dtype), v.to(dtype), idx)

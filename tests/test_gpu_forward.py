@@ -70,6 +70,20 @@ def test_reference_script_shape(device):
                 torch.float32)
 
 
+@pytest.mark.parametrize("kind", ["clusters", "unaligned", "padded", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_lists_made_of_runs_of_eight(device, kind, dtype):
+    # the tokens of a tile share most of their runs (not "scattered": up to 48 distinct runs, several passes);
+    # N = 396 leaves a partial last tile, "padded" puts index 0 into the runs of a short last cluster
+    _check_attn(wl.attn_case("runs", 61, B=2, H=3, N=396, C=32, lists="runs:" + kind), device, dtype)
+
+
+@pytest.mark.parametrize("c,m", [(16, 48), (64, 48), (32, 16), (32, 64), (64, 64), (16, 8)])
+def test_lists_made_of_runs_other_head_dims_and_lengths(device, c, m):
+    _check_attn(wl.attn_case("runs", 62, B=2, H=2, N=200, C=c, M=m, lists="runs:clusters"), device, torch.float32)
+    _check_attn(wl.attn_case("runs", 63, B=1, H=2, N=200, C=c, M=m, lists="runs:scattered"), device, torch.bfloat16)
+
+
 @pytest.mark.parametrize("n", [49, 197, 8, 5])
 def test_partial_tiles(device, n):
     m = min(48, n) if n >= 48 else 4
