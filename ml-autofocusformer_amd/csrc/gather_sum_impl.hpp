@@ -48,7 +48,12 @@ namespace clusten {
 //                         blocks into the row-major output chunk
 //   [P_BASE, +2*P_SLOT)   p pieces of two heads (slot h % 2), piece-transposed: piece (slot group s,
 //                         token t) at (s*8 + t)*16
-template <typename T, int C, int Q>
+//   union path only (FAST kernels):
+//   (over the p slots)    p of one pass re-indexed by distinct run, as MFMA A operands: element
+//                         (k index kq, token t, step s) at ((kq*8 + t)*PM_STRIDE + s)*4;
+//                         distinct-run number of each of the tile's runs; row indices of up to
+//                         U_MAX distinct runs, 8 per run
+template <typename T, int C, int Q, bool UNION>
 struct SumStaging {
     static constexpr int RB = C * (int)sizeof(T);               // bytes per gathered row
     static constexpr int PPR = RB / 16;                         // 16-byte pieces per row
@@ -61,9 +66,17 @@ struct SumStaging {
     static constexpr int NI_P = (P_PIECES + kWave - 1) / kWave;  // accesses for them
     static constexpr int P_BASE = G_BYTES;
     static constexpr int P_SLOT_BYTES = NI_P * 1024;
-    static constexpr int BYTES = G_BYTES + 2 * P_SLOT_BYTES;
     static constexpr int ECH = C / 16;                          // channels per lane = channel blocks
     static constexpr int STEPS = 4 * Q;                         // MFMA steps per chunk
+    // the union path's tables take the place of the two p slots once their pieces are in registers
+    static constexpr int PM_STRIDE = STEPS % 8 == 4 ? STEPS : STEPS + 4;  // floats; odd multiple of 4: conflict-free rows
+    static constexpr int PM_BASE = P_BASE;
+    static constexpr int PM_BYTES = 4 * kTileTokens * PM_STRIDE * 4;
+    static constexpr int USLOT_BASE = PM_BASE + PM_BYTES;       // one byte per run of the tile
+    static constexpr int ULIST_BASE = USLOT_BASE + kWave;
+    static constexpr int U_FIT = (2 * P_SLOT_BYTES - PM_BYTES - kWave) / 32;
+    static constexpr int U_MAX = !UNION || U_FIT < 1 ? 0 : (U_FIT < 16 ? U_FIT : 16);  // distinct runs the union path holds
+    static constexpr int BYTES = G_BYTES + 2 * P_SLOT_BYTES;
     static_assert(RB >= 32 && kWave % PPR == 0, "row size");
 };
 
@@ -76,7 +89,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                                                                 T* __restrict__ out, int H, int N, int M,
                                                                 clusten_strides rs, clusten_strides os,
                                                                 int tiles_per_batch, int total_tiles) {
-    typedef SumStaging<T, C, Q> S;
+    typedef SumStaging<T, C, Q, FAST> S;
     typedef VecIO<T, S::ECH> ChIO;   // the lane's channels of one gathered row
     typedef VecIO<T, S::SPP> PieceIO;
     static_assert(C == 16 || C == 32 || C == 64, "channel blocks of 16");
@@ -142,6 +155,211 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     const int lds_p = (n & 7) * 16;                                     // the lane's token inside a slot group
     // out: lane (n, kq) holds tokens 4*kq + i of channels n*ECH + e
     const bool rows_contiguous = os.n == C;
+
+    // store of one head: lane (n, kq) holds tokens 4*kq + i of channels n*ECH + e.  `whole` = every token of
+    // the tile is written: when the out rows of the tile are contiguous too, they are laid out row-major in
+    // LDS (over the gathered rows) and leave with full-width 16-byte stores.
+    auto store_head = [&](int h, F32x4 (&d)[S::ECH], int tok_lo, int tok_hi, bool whole) {
+        char* out_h = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
+        if (FAST && whole && rows_contiguous) {
+            __syncthreads();  // every operand read of this head is complete: reuse the row area
+            if (kq < 2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v[S::ECH];
+#pragma unroll
+                    for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
+                    *reinterpret_cast<typename ChIO::raw*>(stage + ((4 * kq + i) * C + n * S::ECH) * (int)sizeof(T)) =
+                        ChIO::pack(v);
+                }
+            }
+            __syncthreads();
+            constexpr int NO = (kTileTokens * S::RB + 1023) / 1024;
+            Piece o[NO];
+#pragma unroll
+            for (int i = 0; i < NO; ++i) {
+                o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
+            }
+            __syncthreads();  // the chunk is in registers: the next head's gather may overwrite it
+            const int chunk_bytes = nt * S::RB;
+#pragma unroll
+            for (int i = 0; i < NO; ++i) {
+                const int off = i * 1024 + lane * 16;
+                if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
+            }
+        } else {
+            if (FAST) __syncthreads();  // operand reads complete before the next head's gather
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int tok = 4 * kq + i;
+                if (tok >= tok_lo && tok < tok_hi) {
+                    float v[S::ECH];
+#pragma unroll
+                    for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
+                    *reinterpret_cast<typename ChIO::raw*>(out_h + ((int64_t)tok * os.n + n * S::ECH) * sizeof(T)) =
+                        ChIO::pack(v);
+                }
+            }
+        }
+    };
+
+    if constexpr (FAST && S::U_MAX > 0) {
+        if (!shared_list && (M & 7) == 0) {
+            // ---- union path: lists made of runs of 8 slots, many of them common to several tokens ----
+            // (the neighbourhoods of a cluster-ordered sequence: a run is the 8 members of one cluster.)
+            // Every distinct run is gathered once per head; the p values are re-indexed by distinct run
+            // (zero where a token does not hold the run), so one set of MFMAs serves the 8 tokens.
+            constexpr int PROWS = 16 * Q;     // union rows per pass
+            const int R = M >> 3;             // runs per token
+            const int nruns = nt * R;         // <= 64: lane rho owns run rho = token * R + run
+            int v[8];
+            {
+                const int64_t* lp = idx_tile + (int64_t)min(lane, nruns - 1) * 8;  // the tile's lists are contiguous
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = (int)lp[t];
+            }
+            bool regular = true;  // 8 consecutive rows
+#pragma unroll
+            for (int t = 1; t < 8; ++t) regular = regular && (v[t] == v[0] + t);
+            const int key = regular ? v[0] : ~lane;  // other runs never merge
+
+            // number the distinct keys in order of first appearance
+            uint64_t remaining = nruns >= 64 ? ~0ull : ((1ull << nruns) - 1);
+            // lanes below this one that hold runs of the same token: a run held twice by one token would need
+            // two p values in one place of the re-indexed p
+            const uint64_t same_token_below = ((1ull << lane) - 1) & ~((1ull << (lane / R * R)) - 1);
+            int uslot = 0, U = 0;
+            bool first = false, twice = false;
+            while (remaining != 0 && U < S::U_MAX) {
+                const int sl = __builtin_ctzll(remaining);
+                const int ks = __builtin_amdgcn_readlane(key, sl);
+                const bool hit = key == ks;
+                const uint64_t match = __ballot(hit) & remaining;
+                if (hit) uslot = U;
+                twice = twice || (hit && lane < nruns && (match & same_token_below) != 0);
+                first = first || lane == sl;
+                remaining &= ~match;
+                ++U;
+            }
+            // at most U_MAX distinct runs and no token holds a run twice; other tiles take the per-token passes
+            if (remaining == 0 && __any(twice ? 1 : 0) == 0) {
+                // The p pieces of heads 0 and 1 are on their way into the two p slots: take them into
+                // registers; from then on the slots hold the run tables and the re-indexed p, and the
+                // pieces of the later heads come straight from global memory, one head ahead.
+                typename PieceIO::raw cur[S::NI_P], nxt[S::NI_P];
+                __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                __syncthreads();
+#pragma unroll
+                for (int k = 0; k < S::NI_P; ++k) {
+                    cur[k] = *reinterpret_cast<const typename PieceIO::raw*>(stage + S::P_BASE + (k * kWave + lane) * 16);
+                    nxt[k] = *reinterpret_cast<const typename PieceIO::raw*>(stage + S::P_BASE + S::P_SLOT_BYTES +
+                                                                            (k * kWave + lane) * 16);
+                }
+                __syncthreads();
+                int* ulist = reinterpret_cast<int*>(stage + S::ULIST_BASE);
+                unsigned char* uslots = reinterpret_cast<unsigned char*>(stage + S::USLOT_BASE);
+                float* pm = reinterpret_cast<float*>(stage + S::PM_BASE);
+                if (first) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) ulist[uslot * 8 + t] = v[t];
+                }
+                if (lane < nruns) uslots[lane] = (unsigned char)uslot;
+                __syncthreads();
+
+                // p piece q = 64*k + lane of a head: SPP slots of token q % 8 from slot (q / 8) * SPP on.
+                // They go to union rows prow .. prow + SPP - 1, i.e. pass prow / PROWS, elements
+                // pm[pm_at + (e % 4) * 8 * PM_STRIDE + e / 4].
+                int ppass[S::NI_P], pm_at[S::NI_P];
+                const T* p_src[S::NI_P];
+#pragma unroll
+                for (int k = 0; k < S::NI_P; ++k) {
+                    const int q = k * kWave + lane;
+                    const int j = (q / kTileTokens) * S::SPP;
+                    const int tok = q % kTileTokens;
+                    const bool valid = j < M && tok < nt;
+                    const int prow = valid ? uslots[tok * R + (j >> 3)] * 8 + (j & 7) : 0;
+                    ppass[k] = valid ? prow / PROWS : -1;
+                    const int rr = prow % PROWS;
+                    pm_at[k] = tok * S::PM_STRIDE + (rr >> 2);
+                    p_src[k] = p + (((int64_t)b * H) * N + i0 + min(tok, nt - 1)) * M + min(j, M - S::SPP);
+                }
+                const int total_rows = 8 * U;
+                const float* pm_lane = pm + (kq * kTileTokens + (n & 7)) * S::PM_STRIDE;
+
+                for (int h = 0; h < H; ++h) {
+                    const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+                    if (h >= 1 && h + 1 < H) {
+#pragma unroll
+                        for (int k = 0; k < S::NI_P; ++k) {
+                            nxt[k] = *reinterpret_cast<const typename PieceIO::raw*>(p_src[k] + (int64_t)(h + 1) * N * M);
+                        }
+                    }
+                    F32x4 d[S::ECH];
+#pragma unroll
+                    for (int e = 0; e < S::ECH; ++e) d[e] = F32x4{0.f, 0.f, 0.f, 0.f};
+                    float pv[S::NI_P][S::SPP];
+#pragma unroll
+                    for (int k = 0; k < S::NI_P; ++k) PieceIO::unpack(cur[k], pv[k]);
+
+                    for (int base = 0, pass = 0; base < total_rows; base += PROWS, ++pass) {
+                        const int rows_here = min(PROWS, total_rows - base);
+                        const int rows_batched = (rows_here + 15) & ~15;  // MFMA batches cover 16 rows
+                        __syncthreads();  // the previous pass (or head) has read its operands
+#pragma unroll
+                        for (int i = 0; i < S::NI_G; ++i) {
+                            if (i * S::RPI < rows_batched) {  // rows past the last one repeat it (their p is zero)
+                                const uint32_t urow = (uint32_t)ulist[min(base + i * S::RPI + g_sub, total_rows - 1)];
+                                CLUSTEN_LDS_DMA16(rows_bh + (urow * row_pitch + (uint32_t)(g_pos * 16)), stage + i * 1024);
+                            }
+                        }
+                        // clear the re-indexed p of this pass, then add this pass's pieces
+#pragma unroll
+                        for (int z = lane * 16; z < S::PM_BYTES; z += kWave * 16) {
+                            *reinterpret_cast<F32x4*>(stage + S::PM_BASE + z) = F32x4{0.f, 0.f, 0.f, 0.f};
+                        }
+                        __syncthreads();
+#pragma unroll
+                        for (int k = 0; k < S::NI_P; ++k) {
+                            if (ppass[k] == pass) {
+#pragma unroll
+                                for (int e = 0; e < S::SPP; ++e) {
+                                    pm[pm_at[k] + (e & 3) * kTileTokens * S::PM_STRIDE + (e >> 2)] = pv[k][e];
+                                }
+                            }
+                        }
+                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+                        __syncthreads();
+
+                        // batches of 4 steps (16 union rows = 2 runs); batches past the last row are skipped
+#pragma unroll
+                        for (int sb = 0; sb < S::STEPS; sb += 4) {
+                            if (sb * 4 < rows_here) {
+                                const F32x4 a4 = *reinterpret_cast<const F32x4*>(pm_lane + sb);
+                                typename ChIO::raw g_raw[4];
+#pragma unroll
+                                for (int ss = 0; ss < 4; ++ss) {
+                                    g_raw[ss] = *reinterpret_cast<const typename ChIO::raw*>(stage + 4 * (sb + ss) * S::RB + lds_g);
+                                }
+#pragma unroll
+                                for (int ss = 0; ss < 4; ++ss) {
+                                    float g[S::ECH];
+                                    ChIO::unpack(g_raw[ss], g);
+#pragma unroll
+                                    for (int e = 0; e < S::ECH; ++e) {
+                                        d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[ss], g[e], d[e], 0, 0, 0);
+                                    }
+                                }
+                            }
+                        }
+                    }
+                    store_head(h, d, 0, nt, true);
+#pragma unroll
+                    for (int k = 0; k < S::NI_P; ++k) cur[k] = nxt[k];
+                }
+                return;
+            }
+        }
+    }
 
     // shared list: one pass that serves all tokens; otherwise one pass per token that keeps its row
     const int passes = shared_list ? 1 : nt;
@@ -241,48 +459,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 }
             }
 
-            // store: lane (n, kq) holds tokens 4*kq + i, channels n*ECH + e
-            char* out_h = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
-            if (FAST && shared_list && rows_contiguous) {
-                __syncthreads();  // every operand read of this head is complete: reuse the row area
-                if (kq < 2) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        float v[S::ECH];
-#pragma unroll
-                        for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
-                        *reinterpret_cast<typename ChIO::raw*>(stage + ((4 * kq + i) * C + n * S::ECH) * (int)sizeof(T)) =
-                            ChIO::pack(v);
-                    }
-                }
-                __syncthreads();
-                constexpr int NO = (kTileTokens * S::RB + 1023) / 1024;
-                Piece o[NO];
-#pragma unroll
-                for (int i = 0; i < NO; ++i) {
-                    o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
-                }
-                __syncthreads();  // the chunk is in registers: the next head's gather may overwrite it
-                const int chunk_bytes = nt * S::RB;
-#pragma unroll
-                for (int i = 0; i < NO; ++i) {
-                    const int off = i * 1024 + lane * 16;
-                    if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
-                }
-            } else {
-                if (FAST) __syncthreads();  // operand reads complete before the next head's gather
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int tok = 4 * kq + i;
-                    if (tok >= tok_lo && tok < tok_hi) {
-                        float v[S::ECH];
-#pragma unroll
-                        for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
-                        *reinterpret_cast<typename ChIO::raw*>(out_h + ((int64_t)tok * os.n + n * S::ECH) * sizeof(T)) =
-                            ChIO::pack(v);
-                    }
-                }
-            }
+            store_head(h, d, tok_lo, tok_hi, shared_list);
         }
     }
 }
