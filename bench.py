@@ -169,7 +169,9 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
         return call
 
     real = aff_model.default_ops()
-    ops = SimpleNamespace(qk=timed_call("qk", real.qk), av=timed_call("av", real.av), wf=timed_call("wf", real.wf))
+    ops = SimpleNamespace(**vars(real))
+    ops.qk, ops.av, ops.wf = timed_call("qk", real.qk), timed_call("av", real.av), timed_call("wf", real.wf)
+    ops.attn_softmax = timed_call("bias+mask+blank+softmax", real.attn_softmax)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()
     for layer in net.layers:
         layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)

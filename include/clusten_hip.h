@@ -54,7 +54,7 @@ typedef enum clusten_status {
     CLUSTEN_ERR_BAD_STRIDE = 4,     /* a stride is negative or makes rows overlap */
     CLUSTEN_ERR_WORKSPACE = 5,      /* workspace missing or smaller than *_workspace_bytes() */
     CLUSTEN_ERR_LAUNCH = 6,         /* hipGetLastError() reported a failure after a launch */
-    CLUSTEN_ERR_UNALIGNED = 7       /* clusten_copy_probe only: a pointer is not 16-byte aligned
+    CLUSTEN_ERR_UNALIGNED = 7       /* clusten_copy_probe, clusten_attn_softmax_forward: a pointer is not 16-byte aligned
                                        (the gather ops route unaligned operands to element-wise kernels) */
 } clusten_status;
 
@@ -151,6 +151,24 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
                         const int64_t* nbhd_idx, void* d_weights, void* d_feat,
                         void* workspace, size_t workspace_bytes,
                         clusten_wf_shape shape, int dtype, clusten_stream stream);
+
+/* ---- glue between QK and AV (optional) -------------------------------------------------------- */
+
+/* The arithmetic the model does between CLUSTENQKFunction and CLUSTENAVFunction, in one pass:
+ *   probs[b,h,i,:M], blank_prob[b,h,i] = softmax over the M neighbours and one blank token of
+ *     attn[b,h,i,j] + bias_table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])   and   blank_logit[b,h,i].
+ * It has no entry point in the reference, which writes these steps as tensor expressions
+ * (models/aff_transformer.py:122-147: position-bias gather, two additions, cat with the blank token,
+ * softmax, two slices); it replaces those for inference and leaves the three operators as they are.
+ *   attn (B,H,N,M) and bias_table (rows,H): `dtype` (F32, F16 or BF16), contiguous;
+ *   pe_idx (B,N,M) int64 with values in [0, rows) — unchecked; mask (B,N,M) int64 of 0/1, or NULL;
+ *   blank_logit (B,H,N), probs (B,H,N,M), blank_prob (B,H,N): fp32, contiguous.
+ * shape.C is ignored (pass the head dim).  M <= 64 and M % 4 == 0, else CLUSTEN_ERR_BAD_DIMS;
+ * attn and probs 16-byte aligned, else CLUSTEN_ERR_UNALIGNED. */
+int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx,
+                                 const int64_t* mask, const float* blank_logit, float* probs,
+                                 float* blank_prob, clusten_attn_shape shape, int dtype,
+                                 clusten_stream stream);
 
 /* ---- measurement aid ------------------------------------------------------------------------ */
 

@@ -30,8 +30,9 @@ from .points import knn, space_filling_cluster
 
 def default_ops():
     """The three operators as the HIP library provides them."""
-    from clusten import CLUSTENAVFunction, CLUSTENQKFunction, CLUSTENWFFunction
-    return SimpleNamespace(qk=CLUSTENQKFunction.apply, av=CLUSTENAVFunction.apply, wf=CLUSTENWFFunction.apply)
+    from clusten import CLUSTENAVFunction, CLUSTENQKFunction, CLUSTENWFFunction, _native
+    return SimpleNamespace(qk=CLUSTENQKFunction.apply, av=CLUSTENAVFunction.apply, wf=CLUSTENWFFunction.apply,
+                           attn_softmax=_native.attn_softmax, attn_softmax_supported=_native.attn_softmax_supported)
 
 
 def relative_position_table(img_size):
@@ -106,14 +107,19 @@ class ClusterAttention(nn.Module):
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
 
         bias = self.pos_embed(table)                                                     # (rows, h)
-        attn = attn + bias[pe_idx].permute(0, 3, 1, 2)
-        if cluster_mask is not None and not global_attn:
-            attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
-
         blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)            # (b,h,n,1)
-        attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
-        attn = self.attn_drop(attn)
-        blank, attn = attn[..., -1:], attn[..., :-1]
+        fused = getattr(self.ops, "attn_softmax", None)
+        if (fused is not None and not global_attn and not torch.is_grad_enabled()
+                and not (self.training and self.attn_drop.p > 0) and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
+            # inference: bias gather, mask, blank token and softmax in one kernel
+            attn, blank = fused(attn, bias, pe_idx, cluster_mask, blank)
+        else:
+            attn = attn + bias[pe_idx].permute(0, 3, 1, 2)
+            if cluster_mask is not None and not global_attn:
+                attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
+            attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
+            attn = self.attn_drop(attn)
+            blank, attn = attn[..., -1:], attn[..., :-1]
 
         out = attn @ v if global_attn else self.ops.av(attn, v, member_idx)              # (b,h,n,ch)
         out = out + blank * self.blank_v.reshape(1, h, 1, ch)
@@ -256,10 +262,12 @@ class BasicLayer(nn.Module):
                 if key not in self._grid_cache:
                     self._grid_cache[key] = self.neighbourhoods(pos[:1], h, w, radius, table_width)
                 pos1, ranking, member_idx, mask, pe_idx = self._grid_cache[key]
+                if (key, b) not in self._grid_cache:   # the batch-sized copies the operators read
+                    self._grid_cache[(key, b)] = (member_idx.expand(b, -1, -1).contiguous(),
+                                                  pe_idx.expand(b, -1, -1).contiguous(),
+                                                  None if mask is None else mask.expand(b, -1, -1).contiguous())
+                member_idx, pe_idx, mask = self._grid_cache[(key, b)]
                 pos = pos1.expand(b, -1, -1)
-                member_idx = member_idx.expand(b, -1, -1).contiguous()
-                pe_idx = pe_idx.expand(b, -1, -1)
-                mask = None if mask is None else mask.expand(b, -1, -1)
                 if ranking is not None:
                     feat = feat[:, ranking[0, :, 0]]
             else:

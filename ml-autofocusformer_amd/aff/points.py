@@ -34,10 +34,19 @@ def knn(query, database, k, return_dist=False, chunk_elems=1 << 27):
         for axis in range(q.shape[2]):
             diff = q[:, :, None, axis] - x[:, None, :, axis]
             d2 = diff * diff if d2 is None else d2 + diff * diff
-        dist, idx = torch.sort(d2, dim=2, stable=True)
-        idx_parts.append(idx[:, :, :k])
+        if k * 8 <= n:
+            # few of many: the k smallest of the 64-bit keys (distance bits, index) — non-negative floats order
+            # like their bit patterns, so this is the order of the full stable sort without sorting everything
+            key = (d2.view(torch.int32).long() << 32) | torch.arange(n, device=d2.device)
+            key = torch.topk(key, k, dim=2, largest=False, sorted=True)[0]
+            idx = key & 0xFFFFFFFF
+            dist = (key >> 32).int().view(torch.float32)
+        else:
+            dist, idx = torch.sort(d2, dim=2, stable=True)
+            dist, idx = dist[:, :, :k], idx[:, :, :k]
+        idx_parts.append(idx)
         if return_dist:
-            dist_parts.append(dist[:, :, :k].sqrt())
+            dist_parts.append(dist.sqrt())
     idx = torch.cat(idx_parts) if len(idx_parts) > 1 else idx_parts[0]
     if return_dist:
         return idx, (torch.cat(dist_parts) if len(dist_parts) > 1 else dist_parts[0])

@@ -47,6 +47,7 @@ _PROTOTYPES = {
     "clusten_wf_forward": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
+    "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
 
@@ -292,6 +293,50 @@ def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Ten
                                        _ptr(d_feat), _ptr(ws), ws_bytes, shape, code, _stream(device)),
                "clusten_wf_backward")
     return d_weights, d_feat
+
+
+def attn_softmax_supported(attn: torch.Tensor, m: int) -> bool:
+    """True when `attn_softmax` takes this case: a CUDA tensor of a 16/32-bit float type, M <= 64, M % 4 == 0."""
+    return attn.is_cuda and attn.dtype in (torch.float32, torch.float16, torch.bfloat16) and m <= 64 and m % 4 == 0
+
+
+def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_logit: torch.Tensor):
+    """softmax over M neighbours and one blank token of attn + bias_table[pe_idx] - 100 * (1 - mask) | blank_logit.
+
+    attn (B,H,N,M); bias_table (rows,H), cast to attn's dtype; pe_idx (B,N,M) int64; mask (B,N,M) int64 or None;
+    blank_logit (B,H,N) or (B,H,N,1).  Returns (probs (B,H,N,M) fp32, blank_prob (B,H,N,1) fp32).
+    No autograd: for inference.  The fused form of models/aff_transformer.py:122-147.
+    """
+    lib = load()
+    _require_cuda("attn", attn)
+    device = attn.device
+    for name, t in (("bias_table", bias_table), ("pe_idx", pe_idx), ("blank_logit", blank_logit)):
+        _require_cuda(name, t, device)
+    b, h, n, m = attn.shape
+    if pe_idx.shape != (b, n, m) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")
+    if bias_table.dim() != 2 or bias_table.shape[1] != h:
+        raise RuntimeError("bias_table must have shape (rows, H)")
+    code = _dtype_code(attn, "attn")
+    attn = attn.contiguous()
+    bias_table = bias_table.to(attn.dtype).contiguous()
+    pe_idx = pe_idx.contiguous()
+    if mask is not None:
+        _require_cuda("mask", mask, device)
+        if mask.shape != (b, n, m):
+            raise RuntimeError("mask must have shape (B,N,M)")
+        mask = mask.to(torch.int64).contiguous()
+    blank_logit = blank_logit.reshape(b, h, n).float().contiguous()
+    probs = torch.empty(b, h, n, m, dtype=torch.float32, device=device)
+    blank_prob = torch.empty(b, h, n, 1, dtype=torch.float32, device=device)
+    if probs.numel() == 0:
+        return probs, blank_prob
+    shape = AttnShape(b, h, n, 1, m)
+    with torch.cuda.device(device):
+        _check(lib.clusten_attn_softmax_forward(_ptr(attn), _ptr(bias_table), _ptr(pe_idx), _ptr(mask),
+                                                _ptr(blank_logit), _ptr(probs), _ptr(blank_prob), shape, code,
+                                                _stream(device)), "clusten_attn_softmax_forward")
+    return probs, blank_prob
 
 
 def copy_probe(src: torch.Tensor, dst: torch.Tensor) -> None:

@@ -1,0 +1,103 @@
+// attn_softmax: the arithmetic between the QK and AV operators of local attention, in one pass.
+//
+//   logits[b,h,i,j] = attn[b,h,i,j] + table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])      j < M
+//   logits[b,h,i,M] = blank[b,h,i]                                                          (blank token)
+//   probs[b,h,i,:M], blank_prob[b,h,i] = softmax(logits[b,h,i,:M+1])
+//
+// The reference model spells this out as tensor expressions (models/aff_transformer.py:122-147: a gather of the
+// position-bias table, two additions, a concatenation, a softmax and two slices), each a full pass over
+// (B,H,N,M).  Here a token's M logits are read once and its probabilities written once; pe_idx and mask,
+// which the heads share, are read once per token.
+//
+// 16 lanes per token, 4 consecutive neighbours per lane (M <= 64, M % 4 == 0); a 256-thread workgroup takes 16
+// tokens.  Row maxima and sums are reduced inside the 16-lane rows with xor shuffles.  All arithmetic is fp32.
+#include "launch.hpp"
+
+namespace clusten {
+namespace {
+
+__device__ __forceinline__ float row16_max(float v) {
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__ attn, const T* __restrict__ table,
+                                                           const int64_t* __restrict__ pe_idx,
+                                                           const int64_t* __restrict__ mask,
+                                                           const float* __restrict__ blank, float* __restrict__ probs,
+                                                           float* __restrict__ blank_prob, int H, int N, int M,
+                                                           int64_t tokens) {
+    typedef Quad<T> Q4;
+    const int64_t tok_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const bool tok_live = tok_raw < tokens;
+    const int64_t tok = tok_live ? tok_raw : tokens - 1;  // every lane stays in the shuffles
+    const int sub = threadIdx.x & 15;
+    const int j0 = sub * 4;
+    const bool live = j0 < M;
+    const int jc = live ? j0 : 0;
+    const int64_t b = tok / N;
+    const int64_t i = tok - b * N;
+
+    int64_t pe[4];
+    float off[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        pe[e] = pe_idx[tok * M + jc + e];
+        off[e] = mask ? (float)(1 - mask[tok * M + jc + e]) * -100.f : 0.f;
+    }
+    for (int h = 0; h < H; ++h) {
+        const int64_t row = (b * H + h) * N + i;
+        float x[4];
+        Q4::unpack(*reinterpret_cast<const typename Q4::raw*>(attn + row * M + jc), x);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] = live ? x[e] + (float)to_acc(table[pe[e] * H + h]) + off[e] : -INFINITY;
+        }
+        const float bl = blank[row];
+        const float mx = fmaxf(row16_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]))), bl);
+        float ex[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ex[e] = live ? expf(v[e] - mx) : 0.f;
+        const float eb = expf(bl - mx);
+        const float inv = 1.f / (row16_sum((ex[0] + ex[1]) + (ex[2] + ex[3])) + eb);
+        if (tok_live && live) {
+            float4 o = make_float4(ex[0] * inv, ex[1] * inv, ex[2] * inv, ex[3] * inv);
+            *reinterpret_cast<float4*>(probs + row * M + j0) = o;
+        }
+        if (tok_live && sub == 0) blank_prob[row] = eb * inv;
+    }
+}
+
+template <typename T>
+int launch_typed(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask, const float* blank,
+                 float* probs, float* blank_prob, const clusten_attn_shape& s, hipStream_t stream) {
+    const int64_t tokens = (int64_t)s.B * s.N;
+    const int64_t blocks = (tokens + 15) / 16;
+    hipLaunchKernelGGL((attn_softmax_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank, probs,
+                       blank_prob, s.H, s.N, s.M, tokens);
+    return launch_status();
+}
+
+}  // namespace
+
+int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask,
+                        const float* blank, float* probs, float* blank_prob, clusten_attn_shape s, int dtype,
+                        hipStream_t stream) {
+    switch (dtype) {
+        case CLUSTEN_F32: return launch_typed<float>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
+}  // namespace clusten

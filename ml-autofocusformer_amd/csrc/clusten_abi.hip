@@ -132,6 +132,18 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
     return launch_wf_dfeat(d_feat_new, weights, nbhd_idx, d_feat, workspace, shape, dtype, as_stream(stream));
 }
 
+int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx, const int64_t* mask,
+                                 const float* blank_logit, float* probs, float* blank_prob, clusten_attn_shape shape,
+                                 int dtype, clusten_stream stream) {
+    if (!attn || !bias_table || !pe_idx || !blank_logit || !probs || !blank_prob) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (shape.M > 64 || shape.M % 4 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(attn) || !aligned16(probs)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_attn_softmax(attn, bias_table, pe_idx, mask, blank_logit, probs, blank_prob, shape, dtype,
+                               as_stream(stream));
+}
+
 int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream) {
     if (!src || !dst) return CLUSTEN_ERR_NULL_POINTER;
     if (bytes == 0 || bytes % 16 != 0) return CLUSTEN_ERR_BAD_DIMS;

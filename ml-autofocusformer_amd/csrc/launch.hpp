@@ -36,6 +36,13 @@ size_t wf_dfeat_workspace_bytes(clusten_wf_shape s, int dtype);
 int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* d_feat, void* workspace,
                     clusten_wf_shape s, int dtype, hipStream_t stream);
 
+// probs[b,h,i,:M], blank_prob[b,h,i] = softmax over j <= M of
+//   attn[b,h,i,j] + table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])  (j < M)  and  blank[b,h,i]  (j = M)
+//   attn, table : T;  pe_idx, mask (may be null) : int64 (B,N,M);  blank, probs, blank_prob : fp32.  M <= 64, M % 4 == 0.
+int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask,
+                        const float* blank, float* probs, float* blank_prob, clusten_attn_shape s, int dtype,
+                        hipStream_t stream);
+
 // dst[0:bytes) = src[0:bytes), 16 bytes per lane per step.
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 

@@ -184,6 +184,42 @@ def test_logits_equal_with_hip_operators_and_with_the_oracle(device, amp):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_fused_bias_mask_blank_softmax_equals_the_tensor_expressions(device, dtype, with_mask):
+    from clusten import _native
+    gen = torch.Generator().manual_seed(11)
+    b, h, n, m, rows = 3, 4, 197, 48, 111 * 111
+    attn = (torch.randn(b, h, n, m, generator=gen) * 2).to(dtype).to(device)
+    table = torch.randn(rows, h, generator=gen).to(dtype).to(device)
+    pe_idx = torch.randint(rows, (b, n, m), generator=gen).to(device)
+    blank = torch.randn(b, h, n, 1, generator=gen).to(device)
+    mask = None
+    if with_mask:
+        mask = (torch.rand(b, n, m, generator=gen) > 0.2).long().to(device)
+        mask[0, 5] = 0                      # a token whose neighbours are all padding: only the blank token is left
+    probs, blank_p = _native.attn_softmax(attn, table, pe_idx, mask, blank)
+    # aff_transformer.py:122-147 in fp32 from the same rounded inputs
+    logits = attn.float() + table.float()[pe_idx].permute(0, 3, 1, 2)
+    if mask is not None:
+        logits = logits + (1 - mask.reshape(b, 1, n, m)) * (-100)
+    ref = torch.softmax(torch.cat([logits, blank], dim=-1), dim=-1)
+    assert probs.dtype == torch.float32 and probs.shape == (b, h, n, m) and blank_p.shape == (b, h, n, 1)
+    assert oracle.rel_err(probs, ref[..., :-1]) < 1e-5
+    assert oracle.rel_err(blank_p, ref[..., -1:]) < 1e-5
+    assert torch.allclose(probs.sum(-1, keepdim=True) + blank_p, torch.ones_like(blank_p), atol=1e-5)
+    # other list lengths, and the refusals
+    for m2 in (4, 16, 64):
+        p2, b2 = _native.attn_softmax(attn[..., :1].expand(-1, -1, -1, m2).contiguous(), table,
+                                      pe_idx[..., :1].expand(-1, -1, m2).contiguous(), None, blank)
+        assert torch.allclose(p2.sum(-1, keepdim=True) + b2, torch.ones_like(b2), atol=1e-5)
+        assert torch.allclose(p2, p2[..., :1].expand_as(p2))
+    assert not _native.attn_softmax_supported(attn, 72) and not _native.attn_softmax_supported(attn, 50)
+    with pytest.raises(RuntimeError):
+        _native.attn_softmax(attn.cpu(), table, pe_idx, mask, blank)
+
+
+@pytest.mark.gpu
 def test_operator_dtypes_under_autocast(device):
     """fp16 autocast hands QK fp16 operands and AV / WF fp32 first operands, as in the reference model."""
     from aff.model import default_ops
