@@ -170,6 +170,18 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
                                  float* blank_prob, clusten_attn_shape shape, int dtype,
                                  clusten_stream stream);
 
+/* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
+
+/* K nearest neighbours of 2-D points inside each batch element: for query point q of batch element b,
+ * idx[b,q,0..K) are the indices of the K database points of b nearest to it, ascending Euclidean
+ * distance, equal distances by ascending index; dist (may be NULL) holds the distances.
+ * Replaces knn_keops (models/point_utils.py:27-58; call sites models/aff_transformer.py:298,476), which
+ * delegates to an external library and leaves the order of equal distances to it.
+ *   query (B,Nq,2), database (B,N,2): fp32 contiguous; idx (B,Nq,K): int64; dist (B,Nq,K): fp32.
+ * 1 <= K <= 8 and K <= N, else CLUSTEN_ERR_BAD_DIMS. */
+int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist,
+                  int B, int Nq, int N, int K, clusten_stream stream);
+
 /* ---- measurement aid ------------------------------------------------------------------------ */
 
 /* Plain streaming copy of `bytes` bytes (multiple of 16, both pointers 16-byte aligned) with the

@@ -18,12 +18,18 @@ def knn(query, database, k, return_dist=False, chunk_elems=1 << 27):
     Closed form of `knn_keops` (point_utils.py:27-58): distance = sqrt(sum((q - x)^2)), k smallest, ascending.
     Equal distances are ordered by database index (the reference leaves that order to its library).
     The distance matrix is built from explicit differences, so integer positions give exact squared
-    distances, and in batch chunks so that at most `chunk_elems` distances exist at a time.
+    distances, and in batch chunks so that at most `chunk_elems` distances exist at a time.  This tensor
+    formulation serves CPU tensors (and k > 8 or other than 2-D points on the GPU).
     """
     b, nq, _ = query.shape
     n = database.shape[1]
     query = query.detach().float()
     database = database.detach().float()
+    if query.is_cuda:
+        # on the GPU the search is one scan kernel of the HIP library (same distances, same tie rule)
+        from clusten import _native
+        if _native.knn2d_supported(query, database, k):
+            return _native.knn2d(query, database, k, return_dist=return_dist)
     per_batch = max(1, nq * n)
     step = max(1, chunk_elems // per_batch)
     idx_parts, dist_parts = [], []

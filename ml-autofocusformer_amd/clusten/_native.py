@@ -48,6 +48,7 @@ _PROTOTYPES = {
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
 
@@ -337,6 +338,34 @@ def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Ten
                                                 _ptr(blank_logit), _ptr(probs), _ptr(blank_prob), shape, code,
                                                 _stream(device)), "clusten_attn_softmax_forward")
     return probs, blank_prob
+
+
+def knn2d_supported(query: torch.Tensor, database: torch.Tensor, k: int) -> bool:
+    """True when `knn2d` takes this case: CUDA tensors of 2-D points, 1 <= k <= 8, k <= number of database points."""
+    return (query.is_cuda and database.is_cuda and query.shape[-1] == 2 and database.shape[-1] == 2
+            and 1 <= k <= 8 and k <= database.shape[1])
+
+
+def knn2d(query: torch.Tensor, database: torch.Tensor, k: int, return_dist: bool = False):
+    """Indices (B,Nq,k) int64 [and distances (B,Nq,k) fp32] of the k database points nearest to each query point."""
+    lib = load()
+    _require_cuda("query", query)
+    _require_cuda("database", database, query.device)
+    if query.dim() != 3 or database.dim() != 3 or query.shape[2] != 2 or database.shape[2] != 2 \
+            or query.shape[0] != database.shape[0]:
+        raise RuntimeError("knn2d needs query (B,Nq,2) and database (B,N,2)")
+    device = query.device
+    query = query.detach().float().contiguous()
+    database = database.detach().float().contiguous()
+    b, nq, _ = query.shape
+    n = database.shape[1]
+    idx = torch.empty(b, nq, k, dtype=torch.int64, device=device)
+    dist = torch.empty(b, nq, k, dtype=torch.float32, device=device) if return_dist else None
+    if idx.numel():
+        with torch.cuda.device(device):
+            _check(lib.clusten_knn2d(_ptr(query), _ptr(database), _ptr(idx), _ptr(dist), b, nq, n, k, _stream(device)),
+                   "clusten_knn2d")
+    return (idx, dist) if return_dist else idx
 
 
 def copy_probe(src: torch.Tensor, dst: torch.Tensor) -> None:

@@ -144,6 +144,14 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
                                as_stream(stream));
 }
 
+int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
+                  clusten_stream stream) {
+    if (!query || !database || !idx) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || Nq <= 0 || N <= 0 || K < 1 || K > 8 || K > N) return CLUSTEN_ERR_BAD_DIMS;
+    if ((int64_t)B * ((Nq + 255) / 256) >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    return launch_knn2d(query, database, idx, dist, B, Nq, N, K, as_stream(stream));
+}
+
 int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream) {
     if (!src || !dst) return CLUSTEN_ERR_NULL_POINTER;
     if (bytes == 0 || bytes % 16 != 0) return CLUSTEN_ERR_BAD_DIMS;

@@ -43,6 +43,12 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
                         const float* blank, float* probs, float* blank_prob, clusten_attn_shape s, int dtype,
                         hipStream_t stream);
 
+// idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
+//   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;
+//   idx int64; dist fp32 or null.
+int launch_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
+                 hipStream_t stream);
+
 // dst[0:bytes) = src[0:bytes), 16 bytes per lane per step.
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 

@@ -110,3 +110,23 @@ def test_knn_against_brute_force_and_tie_order():
     self_idx, self_d = knn(p, p, 2, return_dist=True)
     assert torch.equal(self_idx[:, :, 0], torch.arange(100).expand(2, -1))
     assert (self_d[:, :, 0] == 0).all() and (self_d[:, :, 1] >= 1).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("k", [1, 2, 6, 8])
+def test_knn_kernel_equals_the_tensor_formulation(device, k):
+    from clusten import _native
+    gen = torch.Generator().manual_seed(9)
+    for nq, n in ((784, 98), (784, 784), (3136, 392), (37, 2500), (5, 8)):
+        # integer and eighth-of-a-pixel positions: many exactly equal distances
+        q = torch.randint(0, 56, (3, nq, 2), generator=gen).float()
+        x = torch.randint(0, 56 * 8, (3, n, 2), generator=gen).float() / 8
+        ref_idx, ref_dist = knn(q, x, k, return_dist=True)                 # CPU tensors: the tensor formulation
+        idx, dist = _native.knn2d(q.to(device), x.to(device), k, return_dist=True)
+        assert torch.equal(idx.cpu(), ref_idx)
+        # squared distances are exact here; the two square roots may differ by an ulp
+        assert torch.allclose(dist.cpu(), ref_dist, rtol=2.5e-7, atol=0)
+        assert torch.equal(knn(q.to(device), x.to(device), k).cpu(), ref_idx)
+    assert not _native.knn2d_supported(q.to(device), x.to(device), 9)
+    with pytest.raises(RuntimeError):
+        _native.knn2d(q, x, 2)
