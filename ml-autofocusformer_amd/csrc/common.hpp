@@ -180,6 +180,16 @@ struct VecIO {
 template <typename T>
 using Quad = VecIO<T, 4>;
 
+// ---- stores ---------------------------------------------------------------------------------------
+
+// Store of output data that this kernel never reads again, with the non-temporal hint: the L2 streams the
+// line to memory instead of keeping it, so that the outputs (a quarter to a third of a kernel's traffic) do
+// not push the gathered rows, which are re-read many times, out of the cache.
+template <typename V>
+__device__ __forceinline__ void store_streaming(V* p, V v) {
+    __builtin_nontemporal_store(v, p);
+}
+
 // ---- addressing ---------------------------------------------------------------------------------
 
 // Pin a wave-uniform pointer in scalar registers and hide how it was computed, so that

@@ -306,8 +306,8 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                     for (int k = 0; k < NQD; ++k) {
                         if (qvalid[k]) {
                             float o[4] = {val[k][0], val[k][1], val[k][2], val[k][3]};
-                            *reinterpret_cast<typename OutIO::raw*>(out_h + (lane + kWave * k) * 4 * (int)sizeof(T)) =
-                                OutIO::pack(o);
+                            store_streaming(reinterpret_cast<typename OutIO::raw*>(out_h + (lane + kWave * k) * 4 * (int)sizeof(T)),
+                                            OutIO::pack(o));
                         }
                     }
                 }
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
 #pragma unroll
                     for (int i = 0; i < (S::OUT_BYTES + 1023) / 1024; ++i) {
                         const int off = i * 1024 + lane * 16;
-                        if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
+                        if (off < chunk_bytes) store_streaming(reinterpret_cast<Piece*>(out_h + off), o[i]);
                     }
                 } else if (r >= tok_lo && r < tok_hi) {
                     T* out_row = reinterpret_cast<T*>(out_h) + r * M + j0;
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                         const int s0 = 16 * blk + 4 * kq;
                         float v[4] = {d[blk][0], d[blk][1], d[blk][2], d[blk][3]};
                         if (FAST || vec_store) {
-                            if (s0 < mc) *reinterpret_cast<typename OutIO::raw*>(out_row + s0) = OutIO::pack(v);
+                            if (s0 < mc) store_streaming(reinterpret_cast<typename OutIO::raw*>(out_row + s0), OutIO::pack(v));
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {

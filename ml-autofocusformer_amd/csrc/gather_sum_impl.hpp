@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
 #pragma unroll
             for (int i = 0; i < NO; ++i) {
                 const int off = i * 1024 + lane * 16;
-                if (off < chunk_bytes) *reinterpret_cast<Piece*>(out_h + off) = o[i];
+                if (off < chunk_bytes) store_streaming(reinterpret_cast<Piece*>(out_h + off), o[i]);
             }
         } else {
             if (FAST) __syncthreads();  // operand reads complete before the next head's gather
@@ -196,8 +196,8 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                     float v[S::ECH];
 #pragma unroll
                     for (int e = 0; e < S::ECH; ++e) v[e] = d[e][i];
-                    *reinterpret_cast<typename ChIO::raw*>(out_h + ((int64_t)tok * os.n + n * S::ECH) * sizeof(T)) =
-                        ChIO::pack(v);
+                    store_streaming(reinterpret_cast<typename ChIO::raw*>(out_h + ((int64_t)tok * os.n + n * S::ECH) * sizeof(T)),
+                                    ChIO::pack(v));
                 }
             }
         }

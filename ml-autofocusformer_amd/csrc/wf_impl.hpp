@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                     float v[VEC];
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) v[e] = acc[e][ic];
-                    *reinterpret_cast<Piece*>(out_tok + (int64_t)ic * C + c0 + col) = VecIO<T, VEC>::pack(v);
+                    store_streaming(reinterpret_cast<Piece*>(out_tok + (int64_t)ic * C + c0 + col), VecIO<T, VEC>::pack(v));
                 }
             }
         }
