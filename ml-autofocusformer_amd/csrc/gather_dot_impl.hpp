@@ -67,7 +67,9 @@ struct Staging {
     static constexpr int SROW = 16 * QU + 4;                    // floats per token row of the score matrix
     static constexpr int U_BYTES = UNION ? kTileTokens * SROW * 4 : 0;
     static constexpr int G_PLAIN = NI_G * 1024 > OUT_BYTES ? NI_G * 1024 : (OUT_BYTES + 1023) / 1024 * 1024;
-    static constexpr int G_BYTES = G_PLAIN > U_BYTES ? G_PLAIN : (U_BYTES + 1023) / 1024 * 1024;
+    static constexpr int NI_L = Q;                              // accesses for the tile's lists (8 x 16*Q x 8 bytes)
+    static constexpr int G_NEED = UNION ? (U_BYTES > NI_L * 1024 ? U_BYTES : NI_L * 1024) : 0;
+    static constexpr int G_BYTES = G_PLAIN > G_NEED ? G_PLAIN : (G_NEED + 1023) / 1024 * 1024;
     static constexpr int A_BASE = G_BYTES;
     static constexpr int A_SLOT_BYTES = NI_A * 1024;
     static constexpr int ULIST_BASE = A_BASE + 2 * A_SLOT_BYTES;
@@ -158,7 +160,29 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
         // the tile's lists: are they all the same?  (only the first is kept in registers)
         int list0;
         bool same = true;
-        {
+        if constexpr (FAST) {
+            // the nt lists are one contiguous block of nt*M*8 bytes: it travels by LDS-direct load in 1 KiB
+            // accesses (a third of the vector-memory instructions that 8-byte loads per lane need) and is
+            // compared from LDS
+            const int list_bytes = nt * M * 8;
+            const char* idx_bytes = reinterpret_cast<const char*>(idx_tile);
+#pragma unroll
+            for (int i = 0; i < S::NI_L; ++i) {
+                if (i * 1024 < list_bytes) {
+                    CLUSTEN_LDS_DMA16(idx_bytes + min(i * 1024 + lane * 16, list_bytes - 16), stage + i * 1024);
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            __syncthreads();
+            int64_t wide[kTileTokens];
+#pragma unroll
+            for (int t = 0; t < kTileTokens; ++t) {
+                wide[t] = *reinterpret_cast<const int64_t*>(stage + (min(t, nt - 1) * M + slot) * 8);
+            }
+#pragma unroll
+            for (int t = 1; t < kTileTokens; ++t) same = same && (wide[t] == wide[0]);
+            list0 = (int)wide[0];
+        } else {
             int64_t wide[kTileTokens];
 #pragma unroll
             for (int t = 0; t < kTileTokens; ++t) wide[t] = idx_tile[(int64_t)min(t, nt - 1) * M + j0 + slot];
@@ -180,10 +204,11 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 const int nruns = nt * R;         // <= 64: lane rho owns run rho = token * R + run
                 int v[8];
                 {
-                    const int64_t* p = idx_tile + (int64_t)min(lane, nruns - 1) * 8;  // the tile's lists are contiguous
+                    const int64_t* p = reinterpret_cast<const int64_t*>(stage) + min(lane, nruns - 1) * 8;  // lists in LDS
 #pragma unroll
                     for (int t = 0; t < 8; ++t) v[t] = (int)p[t];
                 }
+                __syncthreads();  // the lists are in registers: the staging buffer is free for the gathers
                 bool regular = true;  // 8 consecutive rows
 #pragma unroll
                 for (int t = 1; t < 8; ++t) regular = regular && (v[t] == v[0] + t);
@@ -315,6 +340,8 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 }
             }
         }
+
+        if (FAST) __syncthreads();  // the list block has been read: the staging buffer is free for the gathers
 
         // the list entry of staging row i*RPI + g_sub lives in the lane of that slot
         int src_lane[S::NI_G];
