@@ -132,6 +132,25 @@ def _bench_attn(case, steps, warmup, dtype=None):
             "av_us": round(per[1] * 1e3, 1), "av_GBps": round(nbytes / per[1] / 1e6, 1), "bytes_each": nbytes}
 
 
+def _bench_backward(acase, wcase, steps, warmup):
+    """Backward of the three operators at one shape: microseconds per call (both gradients of each operator)."""
+    import torch
+    from clusten import _native
+
+    d, w = acase.to("cuda"), wcase.to("cuda")
+    q, k, v, idx = d.query, d.key, d.value, d.nbhd_idx
+    attn = torch.softmax(_native.qk_forward(q, k, idx).float(), dim=-1).to(q.dtype)
+    d_attn = torch.randn_like(attn)
+    d_feat = torch.randn_like(q)
+    d_out = torch.randn(w.weights.shape[0], w.weights.shape[1], w.weights.shape[3], w.feat.shape[2],
+                        dtype=w.feat.dtype, device="cuda")
+    _, per, _ = _time_kernels([lambda: _native.qk_backward(d_attn, q, k, idx),
+                               lambda: _native.av_backward(d_feat, attn, v, idx),
+                               lambda: _native.wf_backward(d_out, w.weights, w.feat, w.nbhd_idx)], steps, warmup)
+    return {"qk_backward_us": round(per[0] * 1e3, 1), "av_backward_us": round(per[1] * 1e3, 1),
+            "wf_backward_us": round(per[2] * 1e3, 1)}
+
+
 def _bench_wf(case, steps, warmup):
     import workloads as wl
     from clusten import _native
@@ -307,6 +326,7 @@ def main():
         other["cfg3_bf16_wf_ic4"] = _bench_wf(wl.config3_wf(), args.steps, args.warmup)
         other["cfg2_s1_model_like_lists"] = _bench_attn(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
+        other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:
         out["aff_tiny_224"] = _aff_tiny_throughput()
