@@ -197,6 +197,115 @@ __global__ __launch_bounds__(256) void wf_dweights_kernel(const T* __restrict__ 
     }
 }
 
+// d_w on the matrix cores.  For one output token  D[slot][ic] = sum_c G[slot][c] * dO[ic][c]  with G the rows its
+// list gathers and dO its IC rows of d_out: the shared-list tile product of the QK kernel with the inner
+// channels in the place of the tile's tokens.  One wave per output token; the channels are taken 256 bytes of a
+// row at a time (rows and d_out rows by LDS-direct load, XOR-swizzled so that the 16-byte operand reads of the 16
+// lanes of an MFMA row fall into different bank groups), fp32 MFMA 16x16x4, D accumulated over the column blocks.
+// The result leaves through LDS in the (slot, ic) order of d_w as full-width stores.
+template <typename T, int Q>
+__global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __restrict__ d_out,
+                                                                 const T* __restrict__ feat,
+                                                                 const int64_t* __restrict__ idx, T* __restrict__ d_w,
+                                                                 int N, int Nout, int C, int M, int IC,
+                                                                 int total_tokens) {
+    constexpr int RB = 256;                       // bytes of a row handled per column block
+    constexpr int CB = RB / (int)sizeof(T);       // channels per column block
+    constexpr int ROWS = 16 * Q;                  // list slots (staging rows)
+    constexpr int NI_G = ROWS / 4;                // a wave access moves 4 rows of 256 bytes
+    constexpr int G_BYTES = ROWS * RB;
+    constexpr int VEC = 16 / (int)sizeof(T);      // elements per 16-byte piece
+    constexpr int NU = 4;                         // pieces per lane: a quarter row
+    typedef VecIO<T, VEC> RunIO;
+
+    __shared__ __attribute__((aligned(1024))) char stage[G_BYTES + 8 * RB];
+
+    const int token = xcd_tile(blockIdx.x, total_tokens);
+    if (token < 0) return;
+    const int b = token / Nout;
+    const int lane = threadIdx.x;
+    const int r = lane & 15, kq = lane >> 4;      // MFMA row / k index: the lane holds quarter kq of row r
+    const int g_sub = lane >> 4, g_pos = lane & 15;  // gather side: piece g_pos of staging row 4*i + g_sub
+
+    const int mine = (int)idx[(int64_t)token * M + min(lane, M - 1)];
+    const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
+    const char* g_tok = reinterpret_cast<const char*>(d_out + (int64_t)token * IC * C);
+    const uint32_t row_pitch = (uint32_t)C * sizeof(T);
+
+    uint32_t g_off[NI_G];
+#pragma unroll
+    for (int i = 0; i < NI_G; ++i) {
+        const int srow = 4 * i + g_sub;
+        g_off[i] = (uint32_t)__shfl(mine, min(srow, M - 1)) * row_pitch + (uint32_t)((g_pos ^ (srow & 15)) * 16);
+    }
+    uint32_t a_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int srow = 4 * i + g_sub;
+        a_off[i] = (uint32_t)min(srow, IC - 1) * row_pitch + (uint32_t)((g_pos ^ (srow & 15)) * 16);
+    }
+    int lds_g[NU], lds_a[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        lds_g[u] = r * RB + (((kq * NU + u) ^ r) * 16);
+        lds_a[u] = G_BYTES + (r & 7) * RB + (((kq * NU + u) ^ (r & 7)) * 16);
+    }
+
+    F32x4 d[Q];
+#pragma unroll
+    for (int blk = 0; blk < Q; ++blk) d[blk] = F32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int c0 = 0; c0 < C; c0 += CB) {
+        const uint32_t col_bytes = (uint32_t)c0 * sizeof(T);
+        __syncthreads();  // the previous column block's operands are in registers
+#pragma unroll
+        for (int i = 0; i < 2; ++i) CLUSTEN_LDS_DMA16(g_tok + (a_off[i] + col_bytes), stage + G_BYTES + i * 1024);
+#pragma unroll
+        for (int i = 0; i < NI_G; ++i) CLUSTEN_LDS_DMA16(feat_b + (g_off[i] + col_bytes), stage + i * 1024);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+
+        typename RunIO::raw a_raw[NU];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u]);
+#pragma unroll
+        for (int blk = 0; blk < Q; ++blk) {
+            typename RunIO::raw g_raw[NU];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                g_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] + blk * 16 * RB);
+            }
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                float x[VEC], y[VEC];
+                RunIO::unpack(g_raw[u], x);
+                RunIO::unpack(a_raw[u], y);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) d[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], y[e], d[blk], 0, 0, 0);
+            }
+        }
+    }
+
+    // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of inner channel r; d_w of the token is M*IC contiguous elements
+    __syncthreads();
+    if (r < IC) {
+#pragma unroll
+        for (int blk = 0; blk < Q; ++blk) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int slot = 16 * blk + 4 * kq + e;
+                if (slot < M) reinterpret_cast<T*>(stage)[slot * IC + r] = from_acc<T>(d[blk][e]);
+            }
+        }
+    }
+    __syncthreads();
+    const int out_bytes = M * IC * (int)sizeof(T);
+    char* dst = reinterpret_cast<char*>(d_w + (int64_t)token * M * IC);
+    for (int off = lane * 16; off < out_bytes; off += kWave * 16) {
+        store_streaming(reinterpret_cast<Piece*>(dst + off), *reinterpret_cast<const Piece*>(stage + off));
+    }
+}
+
 // d_feat: one workgroup per output token, threads over channels; per slot the IC products are
 // summed in registers and leave as one atomic per channel onto a contiguous destination row.
 template <typename T, typename A>
@@ -279,6 +388,23 @@ int wf_forward_typed(const void* w, const void* feat, const int64_t* idx, void* 
 template <typename T>
 int wf_dweights_typed(const void* d_out, const void* feat, const int64_t* idx, void* d_w, const clusten_wf_shape& s,
                       hipStream_t stream) {
+    // whole 256-byte row blocks, 32-bit byte offsets inside one batch element of feat, d_w rows in 16-byte pieces
+    const bool tile_ok = (s.C * (int)sizeof(T)) % 256 == 0 && aligned16(feat) && aligned16(d_out) && aligned16(d_w) &&
+                         (int64_t)s.N * s.C * (int64_t)sizeof(T) < ((int64_t)1 << 31) && s.M <= 64 && s.IC <= 8 &&
+                         ((int64_t)s.M * s.IC * sizeof(T)) % 16 == 0;
+    if constexpr (sizeof(T) <= 4) if (tile_ok) {
+        const int total_tokens = s.B * s.Nout;
+        if (s.M <= 48) {
+            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 3>), dim3(xcd_grid(total_tokens)), dim3(kWave), 0, stream,
+                               static_cast<const T*>(d_out), static_cast<const T*>(feat), idx, static_cast<T*>(d_w),
+                               s.N, s.Nout, s.C, s.M, s.IC, total_tokens);
+        } else {
+            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 4>), dim3(xcd_grid(total_tokens)), dim3(kWave), 0, stream,
+                               static_cast<const T*>(d_out), static_cast<const T*>(feat), idx, static_cast<T*>(d_w),
+                               s.N, s.Nout, s.C, s.M, s.IC, total_tokens);
+        }
+        return launch_status();
+    }
     const int64_t total = (int64_t)s.B * s.Nout * s.M * s.IC;
     hipLaunchKernelGGL((wf_dweights_kernel<T>), dim3(elem_grid(total)), dim3(256), 0, stream,
                        static_cast<const T*>(d_out), static_cast<const T*>(feat), idx, static_cast<T*>(d_w), s.B, s.N,
