@@ -163,10 +163,14 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
  *   attn (B,H,N,M) and bias_table (rows,H): `dtype` (F32, F16 or BF16), contiguous;
  *   pe_idx (B,N,M) int64 with values in [0, rows) — unchecked; mask (B,N,M) int64 of 0/1, or NULL;
  *   blank_logit (B,H,N), probs (B,H,N,M), blank_prob (B,H,N): fp32, contiguous.
- * shape.C is ignored (pass the head dim).  M <= 64 and M % 4 == 0, else CLUSTEN_ERR_BAD_DIMS;
- * attn and probs 16-byte aligned, else CLUSTEN_ERR_UNALIGNED. */
+ * blank_logit may be NULL when query (strided (B,H,N,C) like clusten_qk_forward's, `dtype`) and blank_key
+ * ((H,C), fp32, contiguous) are given: the logit is then their dot product per token and head
+ * (`(q * blank_k).sum(-1)`, models/aff_transformer.py:144), computed in fp32 inside the same pass.
+ * M <= 64 and M % 4 == 0, else CLUSTEN_ERR_BAD_DIMS; attn and probs 16-byte aligned, else
+ * CLUSTEN_ERR_UNALIGNED. */
 int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx,
-                                 const int64_t* mask, const float* blank_logit, float* probs,
+                                 const int64_t* mask, const float* blank_logit, const void* query,
+                                 clusten_strides query_strides, const float* blank_key, float* probs,
                                  float* blank_prob, clusten_attn_shape shape, int dtype,
                                  clusten_stream stream);
 

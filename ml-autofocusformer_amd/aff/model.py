@@ -107,13 +107,13 @@ class ClusterAttention(nn.Module):
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
 
         bias = self.pos_embed(table)                                                     # (rows, h)
-        blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)            # (b,h,n,1)
         fused = getattr(self.ops, "attn_softmax", None)
         if (fused is not None and not global_attn and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0) and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
-            # inference: bias gather, mask, blank token and softmax in one kernel
-            attn, blank = fused(attn, bias, pe_idx, cluster_mask, blank)
+            # inference: bias gather, mask, blank-token logit and softmax in one kernel
+            attn, blank = fused(attn, bias, pe_idx, cluster_mask, query=q, blank_key=self.blank_k)
         else:
+            blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)        # (b,h,n,1)
             attn = attn + bias[pe_idx].permute(0, 3, 1, 2)
             if cluster_mask is not None and not global_attn:
                 attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)

@@ -47,7 +47,8 @@ _PROTOTYPES = {
     "clusten_wf_forward": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
-    "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
+                                                   _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
@@ -301,19 +302,24 @@ def attn_softmax_supported(attn: torch.Tensor, m: int) -> bool:
     return attn.is_cuda and attn.dtype in (torch.float32, torch.float16, torch.bfloat16) and m <= 64 and m % 4 == 0
 
 
-def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_logit: torch.Tensor):
-    """softmax over M neighbours and one blank token of attn + bias_table[pe_idx] - 100 * (1 - mask) | blank_logit.
+def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_logit=None,
+                 query=None, blank_key=None):
+    """softmax over M neighbours and one blank token of attn + bias_table[pe_idx] - 100 * (1 - mask) | blank logit.
 
-    attn (B,H,N,M); bias_table (rows,H), cast to attn's dtype; pe_idx (B,N,M) int64; mask (B,N,M) int64 or None;
-    blank_logit (B,H,N) or (B,H,N,1).  Returns (probs (B,H,N,M) fp32, blank_prob (B,H,N,1) fp32).
+    attn (B,H,N,M); bias_table (rows,H), cast to attn's dtype; pe_idx (B,N,M) int64; mask (B,N,M) int64 or None.
+    The blank token's logit is either given, blank_logit (B,H,N) or (B,H,N,1), or computed in the same pass as
+    (query * blank_key).sum(-1) from query (B,H,N,C) (any strides, channel stride 1, attn's dtype) and blank_key (H,C).
+    Returns (probs (B,H,N,M) fp32, blank_prob (B,H,N,1) fp32).
     No autograd: for inference.  The fused form of models/aff_transformer.py:122-147.
     """
     lib = load()
     _require_cuda("attn", attn)
     device = attn.device
-    for name, t in (("bias_table", bias_table), ("pe_idx", pe_idx), ("blank_logit", blank_logit)):
+    for name, t in (("bias_table", bias_table), ("pe_idx", pe_idx)):
         _require_cuda(name, t, device)
     b, h, n, m = attn.shape
+    if blank_logit is None and (query is None or blank_key is None):
+        raise RuntimeError("attn_softmax needs blank_logit, or query and blank_key")
     if pe_idx.shape != (b, n, m) or pe_idx.dtype != torch.int64:
         raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")
     if bias_table.dim() != 2 or bias_table.shape[1] != h:
@@ -327,16 +333,30 @@ def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Ten
         if mask.shape != (b, n, m):
             raise RuntimeError("mask must have shape (B,N,M)")
         mask = mask.to(torch.int64).contiguous()
-    blank_logit = blank_logit.reshape(b, h, n).float().contiguous()
+    qs, c = Strides(0, 0, 0), 1
+    if blank_logit is not None:
+        _require_cuda("blank_logit", blank_logit, device)
+        blank_logit = blank_logit.reshape(b, h, n).float().contiguous()
+        query = blank_key = None
+    else:
+        _require_cuda("query", query, device)
+        _require_cuda("blank_key", blank_key, device)
+        c = query.shape[3]
+        if query.shape[:3] != (b, h, n) or blank_key.numel() != h * c:
+            raise RuntimeError("query must be (B,H,N,C) and blank_key (H,C)")
+        query = _rows(query.to(attn.dtype))
+        qs = _strides(query)
+        blank_key = blank_key.detach().reshape(h, c).float().contiguous()
     probs = torch.empty(b, h, n, m, dtype=torch.float32, device=device)
     blank_prob = torch.empty(b, h, n, 1, dtype=torch.float32, device=device)
     if probs.numel() == 0:
         return probs, blank_prob
-    shape = AttnShape(b, h, n, 1, m)
+    shape = AttnShape(b, h, n, c, m)
     with torch.cuda.device(device):
         _check(lib.clusten_attn_softmax_forward(_ptr(attn), _ptr(bias_table), _ptr(pe_idx), _ptr(mask),
-                                                _ptr(blank_logit), _ptr(probs), _ptr(blank_prob), shape, code,
-                                                _stream(device)), "clusten_attn_softmax_forward")
+                                                _ptr(blank_logit), _ptr(query), qs, _ptr(blank_key), _ptr(probs),
+                                                _ptr(blank_prob), shape, code, _stream(device)),
+               "clusten_attn_softmax_forward")
     return probs, blank_prob
 
 

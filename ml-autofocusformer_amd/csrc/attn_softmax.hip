@@ -1,7 +1,7 @@
 // attn_softmax: the arithmetic between the QK and AV operators of local attention, in one pass.
 //
 //   logits[b,h,i,j] = attn[b,h,i,j] + table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])      j < M
-//   logits[b,h,i,M] = blank[b,h,i]                                                          (blank token)
+//   logits[b,h,i,M] = blank[b,h,i]   or   sum_c q[b,h,i,c] * blank_k[h,c]                     (blank token)
 //   probs[b,h,i,:M], blank_prob[b,h,i] = softmax(logits[b,h,i,:M+1])
 //
 // The reference model spells this out as tensor expressions (models/aff_transformer.py:122-147: a gather of the
@@ -31,7 +31,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__ attn, const T* __restrict__ table,
                                                            const int64_t* __restrict__ pe_idx,
                                                            const int64_t* __restrict__ mask,
-                                                           const float* __restrict__ blank, float* __restrict__ probs,
+                                                           const float* __restrict__ blank, const T* __restrict__ q,
+                                                           clusten_strides qs, const float* __restrict__ blank_k,
+                                                           int C, float* __restrict__ probs,
                                                            float* __restrict__ blank_prob, int H, int N, int M,
                                                            int64_t tokens) {
     typedef Quad<T> Q4;
@@ -61,7 +63,15 @@ __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__
         for (int e = 0; e < 4; ++e) {
             v[e] = live ? x[e] + (float)to_acc(table[pe[e] * H + h]) + off[e] : -INFINITY;
         }
-        const float bl = blank[row];
+        float bl;
+        if (q) {  // the blank token's logit: this token's query against the blank key of the head
+            const T* qrow = q + b * qs.b + h * qs.h + i * qs.n;
+            float part = 0.f;
+            for (int c = sub; c < C; c += 16) part += to_acc(qrow[c]) * blank_k[h * C + c];
+            bl = row16_sum(part);
+        } else {
+            bl = blank[row];
+        }
         const float mx = fmaxf(row16_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]))), bl);
         float ex[4];
 #pragma unroll
@@ -78,24 +88,25 @@ __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__
 
 template <typename T>
 int launch_typed(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask, const float* blank,
-                 float* probs, float* blank_prob, const clusten_attn_shape& s, hipStream_t stream) {
+                 const void* q, clusten_strides qs, const float* blank_k, float* probs, float* blank_prob,
+                 const clusten_attn_shape& s, hipStream_t stream) {
     const int64_t tokens = (int64_t)s.B * s.N;
     const int64_t blocks = (tokens + 15) / 16;
     hipLaunchKernelGGL((attn_softmax_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank, probs,
-                       blank_prob, s.H, s.N, s.M, tokens);
+                       static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank,
+                       static_cast<const T*>(q), qs, blank_k, s.C, probs, blank_prob, s.H, s.N, s.M, tokens);
     return launch_status();
 }
 
 }  // namespace
 
 int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask,
-                        const float* blank, float* probs, float* blank_prob, clusten_attn_shape s, int dtype,
-                        hipStream_t stream) {
+                        const float* blank, const void* q, clusten_strides qs, const float* blank_k, float* probs,
+                        float* blank_prob, clusten_attn_shape s, int dtype, hipStream_t stream) {
     switch (dtype) {
-        case CLUSTEN_F32: return launch_typed<float>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
-        case CLUSTEN_F16: return launch_typed<f16_t>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
-        case CLUSTEN_BF16: return launch_typed<bf16_t>(attn, table, pe_idx, mask, blank, probs, blank_prob, s, stream);
+        case CLUSTEN_F32: return launch_typed<float>(attn, table, pe_idx, mask, blank, q, qs, blank_k, probs, blank_prob, s, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(attn, table, pe_idx, mask, blank, q, qs, blank_k, probs, blank_prob, s, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(attn, table, pe_idx, mask, blank, q, qs, blank_k, probs, blank_prob, s, stream);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }

@@ -133,15 +133,18 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
 }
 
 int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx, const int64_t* mask,
-                                 const float* blank_logit, float* probs, float* blank_prob, clusten_attn_shape shape,
+                                 const float* blank_logit, const void* query, clusten_strides query_strides,
+                                 const float* blank_key, float* probs, float* blank_prob, clusten_attn_shape shape,
                                  int dtype, clusten_stream stream) {
-    if (!attn || !bias_table || !pe_idx || !blank_logit || !probs || !blank_prob) return CLUSTEN_ERR_NULL_POINTER;
+    if (!attn || !bias_table || !pe_idx || !probs || !blank_prob) return CLUSTEN_ERR_NULL_POINTER;
+    if (!blank_logit && !(query && blank_key)) return CLUSTEN_ERR_NULL_POINTER;
+    if (query && !strides_ok(query_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
     if (shape.M > 64 || shape.M % 4 != 0) return CLUSTEN_ERR_BAD_DIMS;
     if (!aligned16(attn) || !aligned16(probs)) return CLUSTEN_ERR_UNALIGNED;
-    return launch_attn_softmax(attn, bias_table, pe_idx, mask, blank_logit, probs, blank_prob, shape, dtype,
-                               as_stream(stream));
+    return launch_attn_softmax(attn, bias_table, pe_idx, mask, blank_logit, blank_logit ? nullptr : query, query_strides,
+                               blank_key, probs, blank_prob, shape, dtype, as_stream(stream));
 }
 
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,

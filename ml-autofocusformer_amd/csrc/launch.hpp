@@ -39,9 +39,10 @@ int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* 
 // probs[b,h,i,:M], blank_prob[b,h,i] = softmax over j <= M of
 //   attn[b,h,i,j] + table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])  (j < M)  and  blank[b,h,i]  (j = M)
 //   attn, table : T;  pe_idx, mask (may be null) : int64 (B,N,M);  blank, probs, blank_prob : fp32.  M <= 64, M % 4 == 0.
+//   With q (strided (B,H,N,C), T) and blank_k ((H,C), fp32) given, blank[b,h,i] is computed here as their dot product.
 int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_idx, const int64_t* mask,
-                        const float* blank, float* probs, float* blank_prob, clusten_attn_shape s, int dtype,
-                        hipStream_t stream);
+                        const float* blank, const void* q, clusten_strides qs, const float* blank_k, float* probs,
+                        float* blank_prob, clusten_attn_shape s, int dtype, hipStream_t stream);
 
 // idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
 //   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;

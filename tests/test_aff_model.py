@@ -208,6 +208,15 @@ def test_fused_bias_mask_blank_softmax_equals_the_tensor_expressions(device, dty
     assert oracle.rel_err(probs, ref[..., :-1]) < 1e-5
     assert oracle.rel_err(blank_p, ref[..., -1:]) < 1e-5
     assert torch.allclose(probs.sum(-1, keepdim=True) + blank_p, torch.ones_like(blank_p), atol=1e-5)
+    # the blank logit computed in the same pass from a (permuted-view) query and the blank key
+    c = 32
+    qsrc = (torch.randn(b, n, h, c, generator=gen) * 0.3).to(dtype).to(device)
+    query = qsrc.permute(0, 2, 1, 3)
+    blank_key = torch.randn(h * c, generator=gen).to(device)
+    probs_q, blank_q = _native.attn_softmax(attn, table, pe_idx, mask, query=query, blank_key=blank_key)
+    blank_ref = (query.float() * blank_key.reshape(1, h, 1, c)).sum(-1, keepdim=True)
+    ref_q = torch.softmax(torch.cat([logits, blank_ref], dim=-1), dim=-1)
+    assert oracle.rel_err(probs_q, ref_q[..., :-1]) < 1e-5 and oracle.rel_err(blank_q, ref_q[..., -1:]) < 1e-5
     # other list lengths, and the refusals
     for m2 in (4, 16, 64):
         p2, b2 = _native.attn_softmax(attn[..., :1].expand(-1, -1, -1, m2).contiguous(), table,
