@@ -32,7 +32,8 @@
 //   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
 //     token's column is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
 //
-// Storage types narrower than fp32 are widened in registers; all products and sums are fp32.
+// fp32 data runs as fp32 MFMA 16x16x4; fp16 / bf16 data goes through the 16-bit matrix instructions as it came
+// from memory (16x16x32, or 16x16x16 for head dim 16): their products are exact in fp32 and all sums are fp32.
 // Rows whose start is not 16-byte aligned, head dims other than 16/32/64 and fp64 take the
 // element-per-thread kernel at the bottom of the file.
 //
@@ -290,27 +291,12 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                         }
                         __syncthreads();  // operands are in registers: the rows make room for the scores
 
-                        float bop[S::EL];
-#pragma unroll
-                        for (int u = 0; u < S::NU; ++u) {
-                            float x[S::VEC];
-                            RunIO::unpack(a_raw[u], x);
-#pragma unroll
-                            for (int e = 0; e < S::VEC; ++e) bop[u * S::VEC + e] = x[e];
-                        }
 #pragma unroll
                         for (int blk = 0; blk < QU; ++blk) {
                             if (blk * 16 < rows_here) {
                                 F32x4 d = F32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                                for (int u = 0; u < S::NU; ++u) {
-                                    float x[S::VEC];
-                                    RunIO::unpack(g_raw[blk][u], x);
-#pragma unroll
-                                    for (int e = 0; e < S::VEC; ++e) {
-                                        d = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], bop[u * S::VEC + e], d, 0, 0, 0);
-                                    }
-                                }
+                                for (int u = 0; u < S::NU; ++u) d = tile_mfma<T>(g_raw[blk][u], a_raw[u], d);
                                 // lane (r, kq): union rows 16*blk + 4*kq .. +3 of token r
                                 if (r < kTileTokens) {
                                     *reinterpret_cast<F32x4*>(stage + (r * S::SROW + 16 * blk + 4 * kq) * 4) = d;
@@ -391,27 +377,12 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 }
                 __syncthreads();  // operands are in registers: the staging buffer may be reused
 
-                float bop[S::EL];
-#pragma unroll
-                for (int u = 0; u < S::NU; ++u) {
-                    float x[S::VEC];
-                    RunIO::unpack(a_raw[u], x);
-#pragma unroll
-                    for (int e = 0; e < S::VEC; ++e) bop[u * S::VEC + e] = x[e];
-                }
                 F32x4 d[Q];
 #pragma unroll
                 for (int blk = 0; blk < Q; ++blk) {
                     d[blk] = F32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int u = 0; u < S::NU; ++u) {
-                        float x[S::VEC];
-                        RunIO::unpack(g_raw[blk][u], x);
-#pragma unroll
-                        for (int e = 0; e < S::VEC; ++e) {
-                            d[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], bop[u * S::VEC + e], d[blk], 0, 0, 0);
-                        }
-                    }
+                    for (int u = 0; u < S::NU; ++u) d[blk] = tile_mfma<T>(g_raw[blk][u], a_raw[u], d[blk]);
                 }
 
                 // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of token r

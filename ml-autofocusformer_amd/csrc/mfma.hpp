@@ -1,6 +1,8 @@
 // Helpers shared by the matrix-core gather kernels (gather_dot, gather_sum).
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace clusten {
@@ -16,5 +18,40 @@ constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 
 #define CLUSTEN_LDS_DMA16(gptr, lptr)                                                       \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr), \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+// D(16x16) += A * B over the channels two lanes hold in one register group of 8 or 16 bytes each: `a` belongs to
+// row lane % 16 of A, `b` to column lane % 16 of B, and lane / 16 selects which quarter of the channel range
+// both cover.  fp32 data goes one channel (k = 4 per instruction) at a time; 16-bit data goes through the
+// 16-bit matrix instructions with the register group as it came from memory (k = 16 or 32 per instruction):
+// products of fp16 / bf16 values are exact in fp32 and the sums are fp32 either way.
+template <typename T, typename Raw>
+__device__ __forceinline__ F32x4 tile_mfma(const Raw& a, const Raw& b, F32x4 d) {
+    if constexpr (sizeof(T) == 4) {
+        constexpr int VEC = (int)sizeof(Raw) / 4;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            d = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(raw_word(a, e)), __uint_as_float(raw_word(b, e)), d,
+                                                     0, 0, 0);
+        }
+        return d;
+    } else if constexpr (sizeof(Raw) == 16) {
+        typedef _Float16 H8 __attribute__((ext_vector_type(8)));
+        typedef __bf16 B8 __attribute__((ext_vector_type(8)));
+        if constexpr (std::is_same<T, f16_t>::value) {
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(H8, a), __builtin_bit_cast(H8, b), d, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(B8, a), __builtin_bit_cast(B8, b), d, 0, 0, 0);
+        }
+    } else {
+        static_assert(sizeof(Raw) == 8, "register groups of 8 or 16 bytes");
+        typedef _Float16 H4 __attribute__((ext_vector_type(4)));
+        typedef short S4 __attribute__((ext_vector_type(4)));
+        if constexpr (std::is_same<T, f16_t>::value) {
+            return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(H4, a), __builtin_bit_cast(H4, b), d, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(S4, a), __builtin_bit_cast(S4, b), d, 0, 0, 0);
+        }
+    }
+}
 
 }  // namespace clusten

@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void wf_dweights_kernel(const T* __restrict__ 
 // list gathers and dO its IC rows of d_out: the shared-list tile product of the QK kernel with the inner
 // channels in the place of the tile's tokens.  One wave per output token; the channels are taken 256 bytes of a
 // row at a time (rows and d_out rows by LDS-direct load, XOR-swizzled so that the 16-byte operand reads of the 16
-// lanes of an MFMA row fall into different bank groups), fp32 MFMA 16x16x4, D accumulated over the column blocks.
+// lanes of an MFMA row fall into different bank groups), 16x16 MFMA blocks, D accumulated over the column blocks.
 // The result leaves through LDS in the (slot, ic) order of d_w as full-width stores.
 template <typename T, int Q>
 __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __restrict__ d_out,
@@ -276,13 +276,7 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
                 g_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] + blk * 16 * RB);
             }
 #pragma unroll
-            for (int u = 0; u < NU; ++u) {
-                float x[VEC], y[VEC];
-                RunIO::unpack(g_raw[u], x);
-                RunIO::unpack(a_raw[u], y);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) d[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(x[e], y[e], d[blk], 0, 0, 0);
-            }
+            for (int u = 0; u < NU; ++u) d[blk] = tile_mfma<T>(g_raw[u], a_raw[u], d[blk]);
         }
     }
 
