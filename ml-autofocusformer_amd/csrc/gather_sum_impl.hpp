@@ -371,6 +371,15 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             fetch_p(0, 0, M, 0);
             if (H > 1) fetch_p(1, 0, M, 1);
         }
+        // FAST: one chunk; the byte offsets of its rows do not depend on the head
+        uint32_t g_off[S::NI_G];
+        if constexpr (FAST) {
+            const int mine = pass == 0 ? list0[0] : (int)idx_tile[(int64_t)pass * M + min(lane, M - 1)];
+#pragma unroll
+            for (int i = 0; i < S::NI_G; ++i) {
+                g_off[i] = (uint32_t)__shfl(mine, min(i * S::RPI + g_sub, M - 1)) * row_pitch + (uint32_t)(g_pos * 16);
+            }
+        }
         for (int h = 0; h < H; ++h) {
             const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
             F32x4 d[S::ECH];
@@ -380,22 +389,27 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             for (int j0 = 0, ch = 0; j0 < (FAST ? 1 : M); j0 += kWave, ++ch) {
                 const int mc = FAST ? M : min(kWave, M - j0);
                 const int slot = min(lane, mc - 1);
-                // this pass's list of the chunk
-                int mine;
-                if (pass == 0 && ch < MAXCH) {
-                    mine = list0[0];
-#pragma unroll
-                    for (int k = 1; k < MAXCH; ++k) mine = (k == ch) ? list0[k] : mine;
-                } else {
-                    mine = (int)idx_tile[(int64_t)pass * M + j0 + slot];
-                }
                 // gather: rows of this chunk -> LDS (and the p pieces when they were not prefetched)
-                if (!FAST) __syncthreads();  // the previous chunk's operand reads are complete
+                if constexpr (FAST) {
 #pragma unroll
-                for (int i = 0; i < S::NI_G; ++i) {
-                    const int srow = min(i * S::RPI + g_sub, mc - 1);
-                    const uint32_t off = (uint32_t)__shfl(mine, srow) * row_pitch + (uint32_t)(g_pos * 16);
-                    CLUSTEN_LDS_DMA16(rows_bh + off, stage + i * 1024);
+                    for (int i = 0; i < S::NI_G; ++i) CLUSTEN_LDS_DMA16(rows_bh + g_off[i], stage + i * 1024);
+                } else {
+                    // this pass's list of the chunk
+                    int mine;
+                    if (pass == 0 && ch < MAXCH) {
+                        mine = list0[0];
+#pragma unroll
+                        for (int k = 1; k < MAXCH; ++k) mine = (k == ch) ? list0[k] : mine;
+                    } else {
+                        mine = (int)idx_tile[(int64_t)pass * M + j0 + slot];
+                    }
+                    __syncthreads();  // the previous chunk's operand reads are complete
+#pragma unroll
+                    for (int i = 0; i < S::NI_G; ++i) {
+                        const int srow = min(i * S::RPI + g_sub, mc - 1);
+                        const uint32_t off = (uint32_t)__shfl(mine, srow) * row_pitch + (uint32_t)(g_pos * 16);
+                        CLUSTEN_LDS_DMA16(rows_bh + off, stage + i * 1024);
+                    }
                 }
                 const int ps = FAST ? (h & 1) : 0;
                 if (!FAST) {
@@ -406,12 +420,12 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 __syncthreads();
 
-                // steps of 4 slots, taken one p piece at a time: all LDS reads of a batch of pieces are
+                // steps of 4 slots, taken one p piece at a time: all LDS reads of a batch of pieces (8 steps) are
                 // issued before its MFMAs so that their latency is paid once per batch, not once per step.
                 // No branches: when the list can end inside the chunk (!EXACT) the operands of the
                 // missing slots are replaced by zeros.
                 constexpr int NPIECE = S::STEPS / S::STEPS_PER_PIECE;
-                constexpr int BATCH = (4 / S::STEPS_PER_PIECE) < 1 ? 1 : (4 / S::STEPS_PER_PIECE);  // pieces per batch = 4 steps
+                constexpr int BATCH = 8 / S::STEPS_PER_PIECE;  // pieces per batch = 8 steps
                 const char* p_lds = stage + S::P_BASE + ps * S::P_SLOT_BYTES + lds_p;
 #pragma unroll
                 for (int sb = 0; sb < NPIECE; sb += BATCH) {
