@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch at the headline workload, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of `bench.py --only {qk,av,wf}`, each counter scaled by what it reads for the copy probe of known
 # size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md.
-MEASURED_TRAFFIC_BYTES = {"qk": 359.58e6 + 154.14e6, "av": 411.01e6 + 102.76e6, "wf": 221.33e6 + 102.76e6}
+MEASURED_TRAFFIC_BYTES = {"qk": 359.56e6 + 154.14e6, "av": 410.98e6 + 102.76e6, "wf": 219.18e6 + 102.76e6}
 
 
 def _time_kernels(fns, steps, warmup):
