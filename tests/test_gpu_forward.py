@@ -255,6 +255,23 @@ def test_wf_full_size_stage1(device):
     assert out.abs().max() <= d.feat.abs().max() * (1 + 1e-6)
 
 
+def test_empty_inputs_give_empty_or_zero_outputs(device):
+    # no batch elements, no tokens, or empty lists: nothing is launched
+    for b, n, m in ((0, 16, 8), (2, 0, 8), (2, 16, 0)):
+        q = torch.randn(b, 2, n, 32, device=device)
+        idx = torch.zeros(b, n, m, dtype=torch.int64, device=device)
+        attn = _native.qk_forward(q, q, idx)
+        assert attn.shape == (b, 2, n, m)
+        feat = _native.av_forward(attn, q, idx)
+        assert feat.shape == (b, 2, n, 32) and (feat == 0).all()
+        w = torch.randn(b, n, m, 4, device=device)
+        f = torch.randn(b, max(n, 1) * 4, 64, device=device)
+        out = _native.wf_forward(w, f, idx)
+        assert out.shape == (b, n, 4, 64) and (out == 0).all()
+        d_q, d_k = _native.qk_backward(torch.zeros_like(attn), q, q, idx)
+        assert d_q.shape == q.shape and (d_q == 0).all() and (d_k == 0).all()
+
+
 def test_copy_probe(device):
     src = torch.randn(1 << 20, device=device)
     dst = torch.zeros_like(src)
