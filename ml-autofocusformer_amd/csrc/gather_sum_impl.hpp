@@ -429,20 +429,18 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 const char* p_lds = stage + S::P_BASE + ps * S::P_SLOT_BYTES + lds_p;
 #pragma unroll
                 for (int sb = 0; sb < NPIECE; sb += BATCH) {
-                    typename PieceIO::raw p_raw[BATCH];
-                    float p_one[BATCH];  // fp32 data: the lane's element of the piece, read on its own
+                    // the lane's A operand of a step is one element of a p piece: element kq of the step's 4 slots,
+                    // read from LDS on its own (no 16-byte read to unpack and select from)
+                    T p_one[BATCH * S::STEPS_PER_PIECE];
                     typename ChIO::raw g_raw[BATCH * S::STEPS_PER_PIECE];
 #pragma unroll
                     for (int q = 0; q < BATCH; ++q) {
                         if (sb + q < NPIECE) {
-                            if constexpr (sizeof(T) == 4) {
-                                p_one[q] = *reinterpret_cast<const float*>(p_lds + (sb + q) * kTileTokens * 16 + kq * 4);
-                            } else {
-                                p_raw[q] = *reinterpret_cast<const typename PieceIO::raw*>(p_lds + (sb + q) * kTileTokens * 16);
-                            }
 #pragma unroll
                             for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
                                 const int s = (sb + q) * S::STEPS_PER_PIECE + ss;
+                                p_one[q * S::STEPS_PER_PIECE + ss] = *reinterpret_cast<const T*>(
+                                    p_lds + (sb + q) * kTileTokens * 16 + (4 * ss + kq) * (int)sizeof(T));
                                 g_raw[q * S::STEPS_PER_PIECE + ss] =
                                     *reinterpret_cast<const typename ChIO::raw*>(stage + 4 * s * S::RB + lds_g);
                             }
@@ -451,20 +449,10 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
 #pragma unroll
                     for (int q = 0; q < BATCH; ++q) {
                         if (sb + q < NPIECE) {
-                            float pv[S::SPP];
-                            if constexpr (sizeof(T) != 4) PieceIO::unpack(p_raw[q], pv);
 #pragma unroll
                             for (int ss = 0; ss < S::STEPS_PER_PIECE; ++ss) {
                                 const int s = (sb + q) * S::STEPS_PER_PIECE + ss;
-                                // element kq of the 4 slots of this step
-                                float aop;
-                                if constexpr (sizeof(T) == 4) {
-                                    aop = p_one[q];
-                                } else {
-                                    aop = pv[4 * ss];
-#pragma unroll
-                                    for (int k = 1; k < 4; ++k) aop = (kq == k) ? pv[4 * ss + k] : aop;
-                                }
+                                float aop = to_acc(p_one[q * S::STEPS_PER_PIECE + ss]);
                                 float g[S::ECH];
                                 ChIO::unpack(g_raw[q * S::STEPS_PER_PIECE + ss], g);
                                 if (!EXACT) {
