@@ -191,6 +191,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     ops = SimpleNamespace(**vars(real))
     ops.qk, ops.av, ops.wf = timed_call("qk", real.qk), timed_call("av", real.av), timed_call("wf", real.wf)
     ops.attn_softmax = timed_call("bias+mask+blank+softmax", real.attn_softmax)
+    ops.qk_clusters, ops.av_clusters = timed_call("qk", real.qk_clusters), timed_call("av", real.av_clusters)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()
     for layer in net.layers:
         layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)
@@ -326,6 +327,15 @@ def main():
         other["cfg3_bf16_wf_ic4"] = _bench_wf(wl.config3_wf(), args.steps, args.warmup)
         other["cfg2_s1_model_like_lists"] = _bench_attn(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
+        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model").to("cuda")
+        cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()   # the same lists as cluster numbers
+        mattn = torch.softmax(_native.qk_forward(mcase.query, mcase.key, mcase.nbhd_idx), dim=-1)
+        _, per_c, _ = _time_kernels([lambda: _native.qk_forward_clusters(mcase.query, mcase.key, cidx),
+                                     lambda: _native.av_forward_clusters(mattn, mcase.value, cidx)],
+                                    args.steps, args.warmup)
+        other["cfg2_s1_model_like_lists_as_cluster_numbers"] = {"qk_us": round(per_c[0] * 1e3, 1),
+                                                                 "av_us": round(per_c[1] * 1e3, 1)}
+        del mcase, cidx, mattn
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:

@@ -152,6 +152,28 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
                         void* workspace, size_t workspace_bytes,
                         clusten_wf_shape shape, int dtype, clusten_stream stream);
 
+/* ---- compact neighbourhood lists (optional) --------------------------------------------------- */
+
+/* QK and AV forward with the neighbourhoods given as cluster numbers instead of row lists.  The reference's
+ * BasicLayer builds nbhd_idx by expanding the nnc nearest clusters of every token into their 8 members
+ * (models/aff_transformer.py:476-480; members of cluster g are rows 8g..8g+7 of the cluster-ordered
+ * sequence, pad slots of the last cluster hold row 0, models/point_utils.py:203-206): an int64 (B,N,8*nnc)
+ * tensor that is 30-55 % of the operators' traffic.  These entry points take the (B,N,nnc) cluster numbers
+ * themselves, as int32 — 1/16 of the bytes — and compute exactly what clusten_qk_forward /
+ * clusten_av_forward compute on the expanded lists:
+ *     nbhd_idx[b,i,8*r+t] = 8*cluster_idx[b,i,r]+t   if that is < N,   else 0.
+ * shape.M = 8 * nnc (a multiple of 8, at most 64).  Tile kernels only: dtype F32/F16/BF16, head dim
+ * 16/32/64 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).  Forward only:
+ * for training expand the lists and use the functions above.  No counterpart in the reference's extension
+ * modules. */
+int clusten_qk_forward_clusters(const void* query, clusten_strides query_strides,
+                                const void* key, clusten_strides key_strides,
+                                const int32_t* cluster_idx, void* attn,
+                                clusten_attn_shape shape, int dtype, clusten_stream stream);
+int clusten_av_forward_clusters(const void* attn, const void* value, clusten_strides value_strides,
+                                const int32_t* cluster_idx, void* feat, clusten_strides feat_strides,
+                                clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* ---- glue between QK and AV (optional) -------------------------------------------------------- */
 
 /* The arithmetic the model does between CLUSTENQKFunction and CLUSTENAVFunction, in one pass:

@@ -32,7 +32,9 @@ def default_ops():
     """The three operators as the HIP library provides them."""
     from clusten import CLUSTENAVFunction, CLUSTENQKFunction, CLUSTENWFFunction, _native
     return SimpleNamespace(qk=CLUSTENQKFunction.apply, av=CLUSTENAVFunction.apply, wf=CLUSTENWFFunction.apply,
-                           attn_softmax=_native.attn_softmax, attn_softmax_supported=_native.attn_softmax_supported)
+                           attn_softmax=_native.attn_softmax, attn_softmax_supported=_native.attn_softmax_supported,
+                           qk_clusters=_native.qk_forward_clusters, av_clusters=_native.av_forward_clusters,
+                           clusters_supported=_native.clusters_supported)
 
 
 def relative_position_table(img_size):
@@ -94,16 +96,22 @@ class ClusterAttention(nn.Module):
         self.proj_drop = nn.Dropout(proj_drop)
         self.ops = ops
 
-    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table):
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None):
         b, n, c = feat.shape
         h = self.num_heads
         ch = c // h
+        # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
+        compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
+                   and getattr(self.ops, "qk_clusters", None) is not None)
         q = (self.q(feat) * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)        # (b,h,n,ch) view
         kv = self.kv(feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
         if global_attn:
             attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
+        elif compact and self.ops.clusters_supported(q, cluster_idx.shape[2]):
+            attn = self.ops.qk_clusters(q, key, cluster_idx)                             # (b,h,n,m)
         else:
+            compact = False
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
 
         bias = self.pos_embed(table)                                                     # (rows, h)
@@ -121,7 +129,12 @@ class ClusterAttention(nn.Module):
             attn = self.attn_drop(attn)
             blank, attn = attn[..., -1:], attn[..., :-1]
 
-        out = attn @ v if global_attn else self.ops.av(attn, v, member_idx)              # (b,h,n,ch)
+        if global_attn:
+            out = attn @ v
+        elif compact:
+            out = self.ops.av_clusters(attn, v, cluster_idx)
+        else:
+            out = self.ops.av(attn, v, member_idx)                                       # (b,h,n,ch)
         out = out + blank * self.blank_v.reshape(1, h, 1, ch)
         out = out.permute(0, 2, 1, 3).reshape(b, n, c)
         return self.proj_drop(self.proj(out))
@@ -141,8 +154,8 @@ class ClusterTransformerBlock(nn.Module):
             self.gamma1 = nn.Parameter(layer_scale * torch.ones(dim))
             self.gamma2 = nn.Parameter(layer_scale * torch.ones(dim))
 
-    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table):
-        a = self.attn(self.norm1(feat), member_idx, cluster_mask, pe_idx, global_attn, table)
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None):
+        a = self.attn(self.norm1(feat), member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx)
         feat = feat + self.drop_path(self.gamma1 * a if self.layer_scale else a)
         f = self.mlp(self.norm2(feat))
         return feat + self.drop_path(self.gamma2 * f if self.layer_scale else f)
@@ -223,7 +236,8 @@ class BasicLayer(nn.Module):
         self._grid_cache = {}
 
     def neighbourhoods(self, pos, h, w, radius, table_width):
-        """(pos reordered, ranking or None, member_idx (b,n,nbhd), mask or None, pe_idx (b,n,nbhd)).
+        """(pos reordered, ranking or None, member_idx (b,n,nbhd), mask or None, pe_idx (b,n,nbhd),
+        cluster numbers (b,n,nnc) int32 or None).
 
         aff_transformer.py:454-487.  The list of token i holds the members of its nnc nearest clusters,
         nearest cluster first; members of cluster g are tokens g*m .. g*m+m-1 of the reordered sequence.
@@ -245,12 +259,16 @@ class BasicLayer(nn.Module):
         nb_pos = pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, d)).reshape(b, n, nnc * m, d)
         rel = nb_pos - (pos.unsqueeze(2) - radius)
         pe_idx = (rel[..., 1] * table_width + rel[..., 0]).long()
-        return pos, ranking, member_idx, mask, pe_idx
+        # with clusters of 8 in cluster order, member_idx[b,i,8r+t] = 8*nearest[b,i,r]+t (0 past the last token):
+        # the cluster numbers alone describe the lists
+        cluster_idx = nearest.to(torch.int32).contiguous() if (ranking is not None and m == 8) else None
+        return pos, ranking, member_idx, mask, pe_idx, cluster_idx
 
     def forward(self, pos, feat, h, w, on_grid, stride, table, radius):
         b, n, d = pos.shape
         table_width = 2 * radius + 1
         global_attn = self.nbhd_size >= n
+        cluster_idx = None
         if global_attn:
             member_idx = mask = None
             rel = (pos[:, None, :, :] + radius) - pos[:, :, None, :]
@@ -261,22 +279,23 @@ class BasicLayer(nn.Module):
                 key = (n, h, w, str(pos.device))
                 if key not in self._grid_cache:
                     self._grid_cache[key] = self.neighbourhoods(pos[:1], h, w, radius, table_width)
-                pos1, ranking, member_idx, mask, pe_idx = self._grid_cache[key]
+                pos1, ranking, member_idx, mask, pe_idx, cluster_idx = self._grid_cache[key]
                 if (key, b) not in self._grid_cache:   # the batch-sized copies the operators read
                     self._grid_cache[(key, b)] = (member_idx.expand(b, -1, -1).contiguous(),
                                                   pe_idx.expand(b, -1, -1).contiguous(),
-                                                  None if mask is None else mask.expand(b, -1, -1).contiguous())
-                member_idx, pe_idx, mask = self._grid_cache[(key, b)]
+                                                  None if mask is None else mask.expand(b, -1, -1).contiguous(),
+                                                  None if cluster_idx is None else cluster_idx.expand(b, -1, -1).contiguous())
+                member_idx, pe_idx, mask, cluster_idx = self._grid_cache[(key, b)]
                 pos = pos1.expand(b, -1, -1)
                 if ranking is not None:
                     feat = feat[:, ranking[0, :, 0]]
             else:
-                pos, ranking, member_idx, mask, pe_idx = self.neighbourhoods(pos, h, w, radius, table_width)
+                pos, ranking, member_idx, mask, pe_idx, cluster_idx = self.neighbourhoods(pos, h, w, radius, table_width)
                 if ranking is not None:
                     feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
 
         for blk in self.blocks:
-            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table)
+            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx)
 
         if self.downsample is not None:
             if global_attn:   # merging after a dense stage: every token is every token's neighbour

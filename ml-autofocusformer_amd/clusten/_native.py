@@ -47,6 +47,8 @@ _PROTOTYPES = {
     "clusten_wf_forward": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
+    "clusten_qk_forward_clusters": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_av_forward_clusters": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
                                                    _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
@@ -295,6 +297,63 @@ def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Ten
                                        _ptr(d_feat), _ptr(ws), ws_bytes, shape, code, _stream(device)),
                "clusten_wf_backward")
     return d_weights, d_feat
+
+
+def clusters_supported(a: torch.Tensor, nnc: int) -> bool:
+    """True when the cluster-number entry points take this case (head dim 16/32/64, at most 8 clusters per token)."""
+    return (a.is_cuda and a.dtype in (torch.float32, torch.float16, torch.bfloat16) and a.shape[3] in (16, 32, 64)
+            and 1 <= nnc <= 8)
+
+
+def _cluster_idx(cluster_idx: torch.Tensor, shape, device) -> torch.Tensor:
+    _require_cuda("cluster_idx", cluster_idx, device)
+    if cluster_idx.dtype != torch.int32 or cluster_idx.dim() != 3 or tuple(cluster_idx.shape[:2]) != tuple(shape):
+        raise RuntimeError("cluster_idx must be int32 of shape (B,N,clusters per token)")
+    return cluster_idx.contiguous()
+
+
+def qk_forward_clusters(query: torch.Tensor, key: torch.Tensor, cluster_idx: torch.Tensor) -> torch.Tensor:
+    """qk_forward on nbhd_idx[b,i,8r+t] = 8*cluster_idx[b,i,r]+t (0 where that is >= N), without building it."""
+    lib = load()
+    _require_cuda("query", query)
+    device = query.device
+    _require_cuda("key", key, device)
+    if query.shape != key.shape or query.dim() != 4 or query.dtype != key.dtype:
+        raise RuntimeError("query and key must be (B,H,N,C) tensors of one dtype")
+    B, H, N, C = query.shape
+    cidx = _cluster_idx(cluster_idx, (B, N), device)
+    shape = AttnShape(B, H, N, C, 8 * cidx.shape[2])
+    query, key = _rows(query), _rows(key)
+    attn = torch.empty((B, H, N, shape.M), dtype=query.dtype, device=device)
+    if attn.numel() == 0:
+        return attn
+    with torch.cuda.device(device):
+        _check(lib.clusten_qk_forward_clusters(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(cidx),
+                                               _ptr(attn), shape, _dtype_code(query, "query"), _stream(device)),
+               "clusten_qk_forward_clusters")
+    return attn
+
+
+def av_forward_clusters(attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.Tensor) -> torch.Tensor:
+    """av_forward on the lists qk_forward_clusters describes; v is cast to attn's dtype like the AV Function does."""
+    lib = load()
+    _require_cuda("attn", attn)
+    device = attn.device
+    _require_cuda("v", v, device)
+    B, H, N, C = v.shape
+    cidx = _cluster_idx(cluster_idx, (B, N), device)
+    if tuple(attn.shape) != (B, H, N, 8 * cidx.shape[2]):
+        raise RuntimeError("attn must be (B,H,N,8 * clusters per token)")
+    shape = AttnShape(B, H, N, C, 8 * cidx.shape[2])
+    attn, v = attn.contiguous(), _rows(v.to(attn.dtype))
+    feat = torch.empty((B, H, N, C), dtype=attn.dtype, device=device)
+    if feat.numel() == 0:
+        return feat
+    with torch.cuda.device(device):
+        _check(lib.clusten_av_forward_clusters(_ptr(attn), _ptr(v), _strides(v), _ptr(cidx), _ptr(feat), _strides(feat),
+                                               shape, _dtype_code(attn, "attn"), _stream(device)),
+               "clusten_av_forward_clusters")
+    return feat
 
 
 def attn_softmax_supported(attn: torch.Tensor, m: int) -> bool:

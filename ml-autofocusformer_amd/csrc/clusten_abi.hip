@@ -132,6 +132,26 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
     return launch_wf_dfeat(d_feat_new, weights, nbhd_idx, d_feat, workspace, shape, dtype, as_stream(stream));
 }
 
+int clusten_qk_forward_clusters(const void* query, clusten_strides query_strides, const void* key,
+                                clusten_strides key_strides, const int32_t* cluster_idx, void* attn,
+                                clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!query || !key || !cluster_idx || !attn) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_gather_dot_clusters(query, query_strides, key, key_strides, cluster_idx, attn, shape, dtype,
+                                      as_stream(stream));
+}
+
+int clusten_av_forward_clusters(const void* attn, const void* value, clusten_strides value_strides,
+                                const int32_t* cluster_idx, void* feat, clusten_strides feat_strides,
+                                clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!attn || !value || !cluster_idx || !feat) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(value_strides, shape.C) || !strides_ok(feat_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_gather_sum_clusters(attn, value, value_strides, cluster_idx, feat, feat_strides, shape, dtype,
+                                      as_stream(stream));
+}
+
 int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx, const int64_t* mask,
                                  const float* blank_logit, const void* query, clusten_strides query_strides,
                                  const float* blank_key, float* probs, float* blank_prob, clusten_attn_shape shape,

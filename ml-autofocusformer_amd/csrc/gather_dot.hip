@@ -10,6 +10,24 @@ int gather_dot_f16(const void*, clusten_strides, const void*, clusten_strides, c
 int gather_dot_bf16(const void*, clusten_strides, const void*, clusten_strides, const int64_t*, void*,
                     const clusten_attn_shape&, hipStream_t);
 
+int gather_dot_clusters_f32(const void*, clusten_strides, const void*, clusten_strides, const int32_t*, void*,
+                            const clusten_attn_shape&, hipStream_t);
+int gather_dot_clusters_f16(const void*, clusten_strides, const void*, clusten_strides, const int32_t*, void*,
+                            const clusten_attn_shape&, hipStream_t);
+int gather_dot_clusters_bf16(const void*, clusten_strides, const void*, clusten_strides, const int32_t*, void*,
+                             const clusten_attn_shape&, hipStream_t);
+
+int launch_gather_dot_clusters(const void* a, clusten_strides as, const void* rows, clusten_strides rs,
+                               const int32_t* cluster_idx, void* out, clusten_attn_shape s, int dtype,
+                               hipStream_t stream) {
+    switch (dtype) {
+        case CLUSTEN_F32: return gather_dot_clusters_f32(a, as, rows, rs, cluster_idx, out, s, stream);
+        case CLUSTEN_F16: return gather_dot_clusters_f16(a, as, rows, rs, cluster_idx, out, s, stream);
+        case CLUSTEN_BF16: return gather_dot_clusters_bf16(a, as, rows, rs, cluster_idx, out, s, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
 int launch_gather_dot(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
                       void* out, clusten_attn_shape s, int dtype, hipStream_t stream) {
     switch (dtype) {

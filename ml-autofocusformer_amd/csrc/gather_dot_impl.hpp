@@ -90,7 +90,10 @@ struct Staging {
 // FAST = the list has at most 64 slots and a multiple of 4 of them: one chunk, and every access to
 // an out row is a whole aligned 16-byte group.  Otherwise lists go 64 slots at a time and the last
 // group of a row may be stored element by element.
-template <typename T, int C, int Q, bool FAST>
+// CLUSTERS (FAST kernels only) = the lists arrive as int32 cluster numbers, M/8 per token: slot j of a token is row
+// 8*g + j%8 of its cluster g = number j/8 (row 0 where that is past the last row, as the padded last cluster of a
+// cluster-ordered sequence is listed); `idx` then points to (B, N, M/8) int32.
+template <typename T, int C, int Q, bool FAST, bool CLUSTERS = false>
 __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restrict__ a, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H, int N, int M,
@@ -120,6 +123,8 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
     const char* a_tile = reinterpret_cast<const char*>(a + (int64_t)b * as.b + (int64_t)i0 * as.n);
     char* out_tile = reinterpret_cast<char*>(out + ((int64_t)b * H * N + i0) * M);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
+    const int32_t* cid_tile = reinterpret_cast<const int32_t*>(idx) + ((int64_t)b * N + i0) * (M >> 3);
+    int cid = 0;  // CLUSTERS: the cluster number of run `lane` of the tile (token lane / R, run lane % R)
     const uint32_t row_pitch = (uint32_t)rs.n * sizeof(T);
 
     // a-rows of head h -> slot h % 2.  Staging row = token; tokens past the end of a partial tile
@@ -161,7 +166,13 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
         // the tile's lists: are they all the same?  (only the first is kept in registers)
         int list0;
         bool same = true;
-        if constexpr (FAST) {
+        if constexpr (CLUSTERS) {
+            const int R = M >> 3, nruns = nt * R;
+            cid = cid_tile[min(lane, nruns - 1)];
+            same = lane >= nruns || cid == __shfl(cid, lane % R);   // against the same run of the tile's first token
+            const int row = __shfl(cid, slot >> 3) * 8 + (slot & 7);
+            list0 = row < N ? row : 0;
+        } else if constexpr (FAST) {
             // the nt lists are one contiguous block of nt*M*8 bytes: it travels by LDS-direct load in 1 KiB
             // accesses (a third of the vector-memory instructions that 8-byte loads per lane need) and is
             // compared from LDS
@@ -204,7 +215,10 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 const int R = M >> 3;             // runs per token
                 const int nruns = nt * R;         // <= 64: lane rho owns run rho = token * R + run
                 int v[8];
-                {
+                if constexpr (CLUSTERS) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) v[t] = cid * 8 + t < N ? cid * 8 + t : 0;
+                } else {
                     const int64_t* p = reinterpret_cast<const int64_t*>(stage) + min(lane, nruns - 1) * 8;  // lists in LDS
 #pragma unroll
                     for (int t = 0; t < 8; ++t) v[t] = (int)p[t];
@@ -340,7 +354,15 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
             const int tok_lo = shared_list ? 0 : pass;
             const int tok_hi = shared_list ? nt : pass + 1;
             // this pass's list: token `pass` of the tile (re-read from L2 for the per-token passes)
-            const int mine = pass == 0 ? list0 : (int)idx_tile[(int64_t)pass * M + j0 + slot];
+            int mine = list0;
+            if (pass > 0) {
+                if constexpr (CLUSTERS) {
+                    const int row = cid_tile[pass * (M >> 3) + (slot >> 3)] * 8 + (slot & 7);
+                    mine = row < N ? row : 0;
+                } else {
+                    mine = (int)idx_tile[(int64_t)pass * M + j0 + slot];
+                }
+            }
             uint32_t g_off[S::NI_G];
 #pragma unroll
             for (int i = 0; i < S::NI_G; ++i) {
@@ -458,12 +480,12 @@ __global__ __launch_bounds__(256) void gather_dot_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q, bool FAST>
+template <typename T, int C, int Q, bool FAST, bool CLUSTERS = false>
 int launch_tile_q(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
                   void* out, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q, FAST>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q, FAST, CLUSTERS>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
                        static_cast<const T*>(a), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, as, rs, tiles_per_batch, total);
     return launch_status();
@@ -488,6 +510,30 @@ int launch_elem(const void* a, clusten_strides as, const void* rows, clusten_str
     hipLaunchKernelGGL((gather_dot_elem_kernel<T>), dim3(grid), dim3(256), 0, stream, static_cast<const T*>(a),
                        static_cast<const T*>(rows), idx, static_cast<T*>(out), s.B, s.H, s.N, s.C, s.M, as, rs);
     return launch_status();
+}
+
+// Lists given as cluster numbers (see CLUSTERS above): `cluster_idx` is (B, N, M/8) int32.  Only the tile kernels
+// take this format: head dim 16/32/64, M a multiple of 8 up to 64, 16-byte aligned rows.
+template <typename T>
+int gather_dot_clusters_typed(const void* a, clusten_strides as, const void* rows, clusten_strides rs,
+                              const int32_t* cluster_idx, void* out, const clusten_attn_shape& s, hipStream_t stream) {
+    const bool vec_ok = rows_aligned16(rows, rs, sizeof(T)) && rows_aligned16(a, as, sizeof(T)) && aligned16(out) &&
+                        slice_fits_int32(rs, s.H, s.N, s.C) && slice_fits_int32(as, s.H, s.N, s.C);
+    if (!vec_ok) return CLUSTEN_ERR_UNALIGNED;
+    if (s.M % 8 != 0 || s.M > 64) return CLUSTEN_ERR_BAD_DIMS;
+    const int64_t* idx = reinterpret_cast<const int64_t*>(cluster_idx);
+    switch (s.C) {
+        case 16:
+            return s.M <= 48 ? launch_tile_q<T, 16, 3, true, true>(a, as, rows, rs, idx, out, s, stream)
+                             : launch_tile_q<T, 16, 4, true, true>(a, as, rows, rs, idx, out, s, stream);
+        case 32:
+            return s.M <= 48 ? launch_tile_q<T, 32, 3, true, true>(a, as, rows, rs, idx, out, s, stream)
+                             : launch_tile_q<T, 32, 4, true, true>(a, as, rows, rs, idx, out, s, stream);
+        case 64:
+            return s.M <= 48 ? launch_tile_q<T, 64, 3, true, true>(a, as, rows, rs, idx, out, s, stream)
+                             : launch_tile_q<T, 64, 4, true, true>(a, as, rows, rs, idx, out, s, stream);
+        default: return CLUSTEN_ERR_BAD_DIMS;
+    }
 }
 
 template <typename T>

@@ -83,7 +83,9 @@ struct SumStaging {
 // FAST = the list has at most 64 slots: one chunk, p-rows of two heads prefetched before the lists
 // are read.  Otherwise lists go 64 slots at a time and the D blocks accumulate over the chunks.
 // EXACT = the list has exactly 16*Q slots (no slot of the chunk is missing).
-template <typename T, int C, int Q, bool FAST, bool EXACT>
+// CLUSTERS (FAST kernels only) = the lists arrive as int32 cluster numbers, M/8 per token: slot j of a token is row
+// 8*g + j%8 of its cluster g = number j/8 (row 0 where that is past the last row); `idx` then points to (B, N, M/8) int32.
+template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false>
 __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H, int N, int M,
@@ -110,6 +112,8 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
 
     const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
+    const int32_t* cid_tile = reinterpret_cast<const int32_t*>(idx) + ((int64_t)b * N + i0) * (M >> 3);
+    int cid = 0;  // CLUSTERS: the cluster number of run `lane` of the tile (token lane / R, run lane % R)
     const uint32_t row_pitch = (uint32_t)rs.n * sizeof(T);
 
     // p pieces of head h, chunk at slot j0 -> slot `ps` of the staging buffer.  Access i moves pieces
@@ -135,6 +139,14 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     constexpr int MAXCH = FAST ? 1 : 4;  // chunks whose first list is kept in registers; longer lists re-read
     int list0[MAXCH];
     bool same = true;
+    if constexpr (CLUSTERS) {
+        const int R = M >> 3, nruns = nt * R;
+        const int slot = min(lane, M - 1);
+        cid = cid_tile[min(lane, nruns - 1)];
+        same = lane >= nruns || cid == __shfl(cid, lane % R);   // against the same run of the tile's first token
+        const int row = __shfl(cid, slot >> 3) * 8 + (slot & 7);
+        list0[0] = row < N ? row : 0;
+    } else
     for (int j0 = 0, ch = 0; j0 < M; j0 += kWave, ++ch) {
         const int mc = min(kWave, M - j0);
         const int slot = min(lane, mc - 1);  // lanes past the list repeat its last slot
@@ -213,7 +225,10 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             const int R = M >> 3;             // runs per token
             const int nruns = nt * R;         // <= 64: lane rho owns run rho = token * R + run
             int v[8];
-            {
+            if constexpr (CLUSTERS) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) v[t] = cid * 8 + t < N ? cid * 8 + t : 0;
+            } else {
                 const int64_t* lp = idx_tile + (int64_t)min(lane, nruns - 1) * 8;  // the tile's lists are contiguous
 #pragma unroll
                 for (int t = 0; t < 8; ++t) v[t] = (int)lp[t];
@@ -374,7 +389,16 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
         // FAST: one chunk; the byte offsets of its rows do not depend on the head
         uint32_t g_off[S::NI_G];
         if constexpr (FAST) {
-            const int mine = pass == 0 ? list0[0] : (int)idx_tile[(int64_t)pass * M + min(lane, M - 1)];
+            int mine = list0[0];
+            if (pass > 0) {
+                const int slot = min(lane, M - 1);
+                if constexpr (CLUSTERS) {
+                    const int row = cid_tile[pass * (M >> 3) + (slot >> 3)] * 8 + (slot & 7);
+                    mine = row < N ? row : 0;
+                } else {
+                    mine = (int)idx_tile[(int64_t)pass * M + slot];
+                }
+            }
 #pragma unroll
             for (int i = 0; i < S::NI_G; ++i) {
                 g_off[i] = (uint32_t)__shfl(mine, min(i * S::RPI + g_sub, M - 1)) * row_pitch + (uint32_t)(g_pos * 16);
@@ -499,13 +523,13 @@ __global__ __launch_bounds__(256) void gather_sum_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q, bool FAST, bool EXACT>
+template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false>
 int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int grid = xcd_grid(total);
-    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT>), dim3(grid), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT, CLUSTERS>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, rs, os, tiles_per_batch, total);
     return launch_status();
@@ -529,6 +553,30 @@ int launch_elem(const void* p, const void* rows, clusten_strides rs, const int64
     hipLaunchKernelGGL((gather_sum_elem_kernel<T>), dim3(grid), dim3(256), 0, stream, static_cast<const T*>(p),
                        static_cast<const T*>(rows), idx, static_cast<T*>(out), s.B, s.H, s.N, s.C, s.M, rs, os);
     return launch_status();
+}
+
+// Lists given as cluster numbers (see CLUSTERS above): `cluster_idx` is (B, N, M/8) int32.  Only the tile kernels
+// take this format: head dim 16/32/64, M a multiple of 8 up to 64, 16-byte aligned rows.
+template <typename T>
+int gather_sum_clusters_typed(const void* p, const void* rows, clusten_strides rs, const int32_t* cluster_idx, void* out,
+                              clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
+    const bool quads_ok = ((int64_t)s.M * sizeof(T)) % 16 == 0 && aligned16(p) && rows_aligned16(rows, rs, sizeof(T)) &&
+                          rows_aligned16(out, os, sizeof(T)) && slice_fits_int32(rs, s.H, s.N, s.C);
+    if (!quads_ok) return CLUSTEN_ERR_UNALIGNED;
+    if (s.M % 8 != 0 || s.M > 64) return CLUSTEN_ERR_BAD_DIMS;
+    const int64_t* idx = reinterpret_cast<const int64_t*>(cluster_idx);
+    switch (s.C) {
+        case 16:
+            return s.M == 48 ? launch_tile_q<T, 16, 3, true, true, true>(p, rows, rs, idx, out, os, s, stream)
+                             : launch_tile_q<T, 16, 4, true, false, true>(p, rows, rs, idx, out, os, s, stream);
+        case 32:
+            return s.M == 48 ? launch_tile_q<T, 32, 3, true, true, true>(p, rows, rs, idx, out, os, s, stream)
+                             : launch_tile_q<T, 32, 4, true, false, true>(p, rows, rs, idx, out, os, s, stream);
+        case 64:
+            return s.M == 48 ? launch_tile_q<T, 64, 3, true, true, true>(p, rows, rs, idx, out, os, s, stream)
+                             : launch_tile_q<T, 64, 4, true, false, true>(p, rows, rs, idx, out, os, s, stream);
+        default: return CLUSTEN_ERR_BAD_DIMS;
+    }
 }
 
 template <typename T>

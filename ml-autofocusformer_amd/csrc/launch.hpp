@@ -11,10 +11,21 @@ namespace clusten {
 int launch_gather_dot(const void* a, clusten_strides a_strides, const void* rows, clusten_strides rows_strides,
                       const int64_t* idx, void* out, clusten_attn_shape s, int dtype, hipStream_t stream);
 
+// The same with the lists given as cluster numbers: cluster_idx (B,N,M/8) int32, slot j of a token = row
+// 8*g + j%8 of its cluster number j/8 (row 0 where that is >= N).  F32/F16/BF16, C in {16,32,64}, M % 8 == 0, M <= 64.
+int launch_gather_dot_clusters(const void* a, clusten_strides a_strides, const void* rows, clusten_strides rows_strides,
+                               const int32_t* cluster_idx, void* out, clusten_attn_shape s, int dtype,
+                               hipStream_t stream);
+
 // out[b,h,i,c] = sum_j p[b,h,i,j] * rows[b,h,idx[b,i,j],c]      (AV forward; QK's d_query)
 //   p : contiguous (B,H,N,M);  rows, out : strided (B,H,N,C)
 int launch_gather_sum(const void* p, const void* rows, clusten_strides rows_strides, const int64_t* idx, void* out,
                       clusten_strides out_strides, clusten_attn_shape s, int dtype, hipStream_t stream);
+
+// The same with the lists given as cluster numbers (see launch_gather_dot_clusters).
+int launch_gather_sum_clusters(const void* p, const void* rows, clusten_strides rows_strides, const int32_t* cluster_idx,
+                               void* out, clusten_strides out_strides, clusten_attn_shape s, int dtype,
+                               hipStream_t stream);
 
 // out[b,h,idx[b,i,j],c] += p[b,h,i,j] * x[b,h,i,c]               (QK's d_key; AV's d_value)
 //   p : contiguous (B,H,N,M);  x : strided (B,H,N,C);  out : contiguous (B,H,N,C), zeroed here.

@@ -84,7 +84,7 @@ def _stage_inputs(b, side, c, gen):
 def test_neighbourhood_lists_are_runs_of_whole_clusters_nearest_first():
     layer = BasicLayer(32, 64, 8, 48, 1, 2, 2.0, ops=oracle_ops())
     pos, _ = _stage_inputs(2, 14, 32, torch.Generator().manual_seed(0))         # 196 tokens: 25 clusters, 4 pads
-    new_pos, ranking, member_idx, mask, pe_idx = layer.neighbourhoods(pos, 14, 14, 55, 111)
+    new_pos, ranking, member_idx, mask, pe_idx, cluster_idx = layer.neighbourhoods(pos, 14, 14, 55, 111)
     b, n, m = member_idx.shape
     assert (n, m) == (196, 48) and mask is not None
     runs = member_idx.reshape(b, n, 6, 8)
@@ -103,6 +103,10 @@ def test_neighbourhood_lists_are_runs_of_whole_clusters_nearest_first():
     d_first = (new_pos - centres.gather(1, (start[..., 0] // 8)[..., None].expand(-1, -1, 2))).norm(dim=-1)
     d_own = (new_pos - centres[:, torch.arange(196) // 8]).norm(dim=-1)
     assert (d_first <= d_own + 1e-6).all()
+    # the cluster numbers alone describe the lists: row 8g+t of cluster g, row 0 past the last token
+    rows = cluster_idx.long().unsqueeze(3) * 8 + torch.arange(8)
+    assert cluster_idx.dtype == torch.int32 and cluster_idx.shape == (b, n, 6)
+    assert torch.equal(torch.where(rows < n, rows, torch.zeros_like(rows)).reshape(b, n, m), member_idx)
     # position-table index = (dy + R) * width + (dx + R) of neighbour minus token
     nb = new_pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, 2)).reshape(b, n, m, 2)
     rel = nb - new_pos[:, :, None]
@@ -139,7 +143,7 @@ def test_merging_keeps_a_quarter_with_reserved_tokens_last_and_orders_channels_i
     layer = BasicLayer(16, 32, 8, 48, 1, 2, 2.0, ops=ops).eval()
     table, r = relative_position_table(64)
     pos, feat = _stage_inputs(2, 16, 16, torch.Generator().manual_seed(4))
-    new_pos, ranking, member_idx, mask, pe_idx = layer.neighbourhoods(pos, 16, 16, r, 2 * r + 1)
+    new_pos, ranking, member_idx, mask, pe_idx, _ = layer.neighbourhoods(pos, 16, 16, r, 2 * r + 1)
     feat = feat.gather(1, ranking.expand(-1, -1, 16))
     merge = layer.downsample
     prob = torch.rand(2, 256, 1)

@@ -255,6 +255,54 @@ def test_wf_full_size_stage1(device):
     assert out.abs().max() <= d.feat.abs().max() * (1 + 1e-6)
 
 
+def _cluster_numbers(b, n, nnc, gen, kind):
+    """(B,N,nnc) int32 cluster numbers: clusters = ceil(N/8); the last one may be short (its pad slots list row 0)."""
+    k = (n + 7) // 8
+    own = torch.arange(n) // 8
+    if kind == "shared":          # every token of a cluster lists the same clusters in the same order
+        per_cluster = torch.stack([torch.randperm(k, generator=gen)[:nnc] for _ in range(b * k)]).reshape(b, k, nnc)
+        return per_cluster[:, own].to(torch.int32).contiguous()
+    width = k if kind == "scattered" else min(12, k)
+    lo = torch.zeros(n, dtype=torch.int64) if kind == "scattered" else (own - width // 2).clamp(0, k - width)
+    pick = torch.rand(b, n, width, generator=gen).argsort(dim=2)[:, :, :nnc] + lo.view(1, n, 1)
+    return pick.to(torch.int32).contiguous()
+
+
+def _expand_clusters(cidx, n):
+    rows = cidx.long().unsqueeze(3) * 8 + torch.arange(8)
+    rows = torch.where(rows < n, rows, torch.zeros_like(rows))
+    return rows.reshape(cidx.shape[0], cidx.shape[1], -1).contiguous()
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_lists_given_as_cluster_numbers(device, kind, dtype):
+    gen = torch.Generator().manual_seed(71)
+    for n, c, nnc in ((396, 32, 6), (200, 64, 8), (64, 16, 2)):
+        b, h = 2, 3
+        q = (torch.randn(b, h, n, c, generator=gen) * c ** -0.5).to(dtype)
+        k = torch.randn(b, h, n, c, generator=gen).to(dtype)
+        v = torch.randn(b, h, n, c, generator=gen).to(dtype)
+        cidx = _cluster_numbers(b, n, nnc, gen, kind)
+        idx = _expand_clusters(cidx, n)
+        assert idx.max() < n and idx.shape == (b, n, 8 * nnc)
+        # against the oracle on the expanded lists ...
+        qr, kr, vr = _ref_inputs(q, k, v)
+        attn_ref = oracle.qk_gather_chunked(qr, kr, idx)
+        attn = _native.qk_forward_clusters(q.to(device), k.to(device), cidx.to(device))
+        assert attn.dtype == dtype and oracle.rel_err(attn, attn_ref) <= TOL[dtype]
+        p = torch.softmax(attn_ref, dim=-1).to(dtype)
+        feat_ref = oracle.av_gather_chunked(_ref_inputs(p)[0], vr, idx)
+        feat = _native.av_forward_clusters(p.to(device), v.to(device), cidx.to(device))
+        assert feat.dtype == dtype and oracle.rel_err(feat, feat_ref) <= TOL[dtype]
+        # ... and against the row-list entry points on the same lists
+        assert oracle.rel_err(attn, _native.qk_forward(q.to(device), k.to(device), idx.to(device)).cpu()) <= TOL[dtype]
+        assert oracle.rel_err(feat, _native.av_forward(p.to(device), v.to(device), idx.to(device)).cpu()) <= TOL[dtype]
+    assert not _native.clusters_supported(q.to(device), 9)
+    with pytest.raises(RuntimeError):
+        _native.qk_forward_clusters(q.to(device), k.to(device), cidx.long().to(device))
+
+
 def test_empty_inputs_give_empty_or_zero_outputs(device):
     # no batch elements, no tokens, or empty lists: nothing is launched
     for b, n, m in ((0, 16, 8), (2, 0, 8), (2, 16, 0)):
