@@ -235,7 +235,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the AFF-Tiny images/s leg")
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
-    ap.add_argument("--only", choices=("qk", "av", "wf", "copy"), default=None,
+    ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd"), default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -269,6 +269,10 @@ def main():
            lambda: _native.av_forward(attn, v, idx),
            lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
     torch.cuda.synchronize()
+    if args.only == "bwd":  # the three backward operators, for profilers
+        print(json.dumps({"only": "bwd", "launches": args.steps + args.warmup,
+                          **_bench_backward(acase, wcase, args.steps, args.warmup)}), flush=True)
+        return
     if args.only:
         if args.only == "copy":  # a plain copy of known traffic, to calibrate a profiler's byte counters
             src = torch.empty(qk_bytes // 8, dtype=torch.float32, device="cuda").normal_()
