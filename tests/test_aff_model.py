@@ -257,6 +257,23 @@ def test_operator_dtypes_under_autocast(device):
 
 
 @pytest.mark.gpu
+def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device):
+    """The configuration the images/s figure is quoted on: every operator call of AFF-Tiny at 224x224 under fp16
+    autocast (cluster-number lists, fused softmax, kNN kernel on the HIP side; tensor expressions on the other)."""
+    from aff.model import default_ops
+    torch.manual_seed(0)
+    hip = aff_tiny(ops=default_ops()).to(device).eval()
+    torch.manual_seed(0)
+    ref = aff_tiny(ops=oracle_ops()).to(device).eval()
+    ref.load_state_dict(hip.state_dict())
+    x = torch.randn(2, 3, 224, 224, generator=torch.Generator().manual_seed(3)).to(device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        y_hip, y_ref = hip(x), ref(x)
+    assert y_hip.shape == (2, 1000) and torch.isfinite(y_hip).all()
+    assert oracle.rel_err(y_hip.float(), y_ref.float()) < 2e-2
+
+
+@pytest.mark.gpu
 def test_aff_tiny_224_forward_and_gradients(device):
     model = aff_tiny().to(device)
     x = torch.randn(2, 3, 224, 224, device=device)
