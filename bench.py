@@ -125,11 +125,27 @@ def _bench_attn(case, steps, warmup, dtype=None):
     B, H, N, C = q.shape
     M = d.nbhd_idx.shape[-1]
     nbytes = wl.attn_bytes(B, H, N, C, M, q.element_size())
-    _, per, _ = _time_kernels([lambda: _native.qk_forward(q, k, d.nbhd_idx),
-                               lambda: _native.av_forward(attn, v, d.nbhd_idx)], steps, warmup)
+    # small shapes: rotate among copies of the inputs so that a launch never finds its data in the 256 MB
+    # memory-side cache (inputs of one QK + AV pair are about 1.7 x nbytes)
+    copies = max(1, min(16, int(700e6 // (1.7 * nbytes)) + 1))
+    sets = [(q, k, v, d.nbhd_idx, attn)] + [tuple(t.clone() for t in (q, k, v, d.nbhd_idx, attn)) for _ in range(copies - 1)]
+    turn = [0, 0]
+
+    def qk():
+        a = sets[turn[0] % copies]
+        turn[0] += 1
+        return _native.qk_forward(a[0], a[1], a[3])
+
+    def av():
+        a = sets[turn[1] % copies]
+        turn[1] += 1
+        return _native.av_forward(a[4], a[2], a[3])
+
+    _, per, _ = _time_kernels([qk, av], steps, warmup)
     return {"shape": "B%d H%d N%d C%d M%d %s" % (B, H, N, C, M, str(q.dtype).replace("torch.", "")),
             "qk_us": round(per[0] * 1e3, 1), "qk_GBps": round(nbytes / per[0] / 1e6, 1),
-            "av_us": round(per[1] * 1e3, 1), "av_GBps": round(nbytes / per[1] / 1e6, 1), "bytes_each": nbytes}
+            "av_us": round(per[1] * 1e3, 1), "av_GBps": round(nbytes / per[1] / 1e6, 1), "bytes_each": nbytes,
+            "input_sets_rotated": copies}
 
 
 def _bench_backward(acase, wcase, steps, warmup):
@@ -159,9 +175,20 @@ def _bench_wf(case, steps, warmup):
     B, Nout, M, IC = d.weights.shape
     N, C = d.feat.shape[1], d.feat.shape[2]
     nbytes = wl.wf_bytes(B, N, Nout, C, M, IC, d.feat.element_size())
-    _, per, _ = _time_kernels([lambda: _native.wf_forward(d.weights, d.feat, d.nbhd_idx)], steps, warmup)
+    copies = max(1, min(16, int(700e6 // nbytes) + 1))   # see _bench_attn
+    sets = [(d.weights, d.feat, d.nbhd_idx)] + [tuple(t.clone() for t in (d.weights, d.feat, d.nbhd_idx))
+                                                for _ in range(copies - 1)]
+    turn = [0]
+
+    def wf():
+        a = sets[turn[0] % copies]
+        turn[0] += 1
+        return _native.wf_forward(*a)
+
+    _, per, _ = _time_kernels([wf], steps, warmup)
     return {"shape": "B%d N%d->%d C%d M%d IC%d %s" % (B, N, Nout, C, M, IC, str(d.feat.dtype).replace("torch.", "")),
-            "wf_us": round(per[0] * 1e3, 1), "wf_GBps": round(nbytes / per[0] / 1e6, 1), "bytes": nbytes}
+            "wf_us": round(per[0] * 1e3, 1), "wf_GBps": round(nbytes / per[0] / 1e6, 1), "bytes": nbytes,
+            "input_sets_rotated": copies}
 
 
 def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
