@@ -171,7 +171,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
             cid = cid_tile[min(lane, nruns - 1)];
             same = lane >= nruns || cid == __shfl(cid, lane % R);   // against the same run of the tile's first token
             const int row = __shfl(cid, slot >> 3) * 8 + (slot & 7);
-            list0 = row < N ? row : 0;
+            list0 = (unsigned)row < (unsigned)N ? row : 0;  // also catches a negative cluster number
         } else if constexpr (FAST) {
             // the nt lists are one contiguous block of nt*M*8 bytes: it travels by LDS-direct load in 1 KiB
             // accesses (a third of the vector-memory instructions that 8-byte loads per lane need) and is
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 int v[8];
                 if constexpr (CLUSTERS) {
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) v[t] = cid * 8 + t < N ? cid * 8 + t : 0;
+                    for (int t = 0; t < 8; ++t) v[t] = (unsigned)(cid * 8 + t) < (unsigned)N ? cid * 8 + t : 0;
                 } else {
                     const int64_t* p = reinterpret_cast<const int64_t*>(stage) + min(lane, nruns - 1) * 8;  // lists in LDS
 #pragma unroll
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
             if (pass > 0) {
                 if constexpr (CLUSTERS) {
                     const int row = cid_tile[pass * (M >> 3) + (slot >> 3)] * 8 + (slot & 7);
-                    mine = row < N ? row : 0;
+                    mine = (unsigned)row < (unsigned)N ? row : 0;  // also catches a negative cluster number
                 } else {
                     mine = (int)idx_tile[(int64_t)pass * M + j0 + slot];
                 }

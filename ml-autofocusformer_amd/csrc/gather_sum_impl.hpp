@@ -145,7 +145,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
         cid = cid_tile[min(lane, nruns - 1)];
         same = lane >= nruns || cid == __shfl(cid, lane % R);   // against the same run of the tile's first token
         const int row = __shfl(cid, slot >> 3) * 8 + (slot & 7);
-        list0[0] = row < N ? row : 0;
+        list0[0] = (unsigned)row < (unsigned)N ? row : 0;  // also catches a negative cluster number
     } else
     for (int j0 = 0, ch = 0; j0 < M; j0 += kWave, ++ch) {
         const int mc = min(kWave, M - j0);
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             int v[8];
             if constexpr (CLUSTERS) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) v[t] = cid * 8 + t < N ? cid * 8 + t : 0;
+                for (int t = 0; t < 8; ++t) v[t] = (unsigned)(cid * 8 + t) < (unsigned)N ? cid * 8 + t : 0;
             } else {
                 const int64_t* lp = idx_tile + (int64_t)min(lane, nruns - 1) * 8;  // the tile's lists are contiguous
 #pragma unroll
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 const int slot = min(lane, M - 1);
                 if constexpr (CLUSTERS) {
                     const int row = cid_tile[pass * (M >> 3) + (slot >> 3)] * 8 + (slot & 7);
-                    mine = row < N ? row : 0;
+                    mine = (unsigned)row < (unsigned)N ? row : 0;  // also catches a negative cluster number
                 } else {
                     mine = (int)idx_tile[(int64_t)pass * M + slot];
                 }
