@@ -190,17 +190,6 @@ __device__ __forceinline__ void store_streaming(V* p, V v) {
     __builtin_nontemporal_store(v, p);
 }
 
-// ---- addressing ---------------------------------------------------------------------------------
-
-// Pin a wave-uniform pointer in scalar registers and hide how it was computed, so that
-// `base + (uint32_t)lane_offset` is selected as the scalar-base + 32-bit-vector-offset addressing
-// mode (one VGPR per access instead of a 64-bit VGPR pair and a 64-bit add).
-template <typename P>
-__device__ __forceinline__ P* uniform_base(P* p) {
-    asm volatile("" : "+s"(p));
-    return p;
-}
-
 // ---- workgroup id -> tile ----------------------------------------------------------------------
 
 // One short-lived one-wave workgroup per tile: on this device many small workgroups stream from HBM

@@ -1,8 +1,8 @@
 // Broadcast-operand FMAs on the DPP data path.
 //
-// The gather kernels multiply a small operand that is the same for every lane (a query row, a
-// row of attention weights, a row of down-sampling weights) with data that differs per lane
-// (the gathered rows).  Keeping the shared operand in LDS would make the LDS the bottleneck: every
+// The scatter kernel multiplies a small operand that is the same for every lane (a row of upstream
+// gradients) with data that differs per lane (rows of the other operand); the down-sampling kernel
+// spreads every token's list over the 16-lane rows of that token the same way.  Keeping the shared operand in LDS would make the LDS the bottleneck: every
 // FMA would need 4 bytes per lane from it.  Instead the shared operand is loaded so that each row
 // of 16 lanes holds the same 16 values of it in one VGPR, and the FMA reads lane `L` of its own
 // row through the DPP `row_newbcast:L` control.  One VALU instruction, no LDS, no scalar loads.
@@ -36,26 +36,6 @@ __device__ __forceinline__ void fma4_rowlane(float& acc, float b0, float b1, flo
         : "v"(b0), "v"(b1), "v"(b2), "v"(b3), "v"(x0), "v"(x1), "v"(x2), "v"(x3), "n"(L));
 }
 
-// acc[t] += b[t][L] * x for 8 accumulators that share the per-lane operand x.
-template <int L>
-__device__ __forceinline__ void fma8_rowlane(float (&acc)[8], float b0, float b1, float b2, float b3, float b4,
-                                             float b5, float b6, float b7, float x) {
-    static_assert(L >= 0 && L < 16, "row lane");
-    asm volatile(
-        "s_nop 1\n\t"
-        "v_fmac_f32_dpp %0, %8, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %1, %9, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %2, %10, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %3, %11, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %4, %12, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %5, %13, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %6, %14, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-        "v_fmac_f32_dpp %7, %15, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf"
-        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),
-          "+v"(acc[7])
-        : "v"(b0), "v"(b1), "v"(b2), "v"(b3), "v"(b4), "v"(b5), "v"(b6), "v"(b7), "v"(x), "n"(L));
-}
-
 // acc += b[L] * x
 template <int L>
 __device__ __forceinline__ void fma1_rowlane(float& acc, float b, float x) {
@@ -65,51 +45,6 @@ __device__ __forceinline__ void fma1_rowlane(float& acc, float b, float x) {
         "v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
         : "+v"(acc)
         : "v"(b), "v"(x), "n"(L));
-}
-
-// acc[v] += b[L] * x[v] for v < VEC (VEC = 1, 2, 4 or 8).
-template <int L, int VEC>
-__device__ __forceinline__ void fma_vec_rowlane(float (&acc)[VEC], float b, const float (&x)[VEC]) {
-    static_assert(L >= 0 && L < 16, "row lane");
-    static_assert(VEC == 1 || VEC == 2 || VEC == 4 || VEC == 8, "vector width");
-    if constexpr (VEC == 1) {
-        asm volatile(
-            "s_nop 1\n\t"
-            "v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
-            : "+v"(acc[0])
-            : "v"(b), "v"(x[0]), "n"(L));
-    } else if constexpr (VEC == 2) {
-        asm volatile(
-            "s_nop 1\n\t"
-            "v_fmac_f32_dpp %0, %2, %3 row_newbcast:%5 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %1, %2, %4 row_newbcast:%5 row_mask:0xf bank_mask:0xf"
-            : "+v"(acc[0]), "+v"(acc[1])
-            : "v"(b), "v"(x[0]), "v"(x[1]), "n"(L));
-    } else if constexpr (VEC == 4) {
-        asm volatile(
-            "s_nop 1\n\t"
-            "v_fmac_f32_dpp %0, %4, %5 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %1, %4, %6 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %2, %4, %7 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %3, %4, %8 row_newbcast:%9 row_mask:0xf bank_mask:0xf"
-            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])
-            : "v"(b), "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "n"(L));
-    } else {
-        asm volatile(
-            "s_nop 1\n\t"
-            "v_fmac_f32_dpp %0, %8, %9 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %1, %8, %10 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %2, %8, %11 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %3, %8, %12 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %4, %8, %13 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %5, %8, %14 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %6, %8, %15 row_newbcast:%17 row_mask:0xf bank_mask:0xf\n\t"
-            "v_fmac_f32_dpp %7, %8, %16 row_newbcast:%17 row_mask:0xf bank_mask:0xf"
-            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),
-              "+v"(acc[7])
-            : "v"(b), "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]),
-              "n"(L));
-    }
 }
 
 // Lane L of the caller's row of 16 lanes, in every lane of that row.
