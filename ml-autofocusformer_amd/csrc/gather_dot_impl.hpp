@@ -10,6 +10,8 @@
 // G the gathered rows, and it runs on the matrix cores as fp32 MFMA 16x16x4 blocks.
 //
 // Data path per head:
+//   0. lists: the tile's 8 lists are one contiguous block; it travels by LDS-direct load and is compared
+//      from LDS (FAST kernels) — 1 KiB accesses instead of 8-byte loads per lane.
 //   1. gather: `global_load_lds_dwordx4` moves the rows from HBM/L2 straight into LDS, 16 bytes per
 //      lane, consecutive lanes on consecutive pieces of one row (row-coalesced: a wave access covers
 //      64/pieces-per-row whole rows).  No VGPRs are held while the data travels, so the bytes a CU
@@ -24,11 +26,15 @@
 //      (tile, head) is a single contiguous chunk of 8*M elements, so the blocks are laid out
 //      row-major in LDS and leave with full-width 16-byte stores (lists of up to 64 slots).
 // One short-lived one-wave workgroup per tile; the latency of its dependent chain (lists, rows,
-// product, store) is hidden by the ~20 other waves resident on the CU.
+// product, store) is hidden by the ~16 other waves resident on the CU.
 //
 //   shared-list path — all tokens of the tile carry the same list (true for every tile of a
 //     cluster-ordered token sequence whose cluster shares its neighbourhood): one gather and one
 //     set of MFMAs per head serve the 8 tokens.
+//   union path — lists that differ but are made of runs of 8 slots of which the tile's tokens share most
+//     (the neighbourhoods of a cluster-ordered sequence: a run is the 8 members of one cluster): every
+//     distinct run is gathered and multiplied once per head, the scores go to an LDS matrix from which
+//     each token picks its own slots.
 //   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
 //     token's column is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
 //
@@ -37,8 +43,9 @@
 // Rows whose start is not 16-byte aligned, head dims other than 16/32/64 and fp64 take the
 // element-per-thread kernel at the bottom of the file.
 //
-// This header holds the templates; gather_dot_{f32,f16,bf16}.hip instantiate them per storage type
-// so that the translation units build in parallel, gather_dot.hip holds the dtype dispatch.
+// This header holds the templates; gather_dot_{f32,f16,bf16}.hip and gather_dot_clusters_{...}.hip (lists
+// given as cluster numbers) instantiate them per storage type so that the translation units build in
+// parallel, gather_dot.hip holds the dtype dispatch.
 #pragma once
 
 #include "launch.hpp"

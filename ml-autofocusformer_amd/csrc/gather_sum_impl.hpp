@@ -26,6 +26,10 @@
 //
 //   shared-list path — all tokens of the tile carry the same list: one gather and one set of MFMAs
 //     per head serve the 8 tokens.
+//   union path — lists that differ but are made of runs of 8 slots of which the tile's tokens share most
+//     (the neighbourhoods of a cluster-ordered sequence): every distinct run is gathered once, the p values
+//     are re-indexed by distinct run in LDS (zero where a token does not hold a run), one set of MFMAs per
+//     pass of 6 or 8 runs serves the 8 tokens.
 //   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
 //     token's row is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
 //
@@ -34,8 +38,9 @@
 // rows whose start is not 16-byte aligned and fp64 take the element-per-thread kernel at the
 // bottom of the file.
 //
-// This header holds the templates; gather_sum_{f32,f16,bf16}.hip instantiate them per storage type
-// so that the translation units build in parallel, gather_sum.hip holds the dtype dispatch.
+// This header holds the templates; gather_sum_{f32,f16,bf16}.hip and gather_sum_clusters_{...}.hip (lists
+// given as cluster numbers) instantiate them per storage type so that the translation units build in
+// parallel, gather_sum.hip holds the dtype dispatch.
 #pragma once
 
 #include "launch.hpp"

@@ -26,8 +26,9 @@
 // Rows that are not a multiple of 256 bytes, more than 4 inner channels, and weight rows that are
 // not whole 16-byte pieces take the element-per-thread kernel.
 //
-// Backward: plain kernels (one thread per d_w element; one wave-row per token for d_feat with one
-// fp32 atomic per (slot, channel)).
+// Backward: d_weights is a tile product on the matrix cores, one wave per output token (see
+// wf_dweights_tile_kernel; other shapes take one thread per element); d_feat is one workgroup per output token,
+// threads over channels, one fp32 atomic per (slot, channel) onto a contiguous destination row.
 //
 // This header holds the templates; wf_{f32,f16,bf16}.hip instantiate them per storage type so that
 // the translation units build in parallel, wf.hip holds the dtype dispatch.
