@@ -1,4 +1,6 @@
 """The synthetic input generators produce what the benchmark configurations describe."""
+import os
+
 import torch
 
 import workloads as wl
@@ -77,3 +79,11 @@ def test_algorithmic_bytes_match_the_published_table():
     assert round(wl.wf_bytes(128, 3136, 784, 64, 48, 1, 4) / 1e6, 1) == 186.3
     assert round(wl.attn_bytes(64, 4, 9216, 32, 48, 2) / 1e6, 1) == 755.0
     assert wl.attn_flops(128, 2, 3136, 32, 48) == 2 * 128 * 2 * 3136 * 48 * 32
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_one():
+    import subprocess
+    import sys as _sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([_sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
