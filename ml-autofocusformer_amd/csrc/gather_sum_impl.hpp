@@ -414,6 +414,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             F32x4 d[S::ECH];
 #pragma unroll
             for (int e = 0; e < S::ECH; ++e) d[e] = F32x4{0.f, 0.f, 0.f, 0.f};
+            bool stored = false;  // the 16-bit shared-list path writes its output itself
 
             for (int j0 = 0, ch = 0; j0 < (FAST ? 1 : M); j0 += kWave, ++ch) {
                 const int mc = FAST ? M : min(kWave, M - j0);
@@ -448,6 +449,71 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 }
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 __syncthreads();
+
+                if constexpr (sizeof(T) == 2 && FAST && EXACT) {
+                    if (shared_list && rows_contiguous) {
+                        // 16-bit data, 48 shared slots: the 16-bit matrix instructions take the operands as they
+                        // lie in LDS.  A (tokens x slots) is a p piece: 8 consecutive slots of a token.  B (slots
+                        // x 16 channels) needs, per lane, consecutive slots of one channel — a column of the
+                        // row-major gathered rows: `ds_read_b64_tr_b16` delivers it (lane r of a group of 16 points
+                        // at 4 channels of slot r / 4; lane n receives channel n of the 4 slots).  One 16x16x32
+                        // step covers slots 0..31, a second one slots 32..47 in the lower half of each lane's k
+                        // values (upper half zero: both steps are the same instruction, so the accumulator chain
+                        // is one the hardware orders by itself); products of 16-bit values are exact in fp32 and
+                        // the sums are fp32.
+                        typedef short S4 __attribute__((ext_vector_type(4)));
+                        typedef __attribute__((address_space(3))) S4* LdsS4;
+                        constexpr int CBN = C / 16;
+                        const char* p_tok = stage + S::P_BASE + ps * S::P_SLOT_BYTES + (n & 7) * 16;
+                        const Piece a32 = *reinterpret_cast<const Piece*>(p_tok + kq * kTileTokens * 16);
+                        const U32x2 a16 =
+                            *reinterpret_cast<const U32x2*>(p_tok + (4 + (kq >> 1)) * kTileTokens * 16 + (kq & 1) * 8);
+                        const char* col = stage + (n >> 2) * S::RB + (n & 3) * 8;  // slot n / 4 of a group of 4, 4 channels
+                        F32x4 dh[CBN];
+#pragma unroll
+                        for (int cb = 0; cb < CBN; ++cb) {
+                            const char* cbp = col + cb * 32;
+                            const S4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(cbp + (8 * kq) * S::RB));
+                            const S4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(cbp + (8 * kq + 4) * S::RB));
+                            const S4 b2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(cbp + (32 + 4 * kq) * S::RB));
+                            const U32x2 lo = __builtin_bit_cast(U32x2, b0), hi = __builtin_bit_cast(U32x2, b1);
+                            const Piece b32 = Piece{lo[0], lo[1], hi[0], hi[1]};
+                            dh[cb] = tile_mfma<T>(a32, b32, F32x4{0.f, 0.f, 0.f, 0.f});
+                            const U32x2 t2 = __builtin_bit_cast(U32x2, b2);
+                            dh[cb] = tile_mfma<T>(Piece{a16[0], a16[1], 0u, 0u}, Piece{t2[0], t2[1], 0u, 0u}, dh[cb]);
+                        }
+                        // lane (n, kq) holds tokens 4*kq + i of channel 16*cb + n: row-major chunk in LDS, then
+                        // full-width stores
+                        __syncthreads();
+                        if (kq < 2) {
+#pragma unroll
+                            for (int cb = 0; cb < CBN; ++cb) {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) {
+                                    reinterpret_cast<T*>(stage)[(4 * kq + i) * C + 16 * cb + n] = from_acc<T>(dh[cb][i]);
+                                }
+                            }
+                        }
+                        __syncthreads();
+                        constexpr int NO = (kTileTokens * S::RB + 1023) / 1024;
+                        Piece o[NO];
+#pragma unroll
+                        for (int i = 0; i < NO; ++i) {
+                            o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
+                        }
+                        __syncthreads();
+                        char* out_h =
+                            reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
+                        const int chunk_bytes = nt * S::RB;
+#pragma unroll
+                        for (int i = 0; i < NO; ++i) {
+                            const int off = i * 1024 + lane * 16;
+                            if (off < chunk_bytes) store_streaming(reinterpret_cast<Piece*>(out_h + off), o[i]);
+                        }
+                        stored = true;
+                        continue;
+                    }
+                }
 
                 // steps of 4 slots, taken one p piece at a time: all LDS reads of a batch of pieces (8 steps) are
                 // issued before its MFMAs so that their latency is paid once per batch, not once per step.
@@ -500,7 +566,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 }
             }
 
-            store_head(h, d, tok_lo, tok_hi, shared_list);
+            if (!stored) store_head(h, d, tok_lo, tok_hi, shared_list);
         }
     }
 }
