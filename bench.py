@@ -219,6 +219,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     ops.qk, ops.av, ops.wf = timed_call("qk", real.qk), timed_call("av", real.av), timed_call("wf", real.wf)
     ops.attn_softmax = timed_call("bias+mask+blank+softmax", real.attn_softmax)
     ops.qk_clusters, ops.av_clusters = timed_call("qk", real.qk_clusters), timed_call("av", real.av_clusters)
+    ops.cluster_attention = timed_call("qk+bias+mask+blank+softmax+av (one kernel)", real.cluster_attention)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()
     for layer in net.layers:
         layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)
@@ -366,7 +367,29 @@ def main():
                                     args.steps, args.warmup)
         other["cfg2_s1_model_like_lists_as_cluster_numbers"] = {"qk_us": round(per_c[0] * 1e3, 1),
                                                                  "av_us": round(per_c[1] * 1e3, 1)}
-        del mcase, cidx, mattn
+        # local attention of one block at the same shape under mixed precision: one kernel against the three
+        # operators' kernels with the softmax kernel between them (what the model ran before)
+        h16 = lambda t: t.to(torch.float16)
+        q16, k16, v16 = h16(mcase.query), h16(mcase.key), h16(mcase.value)
+        gen = torch.Generator().manual_seed(1029)
+        rows = 111 * 111                                  # offsets between two tokens of a 56 x 56 grid
+        table = h16(torch.randn(rows, 2, generator=gen)).cuda()
+        pe_idx = torch.randint(rows, (B, 3136, 48), generator=gen).cuda()
+        blank_k, blank_v = torch.randn(64, generator=gen).cuda(), torch.randn(64, generator=gen).cuda()
+
+        def three_kernels():
+            a = _native.qk_forward_clusters(q16, k16, cidx)
+            p, pb = _native.attn_softmax(a, table, pe_idx, None, query=q16, blank_key=blank_k)
+            return _native.av_forward_clusters(p, v16, cidx)
+
+        _, per_a, _ = _time_kernels([lambda: _native.cluster_attention(q16, k16, v16, cidx, table, pe_idx, None,
+                                                                       blank_k, blank_v), three_kernels],
+                                    args.steps, args.warmup)
+        fused_bytes = 4 * q16.numel() * 2 + cidx.numel() * 4 + pe_idx.numel() * 8
+        other["cfg2_s1_local_attention_fp16_model_like_lists"] = {
+            "one_kernel_us": round(per_a[0] * 1e3, 1), "three_kernels_us": round(per_a[1] * 1e3, 1),
+            "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
+        del mcase, cidx, mattn, q16, k16, v16, pe_idx
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:

@@ -196,6 +196,30 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
                                  float* blank_prob, clusten_attn_shape shape, int dtype,
                                  clusten_stream stream);
 
+/* Local attention of a cluster-ordered token sequence in one kernel (inference): CLUSTENQKFunction, the
+ * arithmetic clusten_attn_softmax_forward describes, CLUSTENAVFunction and the blank token's value
+ * (models/aff_transformer.py:120-155), on lists given as cluster numbers, without the (B,H,N,M) logits and
+ * probabilities ever reaching memory:
+ *   logit[b,h,i,j] = scale * <query[b,h,i], key[b,h,row(i,j)]> + bias_table[pe_idx[b,i,j], h] - 100 * (1 - mask[b,i,j])
+ *   blank[b,h,i]   = scale * <query[b,h,i], blank_key[h]>
+ *   p, p_blank     = softmax over the M neighbours and the blank token
+ *   out[b,h,i]     = sum_j p[b,h,i,j] * value[b,h,row(i,j)] + p_blank[b,h,i] * blank_value[h]
+ *   row(i,j)       = 8 * cluster_idx[b,i,j/8] + j%8, row 0 where that is not in [0,N)
+ * query, key, value, out: strided (B,H,N,C) of `dtype`; bias_table (rows,H) of `dtype`, contiguous;
+ * cluster_idx (B,N,M/8) int32; pe_idx (B,N,M) int64 in [0,rows) — unchecked; mask (B,N,M) int64 of 0/1 or NULL;
+ * blank_key, blank_value (H,C) fp32, contiguous.  Pass the unscaled query and the model's scale, or a scaled
+ * query and 1.  The probabilities are rounded to `dtype` before they weigh the value rows; sums are fp32.
+ * dtype F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and M = 48 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
+ * aligned (else CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
+int clusten_cluster_attention_forward(const void* query, clusten_strides query_strides,
+                                      const void* key, clusten_strides key_strides,
+                                      const void* value, clusten_strides value_strides,
+                                      const int32_t* cluster_idx, const void* bias_table,
+                                      const int64_t* pe_idx, const int64_t* mask,
+                                      const float* blank_key, const float* blank_value,
+                                      void* out, clusten_strides out_strides, float scale,
+                                      clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 
 /* K nearest neighbours of 2-D points inside each batch element: for query point q of batch element b,

@@ -34,7 +34,9 @@ def default_ops():
     return SimpleNamespace(qk=CLUSTENQKFunction.apply, av=CLUSTENAVFunction.apply, wf=CLUSTENWFFunction.apply,
                            attn_softmax=_native.attn_softmax, attn_softmax_supported=_native.attn_softmax_supported,
                            qk_clusters=_native.qk_forward_clusters, av_clusters=_native.av_forward_clusters,
-                           clusters_supported=_native.clusters_supported)
+                           clusters_supported=_native.clusters_supported,
+                           cluster_attention=_native.cluster_attention,
+                           cluster_attention_supported=_native.cluster_attention_supported)
 
 
 def relative_position_table(img_size):
@@ -103,9 +105,18 @@ class ClusterAttention(nn.Module):
         # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
         compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
                    and getattr(self.ops, "qk_clusters", None) is not None)
-        q = (self.q(feat) * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)        # (b,h,n,ch) view
+        q = self.q(feat)
         kv = self.kv(feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
+        one_kernel = getattr(self.ops, "cluster_attention", None)
+        if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
+                and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2])):
+            # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
+            # the values in one kernel; the query scale is applied to the scores inside it
+            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, cluster_idx, self.pos_embed(table),
+                             pe_idx, cluster_mask, self.blank_k, self.blank_v, scale=self.scale)
+            return self.proj_drop(self.proj(out))
+        q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:
             attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
         elif compact and self.ops.clusters_supported(q, cluster_idx.shape[2]):

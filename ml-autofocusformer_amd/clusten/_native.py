@@ -51,6 +51,8 @@ _PROTOTYPES = {
     "clusten_av_forward_clusters": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
                                                    _P]),
+    "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, _P,
+                                                        _P, Strides, ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
@@ -417,6 +419,67 @@ def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Ten
                                                 _ptr(blank_prob), shape, code, _stream(device)),
                "clusten_attn_softmax_forward")
     return probs, blank_prob
+
+
+def cluster_attention_supported(query: torch.Tensor, nnc: int) -> bool:
+    """True when `cluster_attention` takes this case: CUDA fp16 / bf16 queries of head dim 32, six clusters per token."""
+    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16) and query.dim() == 4
+            and query.shape[3] == 32 and nnc == 6)
+
+
+def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cluster_idx: torch.Tensor,
+                      bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_key: torch.Tensor,
+                      blank_value: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Local attention over the members of each token's clusters plus one blank token, in one kernel.
+
+    query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1); cluster_idx (B,N,6) integer;
+    bias_table (rows,H); pe_idx (B,N,48) int64; mask (B,N,48) of 0/1 or None; blank_key, blank_value (H*32,).
+    Returns softmax(scale * q.k + bias - 100 * (1 - mask) | scale * q.blank_key) applied to the gathered values and
+    the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the layout the output
+    projection takes).  No autograd: for inference.  The fused form of models/aff_transformer.py:120-155.
+    """
+    lib = load()
+    _require_cuda("query", query)
+    device = query.device
+    for name, t in (("key", key), ("value", value), ("bias_table", bias_table), ("pe_idx", pe_idx),
+                    ("blank_key", blank_key), ("blank_value", blank_value)):
+        _require_cuda(name, t, device)
+    if query.dim() != 4 or key.shape != query.shape or value.shape != query.shape:
+        raise RuntimeError("query, key and value must be (B,H,N,C) tensors of one shape")
+    b, h, n, c = query.shape
+    cidx = _cluster_idx(cluster_idx, (b, n), device)
+    m = 8 * cidx.shape[2]
+    if pe_idx.shape != (b, n, m) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")
+    if bias_table.dim() != 2 or bias_table.shape[1] != h:
+        raise RuntimeError("bias_table must have shape (rows, H)")
+    if blank_key.numel() != h * c or blank_value.numel() != h * c:
+        raise RuntimeError("blank_key and blank_value must have H*C elements")
+    code = _dtype_code(query, "query")
+    dtype = query.dtype
+    query, key, value = _rows(query), _rows(key.to(dtype)), _rows(value.to(dtype))
+    bias_table = bias_table.detach().to(dtype).contiguous()
+    pe_idx = pe_idx.contiguous()
+    if mask is not None:
+        _require_cuda("mask", mask, device)
+        if mask.shape != (b, n, m):
+            raise RuntimeError("mask must have shape (B,N,M)")
+        mask = mask.to(torch.int64).contiguous()
+    blank_key = blank_key.detach().reshape(h, c).float().contiguous()
+    blank_value = blank_value.detach().reshape(h, c).float().contiguous()
+    out = torch.empty(b, n, h, c, dtype=dtype, device=device)
+    if out.numel() == 0:
+        return out.reshape(b, n, h * c)
+    out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
+    shape = AttnShape(b, h, n, c, m)
+    with torch.cuda.device(device):
+        _check(lib.clusten_cluster_attention_forward(_ptr(query), _strides(query), _ptr(key), _strides(key),
+                                                     _ptr(value), _strides(value), _ptr(cidx), _ptr(bias_table),
+                                                     _ptr(pe_idx), _ptr(mask), _ptr(blank_key), _ptr(blank_value),
+                                                     _ptr(out), _strides(out_view), ctypes.c_float(scale), shape, code,
+                                                     _stream(device)),
+               "clusten_cluster_attention_forward")
+    return out.reshape(b, n, h * c)
 
 
 def knn2d_supported(query: torch.Tensor, database: torch.Tensor, k: int) -> bool:

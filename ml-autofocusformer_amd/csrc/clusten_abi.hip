@@ -167,6 +167,26 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
                                blank_key, probs, blank_prob, shape, dtype, as_stream(stream));
 }
 
+int clusten_cluster_attention_forward(const void* query, clusten_strides query_strides, const void* key,
+                                      clusten_strides key_strides, const void* value, clusten_strides value_strides,
+                                      const int32_t* cluster_idx, const void* bias_table, const int64_t* pe_idx,
+                                      const int64_t* mask, const float* blank_key, const float* blank_value, void* out,
+                                      clusten_strides out_strides, float scale, clusten_attn_shape shape, int dtype,
+                                      clusten_stream stream) {
+    if (!query || !key || !value || !cluster_idx || !bias_table || !pe_idx || !blank_key || !blank_value || !out) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
+        !strides_ok(out_strides, shape.C)) {
+        return CLUSTEN_ERR_BAD_STRIDE;
+    }
+    return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, cluster_idx, bias_table,
+                                    pe_idx, mask, blank_key, blank_value, out, out_strides, scale, shape, dtype,
+                                    as_stream(stream));
+}
+
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
                   clusten_stream stream) {
     if (!query || !database || !idx) return CLUSTEN_ERR_NULL_POINTER;

@@ -55,6 +55,15 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
                         const float* blank, const void* q, clusten_strides qs, const float* blank_k, float* probs,
                         float* blank_prob, clusten_attn_shape s, int dtype, hipStream_t stream);
 
+// Local attention of a cluster-ordered sequence in one kernel (QK, position bias, mask, blank token, softmax, AV,
+// blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16}, C = 32;
+//   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48);
+//   blank_k, blank_v : fp32 (H,C).
+int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
+                             clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
+                             const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
+                             clusten_strides os, float scale, clusten_attn_shape s, int dtype, hipStream_t stream);
+
 // idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
 //   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;
 //   idx int64; dist fp32 or null.

@@ -259,10 +259,15 @@ def test_operator_dtypes_under_autocast(device):
 @pytest.mark.gpu
 def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device):
     """The configuration the images/s figure is quoted on: every operator call of AFF-Tiny at 224x224 under fp16
-    autocast (cluster-number lists, fused softmax, kNN kernel on the HIP side; tensor expressions on the other)."""
+    autocast (local attention in one kernel on cluster-number lists, kNN kernel on the HIP side; tensor expressions
+    on the other)."""
     from aff.model import default_ops
+    ops = default_ops()
+    calls = []
+    one_kernel = ops.cluster_attention
+    ops.cluster_attention = lambda *a, **kw: (calls.append(a[0].dtype), one_kernel(*a, **kw))[1]
     torch.manual_seed(0)
-    hip = aff_tiny(ops=default_ops()).to(device).eval()
+    hip = aff_tiny(ops=ops).to(device).eval()
     torch.manual_seed(0)
     ref = aff_tiny(ops=oracle_ops()).to(device).eval()
     ref.load_state_dict(hip.state_dict())
@@ -271,6 +276,16 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
         y_hip, y_ref = hip(x), ref(x)
     assert y_hip.shape == (2, 1000) and torch.isfinite(y_hip).all()
     assert oracle.rel_err(y_hip.float(), y_ref.float()) < 2e-2
+    # the 25 blocks of the three local-attention stages took the one-kernel path, on fp16 operands
+    assert calls == [torch.float16] * 25
+    # the same model with the three operators and the softmax kernel between them
+    three = default_ops()
+    del three.cluster_attention
+    hip3 = aff_tiny(ops=three).to(device).eval()
+    hip3.load_state_dict(hip.state_dict())
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        y3 = hip3(x)
+    assert oracle.rel_err(y_hip.float(), y3.float()) < 2e-2
 
 
 @pytest.mark.gpu

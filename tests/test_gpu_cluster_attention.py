@@ -1,0 +1,137 @@
+"""GPU parity of the one-kernel local attention (`clusten_cluster_attention_forward`) against the composition
+of the CPU gather oracles and the tensor expressions the reference model writes between its two operators
+(models/aff_transformer.py:120-155), evaluated in fp32 from the same rounded inputs.
+
+Bar: max|x - ref| / max|ref| <= 1e-2 (16-bit data; the probabilities are rounded to the storage type before they
+weigh the values, the output is rounded once).
+"""
+import pytest
+import torch
+
+from clusten import _native
+from conftest import TOL
+from oracle import clusten_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+C, NNC, M = 32, 6, 48
+
+
+def _cluster_numbers(b, n, gen, kind):
+    """(B,N,6) int32 cluster numbers out of ceil(N/8) clusters (the last may be short: its pad slots list row 0)."""
+    k = (n + 7) // 8
+    own = torch.arange(n) // 8
+    if kind == "shared":        # the 8 tokens of a cluster list the same clusters
+        per = torch.stack([torch.randperm(k, generator=gen)[:NNC] for _ in range(b * k)]).reshape(b, k, NNC)
+        return per[:, own].to(torch.int32).contiguous()
+    width = k if kind == "scattered" else min(12, k)       # scattered: up to 48 distinct clusters per tile
+    lo = torch.zeros(n, dtype=torch.int64) if kind == "scattered" else (own - width // 2).clamp(0, k - width)
+    pick = torch.rand(b, n, width, generator=gen).argsort(dim=2)[:, :, :NNC] + lo.view(1, n, 1)
+    if kind == "repeated":      # a cluster listed twice by a token
+        pick[:, :, 3] = pick[:, :, 1]
+    return pick.to(torch.int32).contiguous()
+
+
+def _expand(cidx, n):
+    rows = cidx.long().unsqueeze(3) * 8 + torch.arange(8)
+    rows = torch.where((rows < n) & (rows >= 0), rows, torch.zeros_like(rows))
+    return rows.reshape(cidx.shape[0], cidx.shape[1], -1).contiguous()
+
+
+def _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale):
+    """fp32 evaluation of the model's attention on the expanded lists; returns (B,N,H*C)."""
+    b, h, n, c = q.shape
+    q, k, v, table = q.float(), k.float(), v.float(), table.float()
+    attn = oracle.qk_gather_chunked(q, k, idx) * scale                      # (b,h,n,m)
+    attn = attn + table[pe_idx].permute(0, 3, 1, 2)
+    if mask is not None:
+        attn = attn + (1 - mask.reshape(b, 1, n, -1)) * (-100.0)
+    blank = (q * blank_k.reshape(1, h, 1, c)).sum(-1, keepdim=True) * scale
+    p = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
+    out = oracle.av_gather_chunked(p[..., :-1].contiguous(), v, idx) + p[..., -1:] * blank_v.reshape(1, h, 1, c)
+    return out.permute(0, 2, 1, 3).reshape(b, n, h * c)
+
+
+def _case(b, h, n, gen, kind, dtype, with_mask, rows=97):
+    q = torch.randn(b, h, n, C, generator=gen).to(dtype)
+    k = torch.randn(b, h, n, C, generator=gen).to(dtype)
+    v = torch.randn(b, h, n, C, generator=gen).to(dtype)
+    cidx = _cluster_numbers(b, n, gen, kind)
+    table = torch.randn(rows, h, generator=gen).to(dtype)
+    pe_idx = torch.randint(rows, (b, n, M), generator=gen)
+    idx = _expand(cidx, n)
+    mask = None
+    if with_mask:
+        # pad slots of a short last cluster are masked, as the model's cluster mask does, plus a few others
+        mask = ((cidx.long().unsqueeze(3) * 8 + torch.arange(8)) < n).reshape(b, n, M).long()
+        mask = mask * (torch.rand(b, n, M, generator=gen) > 0.05).long()
+    blank_k = torch.randn(h * C, generator=gen)
+    blank_v = torch.randn(h * C, generator=gen)
+    return q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v
+
+
+def _run(device, case, scale):
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = case
+    ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale)
+    out = _native.cluster_attention(q.to(device), k.to(device), v.to(device), cidx.to(device), table.to(device),
+                                    pe_idx.to(device), None if mask is None else mask.to(device),
+                                    blank_k.to(device), blank_v.to(device), scale=scale)
+    assert out.dtype == q.dtype and out.shape == ref.shape and out.is_contiguous()
+    return oracle.rel_err(out, ref)
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_against_the_oracle_composition(device, kind, dtype):
+    gen = torch.Generator().manual_seed(81)
+    # 396 = 49 whole clusters and one of 4 tokens (a partial tile whose pad rows list row 0); 64: few clusters
+    for b, h, n in ((2, 3, 396), (1, 1, 64), (3, 4, 200)):
+        for with_mask in (False, True):
+            err = _run(device, _case(b, h, n, gen, kind, dtype, with_mask), scale=C ** -0.5)
+            assert err <= TOL[dtype], "%s %s n=%d mask=%s rel err %.3g" % (kind, dtype, n, with_mask, err)
+
+
+def test_strided_operands_and_unit_scale(device):
+    """q / k / v as the views a fused qkv projection leaves (channel stride 1, token stride 3*H*C)."""
+    gen = torch.Generator().manual_seed(82)
+    b, h, n = 2, 2, 136
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True)
+    packed = torch.stack([q, k, v], dim=0).permute(1, 3, 0, 2, 4).contiguous()        # (b, n, 3, h, c)
+    views = packed.to(device).permute(2, 0, 3, 1, 4)                                  # (3, b, h, n, c) views
+    assert not views[0].is_contiguous()
+    ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, 1.0)
+    out = _native.cluster_attention(views[0], views[1], views[2], cidx.to(device), table.to(device), pe_idx.to(device),
+                                    mask.to(device), blank_k.to(device), blank_v.to(device))
+    assert oracle.rel_err(out, ref) <= TOL[torch.float16]
+
+
+def test_equals_the_three_kernel_path(device):
+    """Same lists through qk_forward_clusters + attn_softmax + av_forward_clusters."""
+    gen = torch.Generator().manual_seed(83)
+    b, h, n = 2, 2, 392
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True)
+    d = lambda x: x.to(device)
+    attn = _native.qk_forward_clusters(d(q), d(k), d(cidx))
+    probs, blank = _native.attn_softmax(attn, d(table), d(pe_idx), d(mask), query=d(q), blank_key=d(blank_k))
+    three = _native.av_forward_clusters(probs, d(v), d(cidx)) + blank * d(blank_v).reshape(1, h, 1, C)
+    three = three.permute(0, 2, 1, 3).reshape(b, n, h * C)
+    one = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v))
+    assert oracle.rel_err(one.float().cpu(), three.float().cpu()) <= TOL[torch.float16]
+
+
+def test_unsupported_cases_are_refused(device):
+    gen = torch.Generator().manual_seed(84)
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(1, 2, 64, gen, "near", torch.float16, False)
+    d = lambda x: x.to(device)
+    assert _native.cluster_attention_supported(d(q), 6)
+    assert not _native.cluster_attention_supported(d(q).float(), 6)
+    assert not _native.cluster_attention_supported(d(q), 8)
+    assert not _native.cluster_attention_supported(q, 6)
+    with pytest.raises(RuntimeError):       # fp32 has no fused kernel
+        _native.cluster_attention(d(q).float(), d(k).float(), d(v).float(), d(cidx), d(table), d(pe_idx), None,
+                                  d(blank_k), d(blank_v))
+    with pytest.raises(RuntimeError):       # CPU tensors
+        _native.cluster_attention(q, k, v, cidx, table, pe_idx, None, blank_k, blank_v)
+    empty = _native.cluster_attention(d(q)[:0], d(k)[:0], d(v)[:0], d(cidx)[:0], d(table), d(pe_idx)[:0], None,
+                                      d(blank_k), d(blank_v))
+    assert empty.shape == (0, 64, 2 * C)
