@@ -13,18 +13,20 @@
 // attention layer of the shipped models under mixed precision.
 //
 // One wave owns 8 consecutive tokens (one cluster) and walks the heads.  The tile's 48 cluster numbers are
-// numbered by distinct value (`U` of them, typically 8-14: neighbouring tokens choose among the same clusters);
-// per head the rows of 8 distinct clusters at a time (a pass: 64 rows) travel to LDS by LDS-direct loads, and
-//   QK  S[row][token] = K_pass (64 x 32) * q^T (32 x 8): four 16x16x32 matrix instructions; each token picks its own
+// numbered by distinct value (`U` of them; 7-12 in the shipped models: neighbouring tokens choose among the same
+// clusters); per head the rows of up to 12 distinct clusters at a time (a pass: 96 rows) travel to LDS by
+// LDS-direct loads, and
+//   QK  S[row][token] = K_pass (96 x 32) * q^T (32 x 8): six 16x16x32 matrix instructions; each token picks its own
 //       slots from the score matrix in LDS;
 //   softmax: lane (t = lane / 8, i = lane % 8) holds slots 8*r + i, r < 6, of token t; maxima and sums go across the
 //       8 lanes of a token;
-//   AV  out (8 x 32) = P_pass (8 x 64) * V_pass (64 x 32): the probabilities are written to LDS re-indexed by
+//   AV  out (8 x 32) = P_pass (8 x 96) * V_pass (96 x 32): the probabilities are written to LDS re-indexed by
 //       distinct cluster (zero where a token does not hold the cluster; a cluster held twice adds up), rounded to
 //       the storage type; the V operand needs consecutive rows of one channel per lane, which
 //       `ds_read_b64_tr_b16` delivers from the row-major rows.
-// The next pass's rows (the V rows during the softmax, the next head's K rows during the last AV pass) are
-// requested as soon as the current operands are in registers.
+// The first K and V rows of the next head are requested during the last AV pass of the current one, ahead of its
+// output store, so that a head whose clusters fit one pass never waits for rows.  Tiles with more distinct
+// clusters (up to 48: lists with nothing in common) take further passes.
 //
 // A token whose probabilities are zero for a cluster still multiplies that cluster's V rows by zero: non-finite
 // values in rows a token does not list reach its output as NaN (the unfused operators share this on their
@@ -39,33 +41,72 @@ constexpr int kC = 32;            // head dim
 constexpr int kR = 6;             // clusters per token
 constexpr int kM = 8 * kR;        // neighbours per token
 constexpr int kRB = kC * 2;       // bytes per row
-constexpr int kPassRuns = 8;      // distinct clusters per pass
-constexpr int kPassRows = 64;
+constexpr int kPassRuns = 12;     // distinct clusters per pass
+constexpr int kPassRows = 8 * kPassRuns;
+constexpr int kBlocks = kPassRows / 16;   // 16-row blocks of the score product
+constexpr int kSteps = kPassRows / 32;    // 32-row steps of the value product
+constexpr int kAccesses = kPassRows / 16; // wave accesses (16 rows of 64 bytes) per pass
 constexpr int kSRow = kPassRows + 4;   // floats per token row of the score matrix
-constexpr int kPRow = kPassRows + 8;   // 16-bit elements per token row of the re-indexed probabilities
+constexpr int kPRow = kPassRows + 8;   // 16-bit elements per token row of the re-indexed probabilities; the last 8
+                                       // are never read: cells for the writes of runs outside the pass
 
-constexpr int K_BASE = 0;                                  // 64 K rows
-constexpr int V_BASE = K_BASE + kPassRows * kRB;           // 64 V rows
-constexpr int S_BASE = V_BASE + kPassRows * kRB;           // scores of a pass
-constexpr int P_BASE = S_BASE + kTileTokens * kSRow * 4;   // probabilities of a pass; reused for the output chunk
+// LDS: two row areas and small tables.
+//   [K_BASE, +6144)  K rows of a pass; once they are in registers the score matrix; during the AV passes the
+//                    probabilities of a pass (the next head's K rows are requested only once those are in registers)
+//   [V_BASE, +6144)  V rows of a pass
+constexpr int K_BASE = 0;
+constexpr int S_BASE = K_BASE;
+constexpr int P_BASE = K_BASE;
 constexpr int P_BYTES = kTileTokens * kPRow * 2;
-constexpr int Q_BASE = P_BASE + P_BYTES;                   // q rows of two heads (slot h % 2)
+constexpr int V_BASE = K_BASE + kPassRows * kRB;
+constexpr int O_BASE = V_BASE + kPassRows * kRB;           // output chunk of a head
+constexpr int Q_BASE = O_BASE + kTileTokens * kRB;         // q rows of two heads (slot h % 2)
 constexpr int Q_SLOT = kTileTokens * kRB;
 constexpr int UL_BASE = Q_BASE + 2 * Q_SLOT;               // cluster number of each distinct cluster
 constexpr int PB_BASE = UL_BASE + kTileTokens * kR * 4;    // blank-token probability per token
 constexpr int LDS_BYTES = PB_BASE + kTileTokens * 4;
-static_assert(P_BYTES % 16 == 0 && P_BASE % 16 == 0 && Q_BASE % 16 == 0, "16-byte LDS accesses");
-static_assert(P_BYTES >= kTileTokens * kRB, "the output chunk fits the probability area");
+static_assert(P_BYTES % 16 == 0 && P_BYTES <= kPassRows * kRB, "the probabilities fit the K area");
+static_assert(kTileTokens * kSRow * 4 <= kPassRows * kRB, "the scores fit the K area");
+static_assert(kPassRows % 32 == 0 && Q_BASE % 16 == 0, "whole 32-row steps");
 
+// Reductions over the 8 lanes of a token (lanes 8t .. 8t+7) with data-parallel-primitive moves: neighbours in a
+// quad, the other pair of the quad, then the mirrored lane of the other quad.  Every lane ends with the same value.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float oct_max(float v) {
-#pragma unroll
-    for (int m = 1; m < 8; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    return fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
 }
 __device__ __forceinline__ float oct_sum(float v) {
-#pragma unroll
-    for (int m = 1; m < 8; m <<= 1) v += __shfl_xor(v, m);
-    return v;
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    return v + dpp_move<0x141>(v);
+}
+
+// Keeps a 32-bit byte offset a 32-bit register value at the place of use, so that the access it feeds is encoded
+// as uniform base + lane offset instead of through a 64-bit address per lane held across the loops.
+__device__ __forceinline__ uint32_t lane_offset(uint32_t off) {
+    asm volatile("" : "+v"(off));
+    return off;
+}
+
+// Orders the LDS traffic of the wave (a workgroup is one wave): everything issued so far has completed, and the
+// compiler moves no memory access across.  Unlike __syncthreads() it leaves vector-memory operations in flight.
+__device__ __forceinline__ void lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+}
+// The same, and at most `VM` vector-memory operations (LDS-direct loads, loads, stores; they complete in order)
+// are still in flight.
+template <int VM>
+__device__ __forceinline__ void lds_sync_vm() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(VM) & 0xF0FF);  // vmcnt(VM) lgkmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 }
 
 template <typename T>
@@ -99,25 +140,33 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const uint32_t q_off = (uint32_t)min(g_sub, nt - 1) * (uint32_t)qs.n * 2 + (uint32_t)g_pos * 16;
     auto fetch_q = [&](int h) {
         if (lane < 32) {
-            CLUSTEN_LDS_DMA16(q_tile + (int64_t)h * qs.h * 2 + q_off, stage + Q_BASE + (h & 1) * Q_SLOT);
+            CLUSTEN_LDS_DMA16(q_tile + (int64_t)h * qs.h * 2 + lane_offset(q_off), stage + Q_BASE + (h & 1) * Q_SLOT);
         }
     };
     fetch_q(0);
     if (H > 1) fetch_q(1);
 
-    // per-slot inputs the heads share
-    int pe[kR];
-    float off[kR];
-#pragma unroll
-    for (int r = 0; r < kR; ++r) {
-        pe[r] = (int)pe_idx[tok * kM + 8 * r + i];
-        off[r] = mask ? (float)(1 - mask[tok * kM + 8 * r + i]) * -100.f : 0.f;
-    }
-
-    // number the distinct cluster numbers of the tile in order of first appearance: lane rho < 48 owns run rho =
-    // token * 6 + run
+    // cluster numbers: lane rho < 48 owns run rho = token * 6 + run of the tile
     const int rho = min(lane, kTileTokens * kR - 1);
     const int cid = cluster_idx[((int64_t)b * N + i0 + min(rho / kR, nt - 1)) * kR + rho % kR];
+
+    // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
+    int pe[kR];
+    {
+        int64_t wide[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) wide[r] = pe_idx[tok * kM + 8 * r + i];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) pe[r] = (int)wide[r] & 0x7fffffff;
+        if (mask) {
+#pragma unroll
+            for (int r = 0; r < kR; ++r) wide[r] = mask[tok * kM + 8 * r + i];
+#pragma unroll
+            for (int r = 0; r < kR; ++r) pe[r] |= wide[r] == 0 ? (int)0x80000000 : 0;
+        }
+    }
+
+    // number the distinct cluster numbers in order of first appearance
     uint64_t remaining = (1ull << (kTileTokens * kR)) - 1;
     int uslot = 0, U = 0;
     bool first = false;
@@ -136,7 +185,16 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     int us[kR];  // distinct-cluster number of this lane's token's runs
 #pragma unroll
     for (int r = 0; r < kR; ++r) us[r] = __shfl(uslot, t * kR + r);
-    __syncthreads();
+    // does a token of the tile list a cluster twice?  Bit r: run r repeats an earlier run of the token; its
+    // probability is then added to that run's before the probabilities are laid out by distinct cluster.
+    int repeats = 0;
+#pragma unroll
+    for (int r = 1; r < kR; ++r) {
+#pragma unroll
+        for (int r2 = 0; r2 < r; ++r2) repeats |= us[r] == us[r2] ? 1 << r : 0;
+    }
+    const bool twice = __any(repeats) != 0;
+    lds_sync();
 
     const int total_rows = 8 * U;
     const int passes = (U + kPassRuns - 1) / kPassRuns;
@@ -144,28 +202,54 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const char* k_b = reinterpret_cast<const char*>(k + (int64_t)b * ks.b);
     const char* v_b = reinterpret_cast<const char*>(v + (int64_t)b * vs.b);
 
-    // rows of the distinct clusters 8*pass .. 8*pass+7 of one head -> LDS, 16 rows per access; clusters past the
-    // last one repeat it so that every row of a 32-row step holds data
-    auto gather = [&](const char* rows_bh, uint32_t pitch, int pass, int lds_base) {
-        const int rows_here = min(kPassRows, total_rows - pass * kPassRows);
+    // rows of the distinct clusters 8*pass .. 8*pass+7, as this lane gathers them: access a moves row 16*a + g_sub of
+    // the pass; clusters past the last one repeat it so that every row of a 32-row step holds data
+    auto pass_rows = [&](int pass, uint32_t (&rr)[kAccesses]) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
+        for (int a = 0; a < kAccesses; ++a) {
+            const int urow = a * 16 + g_sub;
+            const int c = ulist[min(pass * kPassRuns + (urow >> 3), U - 1)];
+            const int row = c * 8 + (urow & 7);
+            rr[a] = (unsigned)row < (unsigned)N ? (uint32_t)row : 0u;
+        }
+    };
+    auto gather = [&](const char* rows_bh, uint32_t pitch, const uint32_t (&rr)[kAccesses], int rows_here, int lds_base) {
+#pragma unroll
+        for (int a = 0; a < kAccesses; ++a) {
             if ((a & ~1) * 16 < rows_here) {
-                const int urow = a * 16 + g_sub;
-                const int c = ulist[min(pass * kPassRuns + (urow >> 3), U - 1)];
-                const int row = c * 8 + (urow & 7);
-                const uint32_t rr = (unsigned)row < (unsigned)N ? (uint32_t)row : 0u;
-                CLUSTEN_LDS_DMA16(rows_bh + (rr * pitch + (uint32_t)g_pos * 16), stage + lds_base + a * 1024);
+                CLUSTEN_LDS_DMA16(rows_bh + lane_offset(rr[a] * pitch + (uint32_t)g_pos * 16), stage + lds_base + a * 1024);
             }
         }
     };
-
-    gather(k_b, k_pitch, 0, K_BASE);
+    uint32_t rr0[kAccesses];  // pass 0: used by every head
+    pass_rows(0, rr0);
+    const int rows0 = min(kPassRows, total_rows);
+    gather(k_b, k_pitch, rr0, rows0, K_BASE);
+    gather(v_b, v_pitch, rr0, rows0, V_BASE);
 
     for (int h = 0; h < H; ++h) {
         const char* k_bh = k_b + (int64_t)h * ks.h * 2;
         const char* v_bh = v_b + (int64_t)h * vs.h * 2;
         const char* q_lds = stage + Q_BASE + (h & 1) * Q_SLOT;
+
+        // The first K and V rows of this head were requested during the previous head (or above); the only
+        // vector-memory operation issued after them is that head's output store, which may stay in flight.
+        if (h == 0) {
+            lds_sync_vm<0>();
+        } else {
+            lds_sync_vm<1>();
+        }
+
+        // small per-head operands: their latency passes under the score computation
+        float bias[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            const uint32_t cell = lane_offset(((uint32_t)(pe[r] & 0x7fffffff) * (uint32_t)H + (uint32_t)h) * 2);
+            bias[r] = to_acc(*reinterpret_cast<const T*>(reinterpret_cast<const char*>(table) + cell)) +
+                      (pe[r] < 0 ? -100.f : 0.f);
+        }
+        const float4 bk = *reinterpret_cast<const float4*>(blank_k + h * kC + 4 * i);
+        const float bv[2] = {blank_v[h * kC + r16], blank_v[h * kC + 16 + r16]};
 
         // ---- scores -------------------------------------------------------------------------------------
         float logit[kR];
@@ -173,24 +257,18 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         for (int r = 0; r < kR; ++r) logit[r] = 0.f;
         for (int pass = 0; pass < passes; ++pass) {
             const int rows_here = min(kPassRows, total_rows - pass * kPassRows);
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-            __syncthreads();  // the K rows of this pass (and the q rows) are in LDS; the previous pass has picked
-            Piece kraw[4];
+            if (pass > 0) lds_sync_vm<0>();  // the K rows of this pass are in LDS
+            const Piece qraw = *reinterpret_cast<const Piece*>(q_lds + (r16 & 7) * kRB + kq * 16);
+            Piece kraw[kBlocks];
 #pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
+            for (int blk = 0; blk < kBlocks; ++blk) {
                 if (blk * 16 < rows_here) {
                     kraw[blk] = *reinterpret_cast<const Piece*>(stage + K_BASE + (blk * 16 + r16) * kRB + kq * 16);
                 }
             }
-            const Piece qraw = *reinterpret_cast<const Piece*>(q_lds + (r16 & 7) * kRB + kq * 16);
-            __syncthreads();  // operands are in registers: the K area is free
-            if (pass + 1 < passes) {
-                gather(k_bh, k_pitch, pass + 1, K_BASE);
-            } else {
-                gather(v_bh, v_pitch, 0, V_BASE);
-            }
+            lds_sync();  // the K rows are in registers: their area takes the scores
 #pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
+            for (int blk = 0; blk < kBlocks; ++blk) {
                 if (blk * 16 < rows_here) {
                     const F32x4 d = tile_mfma<T>(kraw[blk], qraw, F32x4{0.f, 0.f, 0.f, 0.f});
                     // lane (r16, kq): pass rows 16*blk + 4*kq .. +3 of token r16
@@ -199,13 +277,19 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
                     }
                 }
             }
-            __syncthreads();
+            lds_sync();
 #pragma unroll
             for (int r = 0; r < kR; ++r) {
-                const int u = us[r] - pass * kPassRuns;
-                if (u >= 0 && u < kPassRuns) {
-                    logit[r] = *reinterpret_cast<const float*>(stage + S_BASE + (t * kSRow + u * 8 + i) * 4);
-                }
+                const unsigned u = (unsigned)(us[r] - pass * kPassRuns);
+                const float sc = *reinterpret_cast<const float*>(
+                    stage + S_BASE + (t * kSRow + (int)min(u, (unsigned)kPassRuns - 1) * 8 + i) * 4);
+                logit[r] = u < (unsigned)kPassRuns ? sc : logit[r];
+            }
+            if (pass + 1 < passes) {
+                lds_sync();  // the scores are picked: the area takes the next K rows
+                uint32_t rr[kAccesses];
+                pass_rows(pass + 1, rr);
+                gather(k_bh, k_pitch, rr, min(kPassRows, total_rows - (pass + 1) * kPassRows), K_BASE);
             }
         }
 
@@ -214,13 +298,12 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
-            x[r] = logit[r] * scale + to_acc(table[(int64_t)pe[r] * H + h]) + off[r];
+            x[r] = logit[r] * scale + bias[r];
             mx = fmaxf(mx, x[r]);
         }
         float part = 0.f;
         {
             const T* qrow = reinterpret_cast<const T*>(q_lds + t * kRB) + 4 * i;
-            const float4 bk = *reinterpret_cast<const float4*>(blank_k + h * kC + 4 * i);
             part = to_acc(qrow[0]) * bk.x + to_acc(qrow[1]) * bk.y + to_acc(qrow[2]) * bk.z + to_acc(qrow[3]) * bk.w;
         }
         const float bl = oct_sum(part) * scale;
@@ -237,79 +320,85 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
 #pragma unroll
         for (int r = 0; r < kR; ++r) p[r] *= inv;
         if (i == 0) *reinterpret_cast<float*>(stage + PB_BASE + t * 4) = eb * inv;
+        if (twice) {
+#pragma unroll
+            for (int r = kR - 1; r >= 1; --r) {
+#pragma unroll
+                for (int r2 = 0; r2 < r; ++r2) {
+                    // the first run with the same cluster collects the probabilities of its repeats
+                    bool firstmatch = us[r] == us[r2] && ((repeats >> r) & 1) && !((repeats >> r2) & 1);
+                    p[r2] += firstmatch ? p[r] : 0.f;
+                }
+            }
+        }
 
         // ---- weighted sum of the V rows --------------------------------------------------------------------------
         F32x4 acc[2] = {F32x4{0.f, 0.f, 0.f, 0.f}, F32x4{0.f, 0.f, 0.f, 0.f}};
         for (int pass = 0; pass < passes; ++pass) {
             const int rows_here = min(kPassRows, total_rows - pass * kPassRows);
-            __syncthreads();  // the previous pass's (or head's) reads of the probability area are complete
-            // probabilities of this pass, re-indexed by distinct cluster: zero, then each lane adds its own
+            lds_sync();  // the previous reads of the probability area (K area) are complete
+            // probabilities of this pass, re-indexed by distinct cluster: zero, then each lane puts in its own
             *reinterpret_cast<Piece*>(stage + P_BASE + lane * 16) = Piece{0u, 0u, 0u, 0u};
+            static_assert(P_BYTES > 1024 && P_BYTES <= 2048, "two accesses clear the probabilities");
             if (lane < (P_BYTES - 1024) / 16) {
                 *reinterpret_cast<Piece*>(stage + P_BASE + 1024 + lane * 16) = Piece{0u, 0u, 0u, 0u};
             }
-            __syncthreads();
+            lds_sync();
+            T* prow = reinterpret_cast<T*>(stage + P_BASE) + t * kPRow + i;
 #pragma unroll
             for (int r = 0; r < kR; ++r) {
-                const int u = us[r] - pass * kPassRuns;
-                if (u >= 0 && u < kPassRuns) {
-                    T* cell = reinterpret_cast<T*>(stage + P_BASE) + t * kPRow + u * 8 + i;
-                    *cell = from_acc<T>(to_acc(*cell) + p[r]);
-                }
+                // runs of other passes, and repeats (already added to their first run), go to the spare cells
+                const unsigned u = ((repeats >> r) & 1) ? ~0u : (unsigned)(us[r] - pass * kPassRuns);
+                prow[min(u, (unsigned)kPassRuns) * 8] = from_acc<T>(p[r]);
             }
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-            __syncthreads();  // the V rows of this pass are in LDS, the probabilities are written
-            Piece a[2];
-            S4 bt[2][2][2];  // [step][channel block][rows 0-3 / 4-7 of the lane's 8]
+            if (pass > 0) {
+                lds_sync_vm<0>();  // the V rows of this pass are in LDS, the probabilities are written
+            } else {
+                lds_sync();
+            }
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
+            for (int s = 0; s < kSteps; ++s) {
                 if (s * 32 < rows_here) {
-                    a[s] = *reinterpret_cast<const Piece*>(stage + P_BASE + ((r16 & 7) * kPRow + 32 * s + 8 * kq) * 2);
+                    const Piece a = *reinterpret_cast<const Piece*>(stage + P_BASE + ((r16 & 7) * kPRow + 32 * s + 8 * kq) * 2);
                     const char* col = stage + V_BASE + (32 * s + 8 * kq + (r16 >> 2)) * kRB + (r16 & 3) * 8;
 #pragma unroll
                     for (int cb = 0; cb < 2; ++cb) {
-                        bt[s][cb][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(col + cb * 32));
-                        bt[s][cb][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(col + cb * 32 + 4 * kRB));
+                        // rows 0-3 and 4-7 of the lane's 8, transposed to channel 16*cb + r16
+                        const S4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(col + cb * 32));
+                        const S4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsS4)(col + cb * 32 + 4 * kRB));
+                        const U32x2 lo = __builtin_bit_cast(U32x2, b0), hi = __builtin_bit_cast(U32x2, b1);
+                        acc[cb] = tile_mfma<T>(a, Piece{lo[0], lo[1], hi[0], hi[1]}, acc[cb]);
                     }
                 }
             }
-            __syncthreads();  // operands are in registers: the V area is free
+            lds_sync();  // the operands have been read: the V area and the probability area are free
             if (pass + 1 < passes) {
-                gather(v_bh, v_pitch, pass + 1, V_BASE);
+                uint32_t rr[kAccesses];
+                pass_rows(pass + 1, rr);
+                gather(v_bh, v_pitch, rr, min(kPassRows, total_rows - (pass + 1) * kPassRows), V_BASE);
             } else if (h + 1 < H) {
-                gather(k_b + (int64_t)(h + 1) * ks.h * 2, k_pitch, 0, K_BASE);
+                gather(k_b + (int64_t)(h + 1) * ks.h * 2, k_pitch, rr0, rows0, K_BASE);
+                gather(v_b + (int64_t)(h + 1) * vs.h * 2, v_pitch, rr0, rows0, V_BASE);
                 if (h + 2 < H) fetch_q(h + 2);
-            }
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (s * 32 < rows_here) {
-#pragma unroll
-                    for (int cb = 0; cb < 2; ++cb) {
-                        const U32x2 lo = __builtin_bit_cast(U32x2, bt[s][cb][0]);
-                        const U32x2 hi = __builtin_bit_cast(U32x2, bt[s][cb][1]);
-                        acc[cb] = tile_mfma<T>(a[s], Piece{lo[0], lo[1], hi[0], hi[1]}, acc[cb]);
-                    }
-                }
             }
         }
 
-        // ---- blank token, output chunk (8 tokens x 32 channels, row-major over the probability area) ---------------
-        __syncthreads();
+        // ---- blank token, output chunk (8 tokens x 32 channels, row-major) -----------------------------------------------
         if (kq < 2) {
             const F32x4 pb = *reinterpret_cast<const F32x4*>(stage + PB_BASE + 16 * kq);
 #pragma unroll
             for (int cb = 0; cb < 2; ++cb) {
-                const float bv = blank_v[h * kC + 16 * cb + r16];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    reinterpret_cast<T*>(stage + P_BASE)[(4 * kq + e) * kC + 16 * cb + r16] =
-                        from_acc<T>(acc[cb][e] + pb[e] * bv);
+                    reinterpret_cast<T*>(stage + O_BASE)[(4 * kq + e) * kC + 16 * cb + r16] =
+                        from_acc<T>(acc[cb][e] + pb[e] * bv[cb]);
                 }
             }
         }
-        __syncthreads();
+        lds_sync();
+        // the head's only store, and the last vector-memory operation it issues (see the wait at the top of the loop)
         if (lane < 32 && g_sub < nt) {
-            const Piece o = *reinterpret_cast<const Piece*>(stage + P_BASE + lane * 16);
+            const Piece o = *reinterpret_cast<const Piece*>(stage + O_BASE + lane * 16);
             char* dst = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)(i0 + g_sub) * os.n);
             store_streaming(reinterpret_cast<Piece*>(dst + g_pos * 16), o);
         }
