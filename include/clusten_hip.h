@@ -220,6 +220,18 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* Layer normalisation over the last axis of an fp32 tensor, written as fp32, fp16 or bf16:
+ *   out[r,c] = (x[r,c] - mean_r) * rsqrt(var_r + eps) * weight[c] + bias[c]      (biased variance)
+ * what `nn.LayerNorm` computes in the reference model before every attention and MLP block
+ * (models/aff_transformer.py:226-240 and the norms at :351, :441, :569-571), with the rounding to 16 bits that
+ * mixed precision applies to the following Linear layer's input done in the same pass when out_dtype asks
+ * for it.  x (rows,C), weight, bias (C): fp32, contiguous, 16-byte aligned (else CLUSTEN_ERR_UNALIGNED);
+ * C in {64,128,256,384,512,768,1024} (else CLUSTEN_ERR_BAD_DIMS); out_dtype F32, F16 or BF16.
+ * Inference only (no statistics are kept for a backward pass).  No counterpart in the reference's extension
+ * modules. */
+int clusten_layer_norm_forward(const float* x, const float* weight, const float* bias, void* out,
+                               int64_t rows, int C, float eps, int out_dtype, clusten_stream stream);
+
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 
 /* K nearest neighbours of 2-D points inside each batch element: for query point q of batch element b,

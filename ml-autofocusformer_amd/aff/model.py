@@ -36,7 +36,20 @@ def default_ops():
                            qk_clusters=_native.qk_forward_clusters, av_clusters=_native.av_forward_clusters,
                            clusters_supported=_native.clusters_supported,
                            cluster_attention=_native.cluster_attention,
-                           cluster_attention_supported=_native.cluster_attention_supported)
+                           cluster_attention_supported=_native.cluster_attention_supported,
+                           layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported)
+
+
+def _layer_norm(norm, x, ops, feeds_linear=False):
+    """`norm(x)` for an nn.LayerNorm; in inference on the GPU through the library's one-pass kernel when `ops` has it.
+
+    `feeds_linear`: the result is only read by Linear layers, so under mixed precision it is produced in the
+    autocast dtype directly (the rounding those layers would apply to their input, done once)."""
+    fn = getattr(ops, "layer_norm", None)
+    if fn is None or torch.is_grad_enabled() or not ops.layer_norm_supported(x):
+        return norm(x)
+    out_dtype = torch.get_autocast_dtype("cuda") if (feeds_linear and torch.is_autocast_enabled("cuda")) else None
+    return fn(x, norm.weight, norm.bias, norm.eps, out_dtype)
 
 
 def relative_position_table(img_size):
@@ -166,9 +179,11 @@ class ClusterTransformerBlock(nn.Module):
             self.gamma2 = nn.Parameter(layer_scale * torch.ones(dim))
 
     def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None):
-        a = self.attn(self.norm1(feat), member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx)
+        ops = self.attn.ops
+        a = self.attn(_layer_norm(self.norm1, feat, ops, True), member_idx, cluster_mask, pe_idx, global_attn, table,
+                      cluster_idx)
         feat = feat + self.drop_path(self.gamma1 * a if self.layer_scale else a)
-        f = self.mlp(self.norm2(feat))
+        f = self.mlp(_layer_norm(self.norm2, feat, ops, True))
         return feat + self.drop_path(self.gamma2 * f if self.layer_scale else f)
 
 
@@ -223,7 +238,7 @@ class ClusterMerging(nn.Module):
         if cluster_mask is not None:
             weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
         merged = self.ops.wf(weights, feat, member_idx).reshape(b, n_out, -1)            # channel = ic * c + c'
-        return pos, self.linear(self.norm(merged))
+        return pos, self.linear(_layer_norm(self.norm, merged, self.ops, True))
 
 
 class BasicLayer(nn.Module):

@@ -53,6 +53,8 @@ _PROTOTYPES = {
                                                    _P]),
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, _P,
                                                         _P, Strides, ctypes.c_float, AttnShape, ctypes.c_int, _P]),
+    "clusten_layer_norm_forward": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
+                                                 ctypes.c_int, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
@@ -480,6 +482,43 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
                                                      _stream(device)),
                "clusten_cluster_attention_forward")
     return out.reshape(b, n, h * c)
+
+
+_LAYER_NORM_WIDTHS = (64, 128, 256, 384, 512, 768, 1024)
+_DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def layer_norm_supported(x: torch.Tensor, out_dtype=None) -> bool:
+    """True when `layer_norm` takes this case: a CUDA fp32 tensor whose last axis has one of the built widths."""
+    return (x.is_cuda and x.dtype == torch.float32 and x.dim() >= 1 and x.shape[-1] in _LAYER_NORM_WIDTHS
+            and (out_dtype is None or out_dtype in _DTYPE_CODES))
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5, out_dtype=None):
+    """F.layer_norm(x, (C,), weight, bias, eps) for fp32 x, returned as `out_dtype` (fp32 unless given): the
+    normalisation in fp32 and the rounding a following mixed-precision Linear applies, in one pass.  No autograd."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    _require_cuda("weight", weight, device)
+    _require_cuda("bias", bias, device)
+    out_dtype = torch.float32 if out_dtype is None else out_dtype
+    if x.dtype != torch.float32 or out_dtype not in _DTYPE_CODES:
+        raise RuntimeError("layer_norm takes fp32 input and writes fp32, fp16 or bf16")
+    c = x.shape[-1]
+    if weight.numel() != c or bias.numel() != c:
+        raise RuntimeError("weight and bias must have as many elements as the last axis of x")
+    x = x.detach().contiguous()
+    weight = weight.detach().float().contiguous()
+    bias = bias.detach().float().contiguous()
+    out = torch.empty(x.shape, dtype=out_dtype, device=device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(device):
+        _check(lib.clusten_layer_norm_forward(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), x.numel() // c, c,
+                                              ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
+               "clusten_layer_norm_forward")
+    return out
 
 
 def knn2d_supported(query: torch.Tensor, database: torch.Tensor, k: int) -> bool:

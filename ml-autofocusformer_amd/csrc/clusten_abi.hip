@@ -187,6 +187,15 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     as_stream(stream));
 }
 
+int clusten_layer_norm_forward(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C,
+                               float eps, int out_dtype, clusten_stream stream) {
+    if (!x || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;
+    if (out_dtype != CLUSTEN_F32 && out_dtype != CLUSTEN_F16 && out_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || C <= 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(bias) || !aligned16(out)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_layer_norm(x, weight, bias, out, rows, C, eps, out_dtype, as_stream(stream));
+}
+
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
                   clusten_stream stream) {
     if (!query || !database || !idx) return CLUSTEN_ERR_NULL_POINTER;

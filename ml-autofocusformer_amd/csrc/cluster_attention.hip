@@ -93,22 +93,6 @@ __device__ __forceinline__ uint32_t lane_offset(uint32_t off) {
     return off;
 }
 
-// Orders the LDS traffic of the wave (a workgroup is one wave): everything issued so far has completed, and the
-// compiler moves no memory access across.  Unlike __syncthreads() it leaves vector-memory operations in flight.
-__device__ __forceinline__ void lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-}
-// The same, and at most `VM` vector-memory operations (LDS-direct loads, loads, stores; they complete in order)
-// are still in flight.
-template <int VM>
-__device__ __forceinline__ void lds_sync_vm() {
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(VM) & 0xF0FF);  // vmcnt(VM) lgkmcnt(0)
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-}
-
 template <typename T>
 __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const T* __restrict__ q, clusten_strides qs, const T* __restrict__ k, clusten_strides ks, const T* __restrict__ v,

@@ -56,7 +56,8 @@ namespace clusten {
 // Geometry of the staging buffer in LDS: rows of RB bytes, filled 1 KiB (one wave access) at a time.
 //   [0, G_BYTES)            gathered rows of one head (16*Q rows); reused to turn the D blocks into
 //                           the row-major output chunk once the operands are in registers
-//   [A_BASE, +2*A_SLOT)     a-rows of two heads (slot h % 2)
+//   [A_BASE, +2*OA_BYTES)   a-rows of two heads (slot h % 2); on the shared-list path of the FAST kernels a slot then
+//                           takes the head's output chunk, so that the row area is free for the next head's rows
 //   union path only (FAST kernels):
 //   [0, G_BYTES)            rows of 2*Q distinct runs per pass; reused for the score matrix of the pass
 //   [ULIST_BASE, +512)      row indices of up to U_MAX distinct runs, 8 per run
@@ -80,7 +81,9 @@ struct Staging {
     static constexpr int G_BYTES = G_PLAIN > G_NEED ? G_PLAIN : (G_NEED + 1023) / 1024 * 1024;
     static constexpr int A_BASE = G_BYTES;
     static constexpr int A_SLOT_BYTES = NI_A * 1024;
-    static constexpr int ULIST_BASE = A_BASE + 2 * A_SLOT_BYTES;
+    static constexpr int OUT_PIECES = (OUT_BYTES + 15) / 16 * 16;
+    static constexpr int OA_BYTES = A_SLOT_BYTES > OUT_PIECES ? A_SLOT_BYTES : OUT_PIECES;  // a-rows, then output chunk
+    static constexpr int ULIST_BASE = A_BASE + 2 * OA_BYTES;
     static constexpr int USLOT_BASE = ULIST_BASE + (UNION ? U_MAX * 8 * 4 : 0);
     static constexpr int BYTES = USLOT_BASE + (UNION ? kWave * 4 : 0);
     static constexpr int EL = C / 4;                            // channels per lane (a quarter row)
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
         const char* a_bh = a_tile + (int64_t)h * as.h * sizeof(T);
 #pragma unroll
         for (int i = 0; i < S::NI_A; ++i) {
-            CLUSTEN_LDS_DMA16(a_bh + a_off[i], stage + S::A_BASE + (h & 1) * S::A_SLOT_BYTES + i * 1024);
+            CLUSTEN_LDS_DMA16(a_bh + a_off[i], stage + S::A_BASE + (h & 1) * S::OA_BYTES + i * 1024);
         }
     };
     fetch_a(0);
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                                 }
                             }
                             a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] +
-                                                                                     (h & 1) * S::A_SLOT_BYTES);
+                                                                                     (h & 1) * S::OA_BYTES);
                         }
                         __syncthreads();  // operands are in registers: the rows make room for the scores
 
@@ -349,6 +352,86 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
         }
 
         if (FAST) __syncthreads();  // the list block has been read: the staging buffer is free for the gathers
+
+        if constexpr (FAST) {
+            if (shared_list) {
+                // ---- shared list: one gather and one set of MFMAs per head serve the 8 tokens; heads pipelined ----
+                // The rows of head h+1 are requested as soon as the operands of head h are in registers; the output
+                // chunk of head h is laid out in the slot its a-rows came from, so the row area stays free, and the
+                // wait for the rows of head h+1 leaves the stores of head h in flight.
+                uint32_t g_off[S::NI_G];
+#pragma unroll
+                for (int i = 0; i < S::NI_G; ++i) {
+                    const int srow = i * S::RPI + g_sub;
+                    g_off[i] = (uint32_t)__shfl(list0, min(srow, mc - 1)) * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16);
+                }
+                auto gather = [&](int h) {
+                    const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+#pragma unroll
+                    for (int i = 0; i < S::NI_G; ++i) CLUSTEN_LDS_DMA16(rows_bh + g_off[i], stage + i * 1024);
+                };
+                constexpr int NO = (S::OUT_BYTES + 1023) / 1024;  // store instructions per head
+                const int chunk_bytes = nt * M * (int)sizeof(T);
+                const bool all_stores = (NO - 1) * 1024 < chunk_bytes;  // each of them has an active lane
+                gather(0);
+                for (int h = 0; h < H; ++h) {
+                    if (h == 0 || !all_stores) {
+                        lds_sync_vm<0>();
+                    } else {
+                        lds_sync_vm<NO>();  // everything but the stores of the previous head
+                    }
+                    typename RunIO::raw g_raw[Q][S::NU];
+                    typename RunIO::raw a_raw[S::NU];
+#pragma unroll
+                    for (int u = 0; u < S::NU; ++u) {
+#pragma unroll
+                        for (int blk = 0; blk < Q; ++blk) {
+                            g_raw[blk][u] =
+                                *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] + blk * 16 * S::RB);
+                        }
+                        a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] + (h & 1) * S::OA_BYTES);
+                    }
+                    lds_sync();  // operands are in registers: the row area and this head's a-row slot are free
+                    if (h + 1 < H) {
+                        gather(h + 1);
+                        if (h + 1 >= 2) fetch_a(h + 1);
+                    }
+                    F32x4 d[Q];
+#pragma unroll
+                    for (int blk = 0; blk < Q; ++blk) {
+                        d[blk] = F32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int u = 0; u < S::NU; ++u) d[blk] = tile_mfma<T>(g_raw[blk][u], a_raw[u], d[blk]);
+                    }
+                    // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of token r: the (tile, head) output is one contiguous
+                    // chunk of nt*M elements; it is laid out row-major in LDS and leaves with full-width 16-byte stores
+                    char* chunk = stage + S::A_BASE + (h & 1) * S::OA_BYTES;
+                    if (r < nt) {
+#pragma unroll
+                        for (int blk = 0; blk < Q; ++blk) {
+                            const int s0 = 16 * blk + 4 * kq;
+                            float v[4] = {d[blk][0], d[blk][1], d[blk][2], d[blk][3]};
+                            if (s0 < mc) {
+                                *reinterpret_cast<typename OutIO::raw*>(chunk + (r * M + s0) * (int)sizeof(T)) = OutIO::pack(v);
+                            }
+                        }
+                    }
+                    lds_sync();
+                    Piece o[NO];
+#pragma unroll
+                    for (int i = 0; i < NO; ++i) {
+                        o[i] = *reinterpret_cast<const Piece*>(chunk + min(i * 1024 + lane * 16, S::OA_BYTES - 16));
+                    }
+                    char* out_h = out_tile + (int64_t)h * N * M * sizeof(T);
+#pragma unroll
+                    for (int i = 0; i < NO; ++i) {
+                        const int off = i * 1024 + lane * 16;
+                        if (off < chunk_bytes) store_streaming(reinterpret_cast<Piece*>(out_h + off), o[i]);
+                    }
+                }
+                return;
+            }
+        }
 
         // the list entry of staging row i*RPI + g_sub lives in the lane of that slot
         int src_lane[S::NI_G];
@@ -402,7 +485,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                             *reinterpret_cast<const typename RunIO::raw*>(stage + lds_g[u] + blk * 16 * S::RB);
                     }
                     a_raw[u] =
-                        *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] + (h & 1) * S::A_SLOT_BYTES);
+                        *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] + (h & 1) * S::OA_BYTES);
                 }
                 __syncthreads();  // operands are in registers: the staging buffer may be reused
 

@@ -64,6 +64,11 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
                              clusten_strides os, float scale, clusten_attn_shape s, int dtype, hipStream_t stream);
 
+// out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C fp32 channels
+//   (C in {64,128,256,384,512,768,1024}); out of dtype F32, F16 or BF16.
+int launch_layer_norm(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                      int out_dtype, hipStream_t stream);
+
 // idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
 //   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;
 //   idx int64; dist fp32 or null.

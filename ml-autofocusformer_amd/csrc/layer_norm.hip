@@ -1,0 +1,102 @@
+// layer_norm: y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias over the last axis of an fp32 tensor,
+// written as fp32, fp16 or bf16.
+//
+// The reference model normalises the token features before every attention and MLP block, before each merge
+// projection and at the end (`nn.LayerNorm`, models/aff_transformer.py:226-240, 351, 441, 569-571); under mixed
+// precision the normalisation runs in fp32 and the Linear layer that follows rounds its input to 16 bits.  This
+// kernel does both in one pass over the rows (64 to 512 channels: a row is a few hundred bytes, which the
+// framework's general kernel handles at a fraction of the memory bandwidth).  It has no counterpart in the
+// reference's extension modules.
+//
+// A row is held by L = min(64, C / 4) lanes, four consecutive channels per lane and step (C / (4 L) steps), so
+// that a wave reads 1 KiB contiguous per access; mean and variance are two reductions over registers (the
+// variance from the centred values, as a two-pass computation gives it), across the lanes of the row with xor
+// shuffles.  All arithmetic is fp32.
+#include "launch.hpp"
+
+namespace clusten {
+namespace {
+
+template <int L>
+__device__ __forceinline__ float row_sum(float v) {
+#pragma unroll
+    for (int m = 1; m < L; m <<= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+template <typename OutT, int L, int V>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                         const float* __restrict__ bias, OutT* __restrict__ out,
+                                                         int64_t rows, float eps) {
+    constexpr int C = 4 * L * V;
+    constexpr int ROWS_PER_WG = 256 / L;
+    const int sub = threadIdx.x % L;
+    const int64_t row_raw = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / L;
+    const bool live = row_raw < rows;
+    const int64_t row = live ? row_raw : rows - 1;  // every lane stays in the shuffles
+    const float* xr = x + row * C;
+    float4 v[V];
+#pragma unroll
+    for (int s = 0; s < V; ++s) v[s] = *reinterpret_cast<const float4*>(xr + 4 * (s * L + sub));
+    float sum = 0.f;
+#pragma unroll
+    for (int s = 0; s < V; ++s) sum += (v[s].x + v[s].y) + (v[s].z + v[s].w);
+    const float mean = row_sum<L>(sum) * (1.f / C);
+    float sq = 0.f;
+#pragma unroll
+    for (int s = 0; s < V; ++s) {
+        v[s].x -= mean, v[s].y -= mean, v[s].z -= mean, v[s].w -= mean;
+        sq += (v[s].x * v[s].x + v[s].y * v[s].y) + (v[s].z * v[s].z + v[s].w * v[s].w);
+    }
+    const float rstd = rsqrtf(row_sum<L>(sq) * (1.f / C) + eps);
+    if (!live) return;
+    OutT* orow = out + row * C;
+#pragma unroll
+    for (int s = 0; s < V; ++s) {
+        const int c = 4 * (s * L + sub);
+        const float4 w = *reinterpret_cast<const float4*>(weight + c);
+        const float4 b = *reinterpret_cast<const float4*>(bias + c);
+        float y[4] = {v[s].x * rstd * w.x + b.x, v[s].y * rstd * w.y + b.y, v[s].z * rstd * w.z + b.z,
+                      v[s].w * rstd * w.w + b.w};
+        *reinterpret_cast<typename Quad<OutT>::raw*>(orow + c) = Quad<OutT>::pack(y);
+    }
+}
+
+template <typename OutT, int L, int V>
+int launch_lv(const float* x, const float* weight, const float* bias, void* out, int64_t rows, float eps,
+              hipStream_t stream) {
+    constexpr int ROWS_PER_WG = 256 / L;
+    const int64_t blocks = (rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
+    hipLaunchKernelGGL((layer_norm_kernel<OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream, x, weight, bias,
+                       static_cast<OutT*>(out), rows, eps);
+    return launch_status();
+}
+
+template <typename OutT>
+int launch_typed(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                 hipStream_t stream) {
+    switch (C) {
+        case 64: return launch_lv<OutT, 16, 1>(x, weight, bias, out, rows, eps, stream);
+        case 128: return launch_lv<OutT, 32, 1>(x, weight, bias, out, rows, eps, stream);
+        case 256: return launch_lv<OutT, 64, 1>(x, weight, bias, out, rows, eps, stream);
+        case 384: return launch_lv<OutT, 32, 3>(x, weight, bias, out, rows, eps, stream);
+        case 512: return launch_lv<OutT, 64, 2>(x, weight, bias, out, rows, eps, stream);
+        case 768: return launch_lv<OutT, 64, 3>(x, weight, bias, out, rows, eps, stream);
+        case 1024: return launch_lv<OutT, 64, 4>(x, weight, bias, out, rows, eps, stream);
+        default: return CLUSTEN_ERR_BAD_DIMS;
+    }
+}
+
+}  // namespace
+
+int launch_layer_norm(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                      int out_dtype, hipStream_t stream) {
+    switch (out_dtype) {
+        case CLUSTEN_F32: return launch_typed<float>(x, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(x, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(x, weight, bias, out, rows, C, eps, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
+}  // namespace clusten

@@ -13,6 +13,23 @@ typedef float F32x4 __attribute__((ext_vector_type(4)));
 // outstanding and leaves the LDS/scalar and export counters alone.
 constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (15 << 8); }
 
+// Orders the LDS traffic of a one-wave workgroup: every LDS access issued so far has completed, and the compiler
+// moves no memory access across.  Unlike __syncthreads(), whose fence also waits for every vector-memory
+// operation, it leaves LDS-direct loads, loads and stores in flight.
+__device__ __forceinline__ void lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+}
+// The same, and at most `VM` vector-memory operations are still in flight.  They complete in the order of issue,
+// so this waits for everything but the last `VM` of them (e.g. output stores issued after a prefetch).
+template <int VM>
+__device__ __forceinline__ void lds_sync_vm() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(VM) & 0xF0FF);  // vmcnt(VM) lgkmcnt(0)
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+}
+
 // One LDS-direct load: every lane moves 16 bytes from its own global address `gptr` to LDS address
 // `lptr` + 16 * lane (`lptr` is wave-uniform).  Completion is tracked by the vector-memory counter.
 #define CLUSTEN_LDS_DMA16(gptr, lptr)                                                       \

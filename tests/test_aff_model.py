@@ -22,6 +22,9 @@ def oracle_ops():
         wf=lambda w, f, idx: oracle.wf_gather(w, f.to(w.dtype), idx))
 
 
+TOL_16 = 1e-2
+
+
 def small_model(ops, **kw):
     cfg = dict(embed_dim=(32, 64, 128, 256), depths=(1, 2, 1, 1), num_heads=(2, 4, 8, 16), mlp_ratio=2.0,
                num_classes=10, img_size=128, drop_path_rate=0.0, ops=ops)
@@ -230,6 +233,33 @@ def test_fused_bias_mask_blank_softmax_equals_the_tensor_expressions(device, dty
     assert not _native.attn_softmax_supported(attn, 72) and not _native.attn_softmax_supported(attn, 50)
     with pytest.raises(RuntimeError):
         _native.attn_softmax(attn.cpu(), table, pe_idx, mask, blank)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_layer_norm_kernel_equals_torch(device, out_dtype):
+    """fp32 statistics and affine transform, one rounding to the output type: F.layer_norm in fp32, then .to()."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(17)
+    for rows, c in (((5, 37), 64), ((3, 200), 128), ((2, 49), 256), ((1, 7), 384), ((4, 13), 512), ((2, 3), 768),
+                    ((3, 5), 1024), ((1,), 64)):
+        x = (torch.randn(*rows, c, generator=gen) * 3 + 1.5).to(device)
+        w = torch.randn(c, generator=gen).to(device)
+        b = torch.randn(c, generator=gen).to(device)
+        ref = torch.nn.functional.layer_norm(x, (c,), w, b, 1e-5)
+        out = _native.layer_norm(x, w, b, 1e-5, out_dtype)
+        assert out.dtype == out_dtype and out.shape == x.shape
+        if out_dtype == torch.float32:
+            assert oracle.rel_err(out, ref) <= 1e-5
+        else:
+            # the fp32 result rounded once: at most one unit in the last place of the 16-bit type from torch's
+            assert oracle.rel_err(out.float(), ref.to(out_dtype).float()) <= (2e-3 if out_dtype == torch.float16 else 1.6e-2)
+            assert oracle.rel_err(out.float(), ref) <= TOL_16
+    assert not _native.layer_norm_supported(x[..., :40].contiguous())
+    assert not _native.layer_norm_supported(x.half())
+    assert not _native.layer_norm_supported(x.cpu())
+    with pytest.raises(RuntimeError):
+        _native.layer_norm(x[..., :40].contiguous(), w[:40], b[:40])
 
 
 @pytest.mark.gpu
