@@ -220,17 +220,30 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
-/* Layer normalisation over the last axis of an fp32 tensor, written as fp32, fp16 or bf16:
+/* Layer normalisation over the last axis, computed in fp32 from fp32, fp16 or bf16 input and written as fp32,
+ * fp16 or bf16:
  *   out[r,c] = (x[r,c] - mean_r) * rsqrt(var_r + eps) * weight[c] + bias[c]      (biased variance)
  * what `nn.LayerNorm` computes in the reference model before every attention and MLP block
  * (models/aff_transformer.py:226-240 and the norms at :351, :441, :569-571), with the rounding to 16 bits that
- * mixed precision applies to the following Linear layer's input done in the same pass when out_dtype asks
- * for it.  x (rows,C), weight, bias (C): fp32, contiguous, 16-byte aligned (else CLUSTEN_ERR_UNALIGNED);
- * C in {64,128,256,384,512,768,1024} (else CLUSTEN_ERR_BAD_DIMS); out_dtype F32, F16 or BF16.
+ * mixed precision applies to the following Linear layer's input (and the widening it applies to a 16-bit
+ * input of the normalisation) done in the same pass.  x (rows,C) of in_dtype, out (rows,C) of out_dtype (F32,
+ * F16 or BF16 each); weight, bias (C) fp32; all contiguous and 16-byte aligned (else CLUSTEN_ERR_UNALIGNED);
+ * C in {64,128,256,384,512,768,1024} (else CLUSTEN_ERR_BAD_DIMS).
  * Inference only (no statistics are kept for a backward pass).  No counterpart in the reference's extension
  * modules. */
-int clusten_layer_norm_forward(const float* x, const float* weight, const float* bias, void* out,
+int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream);
+
+/* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
+ * (models/aff_transformer.py:363-372), in one pass instead of a row lookup, a gather and two multiplications:
+ *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]
+ * table_weights (rows,IC), prob (B,N) or NULL, weights (B,Nout,M,IC): fp32, contiguous; pe_idx (values in
+ * [0,rows) — unchecked), nbhd_idx (values in [0,N) — unchecked; may be NULL when prob is), mask (0/1, or NULL):
+ * int64 (B,Nout,M).  IC = 4 (else CLUSTEN_ERR_BAD_DIMS); table_weights and weights 16-byte aligned (else
+ * CLUSTEN_ERR_UNALIGNED).  Inference only.  No counterpart in the reference's extension modules. */
+int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
+                                  const float* prob, const int64_t* mask, float* weights,
+                                  int B, int N, int Nout, int M, int IC, clusten_stream stream);
 
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 

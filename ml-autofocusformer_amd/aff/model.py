@@ -24,6 +24,7 @@ from types import SimpleNamespace
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from .points import knn, space_filling_cluster
 
@@ -37,7 +38,23 @@ def default_ops():
                            clusters_supported=_native.clusters_supported,
                            cluster_attention=_native.cluster_attention,
                            cluster_attention_supported=_native.cluster_attention_supported,
-                           layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported)
+                           layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
+                           merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported)
+
+
+def _linear(lin, x):
+    """`lin(x)` for an nn.Linear.  In inference under mixed precision the 16-bit copies of weight and bias are kept
+    between calls (autocast makes them anew in every forward); they are remade when the parameters change."""
+    if torch.is_grad_enabled() or not x.is_cuda or not torch.is_autocast_enabled("cuda"):
+        return lin(x)
+    dt = torch.get_autocast_dtype("cuda")
+    key = (dt, lin.weight._version, lin.weight.data_ptr(),
+           None if lin.bias is None else (lin.bias._version, lin.bias.data_ptr()))
+    cache = lin.__dict__.get("_cast_cache")
+    if cache is None or cache[0] != key:
+        cache = (key, lin.weight.detach().to(dt), None if lin.bias is None else lin.bias.detach().to(dt))
+        lin.__dict__["_cast_cache"] = cache      # a plain attribute: no parameter, no buffer, not in the state_dict
+    return F.linear(x if x.dtype == dt else x.to(dt), cache[1], cache[2])
 
 
 def _layer_norm(norm, x, ops, feeds_linear=False):
@@ -91,7 +108,7 @@ class Mlp(nn.Module):
         self.drop = nn.Dropout(drop)
 
     def forward(self, x):
-        return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
+        return self.drop(_linear(self.fc2, self.drop(self.act(_linear(self.fc1, x)))))
 
 
 class ClusterAttention(nn.Module):
@@ -118,17 +135,17 @@ class ClusterAttention(nn.Module):
         # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
         compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
                    and getattr(self.ops, "qk_clusters", None) is not None)
-        q = self.q(feat)
-        kv = self.kv(feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
+        q = _linear(self.q, feat)
+        kv = _linear(self.kv, feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
         one_kernel = getattr(self.ops, "cluster_attention", None)
         if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
                 and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2])):
             # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
             # the values in one kernel; the query scale is applied to the scores inside it
-            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, cluster_idx, self.pos_embed(table),
+            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, cluster_idx, _linear(self.pos_embed, table),
                              pe_idx, cluster_mask, self.blank_k, self.blank_v, scale=self.scale)
-            return self.proj_drop(self.proj(out))
+            return self.proj_drop(_linear(self.proj, out))
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:
             attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
@@ -138,7 +155,7 @@ class ClusterAttention(nn.Module):
             compact = False
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
 
-        bias = self.pos_embed(table)                                                     # (rows, h)
+        bias = _linear(self.pos_embed, table)                                                     # (rows, h)
         fused = getattr(self.ops, "attn_softmax", None)
         if (fused is not None and not global_attn and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0) and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
@@ -161,7 +178,7 @@ class ClusterAttention(nn.Module):
             out = self.ops.av(attn, v, member_idx)                                       # (b,h,n,ch)
         out = out + blank * self.blank_v.reshape(1, h, 1, ch)
         out = out.permute(0, 2, 1, 3).reshape(b, n, c)
-        return self.proj_drop(self.proj(out))
+        return self.proj_drop(_linear(self.proj, out))
 
 
 class ClusterTransformerBlock(nn.Module):
@@ -232,13 +249,20 @@ class ClusterMerging(nn.Module):
         rows = centre.unsqueeze(2).expand(-1, -1, m)
         member_idx = member_idx.gather(1, rows)                                          # (b, n', m)
         pe_idx = pe_idx.gather(1, rows)
-        weights = self.weight_net(table)[pe_idx]                                         # (b, n', m, 4)
-        if learned_prob is not None:
-            weights = weights * learned_prob.gather(1, member_idx.reshape(b, -1, 1)).reshape(b, n_out, m, 1)
-        if cluster_mask is not None:
-            weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
+        table_w = self.weight_net(table)                                                 # (rows, 4)
+        one_pass = getattr(self.ops, "merge_weights", None)
+        if one_pass is not None and not torch.is_grad_enabled() and self.ops.merge_weights_supported(table_w):
+            # inference: lookup, importance of each neighbour and mask in one kernel
+            weights = one_pass(table_w, pe_idx, member_idx, learned_prob,
+                               None if cluster_mask is None else cluster_mask.gather(1, rows))
+        else:
+            weights = table_w[pe_idx]                                                    # (b, n', m, 4)
+            if learned_prob is not None:
+                weights = weights * learned_prob.gather(1, member_idx.reshape(b, -1, 1)).reshape(b, n_out, m, 1)
+            if cluster_mask is not None:
+                weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
         merged = self.ops.wf(weights, feat, member_idx).reshape(b, n_out, -1)            # channel = ic * c + c'
-        return pos, self.linear(_layer_norm(self.norm, merged, self.ops, True))
+        return pos, _linear(self.linear, _layer_norm(self.norm, merged, self.ops, True))
 
 
 class BasicLayer(nn.Module):
@@ -278,10 +302,18 @@ class BasicLayer(nn.Module):
         else:
             pos, centres, members, mask, ranking = space_filling_cluster(pos, m, h, w)
         nearest = knn(pos, centres, nnc)                                                  # (b, n, nnc)
-        pick = nearest.reshape(b, -1, 1).expand(-1, -1, m)
-        member_idx = members.gather(1, pick).reshape(b, n, nnc * m)
-        if mask is not None:
-            mask = mask.gather(1, pick).reshape(b, n, nnc * m)
+        if ranking is not None:
+            # cluster order: cluster g owns tokens g*m .. g*m+m-1, pad slots of the last one hold index 0 and mask 0
+            rows = nearest.unsqueeze(3) * m + torch.arange(m, device=pos.device)
+            valid = rows < n
+            member_idx = torch.where(valid, rows, torch.zeros_like(rows)).reshape(b, n, nnc * m)
+            if mask is not None:
+                mask = valid.reshape(b, n, nnc * m).to(mask.dtype)
+        else:
+            pick = nearest.reshape(b, -1, 1).expand(-1, -1, m)
+            member_idx = members.gather(1, pick).reshape(b, n, nnc * m)
+            if mask is not None:
+                mask = mask.gather(1, pick).reshape(b, n, nnc * m)
         nb_pos = pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, d)).reshape(b, n, nnc * m, d)
         rel = nb_pos - (pos.unsqueeze(2) - radius)
         pe_idx = (rel[..., 1] * table_width + rel[..., 0]).long()
@@ -326,7 +358,7 @@ class BasicLayer(nn.Module):
         if self.downsample is not None:
             if global_attn:   # merging after a dense stage: every token is every token's neighbour
                 member_idx = torch.arange(n, device=feat.device).expand(b, n, n).contiguous()
-            learned_prob = self.prob_net(feat).sigmoid()
+            learned_prob = _linear(self.prob_net, feat).sigmoid()
             reserve_num = math.ceil(h / (stride * 2)) * math.ceil(w / (stride * 2))
             pos, feat = self.downsample(pos, feat, member_idx, mask, learned_prob, stride, pe_idx, reserve_num, table)
         return pos, feat
@@ -335,8 +367,9 @@ class BasicLayer(nn.Module):
 class PatchEmbed(nn.Module):
     """Two stride-2 3x3 convolutions (BatchNorm + GELU between them): one token per 4x4 pixels."""
 
-    def __init__(self, in_chans=3, embed_dim=32, patch_norm=True):
+    def __init__(self, in_chans=3, embed_dim=32, patch_norm=True, ops=None):
         super().__init__()
+        self.ops = ops
         self.proj1 = nn.Conv2d(in_chans, embed_dim // 2, kernel_size=3, stride=2, padding=1)
         self.bn = nn.BatchNorm2d(embed_dim // 2)
         self.act1 = nn.GELU()
@@ -348,7 +381,7 @@ class PatchEmbed(nn.Module):
         b, c, h, w = x.shape
         x = x.flatten(2).transpose(1, 2)
         if self.norm is not None:
-            x = self.norm(x)
+            x = _layer_norm(self.norm, x, self.ops)
         ys, xs = torch.meshgrid(torch.arange(h, device=x.device), torch.arange(w, device=x.device), indexing="ij")
         pos = torch.stack([xs, ys], dim=2).reshape(1, -1, 2).expand(b, -1, -1).to(x.dtype)
         return pos, x, h, w
@@ -365,7 +398,8 @@ class AutoFocusFormer(nn.Module):
         ops = ops if ops is not None else default_ops()
         self.num_classes = num_classes
         self.num_features = embed_dim[-1]
-        self.patch_embed = PatchEmbed(in_chans, embed_dim[0], patch_norm)
+        self.ops = ops
+        self.patch_embed = PatchEmbed(in_chans, embed_dim[0], patch_norm, ops=ops)
         self.pos_drop = nn.Dropout(drop_rate)
         table, self.radius = relative_position_table(img_size)
         self.register_buffer("pre_table", table, persistent=False)
@@ -396,10 +430,10 @@ class AutoFocusFormer(nn.Module):
         for i, layer in enumerate(self.layers):
             pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=self.pre_table,
                            radius=self.radius)
-        return self.norm(x).mean(1)
+        return _layer_norm(self.norm, x, self.ops).mean(1)
 
     def forward(self, x):
-        return self.head(self.forward_features(x))
+        return _linear(self.head, self.forward_features(x)) if isinstance(self.head, nn.Linear) else self.forward_features(x)
 
 
 def aff_tiny(**kw):

@@ -53,8 +53,10 @@ _PROTOTYPES = {
                                                    _P]),
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, _P,
                                                         _P, Strides, ctypes.c_float, AttnShape, ctypes.c_int, _P]),
-    "clusten_layer_norm_forward": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
-                                                 ctypes.c_int, _P]),
+    "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
+                                                 ctypes.c_float, ctypes.c_int, _P]),
+    "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                    ctypes.c_int, ctypes.c_int, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
@@ -489,22 +491,24 @@ _DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
 def layer_norm_supported(x: torch.Tensor, out_dtype=None) -> bool:
-    """True when `layer_norm` takes this case: a CUDA fp32 tensor whose last axis has one of the built widths."""
-    return (x.is_cuda and x.dtype == torch.float32 and x.dim() >= 1 and x.shape[-1] in _LAYER_NORM_WIDTHS
+    """True when `layer_norm` takes this case: a CUDA fp32 / fp16 / bf16 tensor whose last axis has one of the built
+    widths."""
+    return (x.is_cuda and x.dtype in _DTYPE_CODES and x.dim() >= 1 and x.shape[-1] in _LAYER_NORM_WIDTHS
             and (out_dtype is None or out_dtype in _DTYPE_CODES))
 
 
 def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5, out_dtype=None):
-    """F.layer_norm(x, (C,), weight, bias, eps) for fp32 x, returned as `out_dtype` (fp32 unless given): the
-    normalisation in fp32 and the rounding a following mixed-precision Linear applies, in one pass.  No autograd."""
+    """F.layer_norm(x.float(), (C,), weight, bias, eps), returned as `out_dtype` (fp32 unless given): the widening
+    of a 16-bit input, the normalisation in fp32 and the rounding a following mixed-precision Linear applies, in
+    one pass.  No autograd."""
     lib = load()
     _require_cuda("x", x)
     device = x.device
     _require_cuda("weight", weight, device)
     _require_cuda("bias", bias, device)
     out_dtype = torch.float32 if out_dtype is None else out_dtype
-    if x.dtype != torch.float32 or out_dtype not in _DTYPE_CODES:
-        raise RuntimeError("layer_norm takes fp32 input and writes fp32, fp16 or bf16")
+    if x.dtype not in _DTYPE_CODES or out_dtype not in _DTYPE_CODES:
+        raise RuntimeError("layer_norm reads and writes fp32, fp16 or bf16")
     c = x.shape[-1]
     if weight.numel() != c or bias.numel() != c:
         raise RuntimeError("weight and bias must have as many elements as the last axis of x")
@@ -515,9 +519,49 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
     if out.numel() == 0:
         return out
     with torch.cuda.device(device):
-        _check(lib.clusten_layer_norm_forward(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), x.numel() // c, c,
+        _check(lib.clusten_layer_norm_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(weight), _ptr(bias), _ptr(out),
+                                              x.numel() // c, c,
                                               ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
                "clusten_layer_norm_forward")
+    return out
+
+
+def merge_weights_supported(table_weights: torch.Tensor) -> bool:
+    """True when `merge_weights` takes this case: a CUDA table of 4 weights per row."""
+    return table_weights.is_cuda and table_weights.dim() == 2 and table_weights.shape[1] == 4
+
+
+def merge_weights(table_weights: torch.Tensor, pe_idx: torch.Tensor, nbhd_idx: torch.Tensor, prob, mask):
+    """table_weights[pe_idx] * prob.gather(nbhd_idx) * mask as one (B,N',M,4) fp32 tensor: the weights the WF
+    operator takes (models/aff_transformer.py:363-372).  table_weights (rows,4); pe_idx, nbhd_idx (B,N',M) int64;
+    prob (B,N) or (B,N,1) or None; mask (B,N',M) of 0/1 or None.  No autograd: for inference."""
+    lib = load()
+    _require_cuda("table_weights", table_weights)
+    device = table_weights.device
+    _require_cuda("pe_idx", pe_idx, device)
+    _require_cuda("nbhd_idx", nbhd_idx, device)
+    if pe_idx.dim() != 3 or pe_idx.dtype != torch.int64 or nbhd_idx.shape != pe_idx.shape or nbhd_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx and nbhd_idx must be int64 of one shape (B,N',M)")
+    b, n_out, m = pe_idx.shape
+    table_weights = table_weights.detach().float().contiguous()
+    n = 1
+    if prob is not None:
+        _require_cuda("prob", prob, device)
+        prob = prob.detach().reshape(b, -1).float().contiguous()
+        n = prob.shape[1]
+    if mask is not None:
+        _require_cuda("mask", mask, device)
+        if mask.shape != pe_idx.shape:
+            raise RuntimeError("mask must have the shape of pe_idx")
+        mask = mask.to(torch.int64).contiguous()
+    out = torch.empty(b, n_out, m, table_weights.shape[1], dtype=torch.float32, device=device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(device):
+        _check(lib.clusten_merge_weights_forward(_ptr(table_weights), _ptr(pe_idx.contiguous()),
+                                                 _ptr(nbhd_idx.contiguous()), _ptr(prob), _ptr(mask), _ptr(out), b, n,
+                                                 n_out, m, table_weights.shape[1], _stream(device)),
+               "clusten_merge_weights_forward")
     return out
 
 

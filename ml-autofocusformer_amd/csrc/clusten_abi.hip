@@ -187,13 +187,25 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     as_stream(stream));
 }
 
-int clusten_layer_norm_forward(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C,
-                               float eps, int out_dtype, clusten_stream stream) {
+int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
+                               int64_t rows, int C, float eps, int out_dtype, clusten_stream stream) {
     if (!x || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;
     if (out_dtype != CLUSTEN_F32 && out_dtype != CLUSTEN_F16 && out_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (in_dtype != CLUSTEN_F32 && in_dtype != CLUSTEN_F16 && in_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (rows <= 0 || C <= 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
     if (!aligned16(x) || !aligned16(weight) || !aligned16(bias) || !aligned16(out)) return CLUSTEN_ERR_UNALIGNED;
-    return launch_layer_norm(x, weight, bias, out, rows, C, eps, out_dtype, as_stream(stream));
+    return launch_layer_norm(x, in_dtype, weight, bias, out, rows, C, eps, out_dtype, as_stream(stream));
+}
+
+int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
+                                  const float* prob, const int64_t* mask, float* weights, int B, int N, int Nout, int M,
+                                  int IC, clusten_stream stream) {
+    if (!table_weights || !pe_idx || !weights) return CLUSTEN_ERR_NULL_POINTER;
+    if (prob && !nbhd_idx) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || Nout <= 0 || M <= 0 || IC != 4) return CLUSTEN_ERR_BAD_DIMS;
+    if (((int64_t)B * Nout * M + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(table_weights) || !aligned16(weights)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_merge_weights(table_weights, pe_idx, nbhd_idx, prob, mask, weights, B, N, Nout, M, as_stream(stream));
 }
 
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,

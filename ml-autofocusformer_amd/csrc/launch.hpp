@@ -64,10 +64,15 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
                              clusten_strides os, float scale, clusten_attn_shape s, int dtype, hipStream_t stream);
 
-// out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C fp32 channels
-//   (C in {64,128,256,384,512,768,1024}); out of dtype F32, F16 or BF16.
-int launch_layer_norm(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
-                      int out_dtype, hipStream_t stream);
+// out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C channels
+//   (C in {64,128,256,384,512,768,1024}); x and out of dtype F32, F16 or BF16 each, arithmetic in fp32.
+int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,
+                      float eps, int out_dtype, hipStream_t stream);
+
+// w[b,i,j,:4] = table_w[pe_idx[b,i,j], :4] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]   (prob, mask may be null)
+//   table_w (rows,4), prob (B,N), w (B,Nout,M,4): fp32;  pe_idx, nbhd_idx, mask: int64 (B,Nout,M).
+int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,
+                         const int64_t* mask, float* out, int B, int N, int Nout, int M, hipStream_t stream);
 
 // idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
 //   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;

@@ -1,10 +1,10 @@
-// layer_norm: y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias over the last axis of an fp32 tensor,
-// written as fp32, fp16 or bf16.
+// layer_norm: y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias over the last axis of an fp32, fp16 or bf16
+// tensor, computed in fp32 and written as fp32, fp16 or bf16.
 //
 // The reference model normalises the token features before every attention and MLP block, before each merge
 // projection and at the end (`nn.LayerNorm`, models/aff_transformer.py:226-240, 351, 441, 569-571); under mixed
-// precision the normalisation runs in fp32 and the Linear layer that follows rounds its input to 16 bits.  This
-// kernel does both in one pass over the rows (64 to 512 channels: a row is a few hundred bytes, which the
+// precision the normalisation runs in fp32 (a 16-bit input is widened first) and the Linear layer that follows
+// rounds its input to 16 bits.  This kernel does all of that in one pass over the rows (64 to 512 channels: a row is a few hundred bytes, which the
 // framework's general kernel handles at a fraction of the memory bandwidth).  It has no counterpart in the
 // reference's extension modules.
 //
@@ -24,8 +24,8 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
-template <typename OutT, int L, int V>
-__global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+template <typename InT, typename OutT, int L, int V>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__ x, const float* __restrict__ weight,
                                                          const float* __restrict__ bias, OutT* __restrict__ out,
                                                          int64_t rows, float eps) {
     constexpr int C = 4 * L * V;
@@ -34,10 +34,14 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict
     const int64_t row_raw = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / L;
     const bool live = row_raw < rows;
     const int64_t row = live ? row_raw : rows - 1;  // every lane stays in the shuffles
-    const float* xr = x + row * C;
+    const InT* xr = x + row * C;
     float4 v[V];
 #pragma unroll
-    for (int s = 0; s < V; ++s) v[s] = *reinterpret_cast<const float4*>(xr + 4 * (s * L + sub));
+    for (int s = 0; s < V; ++s) {
+        float in[4];
+        Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(xr + 4 * (s * L + sub)), in);
+        v[s] = make_float4(in[0], in[1], in[2], in[3]);
+    }
     float sum = 0.f;
 #pragma unroll
     for (int s = 0; s < V; ++s) sum += (v[s].x + v[s].y) + (v[s].z + v[s].w);
@@ -62,39 +66,50 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict
     }
 }
 
-template <typename OutT, int L, int V>
-int launch_lv(const float* x, const float* weight, const float* bias, void* out, int64_t rows, float eps,
+template <typename InT, typename OutT, int L, int V>
+int launch_lv(const void* x, const float* weight, const float* bias, void* out, int64_t rows, float eps,
               hipStream_t stream) {
     constexpr int ROWS_PER_WG = 256 / L;
     const int64_t blocks = (rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
-    hipLaunchKernelGGL((layer_norm_kernel<OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream, x, weight, bias,
-                       static_cast<OutT*>(out), rows, eps);
+    hipLaunchKernelGGL((layer_norm_kernel<InT, OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const InT*>(x), weight, bias, static_cast<OutT*>(out), rows, eps);
     return launch_status();
 }
 
-template <typename OutT>
-int launch_typed(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+template <typename InT, typename OutT>
+int launch_typed(const void* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
                  hipStream_t stream) {
     switch (C) {
-        case 64: return launch_lv<OutT, 16, 1>(x, weight, bias, out, rows, eps, stream);
-        case 128: return launch_lv<OutT, 32, 1>(x, weight, bias, out, rows, eps, stream);
-        case 256: return launch_lv<OutT, 64, 1>(x, weight, bias, out, rows, eps, stream);
-        case 384: return launch_lv<OutT, 32, 3>(x, weight, bias, out, rows, eps, stream);
-        case 512: return launch_lv<OutT, 64, 2>(x, weight, bias, out, rows, eps, stream);
-        case 768: return launch_lv<OutT, 64, 3>(x, weight, bias, out, rows, eps, stream);
-        case 1024: return launch_lv<OutT, 64, 4>(x, weight, bias, out, rows, eps, stream);
+        case 64: return launch_lv<InT, OutT, 16, 1>(x, weight, bias, out, rows, eps, stream);
+        case 128: return launch_lv<InT, OutT, 32, 1>(x, weight, bias, out, rows, eps, stream);
+        case 256: return launch_lv<InT, OutT, 64, 1>(x, weight, bias, out, rows, eps, stream);
+        case 384: return launch_lv<InT, OutT, 32, 3>(x, weight, bias, out, rows, eps, stream);
+        case 512: return launch_lv<InT, OutT, 64, 2>(x, weight, bias, out, rows, eps, stream);
+        case 768: return launch_lv<InT, OutT, 64, 3>(x, weight, bias, out, rows, eps, stream);
+        case 1024: return launch_lv<InT, OutT, 64, 4>(x, weight, bias, out, rows, eps, stream);
         default: return CLUSTEN_ERR_BAD_DIMS;
+    }
+}
+
+template <typename InT>
+int launch_in(const void* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+              int out_dtype, hipStream_t stream) {
+    switch (out_dtype) {
+        case CLUSTEN_F32: return launch_typed<InT, float>(x, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_F16: return launch_typed<InT, f16_t>(x, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_BF16: return launch_typed<InT, bf16_t>(x, weight, bias, out, rows, C, eps, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }
 
 }  // namespace
 
-int launch_layer_norm(const float* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
-                      int out_dtype, hipStream_t stream) {
-    switch (out_dtype) {
-        case CLUSTEN_F32: return launch_typed<float>(x, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_F16: return launch_typed<f16_t>(x, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_BF16: return launch_typed<bf16_t>(x, weight, bias, out, rows, C, eps, stream);
+int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,
+                      float eps, int out_dtype, hipStream_t stream) {
+    switch (in_dtype) {
+        case CLUSTEN_F32: return launch_in<float>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
+        case CLUSTEN_F16: return launch_in<f16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
+        case CLUSTEN_BF16: return launch_in<bf16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }

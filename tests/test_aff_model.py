@@ -255,11 +255,42 @@ def test_layer_norm_kernel_equals_torch(device, out_dtype):
             # the fp32 result rounded once: at most one unit in the last place of the 16-bit type from torch's
             assert oracle.rel_err(out.float(), ref.to(out_dtype).float()) <= (2e-3 if out_dtype == torch.float16 else 1.6e-2)
             assert oracle.rel_err(out.float(), ref) <= TOL_16
+        # 16-bit input: widened, as mixed precision does before a normalisation
+        for in_dtype in (torch.float16, torch.bfloat16):
+            xin = x.to(in_dtype)
+            ref16 = torch.nn.functional.layer_norm(xin.float(), (c,), w, b, 1e-5)
+            out16 = _native.layer_norm(xin, w, b, 1e-5, out_dtype)
+            assert out16.dtype == out_dtype
+            assert oracle.rel_err(out16.float(), ref16) <= (1e-5 if out_dtype == torch.float32 else TOL_16)
     assert not _native.layer_norm_supported(x[..., :40].contiguous())
-    assert not _native.layer_norm_supported(x.half())
+    assert not _native.layer_norm_supported(x.double())
     assert not _native.layer_norm_supported(x.cpu())
     with pytest.raises(RuntimeError):
         _native.layer_norm(x[..., :40].contiguous(), w[:40], b[:40])
+
+
+@pytest.mark.gpu
+def test_merge_weights_kernel_equals_the_tensor_expressions(device):
+    from clusten import _native
+    gen = torch.Generator().manual_seed(19)
+    b, n, n_out, m, rows = 3, 200, 50, 48, 321
+    table_w = torch.randn(rows, 4, generator=gen).to(device)
+    pe_idx = torch.randint(rows, (b, n_out, m), generator=gen).to(device)
+    nbhd = torch.randint(n, (b, n_out, m), generator=gen).to(device)
+    prob = torch.rand(b, n, 1, generator=gen).to(device)
+    mask = (torch.rand(b, n_out, m, generator=gen) > 0.2).long().to(device)
+    for p, mk in ((prob, mask), (prob, None), (None, mask), (None, None), (prob.half(), mask)):
+        ref = table_w[pe_idx]
+        if p is not None:
+            ref = ref * p.gather(1, nbhd.reshape(b, -1, 1)).reshape(b, n_out, m, 1)
+        if mk is not None:
+            ref = ref * mk.unsqueeze(3)
+        out = _native.merge_weights(table_w, pe_idx, nbhd, p, mk)
+        assert out.dtype == torch.float32 and out.shape == (b, n_out, m, 4)
+        assert torch.equal(out, ref.float())        # one fp32 product per factor, in the same order
+    assert not _native.merge_weights_supported(table_w[:, :3])
+    with pytest.raises(RuntimeError):
+        _native.merge_weights(table_w, pe_idx.int(), nbhd, prob, mask)
 
 
 @pytest.mark.gpu
