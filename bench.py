@@ -192,7 +192,7 @@ def _bench_wf(case, steps, warmup):
 
 
 def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
-    """Images/s of the AFF-Tiny classifier at 224x224 (random weights, N(0,1) images, fp16 autocast, eval mode),
+    """Images/s of the AFF-Tiny classifier at 224x224 (random weights, N(0,1) images, fp16 autocast, eval mode, no_grad),
     timed like the reference's `throughput` (main.py:343-354: 50 untimed and 30 timed forwards), and the share
     of one forward spent in each operator, measured in a separate pass with stream events around the calls."""
     import torch
@@ -221,6 +221,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     ops.qk_clusters, ops.av_clusters = timed_call("qk", real.qk_clusters), timed_call("av", real.av_clusters)
     ops.cluster_attention = timed_call("qk+bias+mask+blank+softmax+av (one kernel)", real.cluster_attention)
     ops.layer_norm = timed_call("layer_norm", real.layer_norm)
+    ops.merge_weights = timed_call("merge_weights", real.merge_weights)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()
     for layer in net.layers:
         layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)
@@ -251,7 +252,10 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     share = {k: round(sum(a.elapsed_time(b) for a, b in v) / total, 4) for k, v in spans.items() if k != "on"}
     share["everything_else"] = round(1.0 - sum(share.values()), 4)
     return {"img_per_s": round(timed * batch / dt, 1), "ms_per_batch": round(dt / timed * 1e3, 2), "batch": batch,
-            "warmup": warmup, "timed": timed, "dtype": "fp16 autocast (QK fp16; AV, WF fp32)",
+            "warmup": warmup, "timed": timed,
+            "dtype": "fp16 autocast (local attention: one fp16 kernel, fp32 sums; WF fp32)",
+            "inference_path": "16-bit weight copies kept between forwards; layer norm, merge weights, kNN and local "
+                              "attention through the HIP library's optional entry points",
             "share_of_forward": share}
 
 

@@ -427,13 +427,17 @@ class AutoFocusFormer(nn.Module):
     def forward_features(self, x):
         pos, x, h, w = self.patch_embed(x)
         x = self.pos_drop(x)
+        table = self.pre_table
+        if not torch.is_grad_enabled() and table.is_cuda and torch.is_autocast_enabled("cuda"):
+            # every block's position-embedding Linear would round the table to 16 bits again
+            table = table.to(torch.get_autocast_dtype("cuda"))
         for i, layer in enumerate(self.layers):
-            pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=self.pre_table,
-                           radius=self.radius)
+            pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=table, radius=self.radius)
         return _layer_norm(self.norm, x, self.ops).mean(1)
 
     def forward(self, x):
-        return _linear(self.head, self.forward_features(x)) if isinstance(self.head, nn.Linear) else self.forward_features(x)
+        x = self.forward_features(x)
+        return _linear(self.head, x) if isinstance(self.head, nn.Linear) else x
 
 
 def aff_tiny(**kw):
