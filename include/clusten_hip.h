@@ -224,7 +224,7 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
  * fp16 or bf16:
  *   out[r,c] = (x[r,c] - mean_r) * rsqrt(var_r + eps) * weight[c] + bias[c]      (biased variance)
  * what `nn.LayerNorm` computes in the reference model before every attention and MLP block
- * (models/aff_transformer.py:226-240 and the norms at :351, :441, :569-571), with the rounding to 16 bits that
+ * (models/aff_transformer.py:220, :231, and the norms at :362, :546, :663), with the rounding to 16 bits that
  * mixed precision applies to the following Linear layer's input (and the widening it applies to a 16-bit
  * input of the normalisation) done in the same pass.  x (rows,C) of in_dtype, out (rows,C) of out_dtype (F32,
  * F16 or BF16 each); weight, bias (C) fp32; all contiguous and 16-byte aligned (else CLUSTEN_ERR_UNALIGNED);
@@ -235,7 +235,7 @@ int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream);
 
 /* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
- * (models/aff_transformer.py:363-372), in one pass instead of a row lookup, a gather and two multiplications:
+ * (models/aff_transformer.py:340-358), in one pass instead of a row lookup, a gather and two multiplications:
  *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]
  * table_weights (rows,IC), prob (B,N) or NULL, weights (B,Nout,M,IC): fp32, contiguous; pe_idx (values in
  * [0,rows) — unchecked), nbhd_idx (values in [0,N) — unchecked; may be NULL when prob is), mask (0/1, or NULL):

@@ -533,7 +533,7 @@ def merge_weights_supported(table_weights: torch.Tensor) -> bool:
 
 def merge_weights(table_weights: torch.Tensor, pe_idx: torch.Tensor, nbhd_idx: torch.Tensor, prob, mask):
     """table_weights[pe_idx] * prob.gather(nbhd_idx) * mask as one (B,N',M,4) fp32 tensor: the weights the WF
-    operator takes (models/aff_transformer.py:363-372).  table_weights (rows,4); pe_idx, nbhd_idx (B,N',M) int64;
+    operator takes (models/aff_transformer.py:340-358).  table_weights (rows,4); pe_idx, nbhd_idx (B,N',M) int64;
     prob (B,N) or (B,N,1) or None; mask (B,N',M) of 0/1 or None.  No autograd: for inference."""
     lib = load()
     _require_cuda("table_weights", table_weights)

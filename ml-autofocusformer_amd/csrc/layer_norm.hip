@@ -2,11 +2,11 @@
 // tensor, computed in fp32 and written as fp32, fp16 or bf16.
 //
 // The reference model normalises the token features before every attention and MLP block, before each merge
-// projection and at the end (`nn.LayerNorm`, models/aff_transformer.py:226-240, 351, 441, 569-571); under mixed
+// projection and at the end (`nn.LayerNorm`, models/aff_transformer.py:220, 231, 362, 546, 663); under mixed
 // precision the normalisation runs in fp32 (a 16-bit input is widened first) and the Linear layer that follows
-// rounds its input to 16 bits.  This kernel does all of that in one pass over the rows (64 to 512 channels: a row is a few hundred bytes, which the
-// framework's general kernel handles at a fraction of the memory bandwidth).  It has no counterpart in the
-// reference's extension modules.
+// rounds its input to 16 bits.  This kernel does all of that in one pass over the rows (64 to 1024 channels: a row
+// is a few hundred bytes, which the framework's general kernel handles at a fraction of the memory bandwidth).  It
+// has no counterpart in the reference's extension modules.
 //
 // A row is held by L = min(64, C / 4) lanes, four consecutive channels per lane and step (C / (4 L) steps), so
 // that a wave reads 1 KiB contiguous per access; mean and variance are two reductions over registers (the

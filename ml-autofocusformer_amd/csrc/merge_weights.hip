@@ -2,7 +2,7 @@
 //
 //   w[b,i,j,:] = table_w[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]
 //
-// (models/aff_transformer.py:363-372: a row lookup in the position-embedding weights, a gather of the learned
+// (models/aff_transformer.py:340-358: a row lookup in the position-embedding weights, a gather of the learned
 // importance of each neighbour, two multiplications — each a pass over the (B,N',M,IC) tensor; prob and mask are
 // optional).  Here one pass: a lane owns one (token, neighbour) pair, reads its three indices, looks up the row of
 // IC = 4 weights (the table is a few hundred KB and stays in cache) and writes 16 bytes next to its neighbours'.
