@@ -25,6 +25,9 @@
 //   3. the D block leaves lane (r, kq) with slots 4*kq..4*kq+3 of token r.  The output of one
 //      (tile, head) is a single contiguous chunk of 8*M elements, so the blocks are laid out
 //      row-major in LDS and leave with full-width 16-byte stores (lists of up to 64 slots).
+//      On the shared-list path the chunk is laid out in the LDS slot the head's a-rows came from, the rows of
+//      the next head are requested as soon as this head's operands are in registers, and the wait for them
+//      leaves this head's stores in flight (LDS-only ordering between the steps, see lds_sync()).
 // One short-lived one-wave workgroup per tile; the latency of its dependent chain (lists, rows,
 // product, store) is hidden by the ~16 other waves resident on the CU.
 //
@@ -438,7 +441,8 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
 #pragma unroll
         for (int i = 0; i < S::NI_G; ++i) src_lane[i] = min(i * S::RPI + g_sub, mc - 1);
 
-        // shared list: one pass that serves all tokens; otherwise one pass per token that keeps its column
+        // shared list (here only in the kernels for long or odd lists; the FAST kernels took the path above): one
+        // pass that serves all tokens; otherwise one pass per token that keeps its column
         const int passes = shared_list ? 1 : nt;
         for (int pass = 0; pass < passes; ++pass) {
             const int tok_lo = shared_list ? 0 : pass;
@@ -499,34 +503,7 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
 
                 // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of token r
                 char* out_h = out_tile + (int64_t)h * N * M * sizeof(T);
-                if (FAST && shared_list) {
-                    // the (tile, head) output is one contiguous chunk of nt*M elements: turn the D blocks
-                    // into it through LDS and write it with full-width 16-byte stores
-                    if (r < nt) {
-#pragma unroll
-                        for (int blk = 0; blk < Q; ++blk) {
-                            const int s0 = 16 * blk + 4 * kq;
-                            float v[4] = {d[blk][0], d[blk][1], d[blk][2], d[blk][3]};
-                            if (s0 < mc) {
-                                *reinterpret_cast<typename OutIO::raw*>(stage + (r * M + s0) * (int)sizeof(T)) =
-                                    OutIO::pack(v);
-                            }
-                        }
-                    }
-                    __syncthreads();
-                    const int chunk_bytes = nt * M * (int)sizeof(T);
-                    Piece o[(S::OUT_BYTES + 1023) / 1024];
-#pragma unroll
-                    for (int i = 0; i < (S::OUT_BYTES + 1023) / 1024; ++i) {
-                        o[i] = *reinterpret_cast<const Piece*>(stage + min(i * 1024 + lane * 16, S::G_BYTES - 16));
-                    }
-                    __syncthreads();  // the chunk is in registers: the next head's gather may overwrite it
-#pragma unroll
-                    for (int i = 0; i < (S::OUT_BYTES + 1023) / 1024; ++i) {
-                        const int off = i * 1024 + lane * 16;
-                        if (off < chunk_bytes) store_streaming(reinterpret_cast<Piece*>(out_h + off), o[i]);
-                    }
-                } else if (r >= tok_lo && r < tok_hi) {
+                if (r >= tok_lo && r < tok_hi) {
                     T* out_row = reinterpret_cast<T*>(out_h) + r * M + j0;
 #pragma unroll
                     for (int blk = 0; blk < Q; ++blk) {
