@@ -245,6 +245,20 @@ int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_
                                   const float* prob, const int64_t* mask, float* weights,
                                   int B, int N, int Nout, int M, int IC, clusten_stream stream);
 
+/* The order in which the reference's balanced clustering lines up the tokens of each image
+ * (`space_filling_cluster`, models/point_utils.py:61-208, default scan-line path with anchors; the ranking of
+ * point_utils.py:139-159):
+ *   ranking[b,:] = stable argsort of  rank * (max ratio of the batch + 1) + ratio,
+ * rank = position of the token's anchor cell on the row-by-row walk (alternating direction) over a rows x cols
+ * grid of cells of cell_w x cell_h, ratio = squared distance to the previous anchor of the walk over (squared
+ * distance to the next + 1e-5); every float operation rounded as the reference's tensor expressions round it.
+ *   pos (B,N,2) fp32 as (x, y), inside the canvas; ranking (B,N) int64; N <= 4096, rows * cols >= 2 (else
+ *   CLUSTEN_ERR_BAD_DIMS); workspace: clusten_scanline_rank_workspace_bytes(B, N) bytes, 16-byte aligned.
+ * No counterpart in the reference's extension modules. */
+size_t clusten_scanline_rank_workspace_bytes(int B, int N);
+int clusten_scanline_rank(const float* pos, int64_t* ranking, void* workspace, size_t workspace_bytes,
+                          int B, int N, int rows, int cols, float cell_w, float cell_h, clusten_stream stream);
+
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 
 /* K nearest neighbours of 2-D points inside each batch element: for query point q of batch element b,

@@ -59,6 +59,13 @@ def knn(query, database, k, return_dist=False, chunk_elems=1 << 27):
     return idx
 
 
+def _anchor_grid(n, m, h, w):
+    """(rows, cols) of the anchor grid: about one anchor per cluster of m of the n tokens (point_utils.py:91-101)."""
+    k = int(math.ceil(n / m))
+    side = (h * w / k) ** 0.5
+    return int(round(h / side)), int(round(w / side))
+
+
 def _scanline_anchors(n, m, h, w, device):
     """Anchor grid of the balanced clustering and its boustrophedon order.
 
@@ -66,10 +73,7 @@ def _scanline_anchors(n, m, h, w, device):
     cells per row).  Follows point_utils.py:91-137: about one anchor per cluster, rows walked left to right
     and right to left alternately.
     """
-    k = int(math.ceil(n / m))
-    side = (h * w / k) ** 0.5
-    rows = int(round(h / side))
-    cols = int(round(w / side))
+    rows, cols = _anchor_grid(n, m, h, w)
     cell = torch.tensor([w / cols, h / rows], device=device)          # float32, as torch.Tensor([...]) gives
     ys, xs = torch.meshgrid(torch.arange(rows, device=device), torch.arange(cols, device=device), indexing="ij")
     # even rows ascend in x, odd rows descend; the row pitch of the key is the image width (point_utils.py:125-129)
@@ -80,6 +84,31 @@ def _scanline_anchors(n, m, h, w, device):
     cells_xy = torch.stack([xs, ys], dim=2).reshape(-1, 2)[order]
     centres = cells_xy * cell + cell / 2 - 0.5
     return rank_of_cell, centres, cell, cols
+
+
+def _scanline_ranking(pos, m, h, w):
+    """(b, n) order of the tokens along the scan-line walk: the tensor formulation (point_utils.py:139-159)."""
+    b, n, d = pos.shape
+    rank_of_cell, centres, cell, cols = _scanline_anchors(n, m, h, w, pos.device)
+    cells = centres.shape[0]
+
+    # neighbours on the curve, extrapolated linearly past both ends
+    prev_c = torch.empty_like(centres)
+    next_c = torch.empty_like(centres)
+    prev_c[1:] = centres[:cells - 1]
+    prev_c[0] = centres[0] - (centres[1] - centres[0])
+    next_c[:cells - 1] = centres[1:]
+    next_c[cells - 1] = centres[cells - 1] + (centres[cells - 1] - centres[cells - 2])
+
+    cell_xy = (pos / cell).floor()
+    cell_id = (cell_xy[..., 0] + cell_xy[..., 1] * cols).long()    # (b, n)
+    rank = rank_of_cell[cell_id]                                    # (b, n) position of the cell on the curve
+    dist_prev = (pos - prev_c[rank]).pow(2).sum(-1)
+    dist_next = (pos - next_c[rank]).pow(2).sum(-1)
+    ratio = dist_prev / (dist_next + 1e-5)
+    key = rank * (ratio.max() + 1) + ratio                          # one float key; max over the whole batch
+    ranking = key.sort(dim=1, stable=True)[1]                       # (b, n)
+    return ranking
 
 
 def space_filling_cluster(pos, m, h, w, no_reorder=False):
@@ -98,25 +127,15 @@ def space_filling_cluster(pos, m, h, w, no_reorder=False):
         pos = pos.detach().float()
         b, n, d = pos.shape
         k = int(math.ceil(n / m))
-        rank_of_cell, centres, cell, cols = _scanline_anchors(n, m, h, w, pos.device)
-        cells = centres.shape[0]
-
-        # neighbours on the curve, extrapolated linearly past both ends
-        prev_c = torch.empty_like(centres)
-        next_c = torch.empty_like(centres)
-        prev_c[1:] = centres[:cells - 1]
-        prev_c[0] = centres[0] - (centres[1] - centres[0])
-        next_c[:cells - 1] = centres[1:]
-        next_c[cells - 1] = centres[cells - 1] + (centres[cells - 1] - centres[cells - 2])
-
-        cell_xy = (pos / cell).floor()
-        cell_id = (cell_xy[..., 0] + cell_xy[..., 1] * cols).long()    # (b, n)
-        rank = rank_of_cell[cell_id]                                    # (b, n) position of the cell on the curve
-        dist_prev = (pos - prev_c[rank]).pow(2).sum(-1)
-        dist_next = (pos - next_c[rank]).pow(2).sum(-1)
-        ratio = dist_prev / (dist_next + 1e-5)
-        key = rank * (ratio.max() + 1) + ratio                          # one float key; max over the whole batch
-        ranking = key.sort(dim=1, stable=True)[1]                       # (b, n)
+        ranking = None
+        if pos.is_cuda:
+            # on the GPU the ranking is two kernels of the HIP library (same float operations, same order)
+            from clusten import _native
+            rows, cols = _anchor_grid(n, m, h, w)
+            if _native.scanline_rank_supported(pos, rows, cols):
+                ranking = _native.scanline_rank(pos, rows, cols, w / cols, h / rows)
+        if ranking is None:
+            ranking = _scanline_ranking(pos, m, h, w)
 
         pos = pos.gather(1, ranking.unsqueeze(2).expand(-1, -1, d))
         if k * m == n:

@@ -57,6 +57,9 @@ _PROTOTYPES = {
                                                  ctypes.c_float, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                     ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
+    "clusten_scanline_rank": (ctypes.c_int, [_P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_float, ctypes.c_float, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
 }
@@ -563,6 +566,33 @@ def merge_weights(table_weights: torch.Tensor, pe_idx: torch.Tensor, nbhd_idx: t
                                                  n_out, m, table_weights.shape[1], _stream(device)),
                "clusten_merge_weights_forward")
     return out
+
+
+def scanline_rank_supported(pos: torch.Tensor, rows: int, cols: int) -> bool:
+    """True when `scanline_rank` takes this case: CUDA (B,N,2) positions, N <= 4096, at least two anchor cells."""
+    return pos.is_cuda and pos.dim() == 3 and pos.shape[2] == 2 and 0 < pos.shape[1] <= 4096 and rows * cols >= 2
+
+
+def scanline_rank(pos: torch.Tensor, rows: int, cols: int, cell_w: float, cell_h: float) -> torch.Tensor:
+    """(B,N) int64: per image the order of the tokens along the scan-line walk over the rows x cols anchor grid
+    (cells of cell_w x cell_h), the ranking of the reference's `space_filling_cluster` (point_utils.py:139-159)."""
+    lib = load()
+    _require_cuda("pos", pos)
+    if pos.dim() != 3 or pos.shape[2] != 2:
+        raise RuntimeError("pos must be (B,N,2)")
+    device = pos.device
+    pos = pos.detach().float().contiguous()
+    b, n, _ = pos.shape
+    ranking = torch.empty(b, n, dtype=torch.int64, device=device)
+    if ranking.numel() == 0:
+        return ranking
+    nbytes = lib.clusten_scanline_rank_workspace_bytes(b, n)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        _check(lib.clusten_scanline_rank(_ptr(pos), _ptr(ranking), _ptr(workspace), nbytes, b, n, rows, cols,
+                                         ctypes.c_float(cell_w), ctypes.c_float(cell_h), _stream(device)),
+               "clusten_scanline_rank")
+    return ranking
 
 
 def knn2d_supported(query: torch.Tensor, database: torch.Tensor, k: int) -> bool:

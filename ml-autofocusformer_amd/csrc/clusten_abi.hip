@@ -208,6 +208,23 @@ int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_
     return launch_merge_weights(table_weights, pe_idx, nbhd_idx, prob, mask, weights, B, N, Nout, M, as_stream(stream));
 }
 
+size_t clusten_scanline_rank_workspace_bytes(int B, int N) {
+    if (B <= 0 || N <= 0) return 0;
+    return scanline_rank_workspace_bytes(B, N);
+}
+
+int clusten_scanline_rank(const float* pos, int64_t* ranking, void* workspace, size_t workspace_bytes, int B, int N,
+                          int rows, int cols, float cell_w, float cell_h, clusten_stream stream) {
+    if (!pos || !ranking || !workspace) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || N > 4096 || rows <= 0 || cols <= 0 || (int64_t)rows * cols < 2 ||
+        (int64_t)rows * cols >= ((int64_t)1 << 24) || !(cell_w > 0.f) || !(cell_h > 0.f)) {
+        return CLUSTEN_ERR_BAD_DIMS;
+    }
+    if (workspace_bytes < scanline_rank_workspace_bytes(B, N)) return CLUSTEN_ERR_WORKSPACE;
+    if (!aligned16(workspace) || (reinterpret_cast<uintptr_t>(pos) & 7u) != 0) return CLUSTEN_ERR_UNALIGNED;
+    return launch_scanline_rank(pos, ranking, workspace, B, N, rows, cols, cell_w, cell_h, as_stream(stream));
+}
+
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
                   clusten_stream stream) {
     if (!query || !database || !idx) return CLUSTEN_ERR_NULL_POINTER;

@@ -74,6 +74,13 @@ int launch_layer_norm(const void* x, int in_dtype, const float* weight, const fl
 int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,
                          const int64_t* mask, float* out, int B, int N, int Nout, int M, hipStream_t stream);
 
+// ranking[b,:] = the order of the tokens of image b along the scan-line walk over a rows x cols anchor grid with
+//   cells of cell_w x cell_h (see scanline_rank.hip).  pos (B,N,2) fp32 as (x, y); ranking (B,N) int64; N <= 4096,
+//   rows * cols >= 2; workspace of scanline_rank_workspace_bytes(B, N) bytes.
+size_t scanline_rank_workspace_bytes(int B, int N);
+int launch_scanline_rank(const float* pos, int64_t* ranking, void* workspace, int B, int N, int rows, int cols,
+                         float cell_w, float cell_h, hipStream_t stream);
+
 // idx[b,q,:K], dist[b,q,:K] = the K (1..8, K <= N) database points of batch element b nearest to query q,
 //   ascending Euclidean distance, equal distances by index.  query (B,Nq,2), database (B,N,2): fp32;
 //   idx int64; dist fp32 or null.

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from aff.points import knn, space_filling_cluster, _scanline_anchors
+from aff.points import knn, space_filling_cluster, _anchor_grid, _scanline_anchors, _scanline_ranking
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "space_filling_cluster.npz")
 CASES = ["grid56", "grid14", "sub784", "sub196", "sub49", "ref_script", "wide", "grid96"]
@@ -130,3 +130,32 @@ def test_knn_kernel_equals_the_tensor_formulation(device, k):
     assert not _native.knn2d_supported(q.to(device), x.to(device), 9)
     with pytest.raises(RuntimeError):
         _native.knn2d(q, x, 2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", CASES)
+def test_ranking_kernel_equals_the_tensor_formulation(device, name):
+    """Bit-identical keys, hence the same order: the fixtures' positions and denser random ones."""
+    from clusten import _native
+    z, pos, m, h, w = _load(name)
+    gen = torch.Generator().manual_seed(23)
+    more = torch.stack([torch.randperm(h * w, generator=gen)[:pos.shape[1]] for _ in range(5)])
+    more = torch.stack([more % w, more // w], dim=2)
+    for p in (pos, more, more.float() + torch.rand(more.shape, generator=gen) * 0.99):
+        p = p.float()
+        ref = _scanline_ranking(p, m, h, w)                                  # CPU tensors: the tensor formulation
+        rows, cols = _anchor_grid(p.shape[1], m, h, w)
+        if p.shape[1] <= 4096:
+            assert _native.scanline_rank_supported(p.to(device), rows, cols)
+            got = _native.scanline_rank(p.to(device), rows, cols, w / cols, h / rows)
+            assert got.dtype == torch.int64 and torch.equal(got.cpu(), ref)
+        else:   # longer sequences keep the tensor formulation on the GPU
+            assert not _native.scanline_rank_supported(p.to(device), rows, cols)
+        # and through the public function: same clusters on both devices
+        cpu = space_filling_cluster(p, m, h, w)
+        gpu = space_filling_cluster(p.to(device), m, h, w)
+        assert torch.equal(gpu[4].cpu(), cpu[4]) and torch.equal(gpu[0].cpu(), cpu[0])
+        assert torch.allclose(gpu[1].cpu(), cpu[1], rtol=1e-6, atol=1e-6)
+    assert not _native.scanline_rank_supported(torch.zeros(1, 5000, 2, device=device), 10, 10)
+    with pytest.raises(RuntimeError):
+        _native.scanline_rank(pos.float(), 4, 4, 1.0, 1.0)
