@@ -34,25 +34,36 @@ MEASURED_TRAFFIC_BYTES = {"qk": 359.56e6 + 154.14e6, "av": 410.98e6 + 102.76e6, 
 
 
 def _time_kernels(fns, steps, warmup):
-    """Run the launch closures `fns` back to back for warmup + steps steps on the current stream.
-    Returns (ms per step over the timed region, [average ms per launch of each closure])."""
+    """Run the launch closures `fns` back to back for warmup + steps steps on the current stream, twice.
+
+    The first timed pass has one event before and one after its `steps` steps and nothing between the launches:
+    its duration is the throughput figure.  The second pass records an event after every launch (a marker on
+    the stream that costs a few microseconds of gap per launch) for the per-kernel averages.
+    Returns (ms per step of the first pass, [average ms per launch of each closure], host wall ms per step)."""
     import torch
 
     for _ in range(warmup):
         for fn in fns:
             fn()
     torch.cuda.synchronize()
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(fns) + 1)] for _ in range(steps)]
-    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    begin.record()
+    for _ in range(steps):
+        for fn in fns:
+            fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    region_ms = begin.elapsed_time(end)
+
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(fns) + 1)] for _ in range(steps)]
     for s in range(steps):
         marks[s][0].record()
         for i, fn in enumerate(fns):
             fn()
             marks[s][i + 1].record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    region_ms = marks[0][0].elapsed_time(marks[-1][-1])
     per = [sum(marks[s][i].elapsed_time(marks[s][i + 1]) for s in range(steps)) / steps for i in range(len(fns))]
     return region_ms / steps, per, wall_ms / steps
 
