@@ -86,13 +86,6 @@ __device__ __forceinline__ float oct_sum(float v) {
     return v + dpp_move<0x141>(v);
 }
 
-// Keeps a 32-bit byte offset a 32-bit register value at the place of use, so that the access it feeds is encoded
-// as uniform base + lane offset instead of through a 64-bit address per lane held across the loops.
-__device__ __forceinline__ uint32_t lane_offset(uint32_t off) {
-    asm volatile("" : "+v"(off));
-    return off;
-}
-
 template <typename T>
 __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const T* __restrict__ q, clusten_strides qs, const T* __restrict__ k, clusten_strides ks, const T* __restrict__ v,

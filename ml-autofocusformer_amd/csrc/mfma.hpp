@@ -30,6 +30,13 @@ __device__ __forceinline__ void lds_sync_vm() {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 }
 
+// Keeps a 32-bit byte offset a 32-bit register value at the place of use, so that the access it feeds is encoded
+// as uniform base + lane offset instead of through a 64-bit address per lane held across the loops.
+__device__ __forceinline__ uint32_t lane_offset(uint32_t off) {
+    asm volatile("" : "+v"(off));
+    return off;
+}
+
 // One LDS-direct load: every lane moves 16 bytes from its own global address `gptr` to LDS address
 // `lptr` + 16 * lane (`lptr` is wave-uniform).  Completion is tracked by the vector-memory counter.
 #define CLUSTEN_LDS_DMA16(gptr, lptr)                                                       \

@@ -71,7 +71,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     const int b = token / Nout;
     const int col = (lane % LPT) * VEC;  // first channel of the lane inside a column block
     const int ic_lane = lane & 3;        // the row of the 4x4 blocks this lane feeds: inner channel
-    const bool ic_live = ic_lane < IC;
 
     const int64_t* list_p = idx + (int64_t)token * M;
     const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
@@ -117,23 +116,27 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             }
             __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
             __syncthreads();
-            // this lane's A operands: weight (its token, slot j, inner channel l % 4)
+            // this lane's A operands: weight (its token, slot j, inner channel l % 4).  Lanes of an inner channel past
+            // IC read the last one: the rows of the 4x4 blocks they feed are never stored.
             const char* w_lane = wbuf + min(tl, ntok - 1) * w_chunk_bytes + min(ic_lane, IC - 1) * (int)sizeof(T);
 
             Piece fv[SLOTS];
+            T wv[SLOTS];
             slot_pipeline<SLOTS, GS>(
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
-                    // row index of slot j: lane j % 16 of list register j / 16, broadcast inside each row of 16
+                    // row index of slot j: lane j % 16 of list register j / 16, broadcast inside each row of 16.
+                    // Row index and row size are below 2^24 and the offset fits 32 bits (checked by the launcher):
+                    // one 24-bit multiply-add, and the access is encoded as uniform base + lane offset.
                     const int row = rowlane_bcast<j % 16>(lst[j / 16]);
-                    const uint32_t off = (uint32_t)((GUARD && j >= mc) ? 0 : row) * row_bytes + lane_bytes;
-                    fv[j] = *reinterpret_cast<const Piece*>(feat_b + off);
+                    const uint32_t off = __umul24((uint32_t)((GUARD && j >= mc) ? 0 : row), row_bytes) + lane_bytes;
+                    fv[j] = *reinterpret_cast<const Piece*>(feat_b + lane_offset(off));
+                    // the weight of the slot comes from LDS with the group's rows, a pipeline group ahead of its use
+                    wv[j] = *reinterpret_cast<const T*>(w_lane + (GUARD ? min(j, mc - 1) : j) * IC * (int)sizeof(T));
                 },
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
-                    const bool live = ic_live && (!GUARD || j < mc);
-                    const int jj = GUARD ? min(j, mc - 1) : j;
-                    const float aop = live ? to_acc(*reinterpret_cast<const T*>(w_lane + jj * IC * (int)sizeof(T))) : 0.f;
+                    const float aop = (!GUARD || j < mc) ? to_acc(wv[j]) : 0.f;
                     float x[VEC];
                     VecIO<T, VEC>::unpack(fv[j], x);
 #pragma unroll
