@@ -360,3 +360,36 @@ def test_aff_tiny_224_forward_and_gradients(device):
     model.train()
     model(x).square().mean().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+@pytest.mark.gpu
+def test_cached_16_bit_weights_follow_the_parameters(device):
+    """Inference under autocast keeps 16-bit copies of the Linear weights between forwards; an in-place update, a
+    load_state_dict and a move of the parameters must all be seen by the next forward."""
+    from aff.model import default_ops
+    model = small_model(default_ops(), img_size=128).to(device)
+    x = torch.randn(2, 3, 128, 128, generator=torch.Generator().manual_seed(5)).to(device)
+
+    def run(m):
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+            return m(x).float()
+
+    y0 = run(model)
+    assert torch.equal(run(model), y0)                      # second forward: from the cached copies
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    with torch.no_grad():                                   # in-place update of one projection and of the classifier
+        model.layers[0].blocks[0].attn.proj.weight.mul_(1.5)
+        model.head.bias.add_(1.0)
+    y1 = run(model)
+    fresh = small_model(default_ops(), img_size=128).to(device)
+    fresh.load_state_dict(model.state_dict())
+    assert torch.equal(y1, run(fresh)) and not torch.equal(y1, y0)
+    model.load_state_dict(state)                            # back to the first weights
+    assert torch.equal(run(model), y0)
+    model.float()                                           # no-op conversion keeps working
+    assert torch.equal(run(model), y0)
+    # training mode and grad mode do not use the cache
+    model.train()
+    with torch.autocast("cuda", dtype=torch.float16):
+        model(x).float().sum().backward()
+    assert model.head.weight.grad is not None
