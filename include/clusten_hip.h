@@ -207,6 +207,8 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
  *   row(i,j)       = 8 * cluster_idx[b,i,j/8] + j%8, row 0 where that is not in [0,N)
  * query, key, value, out: strided (B,H,N,C) of `dtype`; bias_table (rows,H) of `dtype`, contiguous;
  * cluster_idx (B,N,M/8) int32; pe_idx (B,N,M) int64 in [0,rows) — unchecked; mask (B,N,M) int64 of 0/1 or NULL;
+ * with lists_shared != 0 these three are (1,N,.) tensors that serve every batch element (the tokens of a
+ * regular grid have the same neighbourhoods in every image);
  * blank_key, blank_value (H,C) fp32, contiguous.  Pass the unscaled query and the model's scale, or a scaled
  * query and 1.  The probabilities are rounded to `dtype` before they weigh the value rows; sums are fp32.
  * dtype F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and M = 48 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
@@ -215,7 +217,7 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       const void* key, clusten_strides key_strides,
                                       const void* value, clusten_strides value_strides,
                                       const int32_t* cluster_idx, const void* bias_table,
-                                      const int64_t* pe_idx, const int64_t* mask,
+                                      const int64_t* pe_idx, const int64_t* mask, int lists_shared,
                                       const float* blank_key, const float* blank_value,
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);

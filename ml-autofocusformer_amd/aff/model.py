@@ -128,7 +128,9 @@ class ClusterAttention(nn.Module):
         self.proj_drop = nn.Dropout(proj_drop)
         self.ops = ops
 
-    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None):
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None, grid_lists=None):
+        """`grid_lists`: (cluster_idx, pe_idx, cluster_mask) with a leading 1 instead of the batch size, when the
+        lists are the same for every image (tokens of a regular grid); the one-kernel path reads those."""
         b, n, c = feat.shape
         h = self.num_heads
         ch = c // h
@@ -143,8 +145,9 @@ class ClusterAttention(nn.Module):
                 and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2])):
             # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
             # the values in one kernel; the query scale is applied to the scores inside it
-            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, cluster_idx, _linear(self.pos_embed, table),
-                             pe_idx, cluster_mask, self.blank_k, self.blank_v, scale=self.scale)
+            lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
+            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], _linear(self.pos_embed, table),
+                             lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale)
             return self.proj_drop(_linear(self.proj, out))
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:
@@ -195,10 +198,10 @@ class ClusterTransformerBlock(nn.Module):
             self.gamma1 = nn.Parameter(layer_scale * torch.ones(dim))
             self.gamma2 = nn.Parameter(layer_scale * torch.ones(dim))
 
-    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None):
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None, grid_lists=None):
         ops = self.attn.ops
         a = self.attn(_layer_norm(self.norm1, feat, ops, True), member_idx, cluster_mask, pe_idx, global_attn, table,
-                      cluster_idx)
+                      cluster_idx, grid_lists)
         feat = feat + self.drop_path(self.gamma1 * a if self.layer_scale else a)
         f = self.mlp(_layer_norm(self.norm2, feat, ops, True))
         return feat + self.drop_path(self.gamma2 * f if self.layer_scale else f)
@@ -326,7 +329,7 @@ class BasicLayer(nn.Module):
         b, n, d = pos.shape
         table_width = 2 * radius + 1
         global_attn = self.nbhd_size >= n
-        cluster_idx = None
+        cluster_idx = grid_lists = None
         if global_attn:
             member_idx = mask = None
             rel = (pos[:, None, :, :] + radius) - pos[:, :, None, :]
@@ -343,6 +346,8 @@ class BasicLayer(nn.Module):
                                                   pe_idx.expand(b, -1, -1).contiguous(),
                                                   None if mask is None else mask.expand(b, -1, -1).contiguous(),
                                                   None if cluster_idx is None else cluster_idx.expand(b, -1, -1).contiguous())
+                if cluster_idx is not None:
+                    grid_lists = (cluster_idx, pe_idx, mask)           # one image's lists, for the one-kernel attention
                 member_idx, pe_idx, mask, cluster_idx = self._grid_cache[(key, b)]
                 pos = pos1.expand(b, -1, -1)
                 if ranking is not None:
@@ -353,7 +358,7 @@ class BasicLayer(nn.Module):
                     feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
 
         for blk in self.blocks:
-            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx)
+            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists)
 
         if self.downsample is not None:
             if global_attn:   # merging after a dense stage: every token is every token's neighbour

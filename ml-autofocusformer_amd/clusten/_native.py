@@ -51,8 +51,9 @@ _PROTOTYPES = {
     "clusten_av_forward_clusters": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
                                                    _P]),
-    "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, _P,
-                                                        _P, Strides, ctypes.c_float, AttnShape, ctypes.c_int, _P]),
+    "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
+                                                        ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
+                                                        ctypes.c_int, _P]),
     "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
                                                  ctypes.c_float, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -439,8 +440,9 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
                       blank_value: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """Local attention over the members of each token's clusters plus one blank token, in one kernel.
 
-    query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1); cluster_idx (B,N,6) integer;
+    query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
     bias_table (rows,H); pe_idx (B,N,48) int64; mask (B,N,48) of 0/1 or None; blank_key, blank_value (H*32,).
+    cluster_idx, pe_idx and mask may all have a leading 1 instead of B: one set of lists for every image.
     Returns softmax(scale * q.k + bias - 100 * (1 - mask) | scale * q.blank_key) applied to the gathered values and
     the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the layout the output
     projection takes).  No autograd: for inference.  The fused form of models/aff_transformer.py:120-155.
@@ -454,10 +456,12 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     if query.dim() != 4 or key.shape != query.shape or value.shape != query.shape:
         raise RuntimeError("query, key and value must be (B,H,N,C) tensors of one shape")
     b, h, n, c = query.shape
-    cidx = _cluster_idx(cluster_idx, (b, n), device)
+    shared = b != 1 and cluster_idx.dim() == 3 and cluster_idx.shape[0] == 1
+    lb = 1 if shared else b
+    cidx = _cluster_idx(cluster_idx, (lb, n), device)
     m = 8 * cidx.shape[2]
-    if pe_idx.shape != (b, n, m) or pe_idx.dtype != torch.int64:
-        raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")
+    if pe_idx.shape != (lb, n, m) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,M), or (1,N,M) like cluster_idx")
     if bias_table.dim() != 2 or bias_table.shape[1] != h:
         raise RuntimeError("bias_table must have shape (rows, H)")
     if blank_key.numel() != h * c or blank_value.numel() != h * c:
@@ -469,8 +473,8 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     pe_idx = pe_idx.contiguous()
     if mask is not None:
         _require_cuda("mask", mask, device)
-        if mask.shape != (b, n, m):
-            raise RuntimeError("mask must have shape (B,N,M)")
+        if mask.shape != (lb, n, m):
+            raise RuntimeError("mask must have shape (B,N,M), or (1,N,M) like cluster_idx")
         mask = mask.to(torch.int64).contiguous()
     blank_key = blank_key.detach().reshape(h, c).float().contiguous()
     blank_value = blank_value.detach().reshape(h, c).float().contiguous()
@@ -482,7 +486,8 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     with torch.cuda.device(device):
         _check(lib.clusten_cluster_attention_forward(_ptr(query), _strides(query), _ptr(key), _strides(key),
                                                      _ptr(value), _strides(value), _ptr(cidx), _ptr(bias_table),
-                                                     _ptr(pe_idx), _ptr(mask), _ptr(blank_key), _ptr(blank_value),
+                                                     _ptr(pe_idx), _ptr(mask), int(shared), _ptr(blank_key),
+                                                     _ptr(blank_value),
                                                      _ptr(out), _strides(out_view), ctypes.c_float(scale), shape, code,
                                                      _stream(device)),
                "clusten_cluster_attention_forward")

@@ -170,9 +170,9 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
 int clusten_cluster_attention_forward(const void* query, clusten_strides query_strides, const void* key,
                                       clusten_strides key_strides, const void* value, clusten_strides value_strides,
                                       const int32_t* cluster_idx, const void* bias_table, const int64_t* pe_idx,
-                                      const int64_t* mask, const float* blank_key, const float* blank_value, void* out,
-                                      clusten_strides out_strides, float scale, clusten_attn_shape shape, int dtype,
-                                      clusten_stream stream) {
+                                      const int64_t* mask, int lists_shared, const float* blank_key,
+                                      const float* blank_value, void* out, clusten_strides out_strides, float scale,
+                                      clusten_attn_shape shape, int dtype, clusten_stream stream) {
     if (!query || !key || !value || !cluster_idx || !bias_table || !pe_idx || !blank_key || !blank_value || !out) {
         return CLUSTEN_ERR_NULL_POINTER;
     }
@@ -183,8 +183,8 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
         return CLUSTEN_ERR_BAD_STRIDE;
     }
     return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, cluster_idx, bias_table,
-                                    pe_idx, mask, blank_key, blank_value, out, out_strides, scale, shape, dtype,
-                                    as_stream(stream));
+                                    pe_idx, mask, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, shape,
+                                    dtype, as_stream(stream));
 }
 
 int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     clusten_strides vs, const int32_t* __restrict__ cluster_idx, const T* __restrict__ table,
     const int64_t* __restrict__ pe_idx, const int64_t* __restrict__ mask, const float* __restrict__ blank_k,
     const float* __restrict__ blank_v, T* __restrict__ out, clusten_strides os, int H, int N, float scale,
-    int tiles_per_batch, int total_tiles) {
+    int tiles_per_batch, int total_tiles, int lists_shared) {
     typedef short S4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) S4* LdsS4;
 
@@ -110,7 +110,10 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const int g_pos = lane & 3;    //              16-byte piece of the row
     const int t = lane >> 3;       // softmax side: token of the tile (tokens past a partial tile repeat its last one)
     const int i = lane & 7;        //               member of each cluster
-    const int64_t tok = (int64_t)b * N + i0 + min(t, nt - 1);
+    // the token's row in the index tensors: those of batch element 0 serve every image when the lists are shared
+    // (the tokens of a regular grid have the same neighbourhoods in every image)
+    const int64_t list_b = lists_shared ? 0 : b;
+    const int64_t tok = list_b * N + i0 + min(t, nt - 1);
 
     // q rows of head h -> slot h % 2 (lanes 0..31: token lane / 4, piece lane % 4)
     const char* q_tile = reinterpret_cast<const char*>(q + (int64_t)b * qs.b + (int64_t)i0 * qs.n);
@@ -125,7 +128,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
 
     // cluster numbers: lane rho < 48 owns run rho = token * 6 + run of the tile
     const int rho = min(lane, kTileTokens * kR - 1);
-    const int cid = cluster_idx[((int64_t)b * N + i0 + min(rho / kR, nt - 1)) * kR + rho % kR];
+    const int cid = cluster_idx[(list_b * N + i0 + min(rho / kR, nt - 1)) * kR + rho % kR];
 
     // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
     int pe[kR];
@@ -386,13 +389,13 @@ template <typename T>
 int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out, clusten_strides os,
-                 float scale, const clusten_attn_shape& s, hipStream_t stream) {
+                 float scale, int lists_shared, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
                        static_cast<const T*>(q), qs, static_cast<const T*>(k), ks, static_cast<const T*>(v), vs,
                        cluster_idx, static_cast<const T*>(table), pe_idx, mask, blank_k, blank_v, static_cast<T*>(out),
-                       os, s.H, s.N, scale, tiles_per_batch, total);
+                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared);
     return launch_status();
 }
 
@@ -401,7 +404,8 @@ int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strid
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, clusten_attn_shape s, int dtype, hipStream_t stream) {
+                             clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
+                             hipStream_t stream) {
     if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (s.C != kC || s.M != kM) return CLUSTEN_ERR_BAD_DIMS;
     const bool ok = rows_aligned16(q, qs, 2) && rows_aligned16(k, ks, 2) && rows_aligned16(v, vs, 2) &&
@@ -410,10 +414,10 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
     if (!ok) return CLUSTEN_ERR_UNALIGNED;
     if (dtype == CLUSTEN_F16) {
         return launch_typed<f16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                   s, stream);
+                                   lists_shared, s, stream);
     }
-    return launch_typed<bf16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale, s,
-                                stream);
+    return launch_typed<bf16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
+                                lists_shared, s, stream);
 }
 
 }  // namespace clusten

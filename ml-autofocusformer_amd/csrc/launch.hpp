@@ -57,12 +57,14 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
 
 // Local attention of a cluster-ordered sequence in one kernel (QK, position bias, mask, blank token, softmax, AV,
 // blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16}, C = 32;
-//   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48);
+//   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48) — or (1,N,.) each
+//   when lists_shared;
 //   blank_k, blank_v : fp32 (H,C).
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, clusten_attn_shape s, int dtype, hipStream_t stream);
+                             clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
+                             hipStream_t stream);
 
 // out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C channels
 //   (C in {64,128,256,384,512,768,1024}); x and out of dtype F32, F16 or BF16 each, arithmetic in fp32.

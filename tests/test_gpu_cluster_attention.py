@@ -135,3 +135,21 @@ def test_unsupported_cases_are_refused(device):
     empty = _native.cluster_attention(d(q)[:0], d(k)[:0], d(v)[:0], d(cidx)[:0], d(table), d(pe_idx)[:0], None,
                                       d(blank_k), d(blank_v))
     assert empty.shape == (0, 64, 2 * C)
+
+
+def test_lists_shared_by_the_batch(device):
+    """(1,N,.) lists (the tokens of a regular grid) give what their batch-sized copies give."""
+    gen = torch.Generator().manual_seed(85)
+    b, h, n = 3, 2, 200
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True)
+    d = lambda x: x.to(device)
+    c1, p1, m1 = cidx[:1].contiguous(), pe_idx[:1].contiguous(), mask[:1].contiguous()
+    full = _native.cluster_attention(d(q), d(k), d(v), d(c1.expand(b, -1, -1).contiguous()), d(table),
+                                     d(p1.expand(b, -1, -1).contiguous()), d(m1.expand(b, -1, -1).contiguous()),
+                                     d(blank_k), d(blank_v), scale=0.25)
+    shared = _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(p1), d(m1), d(blank_k), d(blank_v), scale=0.25)
+    assert torch.equal(shared, full)
+    no_mask = _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(p1), None, d(blank_k), d(blank_v))
+    assert no_mask.shape == full.shape and torch.isfinite(no_mask.float()).all()
+    with pytest.raises(RuntimeError):       # shared cluster numbers need shared pe_idx
+        _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(pe_idx), None, d(blank_k), d(blank_v))
