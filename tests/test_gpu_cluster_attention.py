@@ -153,3 +153,19 @@ def test_lists_shared_by_the_batch(device):
     assert no_mask.shape == full.shape and torch.isfinite(no_mask.float()).all()
     with pytest.raises(RuntimeError):       # shared cluster numbers need shared pe_idx
         _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(pe_idx), None, d(blank_k), d(blank_v))
+
+
+def test_cluster_numbers_out_of_range_read_row_zero(device):
+    """Negative numbers and numbers past the last cluster list row 0, as the expanded lists of the operators do."""
+    gen = torch.Generator().manual_seed(86)
+    b, h, n = 2, 2, 100                                   # 12 whole clusters and one of 4 tokens
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, False)
+    wild = cidx.clone()
+    hit = torch.rand(wild.shape, generator=gen) < 0.1
+    wild[hit] = torch.tensor([-1, -7, 13, 500, 1 << 20], dtype=torch.int32)[torch.randint(5, (int(hit.sum()),), generator=gen)]
+    idx = _expand(wild, n)
+    assert (idx == 0).sum() > hit.sum()
+    ref = _reference(q, k, v, idx, table, pe_idx, None, blank_k, blank_v, 0.2)
+    d = lambda x: x.to(device)
+    out = _native.cluster_attention(d(q), d(k), d(v), d(wild), d(table), d(pe_idx), None, d(blank_k), d(blank_v), scale=0.2)
+    assert oracle.rel_err(out, ref) <= TOL[torch.float16]
