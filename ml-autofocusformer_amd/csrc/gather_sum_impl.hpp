@@ -33,7 +33,11 @@
 //   per-token path — any other tile: the gather and the MFMAs are repeated per token and only that
 //     token's row is kept.  Exact for arbitrary indices (duplicates, any order), only slower.
 //
-// Storage types narrower than fp32 are widened in registers; all products and sums are fp32.
+// Storage types narrower than fp32 are widened in registers; all products and sums are fp32.  One case goes
+// through the 16-bit matrix instructions instead: fp16 / bf16 data with a shared list of 48 slots.  The p pieces
+// are A operands as they lie in LDS; the B operand (8 consecutive slots of one channel) is a column of the
+// row-major gathered rows, read with `ds_read_b64_tr_b16`; two 16x16x32 steps per 16 channels replace twelve
+// fp32 steps and their conversions (products of 16-bit values are exact in fp32, sums are fp32).
 // Head dims other than 16/32/64, p rows that are not whole 16-byte pieces (M*sizeof(T) % 16 != 0),
 // rows whose start is not 16-byte aligned and fp64 take the element-per-thread kernel at the
 // bottom of the file.
