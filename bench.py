@@ -407,6 +407,8 @@ def main():
             "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
         del mcase, cidx, mattn, q16, k16, v16, pe_idx
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
+        other["cfg2_s1_backward_fp32_model_like_lists"] = _bench_backward(
+            wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:
         out["aff_tiny_224"] = _aff_tiny_throughput()

@@ -11,7 +11,13 @@
 //     destination row are summed in registers and leave the wave as ONE fp32 atomic per (slot,
 //     channel): 8x fewer atomics than one per product, and each wave-wide atomic instruction adds
 //     to whole contiguous rows.
-//   per-token path — one atomic per product, for tiles whose lists differ.
+//   union path — lists that differ but are made of runs of 8 slots of which the tile's tokens share most (the
+//     neighbourhoods of a cluster-ordered sequence: a run is the 8 members of one cluster; a tile of the model's own
+//     lists holds 8-12 distinct runs): the runs are numbered by distinct value as in the forward kernels, p is laid
+//     out in LDS by distinct run and member (zero where a token does not hold the run), and the sums over the tile's
+//     tokens are one small matrix product per head,  D[run member][c] = P^T (members x 8 tokens) * X (8 tokens x C),
+//     on the matrix cores.  One atomic per (distinct run member, channel): 80-100 per lane instead of 384.
+//   per-token path — one atomic per product, for any other tile.
 //
 // The destination is accumulated in fp32: directly in `out` for fp32, in a caller-provided fp32
 // workspace that is rounded once at the end for fp16/bf16.  fp64, head dims other than 16/32/64
@@ -22,6 +28,7 @@
 
 #include "dpp.hpp"
 #include "launch.hpp"
+#include "mfma.hpp"
 
 namespace clusten {
 
@@ -47,6 +54,103 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
     float* out_b = out + (int64_t)b * H * N * C;
+
+    if ((M & 7) == 0 && M <= 64) {
+        // ---- union path: lists made of runs of 8 slots, at most 16 distinct runs in the tile ----
+        constexpr int U_MAX = 16;
+        constexpr int PS = 9;                        // floats per row of the P^T matrix: odd, rows fall into different banks
+        __shared__ float pm[U_MAX * 8 * PS];
+        __shared__ int ulist[U_MAX * 8];
+        const int R = M >> 3;                        // runs per token
+        const int nruns = nt * R;                    // <= 64: lane rho owns run rho = token * R + run
+        int v[8];
+        {
+            const int64_t* run = idx_tile + (int64_t)min(lane, nruns - 1) * 8;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = (int)run[t];
+        }
+        bool regular = true;                         // 8 consecutive rows
+#pragma unroll
+        for (int t = 1; t < 8; ++t) regular = regular && (v[t] == v[0] + t);
+        const int key = regular ? v[0] : ~lane;      // other runs never merge
+        uint64_t remaining = nruns >= 64 ? ~0ull : ((1ull << nruns) - 1);
+        bool differ = false;                         // a shared list is better served by the path below
+        {
+            const int k0 = __shfl(key, lane % R);
+            differ = __any((lane < nruns && key != k0) ? 1 : 0) != 0;
+        }
+        int uslot = 0, U = 0;
+        bool first = false;
+        while (differ && remaining != 0 && U < U_MAX) {
+            const int sl = __builtin_ctzll(remaining);
+            const int ks = __builtin_amdgcn_readlane(key, sl);
+            const bool hit = key == ks;
+            const uint64_t match = __ballot(hit) & remaining;
+            if (hit) uslot = U;
+            first = first || lane == sl;
+            remaining &= ~match;
+            ++U;
+        }
+        if (differ && remaining == 0) {
+            if (first) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) ulist[uslot * 8 + t] = v[t];
+            }
+            const int t8 = lane >> 3, m8 = lane & 7;     // build side: token and run member of the lane
+            const int r16 = lane & 15, kq = lane >> 4;   // matrix side
+            int us[8];                                   // distinct-run number of the lane's token's runs
+#pragma unroll
+            for (int r = 0; r < 8; ++r) us[r] = __shfl(uslot, min(t8 * R + min(r, R - 1), nruns - 1));
+            const int rows_u = 8 * U;
+            for (int h = 0; h < H; ++h) {
+                __syncthreads();  // the previous head's operand reads are complete (and the row table is written)
+                for (int z = lane; z < U_MAX * 8 * PS; z += kWave) pm[z] = 0.f;
+                __syncthreads();
+                if (t8 < nt) {
+                    const T* prow = p + (((int64_t)b * H + h) * N + i0 + t8) * M + m8;
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) {
+                        // the lane owns column t8 of the rows of member m8: repeats of a run by one token add up
+                        if (r < R) pm[(us[r] * 8 + m8) * PS + t8] += to_acc(prow[8 * r]);
+                    }
+                }
+                // B operands: x[token 4*s + kq][channel 16*cb + r16]
+                float xb[2][C / 16];
+                const T* xh = x + (int64_t)b * xs.b + (int64_t)h * xs.h + (int64_t)i0 * xs.n;
+#pragma unroll
+                for (int sx = 0; sx < 2; ++sx) {
+                    const int tok = 4 * sx + kq;
+#pragma unroll
+                    for (int cb = 0; cb < C / 16; ++cb) {
+                        xb[sx][cb] = tok < nt ? to_acc(xh[(int64_t)tok * xs.n + 16 * cb + r16]) : 0.f;
+                    }
+                }
+                __syncthreads();
+                float* out_h = out_b + (int64_t)h * N * C;
+                for (int blk = 0; blk * 16 < rows_u; ++blk) {
+                    const float a0 = pm[(16 * blk + r16) * PS + kq];
+                    const float a1 = pm[(16 * blk + r16) * PS + 4 + kq];
+                    int drow[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) drow[e] = ulist[min(16 * blk + 4 * kq + e, rows_u - 1)];
+#pragma unroll
+                    for (int cb = 0; cb < C / 16; ++cb) {
+                        F32x4 d = F32x4{0.f, 0.f, 0.f, 0.f};
+                        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, xb[0][cb], d, 0, 0, 0);
+                        d = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, xb[1][cb], d, 0, 0, 0);
+                        // lane (r16, kq): members 16*blk + 4*kq .. +3 of channel 16*cb + r16
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (16 * blk + 4 * kq + e < rows_u) {
+                                unsafeAtomicAdd(out_h + (int64_t)drow[e] * C + 16 * cb + r16, d[e]);
+                            }
+                        }
+                    }
+                }
+            }
+            return;
+        }
+    }
 
     for (int h0 = 0; h0 < H; h0 += HPW) {
         const int h_raw = h0 + lane / C;

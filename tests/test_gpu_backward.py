@@ -69,6 +69,28 @@ def test_attn_backward_per_token_lists(device, lists):
     _check_attn_backward(wl.attn_case(lists, 73, B=2, H=4, N=392, C=32, lists=lists), device, torch.float32)
 
 
+@pytest.mark.parametrize("kind", ["clusters", "unaligned", "padded", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_attn_backward_lists_made_of_runs(device, kind, dtype):
+    # the scatter's union path (and its fall-back for tiles with more than 16 distinct runs: "scattered");
+    # N = 396 leaves a partial last tile, "repeated" makes a token list a run twice
+    for c, h, m in ((32, 3, 48), (64, 2, 32), (16, 5, 64)):
+        _check_attn_backward(wl.attn_case("runs", 77, B=2, H=h, N=396, C=c, M=m, lists="runs:" + kind), device, dtype)
+
+
+def test_scatter_union_path_is_bit_exact_on_integer_data(device):
+    g = torch.Generator().manual_seed(78)
+    B, H, N, C = 2, 3, 200, 32
+    idx = wl.model_like_lists(B, N, g)
+    M = idx.shape[-1]
+    q = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    k = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    d_attn = torch.randint(-4, 5, (B, H, N, M), generator=g).float()
+    dq_ref, dk_ref = oracle.qk_gather_backward(d_attn, q, k, idx)
+    dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx.to(device))
+    assert torch.equal(dq.cpu(), dq_ref) and torch.equal(dk.cpu(), dk_ref)
+
+
 @pytest.mark.parametrize("c,h,m,n", [(16, 3, 48, 104), (64, 2, 48, 100), (24, 2, 48, 64), (32, 2, 20, 77),
                                      (32, 5, 144, 160), (32, 2, 5, 40)])
 def test_attn_backward_shapes(device, c, h, m, n):
