@@ -231,6 +231,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     ops.attn_softmax = timed_call("bias+mask+blank+softmax", real.attn_softmax)
     ops.qk_clusters, ops.av_clusters = timed_call("qk", real.qk_clusters), timed_call("av", real.av_clusters)
     ops.cluster_attention = timed_call("qk+bias+mask+blank+softmax+av (one kernel)", real.cluster_attention)
+    ops.dense_attention = timed_call("global attention (one kernel)", real.dense_attention)
     ops.layer_norm = timed_call("layer_norm", real.layer_norm)
     ops.merge_weights = timed_call("merge_weights", real.merge_weights)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()

@@ -222,6 +222,27 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* Attention of every token over every token of a short sequence, fused: the branch the reference model takes in
+ * a stage whose neighbourhood size reaches its number of tokens (models/aff_transformer.py:108-113 and :125-155:
+ * `q @ key^T`, position bias, blank token, softmax, `attn @ v`, blank value), without the (B,H,N,N) logits and
+ * probabilities ever reaching memory:
+ *   logit[b,h,i,j] = scale * <query[b,h,i], key[b,h,j]> + bias_table[pe_idx[b,i,j], h]
+ *   blank[b,h,i]   = scale * <query[b,h,i], blank_key[h]>
+ *   p, p_blank     = softmax over the N tokens and the blank token
+ *   out[b,h,i]     = sum_j p[b,h,i,j] * value[b,h,j] + p_blank[b,h,i] * blank_value[h]
+ * query, key, value, out: strided (B,H,N,C) of `dtype`; bias_table (rows,H) of `dtype`, contiguous; pe_idx (B,N,N)
+ * int64 in [0,rows) — unchecked; blank_key, blank_value (H,C) fp32, contiguous.  shape.M must equal shape.N.
+ * The probabilities are rounded to `dtype` before they weigh the value rows; sums are fp32.
+ * dtype F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and N = M <= 64 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
+ * aligned (else CLUSTEN_ERR_UNALIGNED).  Inference only.  No counterpart in the reference's extension modules. */
+int clusten_dense_attention_forward(const void* query, clusten_strides query_strides,
+                                    const void* key, clusten_strides key_strides,
+                                    const void* value, clusten_strides value_strides,
+                                    const void* bias_table, const int64_t* pe_idx,
+                                    const float* blank_key, const float* blank_value,
+                                    void* out, clusten_strides out_strides, float scale,
+                                    clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* Layer normalisation over the last axis, computed in fp32 from fp32, fp16 or bf16 input and written as fp32,
  * fp16 or bf16:
  *   out[r,c] = (x[r,c] - mean_r) * rsqrt(var_r + eps) * weight[c] + bias[c]      (biased variance)

@@ -38,6 +38,8 @@ def default_ops():
                            clusters_supported=_native.clusters_supported,
                            cluster_attention=_native.cluster_attention,
                            cluster_attention_supported=_native.cluster_attention_supported,
+                           dense_attention=_native.dense_attention,
+                           dense_attention_supported=_native.dense_attention_supported,
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
                            merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported)
 
@@ -148,6 +150,14 @@ class ClusterAttention(nn.Module):
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
             out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], _linear(self.pos_embed, table),
                              lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale)
+            return self.proj_drop(_linear(self.proj, out))
+        dense = getattr(self.ops, "dense_attention", None)
+        if (global_attn and dense is not None and not torch.is_grad_enabled()
+                and not (self.training and self.attn_drop.p > 0)
+                and self.ops.dense_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3))):
+            # inference on 16-bit data, every token attending to every token: one kernel as well
+            out = dense(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, _linear(self.pos_embed, table), pe_idx,
+                        self.blank_k, self.blank_v, scale=self.scale)
             return self.proj_drop(_linear(self.proj, out))
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:

@@ -54,6 +54,8 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
+    "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
+                                                      ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
                                                  ctypes.c_float, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -491,6 +493,59 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
                                                      _ptr(out), _strides(out_view), ctypes.c_float(scale), shape, code,
                                                      _stream(device)),
                "clusten_cluster_attention_forward")
+    return out.reshape(b, n, h * c)
+
+
+def dense_attention_supported(query: torch.Tensor) -> bool:
+    """True when `dense_attention` takes this case: CUDA fp16 / bf16 queries of head dim 32, at most 64 tokens."""
+    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16) and query.dim() == 4
+            and query.shape[3] == 32 and query.shape[2] <= 64)
+
+
+def dense_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bias_table: torch.Tensor,
+                    pe_idx: torch.Tensor, blank_key: torch.Tensor, blank_value: torch.Tensor,
+                    scale: float = 1.0) -> torch.Tensor:
+    """Attention of every token over every token of a short sequence plus one blank token, in one kernel.
+
+    query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1), N <= 64; bias_table (rows,H);
+    pe_idx (B,N,N) int64; blank_key, blank_value (H*32,).  Returns softmax(scale * q.k^T + bias | scale * q.blank_key)
+    applied to the values and the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the
+    layout the output projection takes).  No autograd: for inference.  The fused form of the global branch of
+    models/aff_transformer.py:108-155.
+    """
+    lib = load()
+    _require_cuda("query", query)
+    device = query.device
+    for name, t in (("key", key), ("value", value), ("bias_table", bias_table), ("pe_idx", pe_idx),
+                    ("blank_key", blank_key), ("blank_value", blank_value)):
+        _require_cuda(name, t, device)
+    if query.dim() != 4 or key.shape != query.shape or value.shape != query.shape:
+        raise RuntimeError("query, key and value must be (B,H,N,C) tensors of one shape")
+    b, h, n, c = query.shape
+    if pe_idx.shape != (b, n, n) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,N)")
+    if bias_table.dim() != 2 or bias_table.shape[1] != h:
+        raise RuntimeError("bias_table must have shape (rows, H)")
+    if blank_key.numel() != h * c or blank_value.numel() != h * c:
+        raise RuntimeError("blank_key and blank_value must have H*C elements")
+    code = _dtype_code(query, "query")
+    dtype = query.dtype
+    query, key, value = _rows(query), _rows(key.to(dtype)), _rows(value.to(dtype))
+    bias_table = bias_table.detach().to(dtype).contiguous()
+    pe_idx = pe_idx.contiguous()
+    blank_key = blank_key.detach().reshape(h, c).float().contiguous()
+    blank_value = blank_value.detach().reshape(h, c).float().contiguous()
+    out = torch.empty(b, n, h, c, dtype=dtype, device=device)
+    if out.numel() == 0:
+        return out.reshape(b, n, h * c)
+    out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
+    shape = AttnShape(b, h, n, c, n)
+    with torch.cuda.device(device):
+        _check(lib.clusten_dense_attention_forward(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(value),
+                                                   _strides(value), _ptr(bias_table), _ptr(pe_idx), _ptr(blank_key),
+                                                   _ptr(blank_value), _ptr(out), _strides(out_view),
+                                                   ctypes.c_float(scale), shape, code, _stream(device)),
+               "clusten_dense_attention_forward")
     return out.reshape(b, n, h * c)
 
 

@@ -187,6 +187,24 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     dtype, as_stream(stream));
 }
 
+int clusten_dense_attention_forward(const void* query, clusten_strides query_strides, const void* key,
+                                    clusten_strides key_strides, const void* value, clusten_strides value_strides,
+                                    const void* bias_table, const int64_t* pe_idx, const float* blank_key,
+                                    const float* blank_value, void* out, clusten_strides out_strides, float scale,
+                                    clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!query || !key || !value || !bias_table || !pe_idx || !blank_key || !blank_value || !out) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
+        !strides_ok(out_strides, shape.C)) {
+        return CLUSTEN_ERR_BAD_STRIDE;
+    }
+    return launch_dense_attention(query, query_strides, key, key_strides, value, value_strides, bias_table, pe_idx,
+                                  blank_key, blank_value, out, out_strides, scale, shape, dtype, as_stream(stream));
+}
+
 int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream) {
     if (!x || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;

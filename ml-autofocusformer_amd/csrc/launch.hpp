@@ -66,6 +66,13 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
                              hipStream_t stream);
 
+// Attention of every token over every token (N <= 64) in one kernel: see dense_attention.hip.  q, k, v, out : strided
+//   (B,H,N,C) of T in {F16, BF16}, C = 32; table (rows,H) of T; pe_idx int64 (B,N,N); blank_k, blank_v : fp32 (H,C).
+int launch_dense_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
+                           clusten_strides vs, const void* table, const int64_t* pe_idx, const float* blank_k,
+                           const float* blank_v, void* out, clusten_strides os, float scale, clusten_attn_shape s,
+                           int dtype, hipStream_t stream);
+
 // out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C channels
 //   (C in {64,128,256,384,512,768,1024}); x and out of dtype F32, F16 or BF16 each, arithmetic in fp32.
 int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,

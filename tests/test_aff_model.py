@@ -320,13 +320,16 @@ def test_operator_dtypes_under_autocast(device):
 @pytest.mark.gpu
 def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device):
     """The configuration the images/s figure is quoted on: every operator call of AFF-Tiny at 224x224 under fp16
-    autocast (local attention in one kernel on cluster-number lists, kNN kernel on the HIP side; tensor expressions
+    autocast (local and global attention in one kernel each, kNN kernel on the HIP side; tensor expressions
     on the other)."""
     from aff.model import default_ops
     ops = default_ops()
     calls = []
     one_kernel = ops.cluster_attention
     ops.cluster_attention = lambda *a, **kw: (calls.append(a[0].dtype), one_kernel(*a, **kw))[1]
+    dense_calls = []
+    dense_kernel = ops.dense_attention
+    ops.dense_attention = lambda *a, **kw: (dense_calls.append(a[0].shape[2]), dense_kernel(*a, **kw))[1]
     torch.manual_seed(0)
     hip = aff_tiny(ops=ops).to(device).eval()
     torch.manual_seed(0)
@@ -339,9 +342,12 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     assert oracle.rel_err(y_hip.float(), y_ref.float()) < 2e-2
     # the 25 blocks of the three local-attention stages took the one-kernel path, on fp16 operands
     assert calls == [torch.float16] * 25
+    # and the 5 blocks of the last stage (49 tokens, each attending to all) the dense one
+    assert dense_calls == [49] * 5
     # the same model with the three operators and the softmax kernel between them
     three = default_ops()
     del three.cluster_attention
+    del three.dense_attention
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
