@@ -243,6 +243,21 @@ int clusten_dense_attention_forward(const void* query, clusten_strides query_str
                                     void* out, clusten_strides out_strides, float scale,
                                     clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* A Linear layer on a tall 16-bit activation matrix and a small weight matrix, optionally followed by GELU:
+ *   out[m,n] = act( sum_k x[m,k] * weight[n,k] + bias[n] ),  act = identity (0) or the exact (erf) GELU (1)
+ * what `nn.Linear` (and `nn.GELU` after the first MLP layer) compute around the first-stage attention of the
+ * reference model (models/aff_transformer.py:60-68 q / kv / proj, :181-196 the MLP), where K and Nout are 64 to
+ * 192 and the layer is bound by reading x and writing out once.  x (rows,K) of `dtype` with row stride
+ * x_row_stride elements (a multiple of 8), weight (Nout,K) and bias (Nout, or NULL) of `dtype`, contiguous;
+ * out (rows,Nout) of `dtype`, contiguous; all 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).  Sums are fp32; with
+ * GELU the sum is rounded to `dtype` before the activation, as a separate activation kernel would see it.
+ * dtype F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE); (K,Nout,act) must be one of the combinations
+ * clusten_linear_supported accepts — (64,64|128|192,0|1), (128,64,0), (192,64,0) — else CLUSTEN_ERR_BAD_DIMS.
+ * Inference only.  No counterpart in the reference's extension modules. */
+int clusten_linear_supported(int K, int Nout, int act);
+int clusten_linear_forward(const void* x, int64_t x_row_stride, const void* weight, const void* bias, void* out,
+                           int64_t rows, int K, int Nout, int act, int dtype, clusten_stream stream);
+
 /* Layer normalisation over the last axis, computed in fp32 from fp32, fp16 or bf16 input and written as fp32,
  * fp16 or bf16:
  *   out[r,c] = (x[r,c] - mean_r) * rsqrt(var_r + eps) * weight[c] + bias[c]      (biased variance)

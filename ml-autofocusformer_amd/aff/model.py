@@ -41,14 +41,18 @@ def default_ops():
                            dense_attention=_native.dense_attention,
                            dense_attention_supported=_native.dense_attention_supported,
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
+                           linear=_native.linear, linear_supported=_native.linear_supported,
                            merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported)
 
 
-def _linear(lin, x):
-    """`lin(x)` for an nn.Linear.  In inference under mixed precision the 16-bit copies of weight and bias are kept
-    between calls (autocast makes them anew in every forward); they are remade when the parameters change."""
+def _linear(lin, x, ops=None, gelu=False):
+    """`lin(x)` for an nn.Linear, followed by the exact GELU when `gelu`.  In inference under mixed precision the
+    16-bit copies of weight and bias are kept between calls (autocast makes them anew in every forward; they are
+    remade when the parameters change), and the small layers on many rows go through the library's kernel when
+    `ops` has it."""
     if torch.is_grad_enabled() or not x.is_cuda or not torch.is_autocast_enabled("cuda"):
-        return lin(x)
+        y = lin(x)
+        return F.gelu(y) if gelu else y
     dt = torch.get_autocast_dtype("cuda")
     key = (dt, lin.weight._version, lin.weight.data_ptr(),
            None if lin.bias is None else (lin.bias._version, lin.bias.data_ptr()))
@@ -56,7 +60,12 @@ def _linear(lin, x):
     if cache is None or cache[0] != key:
         cache = (key, lin.weight.detach().to(dt), None if lin.bias is None else lin.bias.detach().to(dt))
         lin.__dict__["_cast_cache"] = cache      # a plain attribute: no parameter, no buffer, not in the state_dict
-    return F.linear(x if x.dtype == dt else x.to(dt), cache[1], cache[2])
+    x = x if x.dtype == dt else x.to(dt)
+    fn = getattr(ops, "linear", None)
+    if fn is not None and ops.linear_supported(x, cache[1], gelu):
+        return fn(x, cache[1], cache[2], gelu)
+    y = F.linear(x, cache[1], cache[2])
+    return F.gelu(y) if gelu else y
 
 
 def _layer_norm(norm, x, ops, feeds_linear=False):
@@ -102,15 +111,17 @@ class DropPath(nn.Module):
 
 
 class Mlp(nn.Module):
-    def __init__(self, dim, hidden, drop=0.0):
+    def __init__(self, dim, hidden, drop=0.0, ops=None):
         super().__init__()
         self.fc1 = nn.Linear(dim, hidden)
         self.act = nn.GELU()
         self.fc2 = nn.Linear(hidden, dim)
         self.drop = nn.Dropout(drop)
+        self.ops = ops
 
     def forward(self, x):
-        return self.drop(_linear(self.fc2, self.drop(self.act(_linear(self.fc1, x)))))
+        hidden = _linear(self.fc1, x, self.ops, gelu=True)        # self.act is the exact GELU
+        return self.drop(_linear(self.fc2, self.drop(hidden), self.ops))
 
 
 class ClusterAttention(nn.Module):
@@ -139,8 +150,8 @@ class ClusterAttention(nn.Module):
         # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
         compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
                    and getattr(self.ops, "qk_clusters", None) is not None)
-        q = _linear(self.q, feat)
-        kv = _linear(self.kv, feat).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
+        q = _linear(self.q, feat, self.ops)
+        kv = _linear(self.kv, feat, self.ops).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
         one_kernel = getattr(self.ops, "cluster_attention", None)
         if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
@@ -150,7 +161,7 @@ class ClusterAttention(nn.Module):
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
             out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], _linear(self.pos_embed, table),
                              lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale)
-            return self.proj_drop(_linear(self.proj, out))
+            return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
         if (global_attn and dense is not None and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0)
@@ -158,7 +169,7 @@ class ClusterAttention(nn.Module):
             # inference on 16-bit data, every token attending to every token: one kernel as well
             out = dense(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, _linear(self.pos_embed, table), pe_idx,
                         self.blank_k, self.blank_v, scale=self.scale)
-            return self.proj_drop(_linear(self.proj, out))
+            return self.proj_drop(_linear(self.proj, out, self.ops))
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:
             attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
@@ -191,7 +202,7 @@ class ClusterAttention(nn.Module):
             out = self.ops.av(attn, v, member_idx)                                       # (b,h,n,ch)
         out = out + blank * self.blank_v.reshape(1, h, 1, ch)
         out = out.permute(0, 2, 1, 3).reshape(b, n, c)
-        return self.proj_drop(_linear(self.proj, out))
+        return self.proj_drop(_linear(self.proj, out, self.ops))
 
 
 class ClusterTransformerBlock(nn.Module):
@@ -202,7 +213,7 @@ class ClusterTransformerBlock(nn.Module):
         self.attn = ClusterAttention(dim, num_heads, attn_drop=attn_drop, proj_drop=drop, ops=ops)
         self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
         self.norm2 = nn.LayerNorm(dim)
-        self.mlp = Mlp(dim, int(dim * mlp_ratio), drop=drop)
+        self.mlp = Mlp(dim, int(dim * mlp_ratio), drop=drop, ops=ops)
         self.layer_scale = isinstance(layer_scale, (int, float)) and layer_scale > 0
         if self.layer_scale:
             self.gamma1 = nn.Parameter(layer_scale * torch.ones(dim))
@@ -275,7 +286,7 @@ class ClusterMerging(nn.Module):
             if cluster_mask is not None:
                 weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
         merged = self.ops.wf(weights, feat, member_idx).reshape(b, n_out, -1)            # channel = ic * c + c'
-        return pos, _linear(self.linear, _layer_norm(self.norm, merged, self.ops, True))
+        return pos, _linear(self.linear, _layer_norm(self.norm, merged, self.ops, True), self.ops)
 
 
 class BasicLayer(nn.Module):
@@ -461,3 +472,48 @@ def aff_tiny(**kw):
                cluster_size=8, nbhd_size=(48, 48, 48, 49), alpha=4.0, ds_rate=0.25, drop_path_rate=0.2)
     cfg.update(kw)
     return AutoFocusFormer(**cfg)
+
+
+class CapturedForward:
+    """One inference forward of `net` at a fixed input shape, recorded into a HIP graph and replayed.
+
+    A forward of the classifier is some 800 kernel launches of 5-100 us each; issued one by one from Python they
+    take as long on the host as on the GPU.  Replaying the recorded graph leaves one launch per forward.  The
+    model's forward has no host synchronisation and every kernel of the library takes the current stream and
+    allocates through the framework, so the recording is the plain forward under `torch.cuda.graph`.
+
+    Replays read the parameters in place (their 16-bit copies are part of the recording: record again after the
+    weights change) and return the same output tensor every time: copy it before the next call if it must outlive
+    it.  `autocast_dtype=None` records without mixed precision.
+    """
+
+    def __init__(self, net, example, autocast_dtype=torch.float16, warmup=3):
+        if not example.is_cuda:
+            raise RuntimeError("CapturedForward records GPU work: the example input must be a CUDA tensor")
+        self.net = net
+        self.autocast_dtype = autocast_dtype
+        self.static_in = example.clone()
+        side = torch.cuda.Stream(device=example.device)
+        side.wait_stream(torch.cuda.current_stream(example.device))
+        with torch.cuda.stream(side):        # library handles, kernel selection and caches settle outside the recording
+            for _ in range(warmup):
+                self._forward()
+        torch.cuda.current_stream(example.device).wait_stream(side)
+        torch.cuda.synchronize(example.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.static_out = self._forward()
+
+    def _forward(self):
+        with torch.no_grad(), torch.autocast("cuda", dtype=self.autocast_dtype or torch.float16,
+                                            enabled=self.autocast_dtype is not None):
+            return self.net(self.static_in)
+
+    def __call__(self, x):
+        if x.shape != self.static_in.shape or x.dtype != self.static_in.dtype:
+            raise RuntimeError("CapturedForward was recorded for inputs of shape %s and dtype %s"
+                               % (tuple(self.static_in.shape), self.static_in.dtype))
+        if x.data_ptr() != self.static_in.data_ptr():
+            self.static_in.copy_(x)
+        self.graph.replay()
+        return self.static_out

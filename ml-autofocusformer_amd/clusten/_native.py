@@ -56,6 +56,9 @@ _PROTOTYPES = {
                                                         ctypes.c_int, _P]),
     "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
                                                       ctypes.c_float, AttnShape, ctypes.c_int, _P]),
+    "clusten_linear_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "clusten_linear_forward": (ctypes.c_int, [_P, ctypes.c_int64, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                             ctypes.c_int, ctypes.c_int, _P]),
     "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
                                                  ctypes.c_float, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -547,6 +550,57 @@ def dense_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                                    ctypes.c_float(scale), shape, code, _stream(device)),
                "clusten_dense_attention_forward")
     return out.reshape(b, n, h * c)
+
+
+_LINEAR_SHAPES = {(64, 64, 0), (64, 128, 0), (64, 192, 0), (128, 64, 0), (192, 64, 0),
+                  (64, 64, 1), (64, 128, 1), (64, 192, 1)}                   # (K, Nout, gelu)
+_LINEAR_MIN_ROWS = 65536
+
+
+def linear_supported(x: torch.Tensor, weight: torch.Tensor, gelu: bool = False) -> bool:
+    """True when `linear` takes this case: a CUDA fp16 / bf16 activation of many rows (the kernel is built for
+    layers that move memory: at least 65536 rows) whose last axis is contiguous and a weight of one of the small
+    shapes it is compiled for."""
+    if not (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and weight.dim() == 2 and x.dim() >= 2):
+        return False
+    nout, k = weight.shape
+    if x.shape[-1] != k or (k, nout, int(gelu)) not in _LINEAR_SHAPES:
+        return False
+    return x.numel() // k >= _LINEAR_MIN_ROWS and x.is_contiguous()
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias, gelu: bool = False) -> torch.Tensor:
+    """`gelu(x @ weight.T + bias)` (or without the GELU) for x (..., K) and weight (Nout, K) of one 16-bit dtype,
+    bias (Nout,) of that dtype or None: `nn.Linear` (+ `nn.GELU`) of models/aff_transformer.py:60-68, 181-196 for
+    the small layers of the first stage.  No autograd: for inference."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    _require_cuda("weight", weight, device)
+    if weight.dim() != 2 or x.dim() < 2 or x.shape[-1] != weight.shape[1]:
+        raise RuntimeError("x must be (..., K) and weight (Nout, K)")
+    if weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise RuntimeError("x, weight and bias must have one dtype")
+    nout, k = weight.shape
+    code = _dtype_code(x, "x")
+    if x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        x2 = x                                       # rows of a wider matrix: read in place
+    else:
+        x2 = x.contiguous().view(-1, k)
+    weight = weight.detach().contiguous()
+    if bias is not None:
+        _require_cuda("bias", bias, device)
+        bias = bias.detach().contiguous()
+        if bias.numel() != nout:
+            raise RuntimeError("bias must have Nout elements")
+    out = torch.empty(x.shape[:-1] + (nout,), dtype=x.dtype, device=device)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(device):
+        _check(lib.clusten_linear_forward(_ptr(x2), x2.stride(0), _ptr(weight), _ptr(bias), _ptr(out), x2.shape[0], k,
+                                          nout, int(bool(gelu)), code, _stream(device)),
+               "clusten_linear_forward")
+    return out
 
 
 _LAYER_NORM_WIDTHS = (64, 128, 256, 384, 512, 768, 1024)

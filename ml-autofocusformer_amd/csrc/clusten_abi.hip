@@ -205,6 +205,18 @@ int clusten_dense_attention_forward(const void* query, clusten_strides query_str
                                   blank_key, blank_value, out, out_strides, scale, shape, dtype, as_stream(stream));
 }
 
+int clusten_linear_supported(int K, int Nout, int act) { return skinny_linear_supported(K, Nout, act) ? 1 : 0; }
+
+int clusten_linear_forward(const void* x, int64_t x_row_stride, const void* weight, const void* bias, void* out,
+                           int64_t rows, int K, int Nout, int act, int dtype, clusten_stream stream) {
+    if (!x || !weight || !out) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || !skinny_linear_supported(K, Nout, act)) return CLUSTEN_ERR_BAD_DIMS;
+    if (x_row_stride < K || 16 * x_row_stride * 2 >= ((int64_t)1 << 32)) return CLUSTEN_ERR_BAD_STRIDE;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || (x_row_stride & 7) != 0) return CLUSTEN_ERR_UNALIGNED;
+    return launch_skinny_linear(x, x_row_stride, weight, bias, out, rows, K, Nout, act, dtype, as_stream(stream));
+}
+
 int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream) {
     if (!x || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;

@@ -73,6 +73,12 @@ int launch_dense_attention(const void* q, clusten_strides qs, const void* k, clu
                            const float* blank_v, void* out, clusten_strides os, float scale, clusten_attn_shape s,
                            int dtype, hipStream_t stream);
 
+// y = act(x W^T + b) for tall x and small W (see skinny_linear.hip): x (M,K) of T with row stride ldx elements,
+//   w (NOUT,K), bias (NOUT) or null, y (M,NOUT), all of T in {F16, BF16}; act 0 = identity, 1 = exact GELU.
+bool skinny_linear_supported(int K, int NOUT, int act);
+int launch_skinny_linear(const void* x, int64_t ldx, const void* w, const void* bias, void* y, int64_t M, int K, int NOUT,
+                         int act, int dtype, hipStream_t stream);
+
 // out[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * weight + bias for `rows` rows of C channels
 //   (C in {64,128,256,384,512,768,1024}); x and out of dtype F32, F16 or BF16 each, arithmetic in fp32.
 int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,

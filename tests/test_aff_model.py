@@ -327,6 +327,9 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     calls = []
     one_kernel = ops.cluster_attention
     ops.cluster_attention = lambda *a, **kw: (calls.append(a[0].dtype), one_kernel(*a, **kw))[1]
+    linear_calls = []
+    linear_kernel = ops.linear
+    ops.linear = lambda *a, **kw: (linear_calls.append(tuple(a[1].shape)), linear_kernel(*a, **kw))[1]
     dense_calls = []
     dense_kernel = ops.dense_attention
     ops.dense_attention = lambda *a, **kw: (dense_calls.append(a[0].shape[2]), dense_kernel(*a, **kw))[1]
@@ -344,15 +347,71 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     assert calls == [torch.float16] * 25
     # and the 5 blocks of the last stage (49 tokens, each attending to all) the dense one
     assert dense_calls == [49] * 5
+    # the Linear layers keep the framework's kernels at this batch size (the library's takes 65536 rows and more)
+    assert linear_calls == []
     # the same model with the three operators and the softmax kernel between them
     three = default_ops()
     del three.cluster_attention
     del three.dense_attention
+    del three.linear
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
         y3 = hip3(x)
     assert oracle.rel_err(y_hip.float(), y3.float()) < 2e-2
+
+
+@pytest.mark.gpu
+def test_aff_tiny_224_small_linear_layers_through_the_library(device):
+    """From 21 images on, the first stage has 65536 rows and more: its q / kv / proj / MLP layers take the library's
+    Linear kernel; the logits agree with the framework's GEMMs."""
+    from aff.model import default_ops
+    ops = default_ops()
+    shapes = []
+    kernel = ops.linear
+    ops.linear = lambda *a, **kw: (shapes.append((tuple(a[1].shape), bool(a[3]) if len(a) > 3 else False)),
+                                   kernel(*a, **kw))[1]
+    torch.manual_seed(0)
+    hip = aff_tiny(ops=ops).to(device).eval()
+    plain = default_ops()
+    del plain.linear
+    ref = aff_tiny(ops=plain).to(device).eval()
+    ref.load_state_dict(hip.state_dict())
+    x = torch.randn(24, 3, 224, 224, generator=torch.Generator().manual_seed(4)).to(device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        y_hip, y_ref = hip(x), ref(x)
+    assert torch.isfinite(y_hip).all()
+    assert oracle.rel_err(y_hip.float(), y_ref.float()) < 1e-2
+    per_block = [((64, 64), False), ((128, 64), False), ((64, 64), False), ((192, 64), True), ((64, 192), False)]
+    assert shapes == per_block * 3        # the merge projection works on a quarter of the rows: below the threshold
+
+
+@pytest.mark.gpu
+def test_recorded_forward_replays_equal_the_eager_forward(device):
+    """The forward recorded into a HIP graph: every replay, with eager forwards and synchronisations between
+    them, gives the eager result bit for bit (the kernels are deterministic and the recording holds no memset)."""
+    from aff.model import CapturedForward
+    torch.manual_seed(0)
+    net = aff_tiny().to(device).eval()
+    gen = torch.Generator().manual_seed(5)
+    xs = [torch.randn(2, 3, 224, 224, generator=gen).to(device) for _ in range(3)]
+
+    def eager(x):
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+            return net(x)
+
+    want = [eager(x).clone() for x in xs]
+    recorded = CapturedForward(net, xs[0])
+    for rep in range(3):
+        for i, x in enumerate(xs):
+            got = recorded(x).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want[i]), "replay %d of input %d" % (rep, i)
+            assert torch.equal(eager(xs[(i + 1) % 3]), want[(i + 1) % 3])
+    with pytest.raises(RuntimeError):
+        recorded(xs[0][:1])
+    with pytest.raises(RuntimeError):
+        CapturedForward(net, xs[0].cpu())
 
 
 @pytest.mark.gpu
