@@ -214,6 +214,7 @@ int clusten_linear_forward(const void* x, int64_t x_row_stride, const void* weig
     if (rows <= 0 || !skinny_linear_supported(K, Nout, act)) return CLUSTEN_ERR_BAD_DIMS;
     if (x_row_stride < K || 16 * x_row_stride * 2 >= ((int64_t)1 << 32)) return CLUSTEN_ERR_BAD_STRIDE;
     if (!aligned16(x) || !aligned16(weight) || !aligned16(out) || (x_row_stride & 7) != 0) return CLUSTEN_ERR_UNALIGNED;
+    if (bias && !aligned16(bias)) return CLUSTEN_ERR_UNALIGNED;
     return launch_skinny_linear(x, x_row_stride, weight, bias, out, rows, K, Nout, act, dtype, as_stream(stream));
 }
 

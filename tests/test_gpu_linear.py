@@ -62,6 +62,34 @@ def test_without_bias_batched_shape_and_row_stride(device):
     assert torch.equal(out.cpu().float(), F.linear(xi.float(), wi.float(), bi.float()))
 
 
+def test_gelu_epilogue_on_every_fp16_value(device):
+    """y = GELU(x I^T): every finite fp16 value through the activation of the epilogue, against the exactly rounded
+    GELU (float64 erfc).  The epilogue approximates erfc to a relative bound, so it stays within one fp16 ulp
+    everywhere, the negative tail included."""
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    vals = bits.view(torch.float16)
+    vals = vals[torch.isfinite(vals)]
+    assert vals.numel() == 63488
+    x = vals.repeat(67)[:65536 * 64].reshape(65536, 64).contiguous()
+    eye = torch.eye(64, dtype=torch.float16)
+    out = _native.linear(x.to(device), eye.to(device), None, True).cpu()
+    x64 = x.double()
+    exact = (x64 * 0.5 * torch.special.erfc(-x64 * 2 ** -0.5)).half()
+
+    def ordered(t):      # fp16 bit patterns as integers that order like the values
+        i = t.view(torch.int16).int()
+        return torch.where(i < 0, -32768 - i, i)
+
+    ulps = (ordered(out) - ordered(exact)).abs()
+    assert int(ulps.max()) <= 1
+    assert int((ulps > 0).sum()) <= 2e-3 * ulps.numel()
+    # and next to the framework's kernel (0.5 x (1 + erf(x / sqrt 2)) in fp32, which cancels in the negative tail)
+    theirs = F.gelu(x.to(device)).cpu()
+    apart = (ordered(out) - ordered(theirs)).abs()
+    assert int(apart.max()) <= 8 and int(apart[x >= -2].max()) <= 1
+    assert (out.float() - theirs.float())[x < -2].abs().max() <= 4e-6      # one ulp of values below 2^-7
+
+
 def test_unsupported_cases_are_refused(device):
     x = torch.zeros(70000, 64, dtype=torch.float16, device=device)
     w = torch.zeros(64, 64, dtype=torch.float16, device=device)
