@@ -202,7 +202,7 @@ def _bench_wf(case, steps, warmup):
             "input_sets_rotated": copies}
 
 
-def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
+def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
     """Images/s of the AFF-Tiny classifier at 224x224 (random weights, N(0,1) images, fp16 autocast, eval mode, no_grad),
     timed like the reference's `throughput` (main.py:343-354: 50 untimed and 30 timed forwards), and the share
     of one forward spent in each operator, measured in a separate pass with stream events around the calls."""
@@ -255,7 +255,31 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
 
-    # the same forward recorded into a HIP graph and replayed (the input copy into the recording's buffer included)
+    # the same forward recorded into a HIP graph and replayed (the input copy into the recording's buffer included);
+    # before the recording PyTorch's TunableOp picks, per Linear shape, the fastest of the GEMM solutions rocBLAS and
+    # hipBLASLt offer (a few seconds, results kept only for this process; the logits are checked against the
+    # untuned forward)
+    gemm_tuning = "library defaults"
+    try:
+        if not tune_gemms:
+            raise RuntimeError("switched off")
+        import tempfile
+        import torch.cuda.tunable as tunable
+        want = forward().float()
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), "clusten_bench_tunableop.csv"))
+        tunable.enable(True)
+        tunable.tuning_enable(True)
+        forward()
+        torch.cuda.synchronize()
+        tunable.tuning_enable(False)
+        got = forward().float()
+        if float((got - want).abs().max()) <= 1e-2 * float(want.abs().max()):
+            gemm_tuning = "PyTorch TunableOp, tuned in this process before the recording"
+        else:
+            tunable.enable(False)
+    except Exception as exc:  # noqa: BLE001 - an optional speed-up: report and go on without it
+        if tune_gemms:
+            gemm_tuning = "library defaults (TunableOp unavailable: %s)" % type(exc).__name__
     recorded = aff_model.CapturedForward(net, x)
     x2 = torch.randn_like(x)
     for _ in range(warmup):
@@ -267,6 +291,10 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     torch.cuda.synchronize()
     dt_graph = time.perf_counter() - t0
     del recorded
+    try:
+        tunable.enable(False)
+    except Exception:  # noqa: BLE001
+        pass
 
     spans["on"] = True
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -279,6 +307,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30):
     share["everything_else"] = round(1.0 - sum(share.values()), 4)
     return {"img_per_s": round(timed * batch / dt_graph, 1), "ms_per_batch": round(dt_graph / timed * 1e3, 2),
             "launch": "one HIP graph replay per forward (aff.model.CapturedForward)",
+            "gemm_selection": gemm_tuning,
             "eager_img_per_s": round(timed * batch / dt, 1), "eager_ms_per_batch": round(dt / timed * 1e3, 2),
             "batch": batch, "warmup": warmup, "timed": timed,
             "dtype": "fp16 autocast (attention: one fp16 kernel per layer, fp32 sums; WF fp32)",
@@ -297,6 +326,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-e2e", action="store_true", help="skip the AFF-Tiny images/s leg")
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd"), default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
@@ -313,7 +344,7 @@ def main():
     _native.load()
     torch.cuda.set_device(0)
     if args.e2e_only:
-        print(json.dumps({"aff_tiny_224": _aff_tiny_throughput()}), flush=True)
+        print(json.dumps({"aff_tiny_224": _aff_tiny_throughput(tune_gemms=not args.no_gemm_tuning)}), flush=True)
         return
 
     B = 128
@@ -429,7 +460,7 @@ def main():
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:
-        out["aff_tiny_224"] = _aff_tiny_throughput()
+        out["aff_tiny_224"] = _aff_tiny_throughput(tune_gemms=not args.no_gemm_tuning)
     if not args.no_cpu:
         out["cpu_baseline"] = _cpu_baseline(acase, wcase, total_bytes, B)
     print(json.dumps(out), flush=True)
