@@ -233,6 +233,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
     ops.cluster_attention = timed_call("qk+bias+mask+blank+softmax+av (one kernel)", real.cluster_attention)
     ops.dense_attention = timed_call("global attention (one kernel)", real.dense_attention)
     ops.layer_norm = timed_call("layer_norm", real.layer_norm)
+    ops.add_layer_norm = timed_call("layer_norm", real.add_layer_norm)
     ops.linear = timed_call("small Linear layers (+GELU) of stage 1", real.linear)
     ops.merge_weights = timed_call("merge_weights", real.merge_weights)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()

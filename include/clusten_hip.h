@@ -272,6 +272,18 @@ int clusten_linear_forward(const void* x, int64_t x_row_stride, const void* weig
 int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream);
 
+/* The residual addition ahead of a layer normalisation, and the normalisation, in one pass:
+ *   sum_out[r,c] = x[r,c] + branch[r,c]   (rounded to x's type, as the framework's addition leaves it)
+ *   out[r,c]     = layer norm of sum_out[r,:] as clusten_layer_norm_forward computes it, written in branch's type
+ * i.e. `feat = shortcut + attn_out; self.norm2(feat)` (models/aff_transformer.py:230-231) and
+ * `feat = feat + mlp_out` followed by the next block's `self.norm1(feat)` (:232, :219) in inference under mixed
+ * precision.  branch and out (rows,C) of branch_dtype, F16 or BF16; x and sum_out (rows,C) of x_dtype, F32 or
+ * branch_dtype (else CLUSTEN_ERR_BAD_DTYPE); sum_out may be x itself; weight, bias (C) fp32; everything contiguous
+ * and 16-byte aligned; C as for clusten_layer_norm_forward.  No counterpart in the reference's extension modules. */
+int clusten_add_layer_norm_forward(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
+                                   const float* weight, const float* bias, void* out, int64_t rows, int C,
+                                   float eps, clusten_stream stream);
+
 /* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
  * (models/aff_transformer.py:340-358), in one pass instead of a row lookup, a gather and two multiplications:
  *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]

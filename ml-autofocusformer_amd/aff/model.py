@@ -42,6 +42,7 @@ def default_ops():
                            dense_attention_supported=_native.dense_attention_supported,
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
                            linear=_native.linear, linear_supported=_native.linear_supported,
+                           add_layer_norm=_native.add_layer_norm, add_layer_norm_supported=_native.add_layer_norm_supported,
                            merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported)
 
 
@@ -78,6 +79,20 @@ def _layer_norm(norm, x, ops, feeds_linear=False):
         return norm(x)
     out_dtype = torch.get_autocast_dtype("cuda") if (feeds_linear and torch.is_autocast_enabled("cuda")) else None
     return fn(x, norm.weight, norm.bias, norm.eps, out_dtype)
+
+
+def _add_layer_norm(norm, x, branch, ops):
+    """(x + branch, norm(x + branch)) — just (x, norm(x)) when `branch` is None — with the norm's output feeding
+    Linear layers only.  In inference under mixed precision addition and norm are one pass of the library's kernel
+    when `ops` has it."""
+    if branch is None:
+        return x, _layer_norm(norm, x, ops, True)
+    fn = getattr(ops, "add_layer_norm", None)
+    if (fn is not None and not torch.is_grad_enabled() and torch.is_autocast_enabled("cuda")
+            and branch.dtype == torch.get_autocast_dtype("cuda") and ops.add_layer_norm_supported(x, branch)):
+        return fn(x, branch, norm.weight, norm.bias, norm.eps)
+    x = x + branch
+    return x, _layer_norm(norm, x, ops, True)
 
 
 def relative_position_table(img_size):
@@ -219,13 +234,16 @@ class ClusterTransformerBlock(nn.Module):
             self.gamma1 = nn.Parameter(layer_scale * torch.ones(dim))
             self.gamma2 = nn.Parameter(layer_scale * torch.ones(dim))
 
-    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None, grid_lists=None):
+    def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None, grid_lists=None,
+                carry=None):
+        """Returns (feat, branch): the block's output is feat + branch.  The addition is left to the caller, which
+        hands `branch` to the next block as `carry` so that it can ride along with that block's first norm."""
         ops = self.attn.ops
-        a = self.attn(_layer_norm(self.norm1, feat, ops, True), member_idx, cluster_mask, pe_idx, global_attn, table,
-                      cluster_idx, grid_lists)
-        feat = feat + self.drop_path(self.gamma1 * a if self.layer_scale else a)
-        f = self.mlp(_layer_norm(self.norm2, feat, ops, True))
-        return feat + self.drop_path(self.gamma2 * f if self.layer_scale else f)
+        feat, x = _add_layer_norm(self.norm1, feat, carry, ops)
+        a = self.attn(x, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx, grid_lists)
+        feat, x = _add_layer_norm(self.norm2, feat, self.drop_path(self.gamma1 * a if self.layer_scale else a), ops)
+        f = self.mlp(x)
+        return feat, self.drop_path(self.gamma2 * f if self.layer_scale else f)
 
 
 class ClusterMerging(nn.Module):
@@ -378,8 +396,11 @@ class BasicLayer(nn.Module):
                 if ranking is not None:
                     feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
 
+        carry = None
         for blk in self.blocks:
-            feat = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists)
+            feat, carry = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists, carry)
+        if carry is not None:
+            feat = feat + carry
 
         if self.downsample is not None:
             if global_attn:   # merging after a dense stage: every token is every token's neighbour

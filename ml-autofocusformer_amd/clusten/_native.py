@@ -61,6 +61,8 @@ _PROTOTYPES = {
                                              ctypes.c_int, ctypes.c_int, _P]),
     "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
                                                  ctypes.c_float, ctypes.c_int, _P]),
+    "clusten_add_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, _P, ctypes.c_int64,
+                                                     ctypes.c_int, ctypes.c_float, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                     ctypes.c_int, ctypes.c_int, _P]),
     "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
@@ -641,6 +643,45 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
                                               ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
                "clusten_layer_norm_forward")
     return out
+
+
+def add_layer_norm_supported(x: torch.Tensor, branch: torch.Tensor) -> bool:
+    """True when `add_layer_norm` takes this case: CUDA tensors of one shape, the branch fp16 / bf16, x fp32 or of
+    the branch's type, the last axis of one of the built widths."""
+    return (x.is_cuda and branch.is_cuda and branch.dtype in (torch.float16, torch.bfloat16)
+            and x.dtype in (torch.float32, branch.dtype) and x.shape == branch.shape and x.dim() >= 1
+            and x.shape[-1] in _LAYER_NORM_WIDTHS)
+
+
+def add_layer_norm(x: torch.Tensor, branch: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5):
+    """(x + branch, F.layer_norm((x + branch).float(), (C,), weight, bias, eps).to(branch.dtype)) in one pass: the
+    residual addition ahead of a norm and the norm (models/aff_transformer.py:230-232, :219).  The sum has x's dtype
+    (fp32, or the branch's 16-bit type) and is rounded before it is normalised, like the separate addition's.
+    No autograd: for inference."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    for name, t in (("branch", branch), ("weight", weight), ("bias", bias)):
+        _require_cuda(name, t, device)
+    if not add_layer_norm_supported(x, branch):
+        raise RuntimeError("add_layer_norm: x fp32 or of the branch's type, branch fp16 / bf16, equal shapes, a built width")
+    c = x.shape[-1]
+    if weight.numel() != c or bias.numel() != c:
+        raise RuntimeError("weight and bias must have as many elements as the last axis of x")
+    x = x.detach().contiguous()
+    branch = branch.detach().contiguous()
+    weight = weight.detach().float().contiguous()
+    bias = bias.detach().float().contiguous()
+    total = torch.empty_like(x)
+    out = torch.empty(x.shape, dtype=branch.dtype, device=device)
+    if out.numel() == 0:
+        return total, out
+    with torch.cuda.device(device):
+        _check(lib.clusten_add_layer_norm_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(branch), _DTYPE_CODES[branch.dtype],
+                                                  _ptr(total), _ptr(weight), _ptr(bias), _ptr(out), x.numel() // c, c,
+                                                  ctypes.c_float(eps), _stream(device)),
+               "clusten_add_layer_norm_forward")
+    return total, out
 
 
 def merge_weights_supported(table_weights: torch.Tensor) -> bool:

@@ -228,6 +228,21 @@ int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight,
     return launch_layer_norm(x, in_dtype, weight, bias, out, rows, C, eps, out_dtype, as_stream(stream));
 }
 
+int clusten_add_layer_norm_forward(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
+                                   const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                                   clusten_stream stream) {
+    if (!x || !branch || !sum_out || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;
+    if (branch_dtype != CLUSTEN_F16 && branch_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (x_dtype != CLUSTEN_F32 && x_dtype != branch_dtype) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || C <= 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(branch) || !aligned16(sum_out) || !aligned16(weight) || !aligned16(bias) ||
+        !aligned16(out)) {
+        return CLUSTEN_ERR_UNALIGNED;
+    }
+    return launch_add_layer_norm(x, x_dtype, branch, branch_dtype, sum_out, weight, bias, out, rows, C, eps,
+                                 as_stream(stream));
+}
+
 int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
                                   const float* prob, const int64_t* mask, float* weights, int B, int N, int Nout, int M,
                                   int IC, clusten_stream stream) {

@@ -84,6 +84,11 @@ int launch_skinny_linear(const void* x, int64_t ldx, const void* w, const void* 
 int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,
                       float eps, int out_dtype, hipStream_t stream);
 
+// sum_out = x + branch (x's type), out = layer norm of sum_out (branch's 16-bit type); x of F32 or branch's type.
+int launch_add_layer_norm(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
+                          const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                          hipStream_t stream);
+
 // w[b,i,j,:4] = table_w[pe_idx[b,i,j], :4] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]   (prob, mask may be null)
 //   table_w (rows,4), prob (B,N), w (B,Nout,M,4): fp32;  pe_idx, nbhd_idx, mask: int64 (B,Nout,M).
 int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,

@@ -5,13 +5,18 @@
 // projection and at the end (`nn.LayerNorm`, models/aff_transformer.py:220, 231, 362, 546, 663); under mixed
 // precision the normalisation runs in fp32 (a 16-bit input is widened first) and the Linear layer that follows
 // rounds its input to 16 bits.  This kernel does all of that in one pass over the rows (64 to 1024 channels: a row
-// is a few hundred bytes, which the framework's general kernel handles at a fraction of the memory bandwidth).  It
-// has no counterpart in the reference's extension modules.
+// is a few hundred bytes, which the framework's general kernel handles at a fraction of the memory bandwidth).  A
+// second form takes the residual addition ahead of the norm along (`x = x + drop_path(branch)` followed by
+// `norm(x)`: models/aff_transformer.py:230-231, and :232 with the next block's :219): it writes the sum, rounded as the
+// framework's addition leaves it, and the normalised row in one pass.  Neither has a counterpart in the
+// reference's extension modules.
 //
 // A row is held by L = min(64, C / 4) lanes, four consecutive channels per lane and step (C / (4 L) steps), so
 // that a wave reads 1 KiB contiguous per access; mean and variance are two reductions over registers (the
 // variance from the centred values, as a two-pass computation gives it), across the lanes of the row with xor
 // shuffles.  All arithmetic is fp32.
+#include <type_traits>
+
 #include "launch.hpp"
 
 namespace clusten {
@@ -24,8 +29,11 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
-template <typename InT, typename OutT, int L, int V>
-__global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__ x, const float* __restrict__ weight,
+// ResT = void: plain layer norm of x.  Otherwise the row normalised is x + branch (the residual connection ahead of
+// the norm), rounded to x's type as the framework's addition would leave it and also written to `sum_out`.
+template <typename InT, typename ResT, typename OutT, int L, int V>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__ x, const ResT* __restrict__ branch,
+                                                         InT* __restrict__ sum_out, const float* __restrict__ weight,
                                                          const float* __restrict__ bias, OutT* __restrict__ out,
                                                          int64_t rows, float eps) {
     constexpr int C = 4 * L * V;
@@ -40,6 +48,15 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__
     for (int s = 0; s < V; ++s) {
         float in[4];
         Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(xr + 4 * (s * L + sub)), in);
+        if constexpr (!std::is_void<ResT>::value) {
+            float br[4];
+            Quad<ResT>::unpack(*reinterpret_cast<const typename Quad<ResT>::raw*>(branch + row * C + 4 * (s * L + sub)), br);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) in[e] = to_acc(from_acc<InT>(in[e] + br[e]));
+            if (live) {
+                *reinterpret_cast<typename Quad<InT>::raw*>(sum_out + row * C + 4 * (s * L + sub)) = Quad<InT>::pack(in);
+            }
+        }
         v[s] = make_float4(in[0], in[1], in[2], in[3]);
     }
     float sum = 0.f;
@@ -66,27 +83,28 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__
     }
 }
 
-template <typename InT, typename OutT, int L, int V>
-int launch_lv(const void* x, const float* weight, const float* bias, void* out, int64_t rows, float eps,
-              hipStream_t stream) {
+template <typename InT, typename ResT, typename OutT, int L, int V>
+int launch_lv(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
+              int64_t rows, float eps, hipStream_t stream) {
     constexpr int ROWS_PER_WG = 256 / L;
     const int64_t blocks = (rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
-    hipLaunchKernelGGL((layer_norm_kernel<InT, OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       static_cast<const InT*>(x), weight, bias, static_cast<OutT*>(out), rows, eps);
+    hipLaunchKernelGGL((layer_norm_kernel<InT, ResT, OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       static_cast<const InT*>(x), static_cast<const ResT*>(branch), static_cast<InT*>(sum_out), weight,
+                       bias, static_cast<OutT*>(out), rows, eps);
     return launch_status();
 }
 
-template <typename InT, typename OutT>
-int launch_typed(const void* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
-                 hipStream_t stream) {
+template <typename InT, typename ResT, typename OutT>
+int launch_typed(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
+                 int64_t rows, int C, float eps, hipStream_t stream) {
     switch (C) {
-        case 64: return launch_lv<InT, OutT, 16, 1>(x, weight, bias, out, rows, eps, stream);
-        case 128: return launch_lv<InT, OutT, 32, 1>(x, weight, bias, out, rows, eps, stream);
-        case 256: return launch_lv<InT, OutT, 64, 1>(x, weight, bias, out, rows, eps, stream);
-        case 384: return launch_lv<InT, OutT, 32, 3>(x, weight, bias, out, rows, eps, stream);
-        case 512: return launch_lv<InT, OutT, 64, 2>(x, weight, bias, out, rows, eps, stream);
-        case 768: return launch_lv<InT, OutT, 64, 3>(x, weight, bias, out, rows, eps, stream);
-        case 1024: return launch_lv<InT, OutT, 64, 4>(x, weight, bias, out, rows, eps, stream);
+        case 64: return launch_lv<InT, ResT, OutT, 16, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 128: return launch_lv<InT, ResT, OutT, 32, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 256: return launch_lv<InT, ResT, OutT, 64, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 384: return launch_lv<InT, ResT, OutT, 32, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 512: return launch_lv<InT, ResT, OutT, 64, 2>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 768: return launch_lv<InT, ResT, OutT, 64, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 1024: return launch_lv<InT, ResT, OutT, 64, 4>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
         default: return CLUSTEN_ERR_BAD_DIMS;
     }
 }
@@ -95,11 +113,20 @@ template <typename InT>
 int launch_in(const void* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
               int out_dtype, hipStream_t stream) {
     switch (out_dtype) {
-        case CLUSTEN_F32: return launch_typed<InT, float>(x, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_F16: return launch_typed<InT, f16_t>(x, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_BF16: return launch_typed<InT, bf16_t>(x, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_F32: return launch_typed<InT, void, float>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_F16: return launch_typed<InT, void, f16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_BF16: return launch_typed<InT, void, bf16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
+}
+
+// x + branch, then the norm, written in the 16-bit type T of the branch: x is fp32 or T
+template <typename T>
+int launch_add(const void* x, int x_dtype, const void* branch, void* sum_out, const float* weight, const float* bias,
+               void* out, int64_t rows, int C, float eps, int t_code, hipStream_t stream) {
+    if (x_dtype == CLUSTEN_F32) return launch_typed<float, T, T>(x, branch, sum_out, weight, bias, out, rows, C, eps, stream);
+    if (x_dtype == t_code) return launch_typed<T, T, T>(x, branch, sum_out, weight, bias, out, rows, C, eps, stream);
+    return CLUSTEN_ERR_BAD_DTYPE;
 }
 
 }  // namespace
@@ -112,6 +139,18 @@ int launch_layer_norm(const void* x, int in_dtype, const float* weight, const fl
         case CLUSTEN_BF16: return launch_in<bf16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
+}
+
+int launch_add_layer_norm(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
+                          const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                          hipStream_t stream) {
+    if (branch_dtype == CLUSTEN_F16) {
+        return launch_add<f16_t>(x, x_dtype, branch, sum_out, weight, bias, out, rows, C, eps, CLUSTEN_F16, stream);
+    }
+    if (branch_dtype == CLUSTEN_BF16) {
+        return launch_add<bf16_t>(x, x_dtype, branch, sum_out, weight, bias, out, rows, C, eps, CLUSTEN_BF16, stream);
+    }
+    return CLUSTEN_ERR_BAD_DTYPE;
 }
 
 }  // namespace clusten

@@ -270,6 +270,38 @@ def test_layer_norm_kernel_equals_torch(device, out_dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("branch_dtype", [torch.float16, torch.bfloat16])
+def test_add_layer_norm_kernel_equals_the_separate_addition_and_norm(device, branch_dtype):
+    """The residual addition ahead of a norm and the norm in one pass: the sum equals the framework's addition bit
+    for bit (fp32 + 16-bit -> fp32; 16-bit + 16-bit -> 16-bit, rounded before it is normalised), the normalised rows
+    are F.layer_norm of that sum in fp32, rounded once."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(23)
+    for x_dtype in (torch.float32, branch_dtype):
+        for rows, c in ((1003, 64), (517, 128), (260, 256), (130, 384), (70, 512), (35, 768), (9, 1024)):
+            x = (torch.randn(rows, c, generator=gen) * 2 + 0.5).to(x_dtype).to(device)
+            branch = torch.randn(rows, c, generator=gen).to(branch_dtype).to(device)
+            w = (torch.rand(c, generator=gen) + 0.5).to(device)
+            b = torch.randn(c, generator=gen).to(device)
+            assert _native.add_layer_norm_supported(x, branch)
+            total, out = _native.add_layer_norm(x, branch, w, b, 1e-5)
+            want_total = x + branch
+            assert total.dtype == want_total.dtype and torch.equal(total, want_total)
+            want = torch.nn.functional.layer_norm(want_total.float(), (c,), w, b, 1e-5)
+            assert out.dtype == branch_dtype
+            err = oracle.rel_err(out.float().cpu(), want.cpu())
+            assert err <= (1e-3 if branch_dtype == torch.float16 else 8e-3), (x_dtype, rows, c, err)
+    x = torch.zeros(4, 3, 64, device=device)
+    assert not _native.add_layer_norm_supported(x, x)                               # fp32 branch
+    assert not _native.add_layer_norm_supported(x.half(), x.bfloat16())             # mixed 16-bit types
+    assert not _native.add_layer_norm_supported(x[..., :48], x[..., :48].half())    # width without a kernel
+    with pytest.raises(RuntimeError):
+        _native.add_layer_norm(x, x, torch.ones(64, device=device), torch.zeros(64, device=device))
+    t, o = _native.add_layer_norm(x[:0], x[:0].half(), torch.ones(64, device=device), torch.zeros(64, device=device))
+    assert t.shape == (0, 3, 64) and o.shape == (0, 3, 64)
+
+
+@pytest.mark.gpu
 def test_merge_weights_kernel_equals_the_tensor_expressions(device):
     from clusten import _native
     gen = torch.Generator().manual_seed(19)
@@ -354,6 +386,7 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     del three.cluster_attention
     del three.dense_attention
     del three.linear
+    del three.add_layer_norm
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
