@@ -284,6 +284,20 @@ int clusten_add_layer_norm_forward(const void* x, int x_dtype, const void* branc
                                    const float* weight, const float* bias, void* out, int64_t rows, int C,
                                    float eps, clusten_stream stream);
 
+/* The index tensors of a stage's local attention from the nearest clusters of every token of a cluster-ordered
+ * sequence (models/aff_transformer.py:476-487), in one pass instead of a gather and some ten tensor operations:
+ *   row(i,j)         = m * nearest[b,i,j/m] + j%m                        (j < nnc*m)
+ *   member_idx[b,i,j] = row(i,j) if row(i,j) < N else 0;   mask[b,i,j] = row(i,j) < N
+ *   pe_idx[b,i,j]    = trunc((y' - (y - radius)) * table_width + (x' - (x - radius))),  (x,y) = pos[b,i],
+ *                      (x',y') = pos[b, member_idx[b,i,j]]    (fp32, each operation rounded on its own)
+ *   cluster_idx[b,i,r] = (int32) nearest[b,i,r]
+ * pos (B,N,2) fp32 as (x,y); nearest (B,N,nnc) int64 with values >= 0; member_idx, pe_idx (B,N,nnc*m) int64;
+ * mask (B,N,nnc*m) int64 or NULL; cluster_idx (B,N,nnc) int32 or NULL; all contiguous.  No counterpart in the
+ * reference's extension modules. */
+int clusten_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* member_idx, int64_t* mask,
+                            int64_t* pe_idx, int32_t* cluster_idx, int B, int N, int nnc, int m, int radius,
+                            int table_width, clusten_stream stream);
+
 /* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
  * (models/aff_transformer.py:340-358), in one pass instead of a row lookup, a gather and two multiplications:
  *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]

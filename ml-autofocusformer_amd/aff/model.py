@@ -43,7 +43,9 @@ def default_ops():
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
                            linear=_native.linear, linear_supported=_native.linear_supported,
                            add_layer_norm=_native.add_layer_norm, add_layer_norm_supported=_native.add_layer_norm_supported,
-                           merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported)
+                           merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported,
+                           neighbour_lists=_native.neighbour_lists,
+                           neighbour_lists_supported=_native.neighbour_lists_supported)
 
 
 def _linear(lin, x, ops=None, gelu=False):
@@ -316,6 +318,7 @@ class BasicLayer(nn.Module):
         super().__init__()
         assert cluster_size > 0
         self.cluster_size, self.nbhd_size = cluster_size, nbhd_size
+        self.ops = ops
         rates = drop_path if isinstance(drop_path, (list, tuple)) else [drop_path] * depth
         self.blocks = nn.ModuleList([
             ClusterTransformerBlock(dim, num_heads, mlp_ratio, drop, attn_drop, rates[i], layer_scale, ops=ops)
@@ -344,6 +347,12 @@ class BasicLayer(nn.Module):
         else:
             pos, centres, members, mask, ranking = space_filling_cluster(pos, m, h, w)
         nearest = knn(pos, centres, nnc)                                                  # (b, n, nnc)
+        one_pass = getattr(self.ops, "neighbour_lists", None)
+        if (ranking is not None and one_pass is not None and not torch.is_grad_enabled()
+                and self.ops.neighbour_lists_supported(pos, nearest)):
+            # the four index tensors in one kernel
+            member_idx, mask, pe_idx, cluster_idx = one_pass(pos, nearest, m, radius, table_width, mask is not None)
+            return pos, ranking, member_idx, mask, pe_idx, (cluster_idx if m == 8 else None)
         if ranking is not None:
             # cluster order: cluster g owns tokens g*m .. g*m+m-1, pad slots of the last one hold index 0 and mask 0
             rows = nearest.unsqueeze(3) * m + torch.arange(m, device=pos.device)

@@ -63,6 +63,8 @@ _PROTOTYPES = {
                                                  ctypes.c_float, ctypes.c_int, _P]),
     "clusten_add_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, _P, ctypes.c_int64,
                                                      ctypes.c_int, ctypes.c_float, _P]),
+    "clusten_neighbour_lists": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                     ctypes.c_int, ctypes.c_int, _P]),
     "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
@@ -682,6 +684,40 @@ def add_layer_norm(x: torch.Tensor, branch: torch.Tensor, weight: torch.Tensor, 
                                                   ctypes.c_float(eps), _stream(device)),
                "clusten_add_layer_norm_forward")
     return total, out
+
+
+def neighbour_lists_supported(pos: torch.Tensor, nearest: torch.Tensor) -> bool:
+    """True when `neighbour_lists` takes this case: CUDA fp32 positions (B,N,2) and int64 cluster numbers (B,N,nnc)."""
+    return (pos.is_cuda and nearest.is_cuda and pos.dtype == torch.float32 and nearest.dtype == torch.int64
+            and pos.dim() == 3 and pos.shape[2] == 2 and nearest.dim() == 3 and nearest.shape[:2] == pos.shape[:2])
+
+
+def neighbour_lists(pos: torch.Tensor, nearest: torch.Tensor, m: int, radius: int, table_width: int, with_mask: bool):
+    """(member_idx, mask or None, pe_idx, cluster_idx) of a cluster-ordered sequence: the members of each token's
+    nearest clusters (clusters of m consecutive rows; rows past the last token become index 0 / mask 0), the row of
+    the relative-position table for every (token, member) pair, and the cluster numbers as int32
+    (models/aff_transformer.py:476-487).  pos (B,N,2) fp32, nearest (B,N,nnc) int64."""
+    lib = load()
+    _require_cuda("pos", pos)
+    device = pos.device
+    _require_cuda("nearest", nearest, device)
+    if not neighbour_lists_supported(pos, nearest):
+        raise RuntimeError("neighbour_lists takes fp32 positions (B,N,2) and int64 cluster numbers (B,N,nnc)")
+    b, n, nnc = nearest.shape
+    pos = pos.contiguous()
+    nearest = nearest.contiguous()
+    member_idx = torch.empty(b, n, nnc * m, dtype=torch.int64, device=device)
+    pe_idx = torch.empty_like(member_idx)
+    mask = torch.empty_like(member_idx) if with_mask else None
+    cluster_idx = torch.empty(b, n, nnc, dtype=torch.int32, device=device)
+    if member_idx.numel() == 0:
+        return member_idx, mask, pe_idx, cluster_idx
+    with torch.cuda.device(device):
+        _check(lib.clusten_neighbour_lists(_ptr(pos), _ptr(nearest), _ptr(member_idx), _ptr(mask), _ptr(pe_idx),
+                                           _ptr(cluster_idx), b, n, nnc, m, int(radius), int(table_width),
+                                           _stream(device)),
+               "clusten_neighbour_lists")
+    return member_idx, mask, pe_idx, cluster_idx
 
 
 def merge_weights_supported(table_weights: torch.Tensor) -> bool:

@@ -243,6 +243,17 @@ int clusten_add_layer_norm_forward(const void* x, int x_dtype, const void* branc
                                  as_stream(stream));
 }
 
+int clusten_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* member_idx, int64_t* mask,
+                            int64_t* pe_idx, int32_t* cluster_idx, int B, int N, int nnc, int m, int radius,
+                            int table_width, clusten_stream stream) {
+    if (!pos || !nearest || !member_idx || !pe_idx) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || nnc <= 0 || m <= 0 || table_width <= 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (((int64_t)B * N * nnc * m + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if ((reinterpret_cast<uintptr_t>(pos) & 7) != 0) return CLUSTEN_ERR_UNALIGNED;
+    return launch_neighbour_lists(pos, nearest, member_idx, mask, pe_idx, cluster_idx, B, N, nnc, m, radius, table_width,
+                                  as_stream(stream));
+}
+
 int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
                                   const float* prob, const int64_t* mask, float* weights, int B, int N, int Nout, int M,
                                   int IC, clusten_stream stream) {

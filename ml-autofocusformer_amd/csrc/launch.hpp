@@ -89,6 +89,12 @@ int launch_add_layer_norm(const void* x, int x_dtype, const void* branch, int br
                           const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
                           hipStream_t stream);
 
+// member_idx, mask (may be null), pe_idx (B,N,nnc*m) int64 and cluster_idx (B,N,nnc) int32 (may be null) from
+//   nearest (B,N,nnc) int64 and pos (B,N,2) fp32: see neighbour_lists.hip.
+int launch_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* member_idx, int64_t* mask, int64_t* pe_idx,
+                           int32_t* cluster_idx, int B, int N, int nnc, int m, int radius, int table_width,
+                           hipStream_t stream);
+
 // w[b,i,j,:4] = table_w[pe_idx[b,i,j], :4] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]   (prob, mask may be null)
 //   table_w (rows,4), prob (B,N), w (B,Nout,M,4): fp32;  pe_idx, nbhd_idx, mask: int64 (B,Nout,M).
 int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,

@@ -302,6 +302,41 @@ def test_add_layer_norm_kernel_equals_the_separate_addition_and_norm(device, bra
 
 
 @pytest.mark.gpu
+def test_neighbour_lists_kernel_equals_the_tensor_expressions(device):
+    """member_idx, mask, pe_idx and the int32 cluster numbers in one kernel: equal, element for element, to the gather
+    and the tensor operations of BasicLayer.neighbourhoods (whole-number and fractional positions, a short last
+    cluster, clusters of 8 and of 5)."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(29)
+    for b, n, nnc, m, radius, frac in ((3, 196, 6, 8, 55, False), (2, 784, 6, 8, 55, False), (2, 203, 4, 5, 30, True),
+                                       (1, 8, 1, 8, 3, False)):
+        k = (n + m - 1) // m
+        pos = torch.randint(0, radius + 1, (b, n, 2), generator=gen).float()
+        if frac:
+            pos = pos + torch.rand(b, n, 2, generator=gen)
+        pos = pos.to(device)
+        nearest = torch.randint(0, k, (b, n, nnc), generator=gen).to(device)
+        width = 2 * radius + 1
+        rows = nearest.unsqueeze(3) * m + torch.arange(m, device=device)
+        valid = rows < n
+        want_members = torch.where(valid, rows, torch.zeros_like(rows)).reshape(b, n, nnc * m)
+        nb_pos = pos.gather(1, want_members.reshape(b, -1, 1).expand(-1, -1, 2)).reshape(b, n, nnc * m, 2)
+        rel = nb_pos - (pos.unsqueeze(2) - radius)
+        want_pe = (rel[..., 1] * width + rel[..., 0]).long()
+        members, mask, pe_idx, cidx = _native.neighbour_lists(pos, nearest, m, radius, width, True)
+        assert torch.equal(members, want_members)
+        assert torch.equal(mask, valid.reshape(b, n, nnc * m).long())
+        assert torch.equal(pe_idx, want_pe)
+        assert cidx.dtype == torch.int32 and torch.equal(cidx.long(), nearest)
+        assert _native.neighbour_lists(pos, nearest, m, radius, width, False)[1] is None
+    assert not _native.neighbour_lists_supported(pos.cpu(), nearest.cpu())
+    assert not _native.neighbour_lists_supported(pos.double(), nearest)
+    assert not _native.neighbour_lists_supported(pos, nearest.int())
+    with pytest.raises(RuntimeError):
+        _native.neighbour_lists(pos.double(), nearest, 8, 3, 7, False)
+
+
+@pytest.mark.gpu
 def test_merge_weights_kernel_equals_the_tensor_expressions(device):
     from clusten import _native
     gen = torch.Generator().manual_seed(19)
@@ -387,6 +422,7 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     del three.dense_attention
     del three.linear
     del three.add_layer_norm
+    del three.neighbour_lists
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
