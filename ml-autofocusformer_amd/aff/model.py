@@ -273,7 +273,9 @@ class ClusterMerging(nn.Module):
             prior = ((pos.long() % spacing.unsqueeze(2).long()).sum(-1) == 0).float()
         score = prior
         if learned_prob is not None:
-            score = score + learned_prob.detach().view(b, n) * self.alpha
+            # widened before the addition (the values are those of the mixed-type addition; the framework's kernel
+            # for mixed types has a fixed cost of some 45 us on this device, however small the tensors)
+            score = score + (learned_prob.detach().view(b, n) * self.alpha).float()
         if not self.reserve_on:
             return score.topk(keep, dim=1, sorted=False)[1]
         reserved = ((pos % (stride * 2)).sum(-1) == 0)
