@@ -97,6 +97,26 @@ def _add_layer_norm(norm, x, branch, ops):
     return x, _layer_norm(norm, x, ops, True)
 
 
+def _autocast_key():
+    return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else None
+
+
+def _table_function(owner, slot, module, table, compute):
+    """`compute()`, a function of `module`'s parameters and of the relative-position table only, kept between
+    inference forwards: the position-bias table of an attention layer and the weight table of a merge are the same
+    for every batch.  Recomputed when a parameter or the table changes (in place or by replacement) or the autocast
+    state does; never kept while gradients are enabled."""
+    if torch.is_grad_enabled() or not table.is_cuda:
+        return compute()
+    key = (tuple((q.data_ptr(), q._version) for q in module.parameters()), table.data_ptr(), table._version, table.dtype,
+           _autocast_key())
+    hit = owner.__dict__.get(slot)
+    if hit is None or hit[0] != key:
+        hit = (key, compute(), table)         # the table is held, so that its address cannot be reused by another one
+        owner.__dict__[slot] = hit
+    return hit[1]
+
+
 def relative_position_table(img_size):
     """(table_width^2, 5) rows (dx, dy, distance, sin, cos) for every offset between two stride-4 tokens.
 
@@ -158,6 +178,10 @@ class ClusterAttention(nn.Module):
         self.proj_drop = nn.Dropout(proj_drop)
         self.ops = ops
 
+    def bias_table(self, table):
+        """(rows, heads) position bias for every row of the relative-position table (aff_transformer.py:125-129)."""
+        return _table_function(self, "_bias_table_cache", self.pos_embed, table, lambda: _linear(self.pos_embed, table))
+
     def forward(self, feat, member_idx, cluster_mask, pe_idx, global_attn, table, cluster_idx=None, grid_lists=None):
         """`grid_lists`: (cluster_idx, pe_idx, cluster_mask) with a leading 1 instead of the batch size, when the
         lists are the same for every image (tokens of a regular grid); the one-kernel path reads those."""
@@ -176,7 +200,7 @@ class ClusterAttention(nn.Module):
             # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
             # the values in one kernel; the query scale is applied to the scores inside it
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
-            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], _linear(self.pos_embed, table),
+            out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], self.bias_table(table),
                              lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale)
             return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
@@ -184,7 +208,7 @@ class ClusterAttention(nn.Module):
                 and not (self.training and self.attn_drop.p > 0)
                 and self.ops.dense_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3))):
             # inference on 16-bit data, every token attending to every token: one kernel as well
-            out = dense(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, _linear(self.pos_embed, table), pe_idx,
+            out = dense(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, self.bias_table(table), pe_idx,
                         self.blank_k, self.blank_v, scale=self.scale)
             return self.proj_drop(_linear(self.proj, out, self.ops))
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
@@ -196,7 +220,7 @@ class ClusterAttention(nn.Module):
             compact = False
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
 
-        bias = _linear(self.pos_embed, table)                                                     # (rows, h)
+        bias = self.bias_table(table)                                                     # (rows, h)
         fused = getattr(self.ops, "attn_softmax", None)
         if (fused is not None and not global_attn and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0) and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
@@ -295,7 +319,8 @@ class ClusterMerging(nn.Module):
         rows = centre.unsqueeze(2).expand(-1, -1, m)
         member_idx = member_idx.gather(1, rows)                                          # (b, n', m)
         pe_idx = pe_idx.gather(1, rows)
-        table_w = self.weight_net(table)                                                 # (rows, 4)
+        table_w = _table_function(self, "_weight_table_cache", self.weight_net, table,
+                                  lambda: self.weight_net(table))                         # (rows, 4)
         one_pass = getattr(self.ops, "merge_weights", None)
         if one_pass is not None and not torch.is_grad_enabled() and self.ops.merge_weights_supported(table_w):
             # inference: lookup, importance of each neighbour and mask in one kernel
@@ -487,8 +512,14 @@ class AutoFocusFormer(nn.Module):
         x = self.pos_drop(x)
         table = self.pre_table
         if not torch.is_grad_enabled() and table.is_cuda and torch.is_autocast_enabled("cuda"):
-            # every block's position-embedding Linear would round the table to 16 bits again
-            table = table.to(torch.get_autocast_dtype("cuda"))
+            # every block's position-embedding Linear would round the table to 16 bits again: one copy, kept
+            dt = torch.get_autocast_dtype("cuda")
+            key = (table.data_ptr(), table._version, dt)
+            hit = self.__dict__.get("_table_cast_cache")
+            if hit is None or hit[0] != key:
+                hit = (key, table.to(dt))
+                self.__dict__["_table_cast_cache"] = hit
+            table = hit[1]
         for i, layer in enumerate(self.layers):
             pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=table, radius=self.radius)
         return _layer_norm(self.norm, x, self.ops).mean(1)

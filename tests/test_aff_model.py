@@ -522,6 +522,21 @@ def test_cached_16_bit_weights_follow_the_parameters(device):
     assert torch.equal(run(model), y0)
     model.float()                                           # no-op conversion keeps working
     assert torch.equal(run(model), y0)
+    # the position-bias table of an attention layer and the weight table of a merge are kept as well: functions of
+    # their parameters and of the relative-position table only
+    with torch.no_grad():
+        model.layers[0].blocks[0].attn.pos_embed.weight.mul_(3.0)
+        model.layers[0].downsample.weight_net[0].bias.add_(0.5)
+    y2 = run(model)
+    fresh = small_model(default_ops(), img_size=128).to(device)
+    fresh.load_state_dict(model.state_dict())
+    assert torch.equal(y2, run(fresh)) and not torch.equal(y2, y0)
+    with torch.no_grad():                                   # without autocast: other tables, not the fp16 ones
+        y_fp32 = model(x)
+        assert torch.equal(y_fp32, fresh(x))
+    assert torch.equal(run(model), y2)
+    model.load_state_dict(state)
+    assert torch.equal(run(model), y0)
     # training mode and grad mode do not use the cache
     model.train()
     with torch.autocast("cuda", dtype=torch.float16):
