@@ -272,6 +272,27 @@ int clusten_linear_forward(const void* x, int64_t x_row_stride, const void* weig
 int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight, const float* bias, void* out,
                                int64_t rows, int C, float eps, int out_dtype, clusten_stream stream);
 
+/* Layer normalisation (as clusten_layer_norm_forward) of rows read in a given order, with a per-channel bias added
+ * first:
+ *   out[g*group + i, :] = layer norm of ( x[g*group + order[i], :] + pre_bias[:] )     i < group, g < rows / group
+ * the norm that ends the patch embedding of the reference model (models/aff_transformer.py:542-546) with the second
+ * convolution's bias and the reordering of the tokens into cluster order (:465-466) taken along.  order (group)
+ * int64, a permutation of 0..group-1, or NULL (then group is ignored); pre_bias (C) of in_dtype or NULL, added with a
+ * rounding to in_dtype as a separate addition would leave it; rows % group == 0 (else CLUSTEN_ERR_BAD_DIMS); the
+ * rest as clusten_layer_norm_forward.  No counterpart in the reference's extension modules. */
+int clusten_layer_norm_rows_forward(const void* x, int in_dtype, const int64_t* order, int group, const void* pre_bias,
+                                    const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                                    int out_dtype, clusten_stream stream);
+
+/* y = GELU(x * scale[c] + shift[c]) over a contiguous (B,C,H,W) tensor of F16 or BF16 data (exact GELU, fp32
+ * arithmetic, one rounding): convolution bias, inference BatchNorm and activation of the patch embedding
+ * (`self.act1(self.bn(self.proj1(x)))`, models/aff_transformer.py:542) in one pass over the convolution's output,
+ * with scale = gamma / sqrt(running_var + eps) and shift = (conv_bias - running_mean) * scale + beta prepared by
+ * the caller.  scale, shift (C) fp32; HW = H*W a multiple of 8 (else CLUSTEN_ERR_BAD_DIMS); x, y 16-byte aligned;
+ * y may be x.  No counterpart in the reference's extension modules. */
+int clusten_channel_affine_gelu_forward(const void* x, const float* scale, const float* shift, void* y, int64_t B, int C,
+                                        int HW, int dtype, clusten_stream stream);
+
 /* The residual addition ahead of a layer normalisation, and the normalisation, in one pass:
  *   sum_out[r,c] = x[r,c] + branch[r,c]   (rounded to x's type, as the framework's addition leaves it)
  *   out[r,c]     = layer norm of sum_out[r,:] as clusten_layer_norm_forward computes it, written in branch's type

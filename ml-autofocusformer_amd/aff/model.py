@@ -44,6 +44,8 @@ def default_ops():
                            linear=_native.linear, linear_supported=_native.linear_supported,
                            add_layer_norm=_native.add_layer_norm, add_layer_norm_supported=_native.add_layer_norm_supported,
                            merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported,
+                           channel_affine_gelu=_native.channel_affine_gelu,
+                           channel_affine_gelu_supported=_native.channel_affine_gelu_supported,
                            neighbour_lists=_native.neighbour_lists,
                            neighbour_lists_supported=_native.neighbour_lists_supported)
 
@@ -81,6 +83,10 @@ def _layer_norm(norm, x, ops, feeds_linear=False):
         return norm(x)
     out_dtype = torch.get_autocast_dtype("cuda") if (feeds_linear and torch.is_autocast_enabled("cuda")) else None
     return fn(x, norm.weight, norm.bias, norm.eps, out_dtype)
+
+
+def _one_pass_norm_available(ops, x):
+    return (getattr(ops, "layer_norm", None) is not None and not torch.is_grad_enabled() and ops.layer_norm_supported(x))
 
 
 def _add_layer_norm(norm, x, branch, ops):
@@ -400,7 +406,20 @@ class BasicLayer(nn.Module):
         cluster_idx = nearest.to(torch.int32).contiguous() if (ranking is not None and m == 8) else None
         return pos, ranking, member_idx, mask, pe_idx, cluster_idx
 
-    def forward(self, pos, feat, h, w, on_grid, stride, table, radius):
+    def grid_order(self, pos1, h, w, radius):
+        """The order (n,) in which this stage, as the first one, takes the tokens of the full grid (`pos1`: the
+        positions of one image), or None when it leaves them as they are; fills the stage's cache of grid lists."""
+        n = pos1.shape[1]
+        if self.nbhd_size >= n:
+            return None
+        key = (n, h, w, str(pos1.device))
+        if key not in self._grid_cache:
+            self._grid_cache[key] = self.neighbourhoods(pos1[:1], h, w, radius, 2 * radius + 1)
+        ranking = self._grid_cache[key][1]
+        return None if ranking is None else ranking[0, :, 0]
+
+    def forward(self, pos, feat, h, w, on_grid, stride, table, radius, feat_ordered=False):
+        """`feat_ordered`: the tokens already stand in the order `grid_order` gave (first stage only)."""
         b, n, d = pos.shape
         table_width = 2 * radius + 1
         global_attn = self.nbhd_size >= n
@@ -425,7 +444,7 @@ class BasicLayer(nn.Module):
                     grid_lists = (cluster_idx, pe_idx, mask)           # one image's lists, for the one-kernel attention
                 member_idx, pe_idx, mask, cluster_idx = self._grid_cache[(key, b)]
                 pos = pos1.expand(b, -1, -1)
-                if ranking is not None:
+                if ranking is not None and not feat_ordered:
                     feat = feat[:, ranking[0, :, 0]]
             else:
                 pos, ranking, member_idx, mask, pe_idx, cluster_idx = self.neighbourhoods(pos, h, w, radius, table_width)
@@ -459,15 +478,65 @@ class PatchEmbed(nn.Module):
         self.proj2 = nn.Conv2d(embed_dim // 2, embed_dim, kernel_size=3, stride=2, padding=1)
         self.norm = nn.LayerNorm(embed_dim) if patch_norm else None
 
-    def forward(self, x):
-        x = self.proj2(self.act1(self.bn(self.proj1(x))))
-        b, c, h, w = x.shape
-        x = x.flatten(2).transpose(1, 2)
-        if self.norm is not None:
-            x = _layer_norm(self.norm, x, self.ops)
+    def _bn_affine(self):
+        """BatchNorm in inference as y = x * scale + shift per channel, the first convolution's bias folded in; kept
+        until a parameter or a running statistic changes."""
+        bn, conv = self.bn, self.proj1
+        parts = [t for t in (bn.weight, bn.bias, bn.running_mean, bn.running_var, conv.bias) if t is not None]
+        key = tuple((t.data_ptr(), t._version) for t in parts)
+        hit = self.__dict__.get("_bn_affine_cache")
+        if hit is None or hit[0] != key:
+            scale = torch.rsqrt(bn.running_var.float() + bn.eps)
+            if bn.weight is not None:
+                scale = scale * bn.weight.float()
+            shift = -bn.running_mean.float() if conv.bias is None else conv.bias.float() - bn.running_mean.float()
+            shift = shift * scale
+            if bn.bias is not None:
+                shift = shift + bn.bias.float()
+            hit = (key, scale.detach(), shift.detach())
+            self.__dict__["_bn_affine_cache"] = hit
+        return hit[1], hit[2]
+
+    def forward(self, x, token_order=None):
+        """`token_order(pos_of_one_image, h, w)`, when given, returns the order (N,) in which the first stage wants
+        the tokens (or None); the tokens then leave in that order when the final norm can take it along, and the
+        fifth return value says whether they did."""
+        fused = getattr(self.ops, "channel_affine_gelu", None)
+        if (fused is not None and not torch.is_grad_enabled() and not self.bn.training and x.is_cuda
+                and torch.is_autocast_enabled("cuda") and self.bn.track_running_stats):
+            # inference: bias, BatchNorm (an affine map per channel) and GELU in one pass over the convolution's output
+            y = F.conv2d(x, self.proj1.weight, None, self.proj1.stride, self.proj1.padding)
+            if self.ops.channel_affine_gelu_supported(y):
+                y = fused(y, *self._bn_affine())
+            else:
+                y = self.act1(self.bn(y if self.proj1.bias is None else y + self.proj1.bias.view(1, -1, 1, 1)))
+        else:
+            y = self.act1(self.bn(self.proj1(x)))
+        b, _, h0, w0 = y.shape
+        h, w = (h0 + 1) // 2, (w0 + 1) // 2
         ys, xs = torch.meshgrid(torch.arange(h, device=x.device), torch.arange(w, device=x.device), indexing="ij")
-        pos = torch.stack([xs, ys], dim=2).reshape(1, -1, 2).expand(b, -1, -1).to(x.dtype)
-        return pos, x, h, w
+        pos = torch.stack([xs, ys], dim=2).reshape(1, -1, 2)
+        order = None
+        if self.norm is not None and token_order is not None and x.is_cuda and not torch.is_grad_enabled():
+            order = token_order(pos.float(), h, w)
+        if order is not None or (self.norm is not None and self.proj2.bias is not None and x.is_cuda
+                                 and not torch.is_grad_enabled()):
+            # the second convolution's bias and the reordering ride along with the norm
+            z = F.conv2d(y, self.proj2.weight, None, self.proj2.stride, self.proj2.padding)
+            z = z.flatten(2).transpose(1, 2).contiguous()
+            if _one_pass_norm_available(self.ops, z):
+                tokens = self.ops.layer_norm(z, self.norm.weight, self.norm.bias, self.norm.eps, None, order,
+                                             self.proj2.bias)
+                return pos.expand(b, -1, -1).to(tokens.dtype), tokens, h, w, order is not None
+            if self.proj2.bias is not None:
+                z = z + self.proj2.bias
+            tokens = self.norm(z)
+            return pos.expand(b, -1, -1).to(tokens.dtype), tokens, h, w, False
+        tokens = self.proj2(y).flatten(2).transpose(1, 2)
+        assert tokens.shape[1] == h * w
+        if self.norm is not None:
+            tokens = _layer_norm(self.norm, tokens, self.ops)
+        return pos.expand(b, -1, -1).to(tokens.dtype), tokens, h, w, False
 
 
 class AutoFocusFormer(nn.Module):
@@ -508,7 +577,8 @@ class AutoFocusFormer(nn.Module):
             nn.init.ones_(mod.weight)
 
     def forward_features(self, x):
-        pos, x, h, w = self.patch_embed(x)
+        first = self.layers[0]
+        pos, x, h, w, ordered = self.patch_embed(x, lambda pos1, h, w: first.grid_order(pos1, h, w, self.radius))
         x = self.pos_drop(x)
         table = self.pre_table
         if not torch.is_grad_enabled() and table.is_cuda and torch.is_autocast_enabled("cuda"):
@@ -521,7 +591,8 @@ class AutoFocusFormer(nn.Module):
                 self.__dict__["_table_cast_cache"] = hit
             table = hit[1]
         for i, layer in enumerate(self.layers):
-            pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=table, radius=self.radius)
+            pos, x = layer(pos, x, h, w, on_grid=(i == 0), stride=2 ** (i + 1), table=table, radius=self.radius,
+                           feat_ordered=(i == 0 and ordered))
         return _layer_norm(self.norm, x, self.ops).mean(1)
 
     def forward(self, x):

@@ -61,6 +61,10 @@ _PROTOTYPES = {
                                              ctypes.c_int, ctypes.c_int, _P]),
     "clusten_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
                                                  ctypes.c_float, ctypes.c_int, _P]),
+    "clusten_layer_norm_rows_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, _P, ctypes.c_int64,
+                                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, _P]),
+    "clusten_channel_affine_gelu_forward": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                          ctypes.c_int, _P]),
     "clusten_add_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, _P, ctypes.c_int64,
                                                      ctypes.c_int, ctypes.c_float, _P]),
     "clusten_neighbour_lists": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -618,10 +622,12 @@ def layer_norm_supported(x: torch.Tensor, out_dtype=None) -> bool:
             and (out_dtype is None or out_dtype in _DTYPE_CODES))
 
 
-def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5, out_dtype=None):
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5, out_dtype=None,
+               order=None, pre_bias=None):
     """F.layer_norm(x.float(), (C,), weight, bias, eps), returned as `out_dtype` (fp32 unless given): the widening
     of a 16-bit input, the normalisation in fp32 and the rounding a following mixed-precision Linear applies, in
-    one pass.  No autograd."""
+    one pass.  With `order` ((N,) int64, a permutation) x is (B,N,C) and row i of every image is the norm of its row
+    order[i]; with `pre_bias` ((C,), x's dtype) the rows are x + pre_bias, rounded to x's dtype.  No autograd."""
     lib = load()
     _require_cuda("x", x)
     device = x.device
@@ -639,11 +645,62 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
     out = torch.empty(x.shape, dtype=out_dtype, device=device)
     if out.numel() == 0:
         return out
+    if order is None and pre_bias is None:
+        with torch.cuda.device(device):
+            _check(lib.clusten_layer_norm_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(weight), _ptr(bias), _ptr(out),
+                                                  x.numel() // c, c,
+                                                  ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
+                   "clusten_layer_norm_forward")
+        return out
+    group = 1
+    if order is not None:
+        _require_cuda("order", order, device)
+        if x.dim() != 3 or order.shape != (x.shape[1],) or order.dtype != torch.int64:
+            raise RuntimeError("order must be an int64 tensor of N entries for x of shape (B,N,C)")
+        order = order.contiguous()
+        group = x.shape[1]
+    if pre_bias is not None:
+        _require_cuda("pre_bias", pre_bias, device)
+        if pre_bias.numel() != c:
+            raise RuntimeError("pre_bias must have as many elements as the last axis of x")
+        pre_bias = pre_bias.detach().to(x.dtype).contiguous()
     with torch.cuda.device(device):
-        _check(lib.clusten_layer_norm_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(weight), _ptr(bias), _ptr(out),
-                                              x.numel() // c, c,
-                                              ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
-               "clusten_layer_norm_forward")
+        _check(lib.clusten_layer_norm_rows_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(order), group, _ptr(pre_bias),
+                                                   _ptr(weight), _ptr(bias), _ptr(out), x.numel() // c, c,
+                                                   ctypes.c_float(eps), _DTYPE_CODES[out_dtype], _stream(device)),
+               "clusten_layer_norm_rows_forward")
+    return out
+
+
+def channel_affine_gelu_supported(x: torch.Tensor) -> bool:
+    """True when `channel_affine_gelu` takes this case: a contiguous CUDA fp16 / bf16 (B,C,H,W) tensor, H*W % 8 == 0."""
+    return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.dim() == 4 and x.is_contiguous()
+            and (x.shape[2] * x.shape[3]) % 8 == 0)
+
+
+def channel_affine_gelu(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor) -> torch.Tensor:
+    """F.gelu(x * scale[None,:,None,None] + shift[None,:,None,None]) in fp32, rounded once to x's 16-bit dtype: bias,
+    inference BatchNorm and GELU after the first convolution of the patch embedding
+    (models/aff_transformer.py:542) in one pass.  No autograd."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    _require_cuda("scale", scale, device)
+    _require_cuda("shift", shift, device)
+    if not channel_affine_gelu_supported(x):
+        raise RuntimeError("channel_affine_gelu takes a contiguous fp16 / bf16 (B,C,H,W) tensor with H*W % 8 == 0")
+    b, c, h, w = x.shape
+    if scale.numel() != c or shift.numel() != c:
+        raise RuntimeError("scale and shift must have C elements")
+    scale = scale.detach().float().contiguous()
+    shift = shift.detach().float().contiguous()
+    out = torch.empty_like(x)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(device):
+        _check(lib.clusten_channel_affine_gelu_forward(_ptr(x), _ptr(scale), _ptr(shift), _ptr(out), b, c, h * w,
+                                                       _DTYPE_CODES[x.dtype], _stream(device)),
+               "clusten_channel_affine_gelu_forward")
     return out
 
 

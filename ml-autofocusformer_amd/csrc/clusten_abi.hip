@@ -228,6 +228,31 @@ int clusten_layer_norm_forward(const void* x, int in_dtype, const float* weight,
     return launch_layer_norm(x, in_dtype, weight, bias, out, rows, C, eps, out_dtype, as_stream(stream));
 }
 
+int clusten_layer_norm_rows_forward(const void* x, int in_dtype, const int64_t* order, int group, const void* pre_bias,
+                                    const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                                    int out_dtype, clusten_stream stream) {
+    if (!x || !weight || !bias || !out) return CLUSTEN_ERR_NULL_POINTER;
+    if (out_dtype != CLUSTEN_F32 && out_dtype != CLUSTEN_F16 && out_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (in_dtype != CLUSTEN_F32 && in_dtype != CLUSTEN_F16 && in_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || C <= 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (order && (group <= 0 || rows % group != 0)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(bias) || !aligned16(out) || (pre_bias && !aligned16(pre_bias))) {
+        return CLUSTEN_ERR_UNALIGNED;
+    }
+    return launch_layer_norm_rows(x, in_dtype, order, order ? group : 1, pre_bias, weight, bias, out, rows, C, eps,
+                                  out_dtype, as_stream(stream));
+}
+
+int clusten_channel_affine_gelu_forward(const void* x, const float* scale, const float* shift, void* y, int64_t B, int C,
+                                        int HW, int dtype, clusten_stream stream) {
+    if (!x || !scale || !shift || !y) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (B <= 0 || C <= 0 || HW <= 0 || HW % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((B * C * HW / 8 + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(y)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_channel_affine_gelu(x, scale, shift, y, B, C, HW, dtype, as_stream(stream));
+}
+
 int clusten_add_layer_norm_forward(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
                                    const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
                                    clusten_stream stream) {

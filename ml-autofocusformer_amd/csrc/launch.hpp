@@ -84,6 +84,15 @@ int launch_skinny_linear(const void* x, int64_t ldx, const void* w, const void* 
 int launch_layer_norm(const void* x, int in_dtype, const float* weight, const float* bias, void* out, int64_t rows, int C,
                       float eps, int out_dtype, hipStream_t stream);
 
+// layer norm of rows read in a given order (order may be null) with a per-channel bias (may be null) added first.
+int launch_layer_norm_rows(const void* x, int in_dtype, const int64_t* order, int group, const void* pre_bias,
+                           const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                           int out_dtype, hipStream_t stream);
+
+// y = GELU(x * scale[c] + shift[c]) over (B,C,HW) of T in {F16, BF16}; HW % 8 == 0.
+int launch_channel_affine_gelu(const void* x, const float* scale, const float* shift, void* y, int64_t B, int C, int HW,
+                               int dtype, hipStream_t stream);
+
 // sum_out = x + branch (x's type), out = layer norm of sum_out (branch's 16-bit type); x of F32 or branch's type.
 int launch_add_layer_norm(const void* x, int x_dtype, const void* branch, int branch_dtype, void* sum_out,
                           const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,

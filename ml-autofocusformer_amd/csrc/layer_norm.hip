@@ -8,8 +8,11 @@
 // is a few hundred bytes, which the framework's general kernel handles at a fraction of the memory bandwidth).  A
 // second form takes the residual addition ahead of the norm along (`x = x + drop_path(branch)` followed by
 // `norm(x)`: models/aff_transformer.py:230-231, and :232 with the next block's :219): it writes the sum, rounded as the
-// framework's addition leaves it, and the normalised row in one pass.  Neither has a counterpart in the
-// reference's extension modules.
+// framework's addition leaves it, and the normalised row in one pass.  A third form reads the rows of every image
+// in a given order and adds a per-channel bias first: the norm at the end of the patch embedding
+// (models/aff_transformer.py:542-546), with the second convolution's bias and the reordering of the tokens into
+// cluster order (:465-466, the first stage) taken along.  None has a counterpart in the reference's extension
+// modules.
 //
 // A row is held by L = min(64, C / 4) lanes, four consecutive channels per lane and step (C / (4 L) steps), so
 // that a wave reads 1 KiB contiguous per access; mean and variance are two reductions over registers (the
@@ -35,19 +38,29 @@ template <typename InT, typename ResT, typename OutT, int L, int V>
 __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__ x, const ResT* __restrict__ branch,
                                                          InT* __restrict__ sum_out, const float* __restrict__ weight,
                                                          const float* __restrict__ bias, OutT* __restrict__ out,
-                                                         int64_t rows, float eps) {
+                                                         int64_t rows, float eps, const int64_t* __restrict__ order,
+                                                         int group, const InT* __restrict__ pre_bias) {
     constexpr int C = 4 * L * V;
     constexpr int ROWS_PER_WG = 256 / L;
     const int sub = threadIdx.x % L;
     const int64_t row_raw = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / L;
     const bool live = row_raw < rows;
     const int64_t row = live ? row_raw : rows - 1;  // every lane stays in the shuffles
-    const InT* xr = x + row * C;
+    // with `order`: output row g * group + i is the norm of input row g * group + order[i] (the rows of every group
+    // of `group` rows, an image's tokens, permuted the same way)
+    const int64_t src = order ? row - row % group + order[row % group] : row;
+    const InT* xr = x + src * C;
     float4 v[V];
 #pragma unroll
     for (int s = 0; s < V; ++s) {
         float in[4];
         Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(xr + 4 * (s * L + sub)), in);
+        if (pre_bias) {  // a per-channel bias the producer left out, added as its own addition would have: rounded
+            float pb[4];
+            Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(pre_bias + 4 * (s * L + sub)), pb);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) in[e] = to_acc(from_acc<InT>(in[e] + pb[e]));
+        }
         if constexpr (!std::is_void<ResT>::value) {
             float br[4];
             Quad<ResT>::unpack(*reinterpret_cast<const typename Quad<ResT>::raw*>(branch + row * C + 4 * (s * L + sub)), br);
@@ -85,37 +98,46 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__
 
 template <typename InT, typename ResT, typename OutT, int L, int V>
 int launch_lv(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
-              int64_t rows, float eps, hipStream_t stream) {
+              int64_t rows, float eps, hipStream_t stream, const int64_t* order = nullptr, int group = 1,
+              const void* pre_bias = nullptr) {
     constexpr int ROWS_PER_WG = 256 / L;
     const int64_t blocks = (rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
     hipLaunchKernelGGL((layer_norm_kernel<InT, ResT, OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream,
                        static_cast<const InT*>(x), static_cast<const ResT*>(branch), static_cast<InT*>(sum_out), weight,
-                       bias, static_cast<OutT*>(out), rows, eps);
+                       bias, static_cast<OutT*>(out), rows, eps, order, group, static_cast<const InT*>(pre_bias));
     return launch_status();
 }
 
 template <typename InT, typename ResT, typename OutT>
 int launch_typed(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
-                 int64_t rows, int C, float eps, hipStream_t stream) {
+                 int64_t rows, int C, float eps, hipStream_t stream, const int64_t* order = nullptr, int group = 1,
+                 const void* pre_bias = nullptr) {
     switch (C) {
-        case 64: return launch_lv<InT, ResT, OutT, 16, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 128: return launch_lv<InT, ResT, OutT, 32, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 256: return launch_lv<InT, ResT, OutT, 64, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 384: return launch_lv<InT, ResT, OutT, 32, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 512: return launch_lv<InT, ResT, OutT, 64, 2>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 768: return launch_lv<InT, ResT, OutT, 64, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
-        case 1024: return launch_lv<InT, ResT, OutT, 64, 4>(x, branch, sum_out, weight, bias, out, rows, eps, stream);
+        case 64: return launch_lv<InT, ResT, OutT, 16, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 128: return launch_lv<InT, ResT, OutT, 32, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 256: return launch_lv<InT, ResT, OutT, 64, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 384: return launch_lv<InT, ResT, OutT, 32, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 512: return launch_lv<InT, ResT, OutT, 64, 2>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 768: return launch_lv<InT, ResT, OutT, 64, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 1024: return launch_lv<InT, ResT, OutT, 64, 4>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
         default: return CLUSTEN_ERR_BAD_DIMS;
     }
 }
 
 template <typename InT>
 int launch_in(const void* x, const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
-              int out_dtype, hipStream_t stream) {
+              int out_dtype, hipStream_t stream, const int64_t* order = nullptr, int group = 1,
+              const void* pre_bias = nullptr) {
     switch (out_dtype) {
-        case CLUSTEN_F32: return launch_typed<InT, void, float>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_F16: return launch_typed<InT, void, f16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
-        case CLUSTEN_BF16: return launch_typed<InT, void, bf16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream);
+        case CLUSTEN_F32:
+            return launch_typed<InT, void, float>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream, order, group,
+                                                  pre_bias);
+        case CLUSTEN_F16:
+            return launch_typed<InT, void, f16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream, order, group,
+                                                  pre_bias);
+        case CLUSTEN_BF16:
+            return launch_typed<InT, void, bf16_t>(x, nullptr, nullptr, weight, bias, out, rows, C, eps, stream, order,
+                                                   group, pre_bias);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }
@@ -137,6 +159,20 @@ int launch_layer_norm(const void* x, int in_dtype, const float* weight, const fl
         case CLUSTEN_F32: return launch_in<float>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
         case CLUSTEN_F16: return launch_in<f16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
         case CLUSTEN_BF16: return launch_in<bf16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
+int launch_layer_norm_rows(const void* x, int in_dtype, const int64_t* order, int group, const void* pre_bias,
+                           const float* weight, const float* bias, void* out, int64_t rows, int C, float eps,
+                           int out_dtype, hipStream_t stream) {
+    switch (in_dtype) {
+        case CLUSTEN_F32:
+            return launch_in<float>(x, weight, bias, out, rows, C, eps, out_dtype, stream, order, group, pre_bias);
+        case CLUSTEN_F16:
+            return launch_in<f16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream, order, group, pre_bias);
+        case CLUSTEN_BF16:
+            return launch_in<bf16_t>(x, weight, bias, out, rows, C, eps, out_dtype, stream, order, group, pre_bias);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }

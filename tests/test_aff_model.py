@@ -337,6 +337,62 @@ def test_neighbour_lists_kernel_equals_the_tensor_expressions(device):
 
 
 @pytest.mark.gpu
+def test_layer_norm_kernel_with_row_order_and_bias(device):
+    """The norm that ends the patch embedding with the reordering of the tokens and the convolution's bias taken
+    along: row i of every image is the norm of (row order[i] + bias), the sum rounded to the input's type."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(31)
+    for in_dtype in (torch.float16, torch.bfloat16, torch.float32):
+        for b, n, c in ((3, 200, 64), (2, 49, 128), (1, 7, 256)):
+            x = (torch.randn(b, n, c, generator=gen) * 2).to(in_dtype).to(device)
+            bias = torch.randn(c, generator=gen).to(device)
+            w = (torch.rand(c, generator=gen) + 0.5).to(device)
+            beta = torch.randn(c, generator=gen).to(device)
+            order = torch.randperm(n, generator=gen).to(device)
+            summed = (x + bias.to(in_dtype)).float()
+            want = torch.nn.functional.layer_norm(summed, (c,), w, beta, 1e-5)
+            tol = 1e-5
+            assert oracle.rel_err(_native.layer_norm(x, w, beta, 1e-5, None, order, bias).cpu(), want[:, order].cpu()) <= tol
+            assert oracle.rel_err(_native.layer_norm(x, w, beta, 1e-5, None, None, bias).cpu(), want.cpu()) <= tol
+            plain = torch.nn.functional.layer_norm(x.float(), (c,), w, beta, 1e-5)
+            assert oracle.rel_err(_native.layer_norm(x, w, beta, 1e-5, None, order).cpu(), plain[:, order].cpu()) <= tol
+    with pytest.raises(RuntimeError):
+        _native.layer_norm(x, w, beta, 1e-5, None, order[:3])
+    with pytest.raises(RuntimeError):
+        _native.layer_norm(x, w, beta, 1e-5, None, None, bias[:5])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_channel_affine_gelu_kernel_equals_bias_batch_norm_gelu(device, dtype):
+    """Convolution bias, inference BatchNorm and GELU as one affine map per channel and one activation."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(37)
+    b, c, h, w = 3, 32, 20, 12
+    x = torch.randn(b, c, h, w, generator=gen).to(dtype).to(device)
+    conv_bias = torch.randn(c, generator=gen).to(device)
+    bn = torch.nn.BatchNorm2d(c).to(device).eval()
+    with torch.no_grad():
+        bn.weight.copy_(torch.rand(c, generator=gen) + 0.5)
+        bn.bias.copy_(torch.randn(c, generator=gen))
+        bn.running_mean.copy_(torch.randn(c, generator=gen))
+        bn.running_var.copy_(torch.rand(c, generator=gen) + 0.3)
+        want = torch.nn.functional.gelu(bn(x.float() + conv_bias.view(1, c, 1, 1)))
+    scale = bn.weight / torch.sqrt(bn.running_var + bn.eps)
+    shift = (conv_bias - bn.running_mean) * scale + bn.bias
+    assert _native.channel_affine_gelu_supported(x)
+    out = _native.channel_affine_gelu(x, scale, shift)
+    assert out.dtype == dtype and out.shape == x.shape
+    assert oracle.rel_err(out.float().cpu(), want.cpu()) <= (1e-3 if dtype == torch.float16 else 8e-3)
+    assert not _native.channel_affine_gelu_supported(x[:, :, :, :5])
+    assert not _native.channel_affine_gelu_supported(x.float())
+    with pytest.raises(RuntimeError):
+        _native.channel_affine_gelu(x.float(), scale, shift)
+    with pytest.raises(RuntimeError):
+        _native.channel_affine_gelu(x, scale[:4], shift)
+
+
+@pytest.mark.gpu
 def test_merge_weights_kernel_equals_the_tensor_expressions(device):
     from clusten import _native
     gen = torch.Generator().manual_seed(19)
@@ -423,6 +479,7 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     del three.linear
     del three.add_layer_norm
     del three.neighbour_lists
+    del three.channel_affine_gelu
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
