@@ -288,7 +288,8 @@ int clusten_layer_norm_rows_forward(const void* x, int in_dtype, const int64_t* 
  * arithmetic, one rounding): convolution bias, inference BatchNorm and activation of the patch embedding
  * (`self.act1(self.bn(self.proj1(x)))`, models/aff_transformer.py:542) in one pass over the convolution's output,
  * with scale = gamma / sqrt(running_var + eps) and shift = (conv_bias - running_mean) * scale + beta prepared by
- * the caller.  scale, shift (C) fp32; HW = H*W a multiple of 8 (else CLUSTEN_ERR_BAD_DIMS); x, y 16-byte aligned;
+ * the caller.  scale, shift (C) fp32; HW = H*W a multiple of 8 and B*C < 65536 (else CLUSTEN_ERR_BAD_DIMS); x, y
+ * 16-byte aligned;
  * y may be x.  No counterpart in the reference's extension modules. */
 int clusten_channel_affine_gelu_forward(const void* x, const float* scale, const float* shift, void* y, int64_t B, int C,
                                         int HW, int dtype, clusten_stream stream);

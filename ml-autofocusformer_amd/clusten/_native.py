@@ -675,7 +675,7 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
 def channel_affine_gelu_supported(x: torch.Tensor) -> bool:
     """True when `channel_affine_gelu` takes this case: a contiguous CUDA fp16 / bf16 (B,C,H,W) tensor, H*W % 8 == 0."""
     return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.dim() == 4 and x.is_contiguous()
-            and (x.shape[2] * x.shape[3]) % 8 == 0)
+            and (x.shape[2] * x.shape[3]) % 8 == 0 and x.shape[0] * x.shape[1] < 65536)
 
 
 def channel_affine_gelu(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor) -> torch.Tensor:

@@ -15,30 +15,34 @@ namespace {
 template <typename T>
 __global__ __launch_bounds__(256) void channel_affine_gelu_kernel(const T* __restrict__ x, const float* __restrict__ scale,
                                                                   const float* __restrict__ shift, T* __restrict__ y, int C,
-                                                                  int HW, int64_t pieces) {
-    const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one 16-byte piece: 8 elements of one channel
-    if (p >= pieces) return;
-    const int c = (int)((p * 8 / HW) % C);
+                                                                  int pieces_per_plane) {
+    // blockIdx.y: the (image, channel) plane; a thread owns 16-byte pieces (8 elements) of it
+    const int c = blockIdx.y % C;
     const float a = scale[c], b = shift[c];
-    float v[8];
-    VecIO<T, 8>::unpack(*reinterpret_cast<const Piece*>(x + p * 8), v);
+    const int64_t plane = (int64_t)blockIdx.y * pieces_per_plane;
+    for (int p = blockIdx.x * 256 + threadIdx.x; p < pieces_per_plane; p += gridDim.x * 256) {
+        float v[8];
+        VecIO<T, 8>::unpack(*reinterpret_cast<const Piece*>(x + (plane + p) * 8), v);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = gelu_erf(v[e] * a + b);
-    *reinterpret_cast<Piece*>(y + p * 8) = VecIO<T, 8>::pack(v);
+        for (int e = 0; e < 8; ++e) v[e] = gelu_erf(v[e] * a + b);
+        *reinterpret_cast<Piece*>(y + (plane + p) * 8) = VecIO<T, 8>::pack(v);
+    }
 }
 
 }  // namespace
 
 int launch_channel_affine_gelu(const void* x, const float* scale, const float* shift, void* y, int64_t B, int C, int HW,
                                int dtype, hipStream_t stream) {
-    const int64_t pieces = B * C * HW / 8;
-    const unsigned blocks = (unsigned)((pieces + 255) / 256);
+    const int pieces = HW / 8;
+    const int64_t planes = B * C;
+    if (planes >= 65536) return CLUSTEN_ERR_BAD_DIMS;
+    const dim3 grid((unsigned)min((pieces + 255) / 256, 64), (unsigned)planes);
     if (dtype == CLUSTEN_F16) {
-        hipLaunchKernelGGL(channel_affine_gelu_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream,
-                           static_cast<const f16_t*>(x), scale, shift, static_cast<f16_t*>(y), C, HW, pieces);
+        hipLaunchKernelGGL(channel_affine_gelu_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), scale,
+                           shift, static_cast<f16_t*>(y), C, pieces);
     } else if (dtype == CLUSTEN_BF16) {
-        hipLaunchKernelGGL(channel_affine_gelu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
-                           static_cast<const bf16_t*>(x), scale, shift, static_cast<bf16_t*>(y), C, HW, pieces);
+        hipLaunchKernelGGL(channel_affine_gelu_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x),
+                           scale, shift, static_cast<bf16_t*>(y), C, pieces);
     } else {
         return CLUSTEN_ERR_BAD_DTYPE;
     }

@@ -248,7 +248,7 @@ int clusten_channel_affine_gelu_forward(const void* x, const float* scale, const
     if (!x || !scale || !shift || !y) return CLUSTEN_ERR_NULL_POINTER;
     if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (B <= 0 || C <= 0 || HW <= 0 || HW % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
-    if ((B * C * HW / 8 + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (B * C >= 65536) return CLUSTEN_ERR_BAD_DIMS;  // one grid row per (image, channel) plane
     if (!aligned16(x) || !aligned16(y)) return CLUSTEN_ERR_UNALIGNED;
     return launch_channel_affine_gelu(x, scale, shift, y, B, C, HW, dtype, as_stream(stream));
 }
