@@ -236,6 +236,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
     ops.add_layer_norm = timed_call("layer_norm", real.add_layer_norm)
     ops.linear = timed_call("small Linear layers (+GELU) of stage 1", real.linear)
     ops.merge_weights = timed_call("merge_weights", real.merge_weights)
+    ops.channel_affine_gelu = timed_call("patch embedding epilogues", real.channel_affine_gelu)
     net = aff_model.aff_tiny(ops=ops).cuda().eval()
     for layer in net.layers:
         layer.neighbourhoods = timed_call("clustering+knn", layer.neighbourhoods)
@@ -317,9 +318,10 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
             "eager_img_per_s": round(timed * batch / dt, 1), "eager_ms_per_batch": round(dt / timed * 1e3, 2),
             "batch": batch, "warmup": warmup, "timed": timed,
             "dtype": "fp16 autocast (attention: one fp16 kernel per layer, fp32 sums; WF fp32)",
-            "inference_path": "16-bit weight copies kept between forwards; layer norm, merge weights, kNN, token "
-                              "ranking, local and global attention and the small Linear layers of stage 1 through "
-                              "the HIP library's optional entry points",
+            "inference_path": "16-bit weight copies, position-bias tables and merge-weight tables kept between "
+                              "forwards; layer norm (with the residual addition ahead of it), merge weights, kNN, token "
+                              "ranking, neighbour lists, local and global attention, the small Linear layers of stage 1 "
+                              "and the patch embedding's epilogues through the HIP library's optional entry points",
             "share_of_forward": share}
 
 
