@@ -320,6 +320,19 @@ int clusten_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* m
                             int64_t* pe_idx, int32_t* cluster_idx, int B, int N, int nnc, int m, int radius,
                             int table_width, clusten_stream stream);
 
+/* The importance score of every token before a merge (`self.prob_net(feat).sigmoid()`, a Linear layer with one
+ * output: models/aff_transformer.py:498), with the last block's residual addition (:232) taken along when branch is
+ * given:
+ *   sum_out[r,:] = x[r,:] + branch[r,:]                 (rounded to x's type; skipped when branch is NULL)
+ *   score[r]     = sigmoid( round_T( <round_T(sum_out[r,:]), weight> + bias ) ), rounded to T
+ * T = dtype, F16 or BF16: the type of weight (C), bias (1 element, or NULL), branch and score (rows); x and sum_out
+ * (rows,C) of x_dtype, F32 or dtype (else CLUSTEN_ERR_BAD_DTYPE); sum_out may be x.  C in {64,128,256,512} (else
+ * CLUSTEN_ERR_BAD_DIMS); everything contiguous, x / branch / sum_out / weight 16-byte aligned.  Inference only.  No
+ * counterpart in the reference's extension modules. */
+int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch, void* sum_out, const void* weight,
+                                  const void* bias, void* score, int64_t rows, int C, int dtype,
+                                  clusten_stream stream);
+
 /* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
  * (models/aff_transformer.py:340-358), in one pass instead of a row lookup, a gather and two multiplications:
  *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]

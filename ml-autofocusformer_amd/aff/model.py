@@ -46,8 +46,20 @@ def default_ops():
                            merge_weights=_native.merge_weights, merge_weights_supported=_native.merge_weights_supported,
                            channel_affine_gelu=_native.channel_affine_gelu,
                            channel_affine_gelu_supported=_native.channel_affine_gelu_supported,
+                           add_row_score=_native.add_row_score, add_row_score_supported=_native.add_row_score_supported,
                            neighbour_lists=_native.neighbour_lists,
                            neighbour_lists_supported=_native.neighbour_lists_supported)
+
+
+def _cast_params(lin, dt):
+    """(key, weight, bias) of an nn.Linear in dtype `dt`, kept until the parameters change."""
+    key = (dt, lin.weight._version, lin.weight.data_ptr(),
+           None if lin.bias is None else (lin.bias._version, lin.bias.data_ptr()))
+    cache = lin.__dict__.get("_cast_cache")
+    if cache is None or cache[0] != key:
+        cache = (key, lin.weight.detach().to(dt), None if lin.bias is None else lin.bias.detach().to(dt))
+        lin.__dict__["_cast_cache"] = cache      # a plain attribute: no parameter, no buffer, not in the state_dict
+    return cache
 
 
 def _linear(lin, x, ops=None, gelu=False):
@@ -59,12 +71,7 @@ def _linear(lin, x, ops=None, gelu=False):
         y = lin(x)
         return F.gelu(y) if gelu else y
     dt = torch.get_autocast_dtype("cuda")
-    key = (dt, lin.weight._version, lin.weight.data_ptr(),
-           None if lin.bias is None else (lin.bias._version, lin.bias.data_ptr()))
-    cache = lin.__dict__.get("_cast_cache")
-    if cache is None or cache[0] != key:
-        cache = (key, lin.weight.detach().to(dt), None if lin.bias is None else lin.bias.detach().to(dt))
-        lin.__dict__["_cast_cache"] = cache      # a plain attribute: no parameter, no buffer, not in the state_dict
+    cache = _cast_params(lin, dt)
     x = x if x.dtype == dt else x.to(dt)
     fn = getattr(ops, "linear", None)
     if fn is not None and ops.linear_supported(x, cache[1], gelu):
@@ -454,13 +461,23 @@ class BasicLayer(nn.Module):
         carry = None
         for blk in self.blocks:
             feat, carry = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists, carry)
+        learned_prob = None
+        scorer = getattr(self.ops, "add_row_score", None)
+        if (self.downsample is not None and scorer is not None and not torch.is_grad_enabled() and feat.is_cuda
+                and torch.is_autocast_enabled("cuda")):
+            # inference: the last residual addition and the importance score of the tokens in one pass
+            _, w16, b16 = _cast_params(self.prob_net, torch.get_autocast_dtype("cuda"))
+            if self.ops.add_row_score_supported(feat, carry, w16):
+                feat, learned_prob = scorer(feat, carry, w16, b16)
+                carry = None
         if carry is not None:
             feat = feat + carry
 
         if self.downsample is not None:
             if global_attn:   # merging after a dense stage: every token is every token's neighbour
                 member_idx = torch.arange(n, device=feat.device).expand(b, n, n).contiguous()
-            learned_prob = _linear(self.prob_net, feat).sigmoid()
+            if learned_prob is None:
+                learned_prob = _linear(self.prob_net, feat).sigmoid()
             reserve_num = math.ceil(h / (stride * 2)) * math.ceil(w / (stride * 2))
             pos, feat = self.downsample(pos, feat, member_idx, mask, learned_prob, stride, pe_idx, reserve_num, table)
         return pos, feat

@@ -65,6 +65,8 @@ _PROTOTYPES = {
                                                       ctypes.c_int, ctypes.c_float, ctypes.c_int, _P]),
     "clusten_channel_affine_gelu_forward": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                           ctypes.c_int, _P]),
+    "clusten_add_row_score_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, _P, _P, _P, _P, ctypes.c_int64, ctypes.c_int,
+                                                    ctypes.c_int, _P]),
     "clusten_add_layer_norm_forward": (ctypes.c_int, [_P, ctypes.c_int, _P, ctypes.c_int, _P, _P, _P, _P, ctypes.c_int64,
                                                      ctypes.c_int, ctypes.c_float, _P]),
     "clusten_neighbour_lists": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -775,6 +777,54 @@ def neighbour_lists(pos: torch.Tensor, nearest: torch.Tensor, m: int, radius: in
                                            _stream(device)),
                "clusten_neighbour_lists")
     return member_idx, mask, pe_idx, cluster_idx
+
+
+def add_row_score_supported(x: torch.Tensor, branch, weight: torch.Tensor) -> bool:
+    """True when `add_row_score` takes this case: CUDA tensors, weight (1,C) or (C,) fp16 / bf16 with C in
+    {64,128,256,512}, x (...,C) fp32 or of weight's type, branch None or of x's shape and weight's type."""
+    if not (x.is_cuda and weight.is_cuda and weight.dtype in (torch.float16, torch.bfloat16)):
+        return False
+    if x.dim() < 1 or x.shape[-1] not in (64, 128, 256, 512) or weight.numel() != x.shape[-1]:
+        return False
+    if x.dtype not in (torch.float32, weight.dtype):
+        return False
+    return branch is None or (branch.is_cuda and branch.dtype == weight.dtype and branch.shape == x.shape)
+
+
+def add_row_score(x: torch.Tensor, branch, weight: torch.Tensor, bias):
+    """(x + branch, sigmoid(F.linear((x + branch).to(T), weight, bias))) with T = weight's 16-bit dtype — or
+    (x, sigmoid(...)) when branch is None: the importance score of the tokens before a merge
+    (models/aff_transformer.py:498) and the residual addition ahead of it, in one pass.  The score has shape
+    x.shape[:-1] + (1,) and dtype T.  No autograd: for inference."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    _require_cuda("weight", weight, device)
+    if not add_row_score_supported(x, branch, weight):
+        raise RuntimeError("add_row_score: weight fp16 / bf16 of 64, 128, 256 or 512 elements, x fp32 or of weight's "
+                           "type, branch of x's shape and weight's type")
+    c = x.shape[-1]
+    code = _DTYPE_CODES[weight.dtype]
+    x = x.detach().contiguous()
+    weight = weight.detach().contiguous()
+    if bias is not None:
+        _require_cuda("bias", bias, device)
+        if bias.numel() != 1 or bias.dtype != weight.dtype:
+            raise RuntimeError("bias must be one element of weight's dtype")
+        bias = bias.detach().contiguous()
+    total = x
+    if branch is not None:
+        branch = branch.detach().contiguous()
+        total = torch.empty_like(x)
+    score = torch.empty(x.shape[:-1] + (1,), dtype=weight.dtype, device=device)
+    if score.numel() == 0:
+        return total, score
+    with torch.cuda.device(device):
+        _check(lib.clusten_add_row_score_forward(_ptr(x), _DTYPE_CODES[x.dtype], _ptr(branch),
+                                                 _ptr(total) if branch is not None else None, _ptr(weight), _ptr(bias),
+                                                 _ptr(score), x.numel() // c, c, code, _stream(device)),
+               "clusten_add_row_score_forward")
+    return total, score
 
 
 def merge_weights_supported(table_weights: torch.Tensor) -> bool:

@@ -279,6 +279,19 @@ int clusten_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* m
                                   as_stream(stream));
 }
 
+int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch, void* sum_out, const void* weight,
+                                  const void* bias, void* score, int64_t rows, int C, int dtype,
+                                  clusten_stream stream) {
+    if (!x || !weight || !score || (branch && !sum_out)) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (x_dtype != CLUSTEN_F32 && x_dtype != dtype) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(weight) || (branch && (!aligned16(branch) || !aligned16(sum_out)))) {
+        return CLUSTEN_ERR_UNALIGNED;
+    }
+    return launch_add_row_score(x, x_dtype, branch, sum_out, weight, bias, score, rows, C, dtype, as_stream(stream));
+}
+
 int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
                                   const float* prob, const int64_t* mask, float* weights, int B, int N, int Nout, int M,
                                   int IC, clusten_stream stream) {

@@ -104,6 +104,10 @@ int launch_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* me
                            int32_t* cluster_idx, int B, int N, int nnc, int m, int radius, int table_width,
                            hipStream_t stream);
 
+// score[r] = sigmoid(<x[r] (+ branch[r]), w> + b) with the sum written to sum_out: see row_score.hip.
+int launch_add_row_score(const void* x, int x_dtype, const void* branch, void* sum_out, const void* w, const void* b,
+                         void* score, int64_t rows, int C, int dtype, hipStream_t stream);
+
 // w[b,i,j,:4] = table_w[pe_idx[b,i,j], :4] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]   (prob, mask may be null)
 //   table_w (rows,4), prob (B,N), w (B,Nout,M,4): fp32;  pe_idx, nbhd_idx, mask: int64 (B,Nout,M).
 int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,

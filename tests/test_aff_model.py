@@ -393,6 +393,35 @@ def test_channel_affine_gelu_kernel_equals_bias_batch_norm_gelu(device, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_add_row_score_kernel_equals_addition_linear_sigmoid(device, dtype):
+    """The importance score of the tokens with the residual addition ahead of it: the sum equals the framework's
+    addition bit for bit, the score is sigmoid(Linear(sum in 16 bits)) with the product rounded to 16 bits first."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(41)
+    for x_dtype in (torch.float32, dtype):
+        for shape, c in (((3, 203), 64), ((2, 77), 128), ((5, 19), 256), ((1, 9), 512)):
+            x = torch.randn(*shape, c, generator=gen).to(x_dtype).to(device)
+            branch = torch.randn(*shape, c, generator=gen).to(dtype).to(device)
+            w = (torch.randn(1, c, generator=gen) * c ** -0.5).to(dtype).to(device)
+            b = torch.randn(1, generator=gen).to(dtype).to(device)
+            for br in (branch, None):
+                assert _native.add_row_score_supported(x, br, w)
+                total, score = _native.add_row_score(x, br, w, b)
+                want_total = x if br is None else x + br
+                assert total.dtype == x.dtype and torch.equal(total, want_total)
+                y = torch.nn.functional.linear(want_total.to(dtype).float(), w.float(), b.float()).to(dtype)
+                want = torch.sigmoid(y.float())
+                assert score.dtype == dtype and score.shape == tuple(shape) + (1,)
+                assert oracle.rel_err(score.float().cpu(), want.cpu()) <= (2e-3 if dtype == torch.float16 else 1.6e-2)
+    assert not _native.add_row_score_supported(x, None, w.float())
+    assert not _native.add_row_score_supported(x[..., :96], None, w[:, :96])
+    assert not _native.add_row_score_supported(x, branch.float(), w)
+    with pytest.raises(RuntimeError):
+        _native.add_row_score(x, None, w.float(), None)
+
+
+@pytest.mark.gpu
 def test_merge_weights_kernel_equals_the_tensor_expressions(device):
     from clusten import _native
     gen = torch.Generator().manual_seed(19)
@@ -479,6 +508,7 @@ def test_aff_tiny_224_logits_equal_with_hip_operators_and_with_the_oracle(device
     del three.linear
     del three.add_layer_norm
     del three.neighbour_lists
+    del three.add_row_score
     del three.channel_affine_gelu
     hip3 = aff_tiny(ops=three).to(device).eval()
     hip3.load_state_dict(hip.state_dict())
