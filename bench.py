@@ -336,7 +336,7 @@ def main():
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
-    ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd"), default=None,
+    ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model"), default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -370,6 +370,11 @@ def main():
            lambda: _native.av_forward(attn, v, idx),
            lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
     torch.cuda.synchronize()
+    if args.only == "bwd-model":  # the same on lists as the model builds them (whole clusters, nearest first)
+        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model")
+        print(json.dumps({"only": "bwd-model", "launches": args.steps + args.warmup,
+                          **_bench_backward(mcase, wcase, args.steps, args.warmup)}), flush=True)
+        return
     if args.only == "bwd":  # the three backward operators, for profilers
         print(json.dumps({"only": "bwd", "launches": args.steps + args.warmup,
                           **_bench_backward(acase, wcase, args.steps, args.warmup)}), flush=True)

@@ -222,6 +222,29 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* The scatter of the two attention backward passes as a gather, for neighbour lists made of whole clusters
+ * (nbhd_idx[b,i,8r+t] = 8 c(b,i,r) + t, the lists of models/aff_transformer.py:476-480):
+ *   y[b,h, 8g+t, :] = sum over the pairs (i,r) with c(b,i,r) = g of  p[b,h,i,8r+t] * x[b,h,i,:]
+ * which equals the d_key of clusten_qk_backward (p = d_attn, x = query) and the d_value of clusten_av_backward
+ * (p = attn, x = d_feat) on such lists, without atomics, zero-fill or workspace, and with sums that do not depend on
+ * the order of execution.  The caller lists the pairs of every cluster once (shared by the heads, and by every
+ * layer that uses the same lists): pairs (B*N*M/8) int32 holds i*8 + r, grouped by (b, g) in any order inside a
+ * group; pair_offsets (B*N/8 + 1) int32 holds the start of every group in it.
+ * p (B,H,N,M) and y (B,H,N,C) contiguous, x strided (B,H,N,C), all of `dtype` (F32, F16 or BF16); every row of y is
+ * written.  C = 32, N % 8 == 0, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the reference's
+ * extension modules. */
+/* First step towards the pair lists clusten_scatter_rows_by_cluster reads: keys[(b*N+i)*M/8 + r] = b*N/8 + c for
+ * every run of 8 list entries nbhd_idx[b,i,8r..8r+7] = 8c..8c+7 with 0 <= 8c <= N-8; any other run sets *not_whole
+ * (which the caller clears first) to 1.  Sorting the keys gives `pairs` (position of each key: i*8 + r), the first
+ * position of every key value `pair_offsets`.  nbhd_idx (B,N,M) int64, keys (B*N*M/8) int32; N % 8 == M % 8 == 0
+ * (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the reference's extension modules. */
+int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M,
+                         clusten_stream stream);
+
+int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides,
+                                    const int32_t* pair_offsets, const int32_t* pairs, void* y,
+                                    clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* Attention of every token over every token of a short sequence, fused: the branch the reference model takes in
  * a stage whose neighbourhood size reaches its number of tokens (models/aff_transformer.py:108-113 and :125-155:
  * `q @ key^T`, position bias, blank token, softmax, `attn @ v`, blank value), without the (B,H,N,N) logits and

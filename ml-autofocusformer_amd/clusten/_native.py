@@ -54,6 +54,8 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
+    "clusten_cluster_keys": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_scatter_rows_by_cluster": (ctypes.c_int, [_P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
                                                       ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_linear_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -195,6 +197,84 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -
     return attn
 
 
+_PAIR_CACHE: "dict" = {}       # lists seen lately -> their pairs by cluster, or None when they are not whole clusters
+_PAIR_CACHE_SIZE = 8
+BY_CLUSTER_MIN_ROWS = 1 << 16  # b*n from which the backward scatters go cluster by cluster
+
+
+def cluster_pairs(nbhd_idx: torch.Tensor):
+    """For lists made of whole clusters (nbhd_idx[b,i,8r+t] = 8 c + t with c = c(b,i,r), every entry a row of the
+    sequence, n and m multiples of 8, m <= 64): (pair_offsets, pairs), int32 tensors that list, for every cluster
+    (b,g), the pairs (i,r) with c(b,i,r) = g as i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other
+    list.  One sort of the b*n*m/8 cluster numbers and one look at the result from the host; the answer is kept for
+    the lists seen lately (the layers of a stage share theirs), keyed by the tensor's memory and version."""
+    if nbhd_idx.dim() != 3 or not nbhd_idx.is_cuda or nbhd_idx.dtype != torch.int64:
+        return None
+    B, N, M = nbhd_idx.shape
+    if B == 0 or N == 0 or N % 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
+        return None
+    key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, nbhd_idx.device.index)
+    hit = _PAIR_CACHE.get(key)
+    if hit is not None:
+        return hit[1]
+    R = M // 8
+    K = N // 8
+    if B * K >= 1 << 31 or B * N * R >= 1 << 31:
+        return None
+    device = nbhd_idx.device
+    keys = torch.empty(B * N * R, dtype=torch.int32, device=device)
+    not_whole = torch.zeros(1, dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        _check(load().clusten_cluster_keys(_ptr(nbhd_idx), _ptr(keys), _ptr(not_whole), B, N, M, _stream(device)),
+               "clusten_cluster_keys")
+    result = None
+    if int(not_whole) == 0:                      # the one host synchronisation
+        ordered, order = torch.sort(keys)
+        pairs = (((order // R) % N) * 8 + order % R).to(torch.int32)
+        offsets = torch.searchsorted(ordered, torch.arange(B * K + 1, dtype=torch.int32, device=device),
+                                     out_int32=True)
+        result = (offsets, pairs)
+    if len(_PAIR_CACHE) >= _PAIR_CACHE_SIZE:
+        _PAIR_CACHE.pop(next(iter(_PAIR_CACHE)))
+    _PAIR_CACHE[key] = (nbhd_idx, result)        # the tensor is held: its address cannot be reused meanwhile
+    return result
+
+
+def scatter_rows_by_cluster(p: torch.Tensor, x: torch.Tensor, pair_lists) -> torch.Tensor:
+    """y (b,h,n,32) with y[b,h,8g+t] = sum over the pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i]: the d_key /
+    d_value of the attention backward passes for lists made of whole clusters, `pair_lists` from `cluster_pairs`."""
+    lib = load()
+    _require_cuda("p", p)
+    device = p.device
+    _require_cuda("x", x, device)
+    if p.dim() != 4 or x.dim() != 4 or p.shape[:3] != x.shape[:3] or p.dtype != x.dtype:
+        raise RuntimeError("p must be (b,h,n,m) and x (b,h,n,c) of one dtype")
+    B, H, N, C = x.shape
+    M = p.shape[3]
+    offsets, pairs = pair_lists
+    if offsets.numel() != B * (N // 8) + 1 or pairs.numel() != B * N * (M // 8) or C != 32 or N % 8 or M % 8:
+        raise RuntimeError("scatter_rows_by_cluster: head dim 32, n and m multiples of 8, pair lists of these lists")
+    code = _dtype_code(p, "p")
+    p, x = p.contiguous(), _rows(x)
+    y = torch.empty((B, H, N, C), dtype=p.dtype, device=device)
+    if y.numel() == 0:
+        return y
+    shape = AttnShape(B, H, N, C, M)
+    with torch.cuda.device(device):
+        _check(lib.clusten_scatter_rows_by_cluster(_ptr(p), _ptr(x), _strides(x), _ptr(offsets), _ptr(pairs), _ptr(y), shape,
+                                                   code, _stream(device)),
+               "clusten_scatter_rows_by_cluster")
+    return y
+
+
+def _pairs_for_backward(nbhd_idx: torch.Tensor, shape) -> "tuple | None":
+    """The pair lists when the backward scatter of this problem goes cluster by cluster: head dim 32, lists made of
+    whole clusters, and enough rows for the sort of the lists to pay."""
+    if shape.C != 32 or shape.B * shape.N < BY_CLUSTER_MIN_ROWS or torch.cuda.is_current_stream_capturing():
+        return None
+    return cluster_pairs(nbhd_idx)
+
+
 def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor):
     """(d_query, d_key), both contiguous (b,h,n,c)."""
     lib = load()
@@ -203,6 +283,11 @@ def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nb
     if tuple(d_attn.shape) != (shape.B, shape.H, shape.N, shape.M) or d_attn.dtype != query.dtype:
         raise RuntimeError("d_attn must be (b,h,n,m) with the dtype of query")
     d_attn = d_attn.contiguous()
+    if d_attn.numel() != 0 and shape.M != 0:
+        lists = _pairs_for_backward(idx, shape)
+        if lists is not None:
+            # lists of whole clusters: d_query is the AV forward on (d_attn, key), d_key a gather cluster by cluster
+            return av_forward(d_attn, key, idx), scatter_rows_by_cluster(d_attn, query, lists)
     query, key = _rows(query), _rows(key)
     d_query = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=query.dtype, device=device)
     d_key = torch.empty_like(d_query)
@@ -257,6 +342,11 @@ def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_
     if tuple(attn.shape) != (shape.B, shape.H, shape.N, shape.M) or attn.dtype != v.dtype:
         raise RuntimeError("attn must be (b,h,n,m) with the dtype of v")
     attn = attn.contiguous()
+    if attn.numel() != 0 and shape.M != 0:
+        lists = _pairs_for_backward(idx, shape)
+        if lists is not None:
+            # lists of whole clusters: d_attn is the QK forward on (d_feat, v), d_v a gather cluster by cluster
+            return qk_forward(d_feat, v, idx), scatter_rows_by_cluster(attn, d_feat, lists)
     d_feat, v = _rows(d_feat), _rows(v)
     d_attn = torch.empty((shape.B, shape.H, shape.N, shape.M), dtype=attn.dtype, device=device)
     d_v = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=attn.dtype, device=device)

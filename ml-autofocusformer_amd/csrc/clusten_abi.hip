@@ -187,6 +187,26 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     dtype, as_stream(stream));
 }
 
+int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M,
+                         clusten_stream stream) {
+    if (!nbhd_idx || !keys || !not_whole) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || M <= 0 || N % 8 != 0 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((int64_t)B * (N / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
+        return CLUSTEN_ERR_BAD_DIMS;
+    }
+    return launch_cluster_keys(nbhd_idx, keys, not_whole, B, N, M, as_stream(stream));
+}
+
+int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const int32_t* pair_offsets,
+                                    const int32_t* pairs, void* y, clusten_attn_shape shape, int dtype,
+                                    clusten_stream stream) {
+    if (!p || !x || !pair_offsets || !pairs || !y) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(x_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_scatter_by_cluster(p, x, x_strides, pair_offsets, pairs, y, shape, dtype, as_stream(stream));
+}
+
 int clusten_dense_attention_forward(const void* query, clusten_strides query_strides, const void* key,
                                     clusten_strides key_strides, const void* value, clusten_strides value_strides,
                                     const void* bias_table, const int64_t* pe_idx, const float* blank_key,

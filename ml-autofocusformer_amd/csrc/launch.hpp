@@ -66,6 +66,11 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
                              hipStream_t stream);
 
+// y[b,h,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i,:]: see scatter_by_cluster.hip.
+int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, hipStream_t stream);
+int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* offsets,
+                              const int32_t* pairs, void* y, clusten_attn_shape s, int dtype, hipStream_t stream);
+
 // Attention of every token over every token (N <= 64) in one kernel: see dense_attention.hip.  q, k, v, out : strided
 //   (B,H,N,C) of T in {F16, BF16}, C = 32; table (rows,H) of T; pe_idx int64 (B,N,N); blank_k, blank_v : fp32 (H,C).
 int launch_dense_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,

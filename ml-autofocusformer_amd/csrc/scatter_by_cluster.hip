@@ -1,0 +1,187 @@
+// scatter_by_cluster: the scatter of the attention backward passes, turned into a gather (no atomics).
+//
+//   y[b,h, idx[b,i,j], :] += p[b,h,i,j] * x[b,h,i,:]          (d_key with p = d_attn, x = query;
+//                                                              d_value with p = attn, x = d_out:
+//                                                              clusten/src/clustenqk_cuda_kernel.cu:96-133,
+//                                                              clustenav_cuda_kernel.cu:96-131)
+//
+// for neighbour lists made of whole clusters: idx[b,i,8r+t] = 8 c(b,i,r) + t, the lists the reference model
+// builds (models/aff_transformer.py:476-480).  Then the 8 rows of cluster g receive
+//
+//   y[b,h, 8g + t, :] = sum over the pairs (i, r) with c(b,i,r) = g of  p[b,h,i,8r+t] * x[b,h,i,:]
+//
+// and, with the pairs of every cluster listed once (a sort of the cluster numbers, shared by the heads and by every
+// layer of a stage), each cluster is an independent small matrix product Y_g (8 x C) = P_g^T (8 x pairs) X_g (pairs x C):
+// one wave per cluster walks the heads, the x rows and the 8-element pieces of p of 32 pairs at a time travel to LDS by
+// LDS-direct loads, and the product runs on `v_mfma_f32_16x16x4_f32` (16-bit data is widened when the operands are
+// read from LDS; rows 8-15 of the instruction are idle).  Every row of y is written exactly once: no atomics, no
+// zero-fill, no fp32 workspace for 16-bit data, and the sums do not depend on the order in which workgroups run.
+// It has no counterpart in the reference's extension modules.
+#include "launch.hpp"
+#include "mfma.hpp"
+
+namespace clusten {
+namespace {
+
+constexpr int kC = 32;           // head dim
+constexpr int kPass = 32;        // pairs per pass
+constexpr int kListMax = 256;    // pairs of a cluster held in LDS at a time
+
+template <typename T>
+__global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __restrict__ p, const T* __restrict__ x,
+                                                                   clusten_strides xs, const int32_t* __restrict__ offsets,
+                                                                   const int32_t* __restrict__ pairs, T* __restrict__ y,
+                                                                   int H, int N, int M, int clusters_per_image,
+                                                                   int total_clusters) {
+    constexpr int EB = (int)sizeof(T);
+    constexpr int ROW_B = kC * EB;                   // bytes of an x row
+    constexpr int PIECE_B = 8 * EB;                  // bytes of the 8 elements of p a pair contributes
+    constexpr int X_BYTES = kPass * ROW_B;
+    constexpr int X_DMA = X_BYTES / 1024;            // LDS-direct loads per pass for the x rows
+    constexpr int ROWS_PER_DMA = 1024 / ROW_B;
+    constexpr int LANES_PER_ROW = ROW_B / 16;
+    constexpr int X_BASE = 0;
+    constexpr int P_BASE = X_BASE + X_BYTES;
+    constexpr int O_BASE = P_BASE + 1024;
+    constexpr int L_BASE = O_BASE + 8 * kC * 4;
+    constexpr int LDS_BYTES = L_BASE + kListMax * 4;
+    __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
+
+    const int unit = xcd_tile(blockIdx.x, total_clusters);
+    if (unit < 0) return;
+    const int b = unit / clusters_per_image;
+    const int g = unit - b * clusters_per_image;
+    const int lane = threadIdx.x;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int first = offsets[unit];
+    const int count = offsets[unit + 1] - first;
+    int* list = reinterpret_cast<int*>(stage + L_BASE);
+
+    // a cluster listed by more than kListMax pairs is taken in segments; the later segments add to what is stored
+    for (int seg = 0; seg == 0 || seg < count; seg += kListMax) {
+        const int n = min(kListMax, count - seg);   // <= 0 only for a cluster nobody lists: its rows become zero
+        lds_sync();
+        for (int e = lane; e < n; e += kWave) list[e] = pairs[first + seg + e];
+        lds_sync();
+        for (int h = 0; h < H; ++h) {
+            const char* x_bh = reinterpret_cast<const char*>(x + (int64_t)b * xs.b + (int64_t)h * xs.h);
+            const char* p_bh = reinterpret_cast<const char*>(p + ((int64_t)b * H + h) * N * M);
+            F32x4 acc[2] = {F32x4{0.f, 0.f, 0.f, 0.f}, F32x4{0.f, 0.f, 0.f, 0.f}};
+            for (int base = 0; base < n; base += kPass) {
+                const int here = min(kPass, n - base);
+                lds_sync();  // the previous pass has been read
+#pragma unroll
+                for (int a = 0; a < X_DMA; ++a) {
+                    const int e = list[base + min(ROWS_PER_DMA * a + lane / LANES_PER_ROW, here - 1)];
+                    CLUSTEN_LDS_DMA16(x_bh + lane_offset((uint32_t)(e >> 3) * (uint32_t)xs.n * EB +
+                                                         (uint32_t)(lane % LANES_PER_ROW) * 16),
+                                      stage + X_BASE + a * 1024);
+                }
+                {
+                    // 32 pieces of PIECE_B bytes: 16 bytes per lane
+                    constexpr int LANES_PER_PIECE = PIECE_B / 16;
+                    if (lane < kPass * LANES_PER_PIECE) {
+                        const int e = list[base + min(lane / LANES_PER_PIECE, here - 1)];
+                        CLUSTEN_LDS_DMA16(p_bh + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * EB +
+                                                             (uint32_t)(lane % LANES_PER_PIECE) * 16),
+                                          stage + P_BASE);
+                    }
+                }
+                lds_sync_vm<0>();
+#pragma unroll
+                for (int s = 0; s < kPass / 4; ++s) {
+                    if (4 * s < here) {
+                        const int pr = 4 * s + kq;
+                        const T* pp = reinterpret_cast<const T*>(stage + P_BASE + pr * PIECE_B) + (r16 & 7);
+                        const float a = (r16 < 8 && pr < here) ? to_acc(*pp) : 0.f;
+                        const T* xp = reinterpret_cast<const T*>(stage + X_BASE + pr * ROW_B) + r16;
+                        const float b0 = to_acc(xp[0]), b1 = to_acc(xp[16]);
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b0, acc[0], 0, 0, 0);
+                        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b1, acc[1], 0, 0, 0);
+                    }
+                }
+            }
+            // rows 4*kq + j of the result (kq < 2: the cluster's 8 rows), channels 16*cb + r16
+            T* y_rows = y + (((int64_t)b * H + h) * N + (int64_t)g * 8) * kC;
+            lds_sync();
+            if (kq < 2) {
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        reinterpret_cast<float*>(stage + O_BASE)[(4 * kq + j) * kC + 16 * cb + r16] = acc[cb][j];
+                    }
+                }
+            }
+            lds_sync();
+            {
+                // 8 rows x 32 channels: four consecutive channels per lane
+                const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
+                float v[4] = {o[0], o[1], o[2], o[3]};
+                if (seg > 0) {
+                    float old[4];
+                    Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(y_rows + lane * 4), old);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += old[e];
+                }
+                *reinterpret_cast<typename Quad<T>::raw*>(y_rows + lane * 4) = Quad<T>::pack(v);
+            }
+        }
+    }
+}
+
+// keys[(b*N + i)*R + r] = b * (N/8) + c for lists made of whole clusters (idx[b,i,8r+t] = 8c + t, 0 <= 8c <= N-8);
+// any other run of 8 entries sets *not_whole to 1.  One thread per run: 64 bytes of the list.
+__global__ __launch_bounds__(256) void cluster_keys_kernel(const int64_t* __restrict__ idx, int32_t* __restrict__ keys,
+                                                           int32_t* __restrict__ not_whole, int N, int R, int64_t runs) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= runs) return;
+    const int64_t* run = idx + e * 8;
+    const int64_t head = run[0];
+    bool ok = (head & 7) == 0 && head >= 0 && head <= N - 8;
+#pragma unroll
+    for (int t = 1; t < 8; ++t) ok = ok && run[t] == head + t;
+    const int64_t b = e / ((int64_t)N * R);
+    keys[e] = ok ? (int32_t)(b * (N / 8) + (head >> 3)) : 0;
+    if (!ok) atomicOr(not_whole, 1);
+}
+
+template <typename T>
+int launch_typed(const void* p, const void* x, clusten_strides xs, const int32_t* offsets, const int32_t* pairs, void* y,
+                 const clusten_attn_shape& s, hipStream_t stream) {
+    const int per_image = s.N / 8;
+    const int64_t total = (int64_t)s.B * per_image;
+    if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
+    hipLaunchKernelGGL((scatter_by_cluster_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWave), 0, stream,
+                       static_cast<const T*>(p), static_cast<const T*>(x), xs, offsets, pairs, static_cast<T*>(y), s.H, s.N,
+                       s.M, per_image, (int)total);
+    return launch_status();
+}
+
+}  // namespace
+
+int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, hipStream_t stream) {
+    const int R = M / 8;
+    const int64_t runs = (int64_t)B * N * R;
+    hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, stream, idx, keys, not_whole,
+                       N, R, runs);
+    return launch_status();
+}
+
+int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* offsets,
+                              const int32_t* pairs, void* y, clusten_attn_shape s, int dtype, hipStream_t stream) {
+    if (s.C != kC || s.N % 8 != 0 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    const size_t eb = dtype_size(dtype);
+    if (!rows_aligned16(x, xs, (int)eb) || !aligned16(p) || !aligned16(y) || !slice_fits_int32(xs, s.H, s.N, s.C) ||
+        (int64_t)s.N * s.M * (int64_t)eb >= ((int64_t)1 << 31)) {
+        return CLUSTEN_ERR_UNALIGNED;
+    }
+    switch (dtype) {
+        case CLUSTEN_F32: return launch_typed<float>(p, x, xs, offsets, pairs, y, s, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(p, x, xs, offsets, pairs, y, s, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(p, x, xs, offsets, pairs, y, s, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
+}  // namespace clusten

@@ -78,6 +78,65 @@ def test_attn_backward_lists_made_of_runs(device, kind, dtype):
         _check_attn_backward(wl.attn_case("runs", 77, B=2, H=h, N=396, C=c, M=m, lists="runs:" + kind), device, dtype)
 
 
+@pytest.fixture
+def by_cluster(monkeypatch):
+    """The cluster-by-cluster scatter for problems of any size (in production it starts at 65536 rows)."""
+    monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
+    _native._PAIR_CACHE.clear()
+    yield
+    _native._PAIR_CACHE.clear()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_attn_backward_cluster_by_cluster(device, dtype, by_cluster):
+    """Lists made of whole clusters: d_key / d_value as a gather over the pairs of every cluster (no atomics)."""
+    g = torch.Generator().manual_seed(79)
+    for B, H, N, nnc in ((2, 3, 200, 6), (1, 2, 392, 6), (3, 1, 64, 8), (2, 2, 24, 3)):
+        idx = wl.model_like_lists(B, N, g, nnc=min(nnc, N // 8))
+        assert _native.cluster_pairs(idx.to(device)) is not None
+        case = wl.attn_case("model", 80, B=B, H=H, N=N, C=32, M=idx.shape[-1])
+        case.nbhd_idx = idx
+        _check_attn_backward(case, device, dtype)
+
+
+def test_cluster_by_cluster_scatter_properties(device, by_cluster):
+    g = torch.Generator().manual_seed(81)
+    B, H, N, C = 2, 3, 200, 32
+    idx = wl.model_like_lists(B, N, g).to(device)
+    M = idx.shape[-1]
+    lists = _native.cluster_pairs(idx)
+    offsets, pairs = lists
+    assert offsets.dtype == torch.int32 and offsets.numel() == B * N // 8 + 1 and int(offsets[-1]) == B * N * M // 8
+    assert _native.cluster_pairs(idx) is lists                       # kept for the lists seen lately
+    # integer-valued data: every product and sum exact, so the result equals the oracle's bit for bit
+    q = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    k = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
+    d_attn = torch.randint(-4, 5, (B, H, N, M), generator=g).float()
+    dq_ref, dk_ref = oracle.qk_gather_backward(d_attn, q, k, idx.cpu())
+    dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx)
+    assert torch.equal(dq.cpu(), dq_ref) and torch.equal(dk.cpu(), dk_ref)
+    # no atomics: two runs on random data give the same bits
+    x = torch.randn(B, H, N, C, generator=g).to(device)
+    p = torch.randn(B, H, N, M, generator=g).to(device)
+    assert torch.equal(_native.scatter_rows_by_cluster(p, x, lists), _native.scatter_rows_by_cluster(p, x, lists))
+    # a cluster nobody lists receives zeros; one listed by more pairs than a wave holds at once is taken in segments
+    lone = torch.zeros(1, 2400, 48, dtype=torch.int64)
+    lone[:] = (torch.arange(48) % 8) + 8 * (torch.arange(48) // 8 + 1)          # everybody lists clusters 1..6
+    lone = lone.to(device)
+    lists2 = _native.cluster_pairs(lone)
+    x2 = torch.randn(1, 2, 2400, C, generator=g)
+    p2 = torch.randn(1, 2, 2400, 48, generator=g)
+    want = oracle.qk_gather_backward(p2, x2, x2, lone.cpu())[1]
+    got = _native.scatter_rows_by_cluster(p2.to(device), x2.to(device), lists2)
+    assert oracle.rel_err(got, want) <= TOL_SCATTER_F32 and float(got[:, :, :8].abs().max()) == 0.0
+    # lists that are not whole clusters keep the atomic path
+    assert _native.cluster_pairs(torch.randint(N, (B, N, M), generator=g).to(device)) is None
+    shifted = idx.clone()
+    shifted[0, 0, :8] += 1
+    assert _native.cluster_pairs(shifted.clamp_(max=N - 1)) is None
+    assert _native.cluster_pairs(idx[:, :, :44].contiguous()) is None
+
+
 def test_scatter_union_path_is_bit_exact_on_integer_data(device):
     g = torch.Generator().manual_seed(78)
     B, H, N, C = 2, 3, 200, 32
