@@ -233,13 +233,27 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
  * p (B,H,N,M) and y (B,H,N,C) contiguous, x strided (B,H,N,C), all of `dtype` (F32, F16 or BF16); every row of y is
  * written.  C = 32, N % 8 == 0, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the reference's
  * extension modules. */
-/* First step towards the pair lists clusten_scatter_rows_by_cluster reads: keys[(b*N+i)*M/8 + r] = b*N/8 + c for
- * every run of 8 list entries nbhd_idx[b,i,8r..8r+7] = 8c..8c+7 with 0 <= 8c <= N-8; any other run sets *not_whole
- * (which the caller clears first) to 1.  Sorting the keys gives `pairs` (position of each key: i*8 + r), the first
- * position of every key value `pair_offsets`.  nbhd_idx (B,N,M) int64, keys (B*N*M/8) int32; N % 8 == M % 8 == 0
- * (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the reference's extension modules. */
-int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M,
+/* First step towards the pair lists clusten_scatter_rows_by_cluster and clusten_wf_backward_by_cluster read:
+ * keys[(b*N+i)*M/8 + r] = b*n_rows/8 + c for every run of 8 list entries nbhd_idx[b,i,8r..8r+7] = 8c..8c+7 with
+ * 0 <= 8c <= n_rows-8 (n_rows: the length of the sequence the lists point into; N for attention, the finer sequence
+ * for WF); any other run sets *not_whole (which the caller clears first) to 1.  Sorting the keys gives `pairs` (the
+ * position of each key: i*8 + r) and `pair_offsets` (the first position of every key value).  nbhd_idx (B,N,M)
+ * int64, keys (B*N*M/8) int32; n_rows % 8 == M % 8 == 0 (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the
+ * reference's extension modules. */
+int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int n_rows,
                          clusten_stream stream);
+
+/* clusten_wf_backward for lists made of whole clusters, the feature gradient as a gather (no atomics, no workspace,
+ * every row of d_feat written once):
+ *   d_feat[b, 8g+t, :] = sum over the pairs (i,r) of cluster (b,g) of  sum_ic weights[b,i,8r+t,ic] * d_feat_new[b,i,ic,:]
+ * with pair_offsets (B*N/8 + 1) and pairs (B*Nout*M/8) as for clusten_scatter_rows_by_cluster (i counts the output
+ * tokens, g the clusters of the N feature rows); d_weights as clusten_wf_backward computes it.  IC = 4, C % 32 == 0,
+ * N % 8 == 0, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS); dtype F32, F16 or BF16.  No counterpart in the
+ * reference's extension modules. */
+int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat,
+                                   const int64_t* nbhd_idx, const int32_t* pair_offsets, const int32_t* pairs,
+                                   void* d_weights, void* d_feat, clusten_wf_shape shape, int dtype,
+                                   clusten_stream stream);
 
 int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides,
                                     const int32_t* pair_offsets, const int32_t* pairs, void* y,

@@ -54,7 +54,8 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
-    "clusten_cluster_keys": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_cluster_keys": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_wf_backward_by_cluster": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
     "clusten_scatter_rows_by_cluster": (ctypes.c_int, [_P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
                                                       ctypes.c_float, AttnShape, ctypes.c_int, _P]),
@@ -202,30 +203,32 @@ _PAIR_CACHE_SIZE = 8
 BY_CLUSTER_MIN_ROWS = 1 << 16  # b*n from which the backward scatters go cluster by cluster
 
 
-def cluster_pairs(nbhd_idx: torch.Tensor):
+def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
     """For lists made of whole clusters (nbhd_idx[b,i,8r+t] = 8 c + t with c = c(b,i,r), every entry a row of the
-    sequence, n and m multiples of 8, m <= 64): (pair_offsets, pairs), int32 tensors that list, for every cluster
-    (b,g), the pairs (i,r) with c(b,i,r) = g as i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other
-    list.  One sort of the b*n*m/8 cluster numbers and one look at the result from the host; the answer is kept for
-    the lists seen lately (the layers of a stage share theirs), keyed by the tensor's memory and version."""
+    sequence of `n_rows` rows the lists point into — n by default —, n_rows and m multiples of 8, m <= 64):
+    (pair_offsets, pairs), int32 tensors that list, for every cluster (b,g), the pairs (i,r) with c(b,i,r) = g as
+    i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other list.  One sort of the b*n*m/8 cluster
+    numbers and one look at the result from the host; the answer is kept for the lists seen lately (the layers of a
+    stage share theirs), keyed by the tensor's memory and version."""
     if nbhd_idx.dim() != 3 or not nbhd_idx.is_cuda or nbhd_idx.dtype != torch.int64:
         return None
     B, N, M = nbhd_idx.shape
-    if B == 0 or N == 0 or N % 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
+    D = N if n_rows is None else int(n_rows)
+    if B == 0 or N == 0 or D <= 0 or D % 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
         return None
-    key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, nbhd_idx.device.index)
+    key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, D, nbhd_idx.device.index)
     hit = _PAIR_CACHE.get(key)
     if hit is not None:
         return hit[1]
     R = M // 8
-    K = N // 8
+    K = D // 8
     if B * K >= 1 << 31 or B * N * R >= 1 << 31:
         return None
     device = nbhd_idx.device
     keys = torch.empty(B * N * R, dtype=torch.int32, device=device)
     not_whole = torch.zeros(1, dtype=torch.int32, device=device)
     with torch.cuda.device(device):
-        _check(load().clusten_cluster_keys(_ptr(nbhd_idx), _ptr(keys), _ptr(not_whole), B, N, M, _stream(device)),
+        _check(load().clusten_cluster_keys(_ptr(nbhd_idx), _ptr(keys), _ptr(not_whole), B, N, M, D, _stream(device)),
                "clusten_cluster_keys")
     result = None
     if int(not_whole) == 0:                      # the one host synchronisation
@@ -405,6 +408,18 @@ def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Ten
     d_feat = torch.empty_like(feat)
     if d_weights.numel() == 0 or d_feat.numel() == 0:
         return d_weights.zero_(), d_feat.zero_()
+    if (shape.IC == 4 and shape.C % 32 == 0 and shape.B * shape.N >= BY_CLUSTER_MIN_ROWS
+            and weights.dtype in (torch.float32, torch.float16, torch.bfloat16)
+            and not torch.cuda.is_current_stream_capturing()):
+        lists = cluster_pairs(idx, shape.N)
+        if lists is not None:
+            # lists of whole clusters: d_feat as a gather over the pairs of every cluster of the feature rows
+            with torch.cuda.device(device):
+                _check(lib.clusten_wf_backward_by_cluster(_ptr(d_feat_new), _ptr(weights), _ptr(feat), _ptr(idx),
+                                                          _ptr(lists[0]), _ptr(lists[1]), _ptr(d_weights), _ptr(d_feat),
+                                                          shape, code, _stream(device)),
+                       "clusten_wf_backward_by_cluster")
+            return d_weights, d_feat
     ws_bytes = lib.clusten_wf_backward_workspace_bytes(shape, code)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
     with torch.cuda.device(device):

@@ -187,14 +187,27 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     dtype, as_stream(stream));
 }
 
-int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M,
+int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int n_rows,
                          clusten_stream stream) {
     if (!nbhd_idx || !keys || !not_whole) return CLUSTEN_ERR_NULL_POINTER;
-    if (B <= 0 || N <= 0 || M <= 0 || N % 8 != 0 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
-    if ((int64_t)B * (N / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
+    if (B <= 0 || N <= 0 || M <= 0 || n_rows <= 0 || n_rows % 8 != 0 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((int64_t)B * (n_rows / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
         return CLUSTEN_ERR_BAD_DIMS;
     }
-    return launch_cluster_keys(nbhd_idx, keys, not_whole, B, N, M, as_stream(stream));
+    return launch_cluster_keys(nbhd_idx, keys, not_whole, B, N, M, n_rows, as_stream(stream));
+}
+
+int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat, const int64_t* nbhd_idx,
+                                   const int32_t* pair_offsets, const int32_t* pairs, void* d_weights, void* d_feat,
+                                   clusten_wf_shape shape, int dtype, clusten_stream stream) {
+    if (!d_feat_new || !weights || !feat || !nbhd_idx || !pair_offsets || !pairs || !d_weights || !d_feat) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_wf_shape(shape)) return st;
+    int st = launch_wf_dweights(d_feat_new, feat, nbhd_idx, d_weights, shape, dtype, as_stream(stream));
+    if (st != CLUSTEN_OK) return st;
+    return launch_wf_dfeat_by_cluster(d_feat_new, weights, pair_offsets, pairs, d_feat, shape, dtype, as_stream(stream));
 }
 
 int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const int32_t* pair_offsets,

@@ -67,7 +67,12 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              hipStream_t stream);
 
 // y[b,h,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i,:]: see scatter_by_cluster.hip.
-int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, hipStream_t stream);
+int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int D,
+                        hipStream_t stream);
+// d_feat[b,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of sum_ic w[b,i,8r+t,ic] * d_out[b,i,ic,:]: see
+//   wf_dfeat_by_cluster.hip.  IC = 4, C % 32 == 0, N % 8 == 0.
+int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
+                               clusten_wf_shape s, int dtype, hipStream_t stream);
 int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* offsets,
                               const int32_t* pairs, void* y, clusten_attn_shape s, int dtype, hipStream_t stream);
 

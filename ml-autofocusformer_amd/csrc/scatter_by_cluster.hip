@@ -130,19 +130,20 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
     }
 }
 
-// keys[(b*N + i)*R + r] = b * (N/8) + c for lists made of whole clusters (idx[b,i,8r+t] = 8c + t, 0 <= 8c <= N-8);
-// any other run of 8 entries sets *not_whole to 1.  One thread per run: 64 bytes of the list.
+// keys[(b*N + i)*R + r] = b * (D/8) + c for lists made of whole clusters of a sequence of D rows (idx[b,i,8r+t] = 8c + t,
+// 0 <= 8c <= D-8); any other run of 8 entries sets *not_whole to 1.  One thread per run: 64 bytes of the list.
 __global__ __launch_bounds__(256) void cluster_keys_kernel(const int64_t* __restrict__ idx, int32_t* __restrict__ keys,
-                                                           int32_t* __restrict__ not_whole, int N, int R, int64_t runs) {
+                                                           int32_t* __restrict__ not_whole, int N, int R, int D,
+                                                           int64_t runs) {
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= runs) return;
     const int64_t* run = idx + e * 8;
     const int64_t head = run[0];
-    bool ok = (head & 7) == 0 && head >= 0 && head <= N - 8;
+    bool ok = (head & 7) == 0 && head >= 0 && head <= D - 8;
 #pragma unroll
     for (int t = 1; t < 8; ++t) ok = ok && run[t] == head + t;
     const int64_t b = e / ((int64_t)N * R);
-    keys[e] = ok ? (int32_t)(b * (N / 8) + (head >> 3)) : 0;
+    keys[e] = ok ? (int32_t)(b * (D / 8) + (head >> 3)) : 0;
     if (!ok) atomicOr(not_whole, 1);
 }
 
@@ -160,11 +161,12 @@ int launch_typed(const void* p, const void* x, clusten_strides xs, const int32_t
 
 }  // namespace
 
-int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, hipStream_t stream) {
+int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int D,
+                        hipStream_t stream) {
     const int R = M / 8;
     const int64_t runs = (int64_t)B * N * R;
     hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, stream, idx, keys, not_whole,
-                       N, R, runs);
+                       N, R, D, runs);
     return launch_status();
 }
 

@@ -1,0 +1,162 @@
+// wf_dfeat_by_cluster: the feature gradient of the WF operator as a gather (no atomics).
+//
+//   d_feat[b, idx[b,i,j], c] += sum_ic d_out[b,i,ic,c] * w[b,i,j,ic]          (clusten/src/clustenwf_cuda_kernel.cu:96-135)
+//
+// for neighbour lists made of whole clusters (idx[b,i,8r+t] = 8 c(b,i,r) + t: the lists a merge of the reference
+// model reads, models/aff_transformer.py:476-480 gathered at :336).  The 8 rows of cluster g of the finer sequence
+// receive
+//
+//   d_feat[b, 8g + t, :] = sum over the pairs (i, r) with c(b,i,r) = g of  sum_ic w[b,i,8r+t,ic] * d_out[b,i,ic,:]
+//
+// With the pairs of every cluster listed once (see scatter_by_cluster.hip: the same sorted pair lists) a pair is one
+// `v_mfma_f32_16x16x4_f32` per 16 channels: A = the pair's 8 x 4 block of weights (32 contiguous elements), B = the
+// four d_out rows of its output token, k = the inner channel.  One wave per cluster takes the channels 32 at a time;
+// d_out rows and weight blocks of 8 pairs at a time travel to LDS by LDS-direct loads (16-bit data is widened when the
+// operands are read).  Every row of d_feat is written exactly once: no atomics, no zero-fill, no workspace.  It has
+// no counterpart in the reference's extension modules.
+#include "launch.hpp"
+#include "mfma.hpp"
+
+namespace clusten {
+namespace {
+
+constexpr int kChunk = 32;       // channels per pass over the pairs
+constexpr int kPass = 8;         // pairs per pass
+constexpr int kListMax = 256;    // pairs of a cluster held in LDS at a time
+constexpr int kIC = 4;           // inner channels: the k of the matrix instruction
+
+template <typename T>
+__global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __restrict__ d_out, const T* __restrict__ w,
+                                                                    const int32_t* __restrict__ offsets,
+                                                                    const int32_t* __restrict__ pairs,
+                                                                    T* __restrict__ d_feat, int N, int Nout, int C, int M,
+                                                                    int clusters_per_image, int total_clusters) {
+    constexpr int EB = (int)sizeof(T);
+    constexpr int ROW_B = kChunk * EB;                 // bytes of a d_out row inside the chunk
+    constexpr int PAIR_B = kIC * ROW_B;                // the four rows of a pair
+    constexpr int X_BYTES = kPass * PAIR_B;
+    constexpr int X_DMA = X_BYTES / 1024;
+    constexpr int LANES_PER_ROW = ROW_B / 16;
+    constexpr int LANES_PER_PAIR = PAIR_B / 16;
+    constexpr int W_B = 8 * kIC * EB;                  // a pair's block of weights
+    constexpr int LANES_PER_W = W_B / 16;
+    constexpr int X_BASE = 0;
+    constexpr int W_BASE = X_BASE + X_BYTES;
+    constexpr int O_BASE = W_BASE + 1024;
+    constexpr int L_BASE = O_BASE + 8 * kChunk * 4;
+    constexpr int LDS_BYTES = L_BASE + kListMax * 4;
+    __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
+
+    const int unit = xcd_tile(blockIdx.x, total_clusters);
+    if (unit < 0) return;
+    const int b = unit / clusters_per_image;
+    const int g = unit - b * clusters_per_image;
+    const int lane = threadIdx.x;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int first = offsets[unit];
+    const int count = offsets[unit + 1] - first;
+    int* list = reinterpret_cast<int*>(stage + L_BASE);
+    const char* d_out_b = reinterpret_cast<const char*>(d_out + (int64_t)b * Nout * kIC * C);
+    const char* w_b = reinterpret_cast<const char*>(w + (int64_t)b * Nout * M * kIC);
+    T* rows_out = d_feat + ((int64_t)b * N + (int64_t)g * 8) * C;
+
+    // a cluster listed by more than kListMax pairs is taken in segments; the later segments add to what is stored
+    for (int seg = 0; seg == 0 || seg < count; seg += kListMax) {
+        const int n = min(kListMax, count - seg);   // <= 0 only for a cluster nobody lists: its rows become zero
+        lds_sync();
+        for (int e = lane; e < n; e += kWave) list[e] = pairs[first + seg + e];
+        lds_sync();
+        for (int c0 = 0; c0 < C; c0 += kChunk) {
+            F32x4 acc[2] = {F32x4{0.f, 0.f, 0.f, 0.f}, F32x4{0.f, 0.f, 0.f, 0.f}};
+            for (int base = 0; base < n; base += kPass) {
+                const int here = min(kPass, n - base);
+                lds_sync();  // the previous pass has been read
+#pragma unroll
+                for (int a = 0; a < X_DMA; ++a) {
+                    // lane -> (pair, inner channel, 16-byte piece of the row)
+                    const int slot = a * 64 + lane;
+                    const int e = list[base + min(slot / LANES_PER_PAIR, here - 1)];
+                    const int ic = (slot / LANES_PER_ROW) % kIC;
+                    CLUSTEN_LDS_DMA16(d_out_b + lane_offset((((uint32_t)(e >> 3) * kIC + (uint32_t)ic) * (uint32_t)C +
+                                                             (uint32_t)c0) * EB + (uint32_t)(lane % LANES_PER_ROW) * 16),
+                                      stage + X_BASE + a * 1024);
+                }
+                if (lane < kPass * LANES_PER_W) {
+                    const int e = list[base + min(lane / LANES_PER_W, here - 1)];
+                    CLUSTEN_LDS_DMA16(w_b + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * (kIC * EB) +
+                                                        (uint32_t)(lane % LANES_PER_W) * 16),
+                                      stage + W_BASE);
+                }
+                lds_sync_vm<0>();
+#pragma unroll
+                for (int pr = 0; pr < kPass; ++pr) {
+                    if (pr < here) {
+                        // A[t][ic] = w[i, 8r + t, ic]; B[ic][c] = d_out[i, ic, c0 + c]
+                        const T* wp = reinterpret_cast<const T*>(stage + W_BASE + pr * W_B) + (r16 & 7) * kIC + kq;
+                        const float a = r16 < 8 ? to_acc(*wp) : 0.f;
+                        const T* xp = reinterpret_cast<const T*>(stage + X_BASE + pr * PAIR_B + kq * ROW_B) + r16;
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, to_acc(xp[0]), acc[0], 0, 0, 0);
+                        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, to_acc(xp[16]), acc[1], 0, 0, 0);
+                    }
+                }
+            }
+            // rows 4*kq + j of the result (kq < 2: the cluster's 8 rows), channels c0 + 16*cb + r16
+            lds_sync();
+            if (kq < 2) {
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        reinterpret_cast<float*>(stage + O_BASE)[(4 * kq + j) * kChunk + 16 * cb + r16] = acc[cb][j];
+                    }
+                }
+            }
+            lds_sync();
+            {
+                // 8 rows x 32 channels: four consecutive channels per lane
+                const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
+                float v[4] = {o[0], o[1], o[2], o[3]};
+                T* dst = rows_out + (int64_t)(lane >> 3) * C + c0 + (lane & 7) * 4;
+                if (seg > 0) {
+                    float old[4];
+                    Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(dst), old);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += old[e];
+                }
+                *reinterpret_cast<typename Quad<T>::raw*>(dst) = Quad<T>::pack(v);
+            }
+        }
+    }
+}
+
+template <typename T>
+int launch_typed(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
+                 const clusten_wf_shape& s, hipStream_t stream) {
+    const int per_image = s.N / 8;
+    const int64_t total = (int64_t)s.B * per_image;
+    if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
+    hipLaunchKernelGGL((wf_dfeat_by_cluster_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWave), 0, stream,
+                       static_cast<const T*>(d_out), static_cast<const T*>(w), offsets, pairs, static_cast<T*>(d_feat), s.N,
+                       s.Nout, s.C, s.M, per_image, (int)total);
+    return launch_status();
+}
+
+}  // namespace
+
+int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
+                               clusten_wf_shape s, int dtype, hipStream_t stream) {
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N % 8 != 0 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    const int64_t eb = (int64_t)dtype_size(dtype);
+    if ((int64_t)s.Nout * kIC * s.C * eb >= ((int64_t)1 << 31) || (int64_t)s.Nout * s.M * kIC * eb >= ((int64_t)1 << 31)) {
+        return CLUSTEN_ERR_BAD_DIMS;
+    }
+    if (!aligned16(d_out) || !aligned16(w) || !aligned16(d_feat)) return CLUSTEN_ERR_UNALIGNED;
+    switch (dtype) {
+        case CLUSTEN_F32: return launch_typed<float>(d_out, w, offsets, pairs, d_feat, s, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(d_out, w, offsets, pairs, d_feat, s, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(d_out, w, offsets, pairs, d_feat, s, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
+}  // namespace clusten

@@ -137,6 +137,55 @@ def test_cluster_by_cluster_scatter_properties(device, by_cluster):
     assert _native.cluster_pairs(idx[:, :, :44].contiguous()) is None
 
 
+def _wf_cluster_lists(B, N, Nout, nnc, gen):
+    """(B,Nout,8*nnc) int64: every output token lists nnc distinct clusters of 8 consecutive feature rows."""
+    K = N // 8
+    pick = torch.rand(B, Nout, K, generator=gen).argsort(dim=2)[:, :, :nnc]
+    return (pick.unsqueeze(3) * 8 + torch.arange(8)).reshape(B, Nout, nnc * 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_wf_backward_cluster_by_cluster(device, dtype, by_cluster):
+    """WF lists made of whole clusters: d_feat as a gather over the pairs of every cluster (no atomics)."""
+    g = torch.Generator().manual_seed(83)
+    for B, N, Nout, C, nnc in ((2, 200, 50, 64, 6), (1, 392, 98, 128, 6), (2, 64, 16, 32, 8), (1, 48, 12, 96, 3)):
+        idx = _wf_cluster_lists(B, N, Nout, nnc, g)
+        assert _native.cluster_pairs(idx.to(device), N) is not None
+        case = wl.wf_case("clusters", 84, B=B, N=N, C=C, IC=4, M=idx.shape[-1], Nout=Nout)
+        case.nbhd_idx = idx
+        _check_wf_backward(case, device, dtype)
+
+
+def test_wf_cluster_by_cluster_properties(device, by_cluster):
+    g = torch.Generator().manual_seed(85)
+    B, N, Nout, C, IC = 2, 200, 50, 64, 4
+    idx = _wf_cluster_lists(B, N, Nout, 6, g)
+    M = idx.shape[-1]
+    # integer-valued data: the result equals the oracle's bit for bit; a second run gives the same bits
+    w = torch.randint(-3, 4, (B, Nout, M, IC), generator=g).float()
+    f = torch.randint(-3, 4, (B, N, C), generator=g).float()
+    d_out = torch.randint(-3, 4, (B, Nout, IC, C), generator=g).float()
+    dw_ref, df_ref = oracle.wf_gather_backward(d_out, w, f, idx)
+    dw, df = _native.wf_backward(d_out.to(device), w.to(device), f.to(device), idx.to(device))
+    assert torch.equal(dw.cpu(), dw_ref) and torch.equal(df.cpu(), df_ref)
+    # a cluster listed by more pairs than a wave holds at once (every output token lists clusters 0..5), and
+    # clusters nobody lists
+    many = (torch.arange(48) % 8 + 8 * (torch.arange(48) // 8)).expand(1, 600, 48).contiguous()
+    w2 = torch.randn(1, 600, 48, IC, generator=g)
+    f2 = torch.randn(1, 160, 32, generator=g)
+    d2 = torch.randn(1, 600, IC, 32, generator=g)
+    want = oracle.wf_gather_backward(d2, w2, f2, many)[1]
+    got = _native.wf_backward(d2.to(device), w2.to(device), f2.to(device), many.to(device))[1]
+    assert oracle.rel_err(got, want) <= TOL_SCATTER_F32 and float(got[:, 48:].abs().max()) == 0.0
+    # other inner channel counts and lists that are not whole clusters keep the atomic kernel
+    case = wl.wf_case("knn", 86, B=2, N=200, C=64, IC=4)
+    assert _native.cluster_pairs(case.nbhd_idx.to(device), 200) is None
+    _check_wf_backward(case, device, torch.float32)
+    case1 = wl.wf_case("ic1", 87, B=1, N=64, C=64, IC=1, M=48, Nout=16)
+    case1.nbhd_idx = _wf_cluster_lists(1, 64, 16, 6, g)
+    _check_wf_backward(case1, device, torch.float32)
+
+
 def test_scatter_union_path_is_bit_exact_on_integer_data(device):
     g = torch.Generator().manual_seed(78)
     B, H, N, C = 2, 3, 200, 32
