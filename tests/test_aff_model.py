@@ -191,6 +191,32 @@ def test_logits_equal_with_hip_operators_and_with_the_oracle(device, amp):
 
 
 @pytest.mark.gpu
+def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkeypatch):
+    """A training step of the model with the backward scatters (d_key, d_value, WF d_feat) running as gathers over
+    sorted pair lists — the model's own lists are made of whole clusters — against the same step on the oracle."""
+    from aff.model import default_ops
+    from clusten import _native
+    monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
+    _native._PAIR_CACHE.clear()
+    seen = []
+    real = _native.cluster_pairs
+    monkeypatch.setattr(_native, "cluster_pairs", lambda *a: (seen.append(real(*a) is not None), real(*a))[1])
+    hip = small_model(default_ops(), img_size=128, num_classes=16).to(device).train()
+    ref = small_model(oracle_ops(), img_size=128, num_classes=16).to(device).train()
+    ref.load_state_dict(hip.state_dict())
+    x = torch.randn(4, 3, 128, 128, generator=torch.Generator().manual_seed(8)).to(device)
+    target = torch.randn(4, 16, generator=torch.Generator().manual_seed(9)).to(device)
+    for model in (hip, ref):
+        ((model(x) - target) ** 2).mean().backward()
+    assert any(seen), "no list of the model took the cluster-by-cluster path"
+    for (name, p), (_, q) in zip(hip.named_parameters(), ref.named_parameters()):
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        # 1e-7: the bias ahead of the BatchNorm has a gradient of zero, both sides hold rounding noise there
+        assert float((p.grad - q.grad).abs().max()) <= 1e-3 * float(q.grad.abs().max()) + 1e-7, name
+    _native._PAIR_CACHE.clear()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("with_mask", [False, True])
 def test_fused_bias_mask_blank_softmax_equals_the_tensor_expressions(device, dtype, with_mask):
