@@ -200,12 +200,15 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -
 
 _PAIR_CACHE: "dict" = {}       # lists seen lately -> their pairs by cluster, or None when they are not whole clusters
 _PAIR_CACHE_SIZE = 8
-BY_CLUSTER_MIN_ROWS = 1 << 16  # b*n from which the backward scatters go cluster by cluster
+_PAD_ENTRY = 1 << 30           # flag of a pair listed under cluster 0 for the pad slots of the short last cluster
+BY_CLUSTER_MIN_ROWS = 1 << 14  # b*n from which the backward scatters go cluster by cluster (the sort of the lists,
+                               # 0.3-0.4 ms per list tensor, is shared by the layers of a stage)
 
 
 def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
     """For lists made of whole clusters (nbhd_idx[b,i,8r+t] = 8 c + t with c = c(b,i,r), every entry a row of the
-    sequence of `n_rows` rows the lists point into — n by default —, n_rows and m multiples of 8, m <= 64):
+    sequence of `n_rows` rows the lists point into — n by default —, m a multiple of 8, m <= 64; the short last
+    cluster of a sequence whose length is not a multiple of 8 is followed by pad slots that hold row 0):
     (pair_offsets, pairs), int32 tensors that list, for every cluster (b,g), the pairs (i,r) with c(b,i,r) = g as
     i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other list.  One sort of the b*n*m/8 cluster
     numbers and one look at the result from the host; the answer is kept for the lists seen lately (the layers of a
@@ -214,15 +217,15 @@ def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
         return None
     B, N, M = nbhd_idx.shape
     D = N if n_rows is None else int(n_rows)
-    if B == 0 or N == 0 or D <= 0 or D % 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
+    if B == 0 or N == 0 or D < 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
         return None
     key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, D, nbhd_idx.device.index)
     hit = _PAIR_CACHE.get(key)
     if hit is not None:
         return hit[1]
     R = M // 8
-    K = D // 8
-    if B * K >= 1 << 31 or B * N * R >= 1 << 31:
+    K = (D + 7) // 8
+    if B * K >= 1 << 30 or B * N * R >= 1 << 30 or N >= 1 << 26:
         return None
     device = nbhd_idx.device
     keys = torch.empty(B * N * R, dtype=torch.int32, device=device)
@@ -232,8 +235,16 @@ def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
                "clusten_cluster_keys")
     result = None
     if int(not_whole) == 0:                      # the one host synchronisation
+        where = torch.arange(B * N * R, dtype=torch.int32, device=device)
+        entries = ((where // R) % N) * 8 + where % R                       # i*8 + r
+        if D % 8:
+            # the pairs that name the short last cluster also feed row 0 with their pad slots: listed a second time,
+            # flagged, under cluster 0 of their image
+            short = (keys % K) == K - 1
+            keys = torch.cat([keys, keys[short] - (K - 1)])
+            entries = torch.cat([entries, entries[short] | _PAD_ENTRY])
         ordered, order = torch.sort(keys)
-        pairs = (((order // R) % N) * 8 + order % R).to(torch.int32)
+        pairs = entries[order].contiguous()
         offsets = torch.searchsorted(ordered, torch.arange(B * K + 1, dtype=torch.int32, device=device),
                                      out_int32=True)
         result = (offsets, pairs)
@@ -255,8 +266,8 @@ def scatter_rows_by_cluster(p: torch.Tensor, x: torch.Tensor, pair_lists) -> tor
     B, H, N, C = x.shape
     M = p.shape[3]
     offsets, pairs = pair_lists
-    if offsets.numel() != B * (N // 8) + 1 or pairs.numel() != B * N * (M // 8) or C != 32 or N % 8 or M % 8:
-        raise RuntimeError("scatter_rows_by_cluster: head dim 32, n and m multiples of 8, pair lists of these lists")
+    if offsets.numel() != B * ((N + 7) // 8) + 1 or pairs.numel() < B * N * (M // 8) or C != 32 or N < 8 or M % 8:
+        raise RuntimeError("scatter_rows_by_cluster: head dim 32, m a multiple of 8, pair lists of these lists")
     code = _dtype_code(p, "p")
     p, x = p.contiguous(), _rows(x)
     y = torch.empty((B, H, N, C), dtype=p.dtype, device=device)

@@ -190,8 +190,8 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
 int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int n_rows,
                          clusten_stream stream) {
     if (!nbhd_idx || !keys || !not_whole) return CLUSTEN_ERR_NULL_POINTER;
-    if (B <= 0 || N <= 0 || M <= 0 || n_rows <= 0 || n_rows % 8 != 0 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
-    if ((int64_t)B * (n_rows / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
+    if (B <= 0 || N <= 0 || M <= 0 || n_rows < 8 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((int64_t)B * ((n_rows + 7) / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
         return CLUSTEN_ERR_BAD_DIMS;
     }
     return launch_cluster_keys(nbhd_idx, keys, not_whole, B, N, M, n_rows, as_stream(stream));

@@ -16,6 +16,9 @@
 // LDS-direct loads, and the product runs on `v_mfma_f32_16x16x4_f32` (16-bit data is widened when the operands are
 // read from LDS; rows 8-15 of the instruction are idle).  Every row of y is written exactly once: no atomics, no
 // zero-fill, no fp32 workspace for 16-bit data, and the sums do not depend on the order in which workgroups run.
+// A sequence whose length is not a multiple of 8 ends in a short cluster, and the lists that name it hold row 0 in
+// the slots past its rows (models/point_utils.py pads member lists with index 0): those slots add to row 0, so the
+// caller lists such a pair a second time, flagged, under cluster 0, where the sum of its pad slots feeds row 0.
 // It has no counterpart in the reference's extension modules.
 #include "launch.hpp"
 #include "mfma.hpp"
@@ -26,6 +29,8 @@ namespace {
 constexpr int kC = 32;           // head dim
 constexpr int kPass = 32;        // pairs per pass
 constexpr int kListMax = 256;    // pairs of a cluster held in LDS at a time
+constexpr int kPadEntry = 1 << 30;   // list entry flag: the pair names the short last cluster; here, for its pad slots
+constexpr int kEntryMask = kPadEntry - 1;
 
 template <typename T>
 __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __restrict__ p, const T* __restrict__ x,
@@ -56,6 +61,8 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
     const int first = offsets[unit];
     const int count = offsets[unit + 1] - first;
     int* list = reinterpret_cast<int*>(stage + L_BASE);
+    const int rows_here = min(8, N - 8 * g);   // the last cluster of a sequence may be short
+    const int pad_from = N & 7;                // ... and the lists that name it hold row 0 in slots pad_from .. 7
 
     // a cluster listed by more than kListMax pairs is taken in segments; the later segments add to what is stored
     for (int seg = 0; seg == 0 || seg < count; seg += kListMax) {
@@ -72,7 +79,7 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
                 lds_sync();  // the previous pass has been read
 #pragma unroll
                 for (int a = 0; a < X_DMA; ++a) {
-                    const int e = list[base + min(ROWS_PER_DMA * a + lane / LANES_PER_ROW, here - 1)];
+                    const int e = list[base + min(ROWS_PER_DMA * a + lane / LANES_PER_ROW, here - 1)] & kEntryMask;
                     CLUSTEN_LDS_DMA16(x_bh + lane_offset((uint32_t)(e >> 3) * (uint32_t)xs.n * EB +
                                                          (uint32_t)(lane % LANES_PER_ROW) * 16),
                                       stage + X_BASE + a * 1024);
@@ -81,7 +88,7 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
                     // 32 pieces of PIECE_B bytes: 16 bytes per lane
                     constexpr int LANES_PER_PIECE = PIECE_B / 16;
                     if (lane < kPass * LANES_PER_PIECE) {
-                        const int e = list[base + min(lane / LANES_PER_PIECE, here - 1)];
+                        const int e = list[base + min(lane / LANES_PER_PIECE, here - 1)] & kEntryMask;
                         CLUSTEN_LDS_DMA16(p_bh + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * EB +
                                                              (uint32_t)(lane % LANES_PER_PIECE) * 16),
                                           stage + P_BASE);
@@ -92,8 +99,16 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
                 for (int s = 0; s < kPass / 4; ++s) {
                     if (4 * s < here) {
                         const int pr = 4 * s + kq;
-                        const T* pp = reinterpret_cast<const T*>(stage + P_BASE + pr * PIECE_B) + (r16 & 7);
-                        const float a = (r16 < 8 && pr < here) ? to_acc(*pp) : 0.f;
+                        const T* pp = reinterpret_cast<const T*>(stage + P_BASE + pr * PIECE_B);
+                        float a = 0.f;
+                        if (pr < here) {
+                            if ((list[base + pr] & kPadEntry) == 0) {
+                                if (r16 < rows_here) a = to_acc(pp[r16]);
+                            } else if (r16 == 0) {
+                                // a pair that names the short last cluster: its pad slots hold row 0, this cluster's first
+                                for (int t = pad_from; t < 8; ++t) a += to_acc(pp[t]);
+                            }
+                        }
                         const T* xp = reinterpret_cast<const T*>(stage + X_BASE + pr * ROW_B) + r16;
                         const float b0 = to_acc(xp[0]), b1 = to_acc(xp[16]);
                         acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b0, acc[0], 0, 0, 0);
@@ -118,20 +133,21 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
                 // 8 rows x 32 channels: four consecutive channels per lane
                 const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
                 float v[4] = {o[0], o[1], o[2], o[3]};
-                if (seg > 0) {
+                if (seg > 0 && (lane >> 3) < rows_here) {
                     float old[4];
                     Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(y_rows + lane * 4), old);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] += old[e];
                 }
-                *reinterpret_cast<typename Quad<T>::raw*>(y_rows + lane * 4) = Quad<T>::pack(v);
+                if ((lane >> 3) < rows_here) *reinterpret_cast<typename Quad<T>::raw*>(y_rows + lane * 4) = Quad<T>::pack(v);
             }
         }
     }
 }
 
-// keys[(b*N + i)*R + r] = b * (D/8) + c for lists made of whole clusters of a sequence of D rows (idx[b,i,8r+t] = 8c + t,
-// 0 <= 8c <= D-8); any other run of 8 entries sets *not_whole to 1.  One thread per run: 64 bytes of the list.
+// keys[(b*N + i)*R + r] = b * ceil(D/8) + c for lists made of whole clusters of a sequence of D rows (idx[b,i,8r+t] = 8c + t;
+// for the short last cluster of a sequence with D % 8 != 0 the slots past its rows hold 0); any other run of 8 entries
+// sets *not_whole to 1.  One thread per run: 64 bytes of the list.
 __global__ __launch_bounds__(256) void cluster_keys_kernel(const int64_t* __restrict__ idx, int32_t* __restrict__ keys,
                                                            int32_t* __restrict__ not_whole, int N, int R, int D,
                                                            int64_t runs) {
@@ -139,18 +155,20 @@ __global__ __launch_bounds__(256) void cluster_keys_kernel(const int64_t* __rest
     if (e >= runs) return;
     const int64_t* run = idx + e * 8;
     const int64_t head = run[0];
-    bool ok = (head & 7) == 0 && head >= 0 && head <= D - 8;
+    // a whole cluster, or the short last one (D % 8 rows) followed by pad slots that hold row 0
+    const int own = (head == D - (D & 7)) ? (D & 7) : 8;
+    bool ok = (head & 7) == 0 && head >= 0 && head < D;
 #pragma unroll
-    for (int t = 1; t < 8; ++t) ok = ok && run[t] == head + t;
+    for (int t = 1; t < 8; ++t) ok = ok && run[t] == (t < own ? head + t : 0);
     const int64_t b = e / ((int64_t)N * R);
-    keys[e] = ok ? (int32_t)(b * (D / 8) + (head >> 3)) : 0;
+    keys[e] = ok ? (int32_t)(b * ((D + 7) / 8) + (head >> 3)) : 0;
     if (!ok) atomicOr(not_whole, 1);
 }
 
 template <typename T>
 int launch_typed(const void* p, const void* x, clusten_strides xs, const int32_t* offsets, const int32_t* pairs, void* y,
                  const clusten_attn_shape& s, hipStream_t stream) {
-    const int per_image = s.N / 8;
+    const int per_image = (s.N + 7) / 8;
     const int64_t total = (int64_t)s.B * per_image;
     if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
     hipLaunchKernelGGL((scatter_by_cluster_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWave), 0, stream,
@@ -172,7 +190,7 @@ int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, i
 
 int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* offsets,
                               const int32_t* pairs, void* y, clusten_attn_shape s, int dtype, hipStream_t stream) {
-    if (s.C != kC || s.N % 8 != 0 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (s.C != kC || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
     const size_t eb = dtype_size(dtype);
     if (!rows_aligned16(x, xs, (int)eb) || !aligned16(p) || !aligned16(y) || !slice_fits_int32(xs, s.H, s.N, s.C) ||
         (int64_t)s.N * s.M * (int64_t)eb >= ((int64_t)1 << 31)) {

@@ -24,6 +24,8 @@ constexpr int kChunk = 32;       // channels per pass over the pairs
 constexpr int kPass = 8;         // pairs per pass
 constexpr int kListMax = 256;    // pairs of a cluster held in LDS at a time
 constexpr int kIC = 4;           // inner channels: the k of the matrix instruction
+constexpr int kPadEntry = 1 << 30;   // list entry flag: see scatter_by_cluster.hip
+constexpr int kEntryMask = kPadEntry - 1;
 
 template <typename T>
 __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __restrict__ d_out, const T* __restrict__ w,
@@ -59,6 +61,8 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
     const char* d_out_b = reinterpret_cast<const char*>(d_out + (int64_t)b * Nout * kIC * C);
     const char* w_b = reinterpret_cast<const char*>(w + (int64_t)b * Nout * M * kIC);
     T* rows_out = d_feat + ((int64_t)b * N + (int64_t)g * 8) * C;
+    const int rows_here = min(8, N - 8 * g);   // the last cluster of a sequence may be short
+    const int pad_from = N & 7;                // ... and the lists that name it hold row 0 in slots pad_from .. 7
 
     // a cluster listed by more than kListMax pairs is taken in segments; the later segments add to what is stored
     for (int seg = 0; seg == 0 || seg < count; seg += kListMax) {
@@ -75,14 +79,14 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
                 for (int a = 0; a < X_DMA; ++a) {
                     // lane -> (pair, inner channel, 16-byte piece of the row)
                     const int slot = a * 64 + lane;
-                    const int e = list[base + min(slot / LANES_PER_PAIR, here - 1)];
+                    const int e = list[base + min(slot / LANES_PER_PAIR, here - 1)] & kEntryMask;
                     const int ic = (slot / LANES_PER_ROW) % kIC;
                     CLUSTEN_LDS_DMA16(d_out_b + lane_offset((((uint32_t)(e >> 3) * kIC + (uint32_t)ic) * (uint32_t)C +
                                                              (uint32_t)c0) * EB + (uint32_t)(lane % LANES_PER_ROW) * 16),
                                       stage + X_BASE + a * 1024);
                 }
                 if (lane < kPass * LANES_PER_W) {
-                    const int e = list[base + min(lane / LANES_PER_W, here - 1)];
+                    const int e = list[base + min(lane / LANES_PER_W, here - 1)] & kEntryMask;
                     CLUSTEN_LDS_DMA16(w_b + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * (kIC * EB) +
                                                         (uint32_t)(lane % LANES_PER_W) * 16),
                                       stage + W_BASE);
@@ -92,8 +96,14 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
                 for (int pr = 0; pr < kPass; ++pr) {
                     if (pr < here) {
                         // A[t][ic] = w[i, 8r + t, ic]; B[ic][c] = d_out[i, ic, c0 + c]
-                        const T* wp = reinterpret_cast<const T*>(stage + W_BASE + pr * W_B) + (r16 & 7) * kIC + kq;
-                        const float a = r16 < 8 ? to_acc(*wp) : 0.f;
+                        const T* wp = reinterpret_cast<const T*>(stage + W_BASE + pr * W_B) + kq;
+                        float a = 0.f;
+                        if ((list[base + pr] & kPadEntry) == 0) {
+                            if (r16 < rows_here) a = to_acc(wp[r16 * kIC]);
+                        } else if (r16 == 0) {
+                            // a pair that names the short last cluster: its pad slots hold row 0, this cluster's first
+                            for (int t = pad_from; t < 8; ++t) a += to_acc(wp[t * kIC]);
+                        }
                         const T* xp = reinterpret_cast<const T*>(stage + X_BASE + pr * PAIR_B + kq * ROW_B) + r16;
                         acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, to_acc(xp[0]), acc[0], 0, 0, 0);
                         acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, to_acc(xp[16]), acc[1], 0, 0, 0);
@@ -117,13 +127,13 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
                 const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
                 float v[4] = {o[0], o[1], o[2], o[3]};
                 T* dst = rows_out + (int64_t)(lane >> 3) * C + c0 + (lane & 7) * 4;
-                if (seg > 0) {
+                if (seg > 0 && (lane >> 3) < rows_here) {
                     float old[4];
                     Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(dst), old);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] += old[e];
                 }
-                *reinterpret_cast<typename Quad<T>::raw*>(dst) = Quad<T>::pack(v);
+                if ((lane >> 3) < rows_here) *reinterpret_cast<typename Quad<T>::raw*>(dst) = Quad<T>::pack(v);
             }
         }
     }
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
 template <typename T>
 int launch_typed(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
                  const clusten_wf_shape& s, hipStream_t stream) {
-    const int per_image = s.N / 8;
+    const int per_image = (s.N + 7) / 8;
     const int64_t total = (int64_t)s.B * per_image;
     if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
     hipLaunchKernelGGL((wf_dfeat_by_cluster_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWave), 0, stream,
@@ -145,7 +155,7 @@ int launch_typed(const void* d_out, const void* w, const int32_t* offsets, const
 
 int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
                                clusten_wf_shape s, int dtype, hipStream_t stream) {
-    if (s.IC != kIC || s.C % kChunk != 0 || s.N % 8 != 0 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
     const int64_t eb = (int64_t)dtype_size(dtype);
     if ((int64_t)s.Nout * kIC * s.C * eb >= ((int64_t)1 << 31) || (int64_t)s.Nout * s.M * kIC * eb >= ((int64_t)1 << 31)) {
         return CLUSTEN_ERR_BAD_DIMS;

@@ -99,6 +99,38 @@ def test_attn_backward_cluster_by_cluster(device, dtype, by_cluster):
         _check_attn_backward(case, device, dtype)
 
 
+def _padded_model_lists(B, N, nnc, gen):
+    """Lists over a sequence whose last cluster is short: (B,N,8*nnc), clusters chosen at random per token, the
+    slots past the last row hold index 0 (as the model pads them)."""
+    K = (N + 7) // 8
+    pick = torch.rand(B, N, K, generator=gen).argsort(dim=2)[:, :, :nnc]
+    rows = pick.unsqueeze(3) * 8 + torch.arange(8)
+    return torch.where(rows < N, rows, torch.zeros_like(rows)).reshape(B, N, nnc * 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_backward_cluster_by_cluster_with_a_short_last_cluster(device, dtype, by_cluster):
+    """196 tokens = 24 clusters and one of 4: the lists that name it hold row 0 in their last slots, and those slots'
+    contributions must reach row 0 (attention scatters and the WF feature gradient)."""
+    g = torch.Generator().manual_seed(88)
+    for B, H, N in ((2, 2, 196), (1, 3, 100), (2, 1, 13)):
+        idx = _padded_model_lists(B, N, min(6, (N + 7) // 8), g)
+        assert (idx == 0).sum() > B * N // 8
+        assert _native.cluster_pairs(idx.to(device)) is not None
+        case = wl.attn_case("padded", 89, B=B, H=H, N=N, C=32, M=idx.shape[-1], lists="random")
+        case.nbhd_idx = idx
+        _check_attn_backward(case, device, dtype)
+    B, N, Nout, C = 2, 196, 49, 64
+    K = (N + 7) // 8
+    pick = torch.rand(B, Nout, K, generator=g).argsort(dim=2)[:, :, :6]
+    rows = pick.unsqueeze(3) * 8 + torch.arange(8)
+    idx = torch.where(rows < N, rows, torch.zeros_like(rows)).reshape(B, Nout, 48)
+    assert _native.cluster_pairs(idx.to(device), N) is not None
+    case = wl.wf_case("padded", 90, B=B, N=N, C=C, IC=4, M=48, Nout=Nout)
+    case.nbhd_idx = idx
+    _check_wf_backward(case, device, dtype)
+
+
 def test_cluster_by_cluster_scatter_properties(device, by_cluster):
     g = torch.Generator().manual_seed(81)
     B, H, N, C = 2, 3, 200, 32
