@@ -69,9 +69,12 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 #pragma unroll
             for (int t = 0; t < 8; ++t) v[t] = (int)run[t];
         }
-        bool regular = true;                         // 8 consecutive rows
+        // 8 consecutive rows, or the short last cluster of the sequence followed by the row 0 its pad slots hold:
+        // either way the first row tells the other seven
+        const int own = ((N & 7) != 0 && v[0] == N - (N & 7)) ? (N & 7) : 8;
+        bool regular = true;
 #pragma unroll
-        for (int t = 1; t < 8; ++t) regular = regular && (v[t] == v[0] + t);
+        for (int t = 1; t < 8; ++t) regular = regular && (v[t] == (t < own ? v[0] + t : 0));
         const int key = regular ? v[0] : ~lane;      // other runs never merge
         uint64_t remaining = nruns >= 64 ? ~0ull : ((1ull << nruns) - 1);
         bool differ = false;                         // a shared list is better served by the path below
