@@ -200,19 +200,24 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -
 
 _PAIR_CACHE: "dict" = {}       # lists seen lately -> their pairs by cluster, or None when they are not whole clusters
 _PAIR_CACHE_SIZE = 8
+WF_BY_CLUSTER_MIN_ROWS = 1 << 14   # b*n (feature rows) from which WF's d_feat goes cluster by cluster: a merge's list
+                                   # tensor is used once, so its sort must pay within that one call
+_SEEN_ONCE = object()          # cache value of a list tensor met once, whose pair lists have not been made yet
 _PAD_ENTRY = 1 << 30           # flag of a pair listed under cluster 0 for the pad slots of the short last cluster
-BY_CLUSTER_MIN_ROWS = 1 << 14  # b*n from which the backward scatters go cluster by cluster (the sort of the lists,
-                               # 0.3-0.4 ms per list tensor, is shared by the layers of a stage)
+BY_CLUSTER_MIN_ROWS = 1 << 12  # b*n from which the backward scatters go cluster by cluster, from the second use of a
+                               # list tensor on (the sort of the lists, 0.3-0.4 ms, is shared by the layers of a stage)
 
 
-def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
+def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None, on_second_sight: bool = False):
     """For lists made of whole clusters (nbhd_idx[b,i,8r+t] = 8 c + t with c = c(b,i,r), every entry a row of the
     sequence of `n_rows` rows the lists point into — n by default —, m a multiple of 8, m <= 64; the short last
     cluster of a sequence whose length is not a multiple of 8 is followed by pad slots that hold row 0):
     (pair_offsets, pairs), int32 tensors that list, for every cluster (b,g), the pairs (i,r) with c(b,i,r) = g as
     i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other list.  One sort of the b*n*m/8 cluster
     numbers and one look at the result from the host; the answer is kept for the lists seen lately (the layers of a
-    stage share theirs), keyed by the tensor's memory and version."""
+    stage share theirs), keyed by the tensor's memory and version.  With `on_second_sight` a list tensor met for the
+    first time is only remembered (None is returned) and the pair lists are made when it comes again: lists used once
+    never pay for the sort."""
     if nbhd_idx.dim() != 3 or not nbhd_idx.is_cuda or nbhd_idx.dtype != torch.int64:
         return None
     B, N, M = nbhd_idx.shape
@@ -221,8 +226,14 @@ def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
         return None
     key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, D, nbhd_idx.device.index)
     hit = _PAIR_CACHE.get(key)
-    if hit is not None:
+    if hit is not None and hit[1] is not _SEEN_ONCE:
         return hit[1]
+    if hit is None and on_second_sight:
+        if len(_PAIR_CACHE) >= _PAIR_CACHE_SIZE:
+            _PAIR_CACHE.pop(next(iter(_PAIR_CACHE)))
+        _PAIR_CACHE[key] = (nbhd_idx, _SEEN_ONCE)
+        return None
+    _PAIR_CACHE.pop(key, None)
     R = M // 8
     K = (D + 7) // 8
     if B * K >= 1 << 30 or B * N * R >= 1 << 30 or N >= 1 << 26:
@@ -286,7 +297,7 @@ def _pairs_for_backward(nbhd_idx: torch.Tensor, shape) -> "tuple | None":
     whole clusters, and enough rows for the sort of the lists to pay."""
     if shape.C != 32 or shape.B * shape.N < BY_CLUSTER_MIN_ROWS or torch.cuda.is_current_stream_capturing():
         return None
-    return cluster_pairs(nbhd_idx)
+    return cluster_pairs(nbhd_idx, on_second_sight=BY_CLUSTER_MIN_ROWS > 0)
 
 
 def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor):
@@ -419,7 +430,7 @@ def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Ten
     d_feat = torch.empty_like(feat)
     if d_weights.numel() == 0 or d_feat.numel() == 0:
         return d_weights.zero_(), d_feat.zero_()
-    if (shape.IC == 4 and shape.C % 32 == 0 and shape.B * shape.N >= BY_CLUSTER_MIN_ROWS
+    if (shape.IC == 4 and shape.C % 32 == 0 and shape.B * shape.N >= WF_BY_CLUSTER_MIN_ROWS
             and weights.dtype in (torch.float32, torch.float16, torch.bfloat16)
             and not torch.cuda.is_current_stream_capturing()):
         lists = cluster_pairs(idx, shape.N)

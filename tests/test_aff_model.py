@@ -197,6 +197,7 @@ def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkey
     from aff.model import default_ops
     from clusten import _native
     monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
+    monkeypatch.setattr(_native, "WF_BY_CLUSTER_MIN_ROWS", 0)
     _native._PAIR_CACHE.clear()
     seen = []
     real = _native.cluster_pairs

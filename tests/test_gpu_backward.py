@@ -82,6 +82,7 @@ def test_attn_backward_lists_made_of_runs(device, kind, dtype):
 def by_cluster(monkeypatch):
     """The cluster-by-cluster scatter for problems of any size (in production it starts at 65536 rows)."""
     monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
+    monkeypatch.setattr(_native, "WF_BY_CLUSTER_MIN_ROWS", 0)
     _native._PAIR_CACHE.clear()
     yield
     _native._PAIR_CACHE.clear()
@@ -161,6 +162,11 @@ def test_cluster_by_cluster_scatter_properties(device, by_cluster):
     want = oracle.qk_gather_backward(p2, x2, x2, lone.cpu())[1]
     got = _native.scatter_rows_by_cluster(p2.to(device), x2.to(device), lists2)
     assert oracle.rel_err(got, want) <= TOL_SCATTER_F32 and float(got[:, :, :8].abs().max()) == 0.0
+    # in production a list tensor is only remembered when it is first met; its pair lists are made when it comes again
+    _native._PAIR_CACHE.clear()
+    assert _native.cluster_pairs(idx, on_second_sight=True) is None
+    again = _native.cluster_pairs(idx, on_second_sight=True)
+    assert again is not None and torch.equal(again[1], pairs) and _native.cluster_pairs(idx, on_second_sight=True) is again
     # lists that are not whole clusters keep the atomic path
     assert _native.cluster_pairs(torch.randint(N, (B, N, M), generator=g).to(device)) is None
     shifted = idx.clone()
