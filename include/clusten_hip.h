@@ -370,6 +370,16 @@ int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch
                                   const void* bias, void* score, int64_t rows, int C, int dtype,
                                   clusten_stream stream);
 
+/* Gradient of the relative-position bias table of an attention layer, the backward of
+ * `pe_table.gather(index=pe_idx...)` added to the logits (models/aff_transformer.py:131-133):
+ *   d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]
+ * summed per workgroup in LDS before it reaches memory.  d_logit (B,H,N,M) of `dtype` (F32, F16 or BF16), pe_idx
+ * (B,N,M) int64 (entries outside [0,rows) are skipped), d_table (rows,H) fp32, zeroed by the caller; all
+ * contiguous.  rows <= 16000 (else CLUSTEN_ERR_BAD_DIMS).  The order of the additions varies from run to run, as a
+ * scatter-add's does.  No counterpart in the reference's extension modules. */
+int clusten_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M,
+                            int rows, int dtype, clusten_stream stream);
+
 /* The `weights` operand of clusten_wf_forward as the reference model builds it before a merge
  * (models/aff_transformer.py:340-358), in one pass instead of a row lookup, a gather and two multiplications:
  *   weights[b,i,j,:] = table_weights[pe_idx[b,i,j], :] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]

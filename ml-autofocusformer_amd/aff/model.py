@@ -47,6 +47,7 @@ def default_ops():
                            channel_affine_gelu=_native.channel_affine_gelu,
                            channel_affine_gelu_supported=_native.channel_affine_gelu_supported,
                            add_row_score=_native.add_row_score, add_row_score_supported=_native.add_row_score_supported,
+                           bias_table_grad=_native.bias_table_grad,
                            neighbour_lists=_native.neighbour_lists,
                            neighbour_lists_supported=_native.neighbour_lists_supported)
 
@@ -117,6 +118,31 @@ def _table_rows(table, idx):
     batch 64 on this device: nine tenths of a training step)."""
     k = table.shape[1]
     return table.gather(0, idx.reshape(-1, 1).expand(-1, k)).reshape(*idx.shape, k)
+
+
+class _PositionBias(torch.autograd.Function):
+    """bias[pe_idx] laid out as (b, h, n, m), with the table's gradient from the library's kernel (sums per workgroup
+    in LDS) instead of the framework's scatter-add of b*h*n*m values into a table of 12 000 rows."""
+
+    @staticmethod
+    def forward(ctx, bias, pe_idx, grad_kernel):
+        ctx.save_for_backward(pe_idx)
+        ctx.rows, ctx.dtype, ctx.grad_kernel = bias.shape[0], bias.dtype, grad_kernel
+        return _table_rows(bias, pe_idx).permute(0, 3, 1, 2)
+
+    @staticmethod
+    def backward(ctx, grad):
+        (pe_idx,) = ctx.saved_tensors
+        return ctx.grad_kernel(grad, pe_idx, ctx.rows).to(ctx.dtype), None, None
+
+
+def _position_bias(bias, pe_idx, ops):
+    """(b, h, n, m) position bias of an attention layer: row pe_idx[b,i,j] of the (rows, h) table for every pair."""
+    kernel = getattr(ops, "bias_table_grad", None)
+    if (kernel is not None and torch.is_grad_enabled() and bias.requires_grad and bias.is_cuda
+            and bias.dtype in (torch.float32, torch.float16, torch.bfloat16) and bias.shape[0] <= 16000):
+        return _PositionBias.apply(bias, pe_idx, kernel)
+    return _table_rows(bias, pe_idx).permute(0, 3, 1, 2)
 
 
 def _autocast_key():
@@ -250,7 +276,7 @@ class ClusterAttention(nn.Module):
             attn, blank = fused(attn, bias, pe_idx, cluster_mask, query=q, blank_key=self.blank_k)
         else:
             blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)        # (b,h,n,1)
-            attn = attn + _table_rows(bias, pe_idx).permute(0, 3, 1, 2)
+            attn = attn + _position_bias(bias, pe_idx, self.ops)
             if cluster_mask is not None and not global_attn:
                 attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
             attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)

@@ -74,6 +74,8 @@ _PROTOTYPES = {
                                                      ctypes.c_int, ctypes.c_float, _P]),
     "clusten_neighbour_lists": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                               ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_bias_table_grad": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.c_int, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                     ctypes.c_int, ctypes.c_int, _P]),
     "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
@@ -952,6 +954,34 @@ def add_row_score(x: torch.Tensor, branch, weight: torch.Tensor, bias):
                                                  _ptr(score), x.numel() // c, c, code, _stream(device)),
                "clusten_add_row_score_forward")
     return total, score
+
+
+def bias_table_grad_supported(d_logit: torch.Tensor, rows: int) -> bool:
+    """True when `bias_table_grad` takes this case: a CUDA fp32 / fp16 / bf16 (B,H,N,M) gradient, at most 16000 rows."""
+    return d_logit.is_cuda and d_logit.dtype in _DTYPE_CODES and d_logit.dim() == 4 and 0 < rows <= 16000
+
+
+def bias_table_grad(d_logit: torch.Tensor, pe_idx: torch.Tensor, rows: int) -> torch.Tensor:
+    """d_table (rows,H) fp32 with d_table[pe_idx[b,i,j], h] = sum of d_logit[b,h,i,j]: the backward of the position-bias
+    lookup of an attention layer (models/aff_transformer.py:131-133).  d_logit (B,H,N,M), pe_idx (B,N,M) int64."""
+    lib = load()
+    _require_cuda("d_logit", d_logit)
+    device = d_logit.device
+    _require_cuda("pe_idx", pe_idx, device)
+    if not bias_table_grad_supported(d_logit, rows):
+        raise RuntimeError("bias_table_grad takes a fp32 / fp16 / bf16 (B,H,N,M) gradient and a table of at most 16000 rows")
+    B, H, N, M = d_logit.shape
+    if pe_idx.shape != (B, N, M) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")
+    d_logit, pe_idx = d_logit.contiguous(), pe_idx.contiguous()
+    d_table = torch.zeros(rows, H, dtype=torch.float32, device=device)
+    if d_logit.numel() == 0:
+        return d_table
+    with torch.cuda.device(device):
+        _check(lib.clusten_bias_table_grad(_ptr(d_logit), _ptr(pe_idx), _ptr(d_table), B, H, N, M, rows,
+                                           _DTYPE_CODES[d_logit.dtype], _stream(device)),
+               "clusten_bias_table_grad")
+    return d_table
 
 
 def merge_weights_supported(table_weights: torch.Tensor) -> bool:

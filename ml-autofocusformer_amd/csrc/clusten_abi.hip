@@ -325,6 +325,14 @@ int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch
     return launch_add_row_score(x, x_dtype, branch, sum_out, weight, bias, score, rows, C, dtype, as_stream(stream));
 }
 
+int clusten_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M,
+                            int rows, int dtype, clusten_stream stream) {
+    if (!d_logit || !pe_idx || !d_table) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (B <= 0 || H <= 0 || H > 65535 || N <= 0 || M <= 0 || rows <= 0) return CLUSTEN_ERR_BAD_DIMS;
+    return launch_bias_table_grad(d_logit, pe_idx, d_table, B, H, N, M, rows, dtype, as_stream(stream));
+}
+
 int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_idx, const int64_t* nbhd_idx,
                                   const float* prob, const int64_t* mask, float* weights, int B, int N, int Nout, int M,
                                   int IC, clusten_stream stream) {

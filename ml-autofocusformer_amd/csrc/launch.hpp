@@ -118,6 +118,10 @@ int launch_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* me
 int launch_add_row_score(const void* x, int x_dtype, const void* branch, void* sum_out, const void* w, const void* b,
                          void* score, int64_t rows, int C, int dtype, hipStream_t stream);
 
+// d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]; d_table (rows,H) fp32 zeroed by the caller, rows <= 16000.
+int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M, int rows,
+                           int dtype, hipStream_t stream);
+
 // w[b,i,j,:4] = table_w[pe_idx[b,i,j], :4] * prob[b, nbhd_idx[b,i,j]] * mask[b,i,j]   (prob, mask may be null)
 //   table_w (rows,4), prob (B,N), w (B,Nout,M,4): fp32;  pe_idx, nbhd_idx, mask: int64 (B,Nout,M).
 int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int64_t* nbhd_idx, const float* prob,

@@ -449,6 +449,29 @@ def test_add_row_score_kernel_equals_addition_linear_sigmoid(device, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_bias_table_grad_kernel_equals_the_scatter_add(device, dtype):
+    """Gradient of the position-bias table: per-workgroup sums in LDS against index_add in fp64."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(43)
+    for b, h, n, m, rows in ((3, 2, 200, 48, 12321), (2, 8, 49, 49, 12321), (1, 1, 5, 8, 7), (4, 16, 64, 48, 16000)):
+        g = torch.randn(b, h, n, m, generator=gen).to(dtype)
+        # positions near the table's centre, as relative offsets of neighbours are, plus a few anywhere
+        idx = (rows // 2 + torch.randint(-min(60, rows // 2), min(61, rows - rows // 2), (b, n, m), generator=gen))
+        far = torch.rand(b, n, m, generator=gen) < 0.05
+        idx[far] = torch.randint(rows, (int(far.sum()),), generator=gen)
+        want = torch.zeros(rows, h, dtype=torch.float64)
+        want.index_add_(0, idx.reshape(-1), g.double().permute(0, 2, 3, 1).reshape(-1, h))
+        got = _native.bias_table_grad(g.to(device), idx.to(device), rows)
+        assert got.dtype == torch.float32 and got.shape == (rows, h)
+        assert oracle.rel_err(got.cpu().double(), want) <= 1e-5
+    assert not _native.bias_table_grad_supported(g.to(device), 16001)
+    assert not _native.bias_table_grad_supported(g, 100)
+    with pytest.raises(RuntimeError):
+        _native.bias_table_grad(g.to(device), idx.to(device)[:, :, :3], rows)
+
+
+@pytest.mark.gpu
 def test_merge_weights_kernel_equals_the_tensor_expressions(device):
     from clusten import _native
     gen = torch.Generator().manual_seed(19)
