@@ -30,9 +30,19 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
     for (int b = 0; b < B; ++b) {
         const int64_t* idx_b = pe_idx + (int64_t)b * per_image;
         const T* g_bh = d_logit + ((int64_t)b * H + h) * per_image;
-        for (int64_t e = lo + threadIdx.x; e < hi; e += kGradThreads) {
-            const int64_t r = idx_b[e];
-            if ((uint64_t)r < (uint64_t)rows) atomicAdd(&col[r], to_acc(g_bh[e]));
+        for (int64_t e0 = lo + threadIdx.x; e0 < hi; e0 += 4 * kGradThreads) {
+            int64_t r[4];
+            float g[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {   // four independent loads before the first addition
+                const int64_t e = e0 + k * kGradThreads;
+                r[k] = e < hi ? idx_b[e] : -1;
+                g[k] = e < hi ? to_acc(g_bh[e]) : 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if ((uint64_t)r[k] < (uint64_t)rows) atomicAdd(&col[r[k]], g[k]);
+            }
         }
     }
     __syncthreads();
@@ -48,9 +58,10 @@ int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_
                            int dtype, hipStream_t stream) {
     if (rows > kGradRowsMax) return CLUSTEN_ERR_BAD_DIMS;
     const int64_t per_image = (int64_t)N * M;
-    // some 512 workgroups in all, each with enough elements to amortise clearing and flushing its column
-    int slices = max(1, 512 / H);
-    while (slices > 1 && per_image * B / slices < 4 * (int64_t)rows) slices /= 2;
+    // a workgroup per head and some 16 000 values: clearing its column of the table (rows words) and flushing the rows
+    // it touched stay small next to that, and the device gets thousands of workgroups to overlap their latencies
+    const int64_t want = (per_image * B + 16383) / 16384;
+    const int slices = (int)max((int64_t)1, min(want, min(per_image, (int64_t)8192)));
     const int64_t per_slice = (per_image + slices - 1) / slices;
     const dim3 grid((unsigned)slices, (unsigned)H);
     switch (dtype) {
