@@ -370,6 +370,18 @@ int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch
                                   const void* bias, void* score, int64_t rows, int C, int dtype,
                                   clusten_stream stream);
 
+/* Backward of clusten_attn_softmax_forward with respect to its logits:
+ *   s = sum_j probs[r,j] * d_probs[r,j] + blank_prob[r] * d_blank_prob[r]
+ *   d_logit[r,j] = probs[r,j] * (d_probs[r,j] - s);   d_blank_logit[r] = blank_prob[r] * (d_blank_prob[r] - s)
+ * for the `rows` = B*H*N rows of M neighbours.  d_logit is the gradient of the attention logits, and, through
+ * clusten_bias_table_grad, of the bias table (both enter the softmax as a sum; the mask is a constant).  probs,
+ * d_probs (rows,M), blank_prob, d_blank_prob, d_blank_logit (rows) fp32; d_logit (rows,M) of `dtype` (F32, F16 or
+ * BF16); M <= 64, M % 4 == 0 (else CLUSTEN_ERR_BAD_DIMS); 16-byte aligned.  No counterpart in the reference's
+ * extension modules. */
+int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
+                                  const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
+                                  int dtype, clusten_stream stream);
+
 /* Gradient of the relative-position bias table of an attention layer, the backward of
  * `pe_table.gather(index=pe_idx...)` added to the logits (models/aff_transformer.py:131-133):
  *   d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]

@@ -48,6 +48,7 @@ def default_ops():
                            channel_affine_gelu_supported=_native.channel_affine_gelu_supported,
                            add_row_score=_native.add_row_score, add_row_score_supported=_native.add_row_score_supported,
                            bias_table_grad=_native.bias_table_grad,
+                           attn_softmax_backward=_native.attn_softmax_backward,
                            neighbour_lists=_native.neighbour_lists,
                            neighbour_lists_supported=_native.neighbour_lists_supported)
 
@@ -134,6 +135,27 @@ class _PositionBias(torch.autograd.Function):
     def backward(ctx, grad):
         (pe_idx,) = ctx.saved_tensors
         return ctx.grad_kernel(grad, pe_idx, ctx.rows).to(ctx.dtype), None, None
+
+
+class _AttnSoftmax(torch.autograd.Function):
+    """Position bias, padding mask, blank token and softmax between QK and AV as one kernel forward and one backward
+    (aff_transformer.py:125-147), with the bias table's gradient from `bias_table_grad`: the training counterpart of
+    the inference path's `attn_softmax`."""
+
+    @staticmethod
+    def forward(ctx, attn, bias, pe_idx, mask, blank_logit, ops):
+        probs, blank_prob = ops.attn_softmax(attn, bias, pe_idx, mask, blank_logit=blank_logit)
+        ctx.save_for_backward(probs, blank_prob, pe_idx)
+        ctx.meta = (attn.dtype, bias.shape[0], bias.dtype, blank_logit.dtype, ops)
+        return probs, blank_prob
+
+    @staticmethod
+    def backward(ctx, d_probs, d_blank_prob):
+        probs, blank_prob, pe_idx = ctx.saved_tensors
+        attn_dtype, rows, bias_dtype, blank_dtype, ops = ctx.meta
+        d_logit, d_blank = ops.attn_softmax_backward(probs, blank_prob, d_probs, d_blank_prob, attn_dtype)
+        d_bias = ops.bias_table_grad(d_logit, pe_idx, rows).to(bias_dtype)
+        return d_logit, d_bias, None, None, d_blank.to(blank_dtype), None
 
 
 def _position_bias(bias, pe_idx, ops):
@@ -276,12 +298,20 @@ class ClusterAttention(nn.Module):
             attn, blank = fused(attn, bias, pe_idx, cluster_mask, query=q, blank_key=self.blank_k)
         else:
             blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)        # (b,h,n,1)
-            attn = attn + _position_bias(bias, pe_idx, self.ops)
-            if cluster_mask is not None and not global_attn:
-                attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
-            attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
-            attn = self.attn_drop(attn)
-            blank, attn = attn[..., -1:], attn[..., :-1]
+            if (fused is not None and getattr(self.ops, "attn_softmax_backward", None) is not None
+                    and getattr(self.ops, "bias_table_grad", None) is not None and torch.is_grad_enabled()
+                    and not global_attn and attn.is_cuda and bias.shape[0] <= 16000
+                    and not (self.training and self.attn_drop.p > 0)
+                    and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
+                # training: the same glue as one kernel forward and one backward
+                attn, blank = _AttnSoftmax.apply(attn, bias, pe_idx, cluster_mask, blank, self.ops)
+            else:
+                attn = attn + _position_bias(bias, pe_idx, self.ops)
+                if cluster_mask is not None and not global_attn:
+                    attn = attn + (1 - cluster_mask.reshape(b, 1, n, -1)) * (-100)
+                attn = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
+                attn = self.attn_drop(attn)
+                blank, attn = attn[..., -1:], attn[..., :-1]
 
         if global_attn:
             out = attn @ v

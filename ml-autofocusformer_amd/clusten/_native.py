@@ -74,6 +74,8 @@ _PROTOTYPES = {
                                                      ctypes.c_int, ctypes.c_float, _P]),
     "clusten_neighbour_lists": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                               ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_attn_softmax_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                    _P]),
     "clusten_bias_table_grad": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                               ctypes.c_int, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -571,6 +573,34 @@ def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Ten
                                                 _ptr(blank_prob), shape, code, _stream(device)),
                "clusten_attn_softmax_forward")
     return probs, blank_prob
+
+
+def attn_softmax_backward(probs: torch.Tensor, blank_prob: torch.Tensor, d_probs: torch.Tensor,
+                          d_blank_prob: torch.Tensor, logit_dtype):
+    """(d_logit (B,H,N,M) of logit_dtype, d_blank_logit (B,H,N,1) fp32): the backward of `attn_softmax` with respect
+    to the attention logits (= the gradient of the gathered bias too) and to the blank token's logit."""
+    lib = load()
+    _require_cuda("probs", probs)
+    device = probs.device
+    if probs.dim() != 4 or probs.dtype != torch.float32 or logit_dtype not in _DTYPE_CODES:
+        raise RuntimeError("probs must be fp32 (B,H,N,M); logits fp32, fp16 or bf16")
+    b, h, n, m = probs.shape
+    if m > 64 or m % 4:
+        raise RuntimeError("attn_softmax_backward: M <= 64, M % 4 == 0")
+    probs = probs.contiguous()
+    d_probs = d_probs.to(torch.float32).expand_as(probs).contiguous()
+    blank_prob = blank_prob.reshape(b, h, n).float().contiguous()
+    d_blank_prob = d_blank_prob.to(torch.float32).expand(b, h, n, 1).reshape(b, h, n).contiguous()
+    d_logit = torch.empty(b, h, n, m, dtype=logit_dtype, device=device)
+    d_blank_logit = torch.empty(b, h, n, 1, dtype=torch.float32, device=device)
+    if d_logit.numel() == 0:
+        return d_logit, d_blank_logit
+    with torch.cuda.device(device):
+        _check(lib.clusten_attn_softmax_backward(_ptr(probs), _ptr(blank_prob), _ptr(d_probs), _ptr(d_blank_prob),
+                                                 _ptr(d_logit), _ptr(d_blank_logit), b * h * n, m,
+                                                 _DTYPE_CODES[logit_dtype], _stream(device)),
+               "clusten_attn_softmax_backward")
+    return d_logit, d_blank_logit
 
 
 def cluster_attention_supported(query: torch.Tensor, nnc: int) -> bool:

@@ -111,4 +111,64 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
     }
 }
 
+// Backward of the softmax over the M neighbours and the blank token:
+//   s = sum_j p_j dp_j + p_blank dp_blank;   d_logit_j = p_j (dp_j - s);   d_blank_logit = p_blank (dp_blank - s)
+// (the bias, the mask and the logits enter the softmax as a sum, so d_logit is the gradient of each of them).
+// One row per 16 lanes, four consecutive neighbours per lane; probs, d_probs fp32, d_logit of the logits' type.
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_softmax_backward_kernel(const float* __restrict__ probs,
+                                                                    const float* __restrict__ blank_prob,
+                                                                    const float* __restrict__ d_probs,
+                                                                    const float* __restrict__ d_blank_prob,
+                                                                    T* __restrict__ d_logit, float* __restrict__ d_blank_logit,
+                                                                    int64_t rows, int M) {
+    const int sub = threadIdx.x & 15;
+    const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const bool live = row_raw < rows;
+    const int64_t row = live ? row_raw : rows - 1;  // every lane stays in the shuffles
+    const bool mine = 4 * sub < M;
+    float4 p = make_float4(0.f, 0.f, 0.f, 0.f), dp = p;
+    if (mine) {
+        p = *reinterpret_cast<const float4*>(probs + row * M + 4 * sub);
+        dp = *reinterpret_cast<const float4*>(d_probs + row * M + 4 * sub);
+    }
+    const float pb = blank_prob[row], dpb = d_blank_prob[row];
+    float s = (p.x * dp.x + p.y * dp.y) + (p.z * dp.z + p.w * dp.w);
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) s += __shfl_xor(s, m);
+    s += pb * dpb;
+    if (!live) return;
+    if (mine) {
+        float v[4] = {p.x * (dp.x - s), p.y * (dp.y - s), p.z * (dp.z - s), p.w * (dp.w - s)};
+        *reinterpret_cast<typename Quad<T>::raw*>(d_logit + row * M + 4 * sub) = Quad<T>::pack(v);
+    }
+    if (sub == 0) d_blank_logit[row] = pb * (dpb - s);
+}
+
+}  // namespace
+
+int launch_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
+                                 const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
+                                 int dtype, hipStream_t stream) {
+    const unsigned blocks = (unsigned)((rows + 15) / 16);
+    switch (dtype) {
+        case CLUSTEN_F32:
+            hipLaunchKernelGGL(attn_softmax_backward_kernel<float>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
+                               d_probs, d_blank_prob, static_cast<float*>(d_logit), d_blank_logit, rows, M);
+            break;
+        case CLUSTEN_F16:
+            hipLaunchKernelGGL(attn_softmax_backward_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
+                               d_probs, d_blank_prob, static_cast<f16_t*>(d_logit), d_blank_logit, rows, M);
+            break;
+        case CLUSTEN_BF16:
+            hipLaunchKernelGGL(attn_softmax_backward_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
+                               d_probs, d_blank_prob, static_cast<bf16_t*>(d_logit), d_blank_logit, rows, M);
+            break;
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+    return launch_status();
+}
+
 }  // namespace clusten

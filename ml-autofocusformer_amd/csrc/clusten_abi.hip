@@ -325,6 +325,17 @@ int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch
     return launch_add_row_score(x, x_dtype, branch, sum_out, weight, bias, score, rows, C, dtype, as_stream(stream));
 }
 
+int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
+                                  const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
+                                  int dtype, clusten_stream stream) {
+    if (!probs || !blank_prob || !d_probs || !d_blank_prob || !d_logit || !d_blank_logit) return CLUSTEN_ERR_NULL_POINTER;
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (rows <= 0 || M <= 0 || M > 64 || M % 4 != 0 || (rows + 15) / 16 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(probs) || !aligned16(d_probs) || !aligned16(d_logit)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_attn_softmax_backward(probs, blank_prob, d_probs, d_blank_prob, d_logit, d_blank_logit, rows, M, dtype,
+                                        as_stream(stream));
+}
+
 int clusten_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M,
                             int rows, int dtype, clusten_stream stream) {
     if (!d_logit || !pe_idx || !d_table) return CLUSTEN_ERR_NULL_POINTER;

@@ -118,6 +118,11 @@ int launch_neighbour_lists(const float* pos, const int64_t* nearest, int64_t* me
 int launch_add_row_score(const void* x, int x_dtype, const void* branch, void* sum_out, const void* w, const void* b,
                          void* score, int64_t rows, int C, int dtype, hipStream_t stream);
 
+// d_logit = probs * (d_probs - s), d_blank_logit = blank_prob * (d_blank_prob - s), s the row's sum of p * dp.
+int launch_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
+                                 const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
+                                 int dtype, hipStream_t stream);
+
 // d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]; d_table (rows,H) fp32 zeroed by the caller, rows <= 16000.
 int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M, int rows,
                            int dtype, hipStream_t stream);

@@ -449,6 +449,41 @@ def test_add_row_score_kernel_equals_addition_linear_sigmoid(device, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_attention_glue_training_function_matches_autograd_through_the_expressions(device, dtype, with_mask):
+    """Bias lookup, mask, blank token and softmax as one kernel forward and one backward (training): outputs and the
+    gradients of the logits, the bias table and the blank logit against autograd through the tensor expressions."""
+    from aff.model import _AttnSoftmax, default_ops
+    ops = default_ops()
+    gen = torch.Generator().manual_seed(47)
+    b, h, n, m, rows = 2, 3, 50, 48, 211
+    attn = torch.randn(b, h, n, m, generator=gen).to(dtype).to(device).requires_grad_()
+    bias = torch.randn(rows, h, generator=gen).to(dtype).to(device).requires_grad_()
+    blank = torch.randn(b, h, n, 1, generator=gen).to(device).requires_grad_()
+    pe_idx = torch.randint(rows, (b, n, m), generator=gen).to(device)
+    mask = (torch.rand(b, n, m, generator=gen) > 0.1).long().to(device) if with_mask else None
+    g_p = torch.randn(b, h, n, m, generator=gen).to(device)
+    g_b = torch.randn(b, h, n, 1, generator=gen).to(device)
+
+    probs, blank_prob = _AttnSoftmax.apply(attn, bias, pe_idx, mask, blank, ops)
+    ((probs * g_p).sum() + (blank_prob * g_b).sum()).backward()
+    got = (probs.detach(), blank_prob.detach(), attn.grad.clone(), bias.grad.clone(), blank.grad.clone())
+    attn.grad = bias.grad = blank.grad = None
+
+    x = attn.float() + bias.float()[pe_idx].permute(0, 3, 1, 2)
+    if mask is not None:
+        x = x + (1 - mask.reshape(b, 1, n, m)) * (-100)
+    p = torch.softmax(torch.cat([x, blank], dim=-1), dim=-1)
+    ((p[..., :-1] * g_p).sum() + (p[..., -1:] * g_b).sum()).backward()
+    want = (p[..., :-1].detach(), p[..., -1:].detach(), attn.grad, bias.grad, blank.grad)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    for name, a, w in zip(("probs", "blank_prob", "d_attn", "d_bias", "d_blank"), got, want):
+        assert a.shape == w.shape and a.dtype == w.dtype, name
+        assert oracle.rel_err(a.float().cpu(), w.float().cpu()) <= tol, name
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_bias_table_grad_kernel_equals_the_scatter_add(device, dtype):
     """Gradient of the position-bias table: per-workgroup sums in LDS against index_add in fp64."""
