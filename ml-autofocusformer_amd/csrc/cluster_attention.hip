@@ -91,15 +91,21 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const T* __restrict__ q, clusten_strides qs, const T* __restrict__ k, clusten_strides ks, const T* __restrict__ v,
     clusten_strides vs, const int32_t* __restrict__ cluster_idx, const T* __restrict__ table,
     const int64_t* __restrict__ pe_idx, const int64_t* __restrict__ mask, const float* __restrict__ blank_k,
-    const float* __restrict__ blank_v, T* __restrict__ out, clusten_strides os, int H, int N, float scale,
-    int tiles_per_batch, int total_tiles, int lists_shared) {
+    const float* __restrict__ blank_v, T* __restrict__ out, clusten_strides os, int H_all, int N, float scale,
+    int tiles_per_batch, int total_tiles, int lists_shared, int head_groups) {
     typedef short S4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) S4* LdsS4;
 
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
+    // a workgroup serves the heads [h0, h0 + H) of its tile (see head_groups_for())
+    const int unit = xcd_tile(blockIdx.x, total_tiles * head_groups);
+    if (unit < 0) return;
+    const int tile = unit / head_groups;
+    const int heads_per_group = (H_all + head_groups - 1) / head_groups;
+    const int h0 = (unit - tile * head_groups) * heads_per_group;
+    const int H = min(heads_per_group, H_all - h0);
+    if (H <= 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
@@ -116,7 +122,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const int64_t tok = list_b * N + i0 + min(t, nt - 1);
 
     // q rows of head h -> slot h % 2 (lanes 0..31: token lane / 4, piece lane % 4)
-    const char* q_tile = reinterpret_cast<const char*>(q + (int64_t)b * qs.b + (int64_t)i0 * qs.n);
+    const char* q_tile = reinterpret_cast<const char*>(q + (int64_t)b * qs.b + (int64_t)h0 * qs.h + (int64_t)i0 * qs.n);
     const uint32_t q_off = (uint32_t)min(g_sub, nt - 1) * (uint32_t)qs.n * 2 + (uint32_t)g_pos * 16;
     auto fetch_q = [&](int h) {
         if (lane < 32) {
@@ -179,8 +185,8 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const int total_rows = 8 * U;
     const int passes = (U + kPassRuns - 1) / kPassRuns;
     const uint32_t k_pitch = (uint32_t)ks.n * 2, v_pitch = (uint32_t)vs.n * 2;
-    const char* k_b = reinterpret_cast<const char*>(k + (int64_t)b * ks.b);
-    const char* v_b = reinterpret_cast<const char*>(v + (int64_t)b * vs.b);
+    const char* k_b = reinterpret_cast<const char*>(k + (int64_t)b * ks.b + (int64_t)h0 * ks.h);
+    const char* v_b = reinterpret_cast<const char*>(v + (int64_t)b * vs.b + (int64_t)h0 * vs.h);
 
     // rows of the distinct clusters 8*pass .. 8*pass+7, as this lane gathers them: access a moves row 16*a + g_sub of
     // the pass; clusters past the last one repeat it so that every row of a 32-row step holds data
@@ -224,12 +230,12 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         float bias[kR];
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
-            const uint32_t cell = lane_offset(((uint32_t)(pe[r] & 0x7fffffff) * (uint32_t)H + (uint32_t)h) * 2);
+            const uint32_t cell = lane_offset(((uint32_t)(pe[r] & 0x7fffffff) * (uint32_t)H_all + (uint32_t)(h0 + h)) * 2);
             bias[r] = to_acc(*reinterpret_cast<const T*>(reinterpret_cast<const char*>(table) + cell)) +
                       (pe[r] < 0 ? -100.f : 0.f);
         }
-        const float4 bk = *reinterpret_cast<const float4*>(blank_k + h * kC + 4 * i);
-        const float bv[2] = {blank_v[h * kC + r16], blank_v[h * kC + 16 + r16]};
+        const float4 bk = *reinterpret_cast<const float4*>(blank_k + (h0 + h) * kC + 4 * i);
+        const float bv[2] = {blank_v[(h0 + h) * kC + r16], blank_v[(h0 + h) * kC + 16 + r16]};
 
         // ---- scores -------------------------------------------------------------------------------------
         float logit[kR];
@@ -379,7 +385,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         // the head's only store, and the last vector-memory operation it issues (see the wait at the top of the loop)
         if (lane < 32 && g_sub < nt) {
             const Piece o = *reinterpret_cast<const Piece*>(stage + O_BASE + lane * 16);
-            char* dst = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)(i0 + g_sub) * os.n);
+            char* dst = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)(h0 + h) * os.h + (int64_t)(i0 + g_sub) * os.n);
             store_streaming(reinterpret_cast<Piece*>(dst + g_pos * 16), o);
         }
     }
@@ -392,10 +398,11 @@ int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strid
                  float scale, int lists_shared, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
+    const int groups = head_groups_for(total, s.H);  // 196 tokens x 8 heads, B = 128: 69.6 -> 63.9 us
+    hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total * groups)), dim3(kWave), 0, stream,
                        static_cast<const T*>(q), qs, static_cast<const T*>(k), ks, static_cast<const T*>(v), vs,
                        cluster_idx, static_cast<const T*>(table), pe_idx, mask, blank_k, blank_v, static_cast<T*>(out),
-                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared);
+                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups);
     return launch_status();
 }
 

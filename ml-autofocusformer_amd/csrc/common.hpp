@@ -208,6 +208,13 @@ __device__ __forceinline__ int xcd_tile(int wg, int total) {
 // Grid size that xcd_tile() needs to cover `total` tiles.
 inline int xcd_grid(int total) { return ((total + kXcds - 1) / kXcds) * kXcds; }
 
+// Head groups per tile for the kernels in which one wave walks the heads of a tile: with few tiles and many
+// heads (the late stages of a model) the device is short of waves, and the heads of a tile are dealt to two
+// workgroups.  Measured at B = 128, fp32: 196 tokens x 8 heads 32 -> 27.6 us (QK), 33.4 -> 29.8 us (AV); 49 tokens x
+// 16 heads 20.1 -> 16.1 us, 24.6 -> 17.4 us; four or eight groups are no faster, and at 784 tokens x 4 heads (12 544
+// tiles) two groups cost AV 3 %.
+inline int head_groups_for(int total_tiles, int H) { return (total_tiles < 8192 && H >= 4) ? 2 : 1; }
+
 // ---- host-side argument checks ------------------------------------------------------------------
 
 inline bool dtype_ok(int dtype) { return dtype >= CLUSTEN_F32 && dtype <= CLUSTEN_F64; }

@@ -109,9 +109,9 @@ struct Staging {
 template <typename T, int C, int Q, bool FAST, bool CLUSTERS = false>
 __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restrict__ a, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
-                                                                T* __restrict__ out, int H, int N, int M,
+                                                                T* __restrict__ out, int H_all, int N, int M,
                                                                 clusten_strides as, clusten_strides rs,
-                                                                int tiles_per_batch, int total_tiles) {
+                                                                int tiles_per_batch, int total_tiles, int head_groups) {
     typedef Staging<T, C, Q, FAST> S;
     typedef VecIO<T, S::VEC> RunIO;
     typedef VecIO<T, 4> OutIO;
@@ -120,8 +120,15 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
 
     __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
 
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
+    // a workgroup serves the heads [h0, h0 + H) of its tile: short sequences with many heads are launched with
+    // several head groups per tile (neighbours in the grid, so the later ones find the tile's lists in the L2)
+    const int unit = xcd_tile(blockIdx.x, total_tiles * head_groups);
+    if (unit < 0) return;
+    const int tile = unit / head_groups;
+    const int heads_per_group = (H_all + head_groups - 1) / head_groups;
+    const int h0 = (unit - tile * head_groups) * heads_per_group;
+    const int H = min(heads_per_group, H_all - h0);
+    if (H <= 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
@@ -132,9 +139,9 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
     const int g_sub = lane / S::PPR;
     const int g_pos = lane % S::PPR;
 
-    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b);
-    const char* a_tile = reinterpret_cast<const char*>(a + (int64_t)b * as.b + (int64_t)i0 * as.n);
-    char* out_tile = reinterpret_cast<char*>(out + ((int64_t)b * H * N + i0) * M);
+    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b + (int64_t)h0 * rs.h);
+    const char* a_tile = reinterpret_cast<const char*>(a + (int64_t)b * as.b + (int64_t)h0 * as.h + (int64_t)i0 * as.n);
+    char* out_tile = reinterpret_cast<char*>(out + (((int64_t)b * H_all + h0) * N + i0) * M);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
     const int32_t* cid_tile = reinterpret_cast<const int32_t*>(idx) + ((int64_t)b * N + i0) * (M >> 3);
     int cid = 0;  // CLUSTERS: the cluster number of run `lane` of the tile (token lane / R, run lane % R)
@@ -555,9 +562,10 @@ int launch_tile_q(const void* a, clusten_strides as, const void* rows, clusten_s
                   void* out, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q, FAST, CLUSTERS>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
-                       static_cast<const T*>(a), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
-                       s.M, as, rs, tiles_per_batch, total);
+    const int groups = head_groups_for(total, s.H);
+    hipLaunchKernelGGL((gather_dot_tile_kernel<T, C, Q, FAST, CLUSTERS>), dim3(xcd_grid(total * groups)), dim3(kWave), 0,
+                       stream, static_cast<const T*>(a), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
+                       s.M, as, rs, tiles_per_batch, total, groups);
     return launch_status();
 }
 

@@ -97,9 +97,9 @@ struct SumStaging {
 template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false>
 __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
-                                                                T* __restrict__ out, int H, int N, int M,
+                                                                T* __restrict__ out, int H_all, int N, int M,
                                                                 clusten_strides rs, clusten_strides os,
-                                                                int tiles_per_batch, int total_tiles) {
+                                                                int tiles_per_batch, int total_tiles, int head_groups) {
     typedef SumStaging<T, C, Q, FAST> S;
     typedef VecIO<T, S::ECH> ChIO;   // the lane's channels of one gathered row
     typedef VecIO<T, S::SPP> PieceIO;
@@ -108,8 +108,15 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
 
     __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
 
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
+    // a workgroup serves the heads [h0, h0 + H) of its tile: short sequences with many heads are launched with
+    // several head groups per tile (neighbours in the grid, so the later ones find the tile's lists in the L2)
+    const int unit = xcd_tile(blockIdx.x, total_tiles * head_groups);
+    if (unit < 0) return;
+    const int tile = unit / head_groups;
+    const int heads_per_group = (H_all + head_groups - 1) / head_groups;
+    const int h0 = (unit - tile * head_groups) * heads_per_group;
+    const int H = min(heads_per_group, H_all - h0);
+    if (H <= 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
     const int nt = min(kTileTokens, N - i0);
@@ -119,7 +126,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     const int g_sub = lane / S::PPR;  // gather side: in access i this lane moves one piece of row i*RPI + g_sub
     const int g_pos = lane % S::PPR;
 
-    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b);
+    const char* rows_b = reinterpret_cast<const char*>(rows + (int64_t)b * rs.b + (int64_t)h0 * rs.h);
     const int64_t* idx_tile = idx + ((int64_t)b * N + i0) * M;
     const int32_t* cid_tile = reinterpret_cast<const int32_t*>(idx) + ((int64_t)b * N + i0) * (M >> 3);
     int cid = 0;  // CLUSTERS: the cluster number of run `lane` of the tile (token lane / R, run lane % R)
@@ -129,7 +136,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     // 64*i + lane; piece q is slot group q / 8 of token q % 8 (tokens past the end of a partial tile
     // repeat its last token, slot groups past the end of the list repeat its last group).
     auto fetch_p = [&](int h, int j0, int mc, int ps) {
-        const char* p_head = reinterpret_cast<const char*>(p + (((int64_t)b * H + h) * N + i0) * M + j0);
+        const char* p_head = reinterpret_cast<const char*>(p + (((int64_t)b * H_all + h0 + h) * N + i0) * M + j0);
 #pragma unroll
         for (int i = 0; i < S::NI_P; ++i) {
             const int q = i * kWave + lane;
@@ -181,7 +188,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     // the tile is written: when the out rows of the tile are contiguous too, they are laid out row-major in
     // LDS (over the gathered rows) and leave with full-width 16-byte stores.
     auto store_head = [&](int h, F32x4 (&d)[S::ECH], int tok_lo, int tok_hi, bool whole) {
-        char* out_h = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
+        char* out_h = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)(h0 + h) * os.h + (int64_t)i0 * os.n);
         if (FAST && whole && rows_contiguous) {
             __syncthreads();  // every operand read of this head is complete: reuse the row area
             if (kq < 2) {
@@ -308,7 +315,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                     ppass[k] = valid ? prow / PROWS : -1;
                     const int rr = prow % PROWS;
                     pm_at[k] = tok * S::PM_STRIDE + (rr >> 2);
-                    p_src[k] = p + (((int64_t)b * H) * N + i0 + min(tok, nt - 1)) * M + min(j, M - S::SPP);
+                    p_src[k] = p + (((int64_t)b * H_all + h0) * N + i0 + min(tok, nt - 1)) * M + min(j, M - S::SPP);
                 }
                 const int total_rows = 8 * U;
                 const float* pm_lane = pm + (kq * kTileTokens + (n & 7)) * S::PM_STRIDE;
@@ -510,7 +517,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                         }
                         __syncthreads();
                         char* out_h =
-                            reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)h * os.h + (int64_t)i0 * os.n);
+                            reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)(h0 + h) * os.h + (int64_t)i0 * os.n);
                         const int chunk_bytes = nt * S::RB;
 #pragma unroll
                         for (int i = 0; i < NO; ++i) {
@@ -606,10 +613,11 @@ int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    const int grid = xcd_grid(total);
+    const int groups = head_groups_for(total, s.H);
+    const int grid = xcd_grid(total * groups);
     hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT, CLUSTERS>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
-                       s.M, rs, os, tiles_per_batch, total);
+                       s.M, rs, os, tiles_per_batch, total, groups);
     return launch_status();
 }
 
