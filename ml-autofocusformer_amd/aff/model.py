@@ -82,6 +82,30 @@ def _linear(lin, x, ops=None, gelu=False):
     return F.gelu(y) if gelu else y
 
 
+def _linear_pair(first, second, x, ops=None):
+    """`(first(x), second(x))` for two nn.Linear layers that read the same input (the query and the key / value
+    projections of an attention layer, aff_transformer.py:103-106).  In inference under mixed precision they run as
+    one matrix product over the stacked 16-bit weights, kept between calls like the single copies; the results are
+    the two column ranges of its output (views).  Layers that the library's small-layer kernel takes stay apart."""
+    if (torch.is_grad_enabled() or not x.is_cuda or not torch.is_autocast_enabled("cuda")
+            or first.bias is None or second.bias is None):
+        return _linear(first, x, ops), _linear(second, x, ops)
+    dt = torch.get_autocast_dtype("cuda")
+    a, b = _cast_params(first, dt), _cast_params(second, dt)
+    x = x if x.dtype == dt else x.to(dt)
+    fn = getattr(ops, "linear", None)
+    if fn is not None and ops.linear_supported(x, a[1], False) and ops.linear_supported(x, b[1], False):
+        return fn(x, a[1], a[2], False), fn(x, b[1], b[2], False)
+    key = (a[0], b[0])
+    cache = first.__dict__.get("_pair_cache")
+    if cache is None or cache[0] != key:
+        cache = (key, torch.cat([a[1], b[1]], 0), torch.cat([a[2], b[2]], 0))
+        first.__dict__["_pair_cache"] = cache    # a plain attribute, like _cast_cache
+    y = F.linear(x, cache[1], cache[2])
+    n_first = a[1].shape[0]
+    return y[..., :n_first], y[..., n_first:]
+
+
 def _layer_norm(norm, x, ops, feeds_linear=False):
     """`norm(x)` for an nn.LayerNorm; in inference on the GPU through the library's one-pass kernel when `ops` has it.
 
@@ -261,8 +285,8 @@ class ClusterAttention(nn.Module):
         # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
         compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
                    and getattr(self.ops, "qk_clusters", None) is not None)
-        q = _linear(self.q, feat, self.ops)
-        kv = _linear(self.kv, feat, self.ops).view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                   # (2,b,h,n,ch) view
+        q, kv = _linear_pair(self.q, self.kv, feat, self.ops)
+        kv = kv.view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                                                 # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
         one_kernel = getattr(self.ops, "cluster_attention", None)
         if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
