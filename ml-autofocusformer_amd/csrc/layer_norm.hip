@@ -14,8 +14,8 @@
 // cluster order (:465-466, the first stage) taken along.  None has a counterpart in the reference's extension
 // modules.
 //
-// A row is held by L = min(64, C / 4) lanes, four consecutive channels per lane and step (C / (4 L) steps), so
-// that a wave reads 1 KiB contiguous per access; mean and variance are two reductions over registers (the
+// A row is held by L lanes, W consecutive channels per lane and step (W = 8 when a 16-bit tensor is among the
+// operands, so that their accesses are 16 bytes per lane, else 4), C / (W L) steps; mean and variance are two reductions over registers (the
 // variance from the centred values, as a two-pass computation gives it), across the lanes of the row with xor
 // shuffles.  All arithmetic is fp32.
 #include <type_traits>
@@ -32,15 +32,45 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
+// W consecutive elements of a row (4 or 8) between memory and fp32 registers, in 16-byte accesses where W elements
+// fill them.
+template <typename T, int W>
+__device__ __forceinline__ void load_run(const T* p, float (&x)[W]) {
+    if constexpr (W == 4) {
+        Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(p), x);
+    } else if constexpr (sizeof(T) == 2) {
+        VecIO<T, 8>::unpack(*reinterpret_cast<const typename VecIO<T, 8>::raw*>(p), x);
+    } else {
+        float lo[4], hi[4];
+        Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(p), lo);
+        Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(p + 4), hi);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = lo[e], x[4 + e] = hi[e];
+    }
+}
+template <typename T, int W>
+__device__ __forceinline__ void store_run(T* p, const float (&x)[W]) {
+    if constexpr (W == 4) {
+        *reinterpret_cast<typename Quad<T>::raw*>(p) = Quad<T>::pack(x);
+    } else if constexpr (sizeof(T) == 2) {
+        *reinterpret_cast<typename VecIO<T, 8>::raw*>(p) = VecIO<T, 8>::pack(x);
+    } else {
+        const float lo[4] = {x[0], x[1], x[2], x[3]}, hi[4] = {x[4], x[5], x[6], x[7]};
+        *reinterpret_cast<typename Quad<T>::raw*>(p) = Quad<T>::pack(lo);
+        *reinterpret_cast<typename Quad<T>::raw*>(p + 4) = Quad<T>::pack(hi);
+    }
+}
+
 // ResT = void: plain layer norm of x.  Otherwise the row normalised is x + branch (the residual connection ahead of
 // the norm), rounded to x's type as the framework's addition would leave it and also written to `sum_out`.
-template <typename InT, typename ResT, typename OutT, int L, int V>
+// A row is held by L lanes, W consecutive channels per lane and step, V steps: C = W * L * V.
+template <typename InT, typename ResT, typename OutT, int L, int V, int W>
 __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__ x, const ResT* __restrict__ branch,
                                                          InT* __restrict__ sum_out, const float* __restrict__ weight,
                                                          const float* __restrict__ bias, OutT* __restrict__ out,
                                                          int64_t rows, float eps, const int64_t* __restrict__ order,
                                                          int group, const InT* __restrict__ pre_bias) {
-    constexpr int C = 4 * L * V;
+    constexpr int C = W * L * V;
     constexpr int ROWS_PER_WG = 256 / L;
     const int sub = threadIdx.x % L;
     const int64_t row_raw = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / L;
@@ -50,59 +80,70 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const InT* __restrict__
     // of `group` rows, an image's tokens, permuted the same way)
     const int64_t src = order ? row - row % group + order[row % group] : row;
     const InT* xr = x + src * C;
-    float4 v[V];
+    float v[V][W];
 #pragma unroll
     for (int s = 0; s < V; ++s) {
-        float in[4];
-        Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(xr + 4 * (s * L + sub)), in);
+        const int c = W * (s * L + sub);
+        load_run<InT, W>(xr + c, v[s]);
         if (pre_bias) {  // a per-channel bias the producer left out, added as its own addition would have: rounded
-            float pb[4];
-            Quad<InT>::unpack(*reinterpret_cast<const typename Quad<InT>::raw*>(pre_bias + 4 * (s * L + sub)), pb);
+            float pb[W];
+            load_run<InT, W>(pre_bias + c, pb);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) in[e] = to_acc(from_acc<InT>(in[e] + pb[e]));
+            for (int e = 0; e < W; ++e) v[s][e] = to_acc(from_acc<InT>(v[s][e] + pb[e]));
         }
         if constexpr (!std::is_void<ResT>::value) {
-            float br[4];
-            Quad<ResT>::unpack(*reinterpret_cast<const typename Quad<ResT>::raw*>(branch + row * C + 4 * (s * L + sub)), br);
+            float br[W];
+            load_run<ResT, W>(branch + row * C + c, br);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) in[e] = to_acc(from_acc<InT>(in[e] + br[e]));
-            if (live) {
-                *reinterpret_cast<typename Quad<InT>::raw*>(sum_out + row * C + 4 * (s * L + sub)) = Quad<InT>::pack(in);
-            }
+            for (int e = 0; e < W; ++e) v[s][e] = to_acc(from_acc<InT>(v[s][e] + br[e]));
+            if (live) store_run<InT, W>(sum_out + row * C + c, v[s]);
         }
-        v[s] = make_float4(in[0], in[1], in[2], in[3]);
     }
+    // sums in the order ((a + b) + (c + d)) per group of four, groups in channel order
     float sum = 0.f;
 #pragma unroll
-    for (int s = 0; s < V; ++s) sum += (v[s].x + v[s].y) + (v[s].z + v[s].w);
+    for (int s = 0; s < V; ++s) {
+#pragma unroll
+        for (int e = 0; e < W; e += 4) sum += (v[s][e] + v[s][e + 1]) + (v[s][e + 2] + v[s][e + 3]);
+    }
     const float mean = row_sum<L>(sum) * (1.f / C);
     float sq = 0.f;
 #pragma unroll
     for (int s = 0; s < V; ++s) {
-        v[s].x -= mean, v[s].y -= mean, v[s].z -= mean, v[s].w -= mean;
-        sq += (v[s].x * v[s].x + v[s].y * v[s].y) + (v[s].z * v[s].z + v[s].w * v[s].w);
+#pragma unroll
+        for (int e = 0; e < W; ++e) v[s][e] -= mean;
+#pragma unroll
+        for (int e = 0; e < W; e += 4) {
+            sq += (v[s][e] * v[s][e] + v[s][e + 1] * v[s][e + 1]) + (v[s][e + 2] * v[s][e + 2] + v[s][e + 3] * v[s][e + 3]);
+        }
     }
     const float rstd = rsqrtf(row_sum<L>(sq) * (1.f / C) + eps);
     if (!live) return;
     OutT* orow = out + row * C;
 #pragma unroll
     for (int s = 0; s < V; ++s) {
-        const int c = 4 * (s * L + sub);
-        const float4 w = *reinterpret_cast<const float4*>(weight + c);
-        const float4 b = *reinterpret_cast<const float4*>(bias + c);
-        float y[4] = {v[s].x * rstd * w.x + b.x, v[s].y * rstd * w.y + b.y, v[s].z * rstd * w.z + b.z,
-                      v[s].w * rstd * w.w + b.w};
-        *reinterpret_cast<typename Quad<OutT>::raw*>(orow + c) = Quad<OutT>::pack(y);
+        const int c = W * (s * L + sub);
+        float y[W];
+#pragma unroll
+        for (int e = 0; e < W; e += 4) {
+            const float4 w = *reinterpret_cast<const float4*>(weight + c + e);
+            const float4 b = *reinterpret_cast<const float4*>(bias + c + e);
+            y[e] = v[s][e] * rstd * w.x + b.x;
+            y[e + 1] = v[s][e + 1] * rstd * w.y + b.y;
+            y[e + 2] = v[s][e + 2] * rstd * w.z + b.z;
+            y[e + 3] = v[s][e + 3] * rstd * w.w + b.w;
+        }
+        store_run<OutT, W>(orow + c, y);
     }
 }
 
-template <typename InT, typename ResT, typename OutT, int L, int V>
+template <typename InT, typename ResT, typename OutT, int L, int V, int W = 4>
 int launch_lv(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
               int64_t rows, float eps, hipStream_t stream, const int64_t* order = nullptr, int group = 1,
               const void* pre_bias = nullptr) {
     constexpr int ROWS_PER_WG = 256 / L;
     const int64_t blocks = (rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
-    hipLaunchKernelGGL((layer_norm_kernel<InT, ResT, OutT, L, V>), dim3((unsigned)blocks), dim3(256), 0, stream,
+    hipLaunchKernelGGL((layer_norm_kernel<InT, ResT, OutT, L, V, W>), dim3((unsigned)blocks), dim3(256), 0, stream,
                        static_cast<const InT*>(x), static_cast<const ResT*>(branch), static_cast<InT*>(sum_out), weight,
                        bias, static_cast<OutT*>(out), rows, eps, order, group, static_cast<const InT*>(pre_bias));
     return launch_status();
@@ -112,16 +153,32 @@ template <typename InT, typename ResT, typename OutT>
 int launch_typed(const void* x, const void* branch, void* sum_out, const float* weight, const float* bias, void* out,
                  int64_t rows, int C, float eps, hipStream_t stream, const int64_t* order = nullptr, int group = 1,
                  const void* pre_bias = nullptr) {
+    // eight channels per lane (16-byte accesses to 16-bit rows) when a 16-bit tensor is among the operands
+    constexpr bool wide = sizeof(InT) == 2 || sizeof(OutT) == 2;
+#define CLUSTEN_LN_ARGS x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias
+    if constexpr (wide) {
+        switch (C) {
+            case 64: return launch_lv<InT, ResT, OutT, 8, 1, 8>(CLUSTEN_LN_ARGS);
+            case 128: return launch_lv<InT, ResT, OutT, 16, 1, 8>(CLUSTEN_LN_ARGS);
+            case 256: return launch_lv<InT, ResT, OutT, 32, 1, 8>(CLUSTEN_LN_ARGS);
+            case 384: return launch_lv<InT, ResT, OutT, 16, 3, 8>(CLUSTEN_LN_ARGS);
+            case 512: return launch_lv<InT, ResT, OutT, 64, 1, 8>(CLUSTEN_LN_ARGS);
+            case 768: return launch_lv<InT, ResT, OutT, 32, 3, 8>(CLUSTEN_LN_ARGS);
+            case 1024: return launch_lv<InT, ResT, OutT, 64, 2, 8>(CLUSTEN_LN_ARGS);
+            default: return CLUSTEN_ERR_BAD_DIMS;
+        }
+    }
     switch (C) {
-        case 64: return launch_lv<InT, ResT, OutT, 16, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 128: return launch_lv<InT, ResT, OutT, 32, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 256: return launch_lv<InT, ResT, OutT, 64, 1>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 384: return launch_lv<InT, ResT, OutT, 32, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 512: return launch_lv<InT, ResT, OutT, 64, 2>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 768: return launch_lv<InT, ResT, OutT, 64, 3>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
-        case 1024: return launch_lv<InT, ResT, OutT, 64, 4>(x, branch, sum_out, weight, bias, out, rows, eps, stream, order, group, pre_bias);
+        case 64: return launch_lv<InT, ResT, OutT, 16, 1>(CLUSTEN_LN_ARGS);
+        case 128: return launch_lv<InT, ResT, OutT, 32, 1>(CLUSTEN_LN_ARGS);
+        case 256: return launch_lv<InT, ResT, OutT, 64, 1>(CLUSTEN_LN_ARGS);
+        case 384: return launch_lv<InT, ResT, OutT, 32, 3>(CLUSTEN_LN_ARGS);
+        case 512: return launch_lv<InT, ResT, OutT, 64, 2>(CLUSTEN_LN_ARGS);
+        case 768: return launch_lv<InT, ResT, OutT, 64, 3>(CLUSTEN_LN_ARGS);
+        case 1024: return launch_lv<InT, ResT, OutT, 64, 4>(CLUSTEN_LN_ARGS);
         default: return CLUSTEN_ERR_BAD_DIMS;
     }
+#undef CLUSTEN_LN_ARGS
 }
 
 template <typename InT>
