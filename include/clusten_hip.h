@@ -5,9 +5,11 @@
  * Every entry point
  *   - takes plain device pointers, sizes, element strides, a dtype code and a HIP stream;
  *   - enqueues its kernels on that stream and returns without synchronising;
- *   - never allocates or frees memory (scratch comes in through a workspace argument);
+ *   - never allocates or frees memory (scratch comes in through a workspace argument; the one entry point
+ *     without such an argument, clusten_qk_backward_static, uses a fixed device array of the library);
  *   - returns a clusten_status (0 = ok) instead of throwing;
- *   - is re-entrant: the library keeps no mutable global state.
+ *   - is re-entrant: the library keeps no mutable global state (clusten_qk_backward_static excepted: calls
+ *     that overlap in time on one GPU share its scratch array and race).
  *
  * The entry points stand in for the six functions the reference binds through pybind11
  * (three extension modules, each exporting `forward` and `backward`):
@@ -54,8 +56,10 @@ typedef enum clusten_status {
     CLUSTEN_ERR_BAD_STRIDE = 4,     /* a stride is negative or makes rows overlap */
     CLUSTEN_ERR_WORKSPACE = 5,      /* workspace missing or smaller than *_workspace_bytes() */
     CLUSTEN_ERR_LAUNCH = 6,         /* hipGetLastError() reported a failure after a launch */
-    CLUSTEN_ERR_UNALIGNED = 7       /* clusten_copy_probe, clusten_attn_softmax_forward: a pointer is not 16-byte aligned
+    CLUSTEN_ERR_UNALIGNED = 7,      /* clusten_copy_probe, clusten_attn_softmax_forward: a pointer is not 16-byte aligned
                                        (the gather ops route unaligned operands to element-wise kernels) */
+    CLUSTEN_ERR_TOO_LARGE = 8       /* clusten_qk_backward_static: the problem needs more scratch than
+                                       CLUSTEN_STATIC_SCRATCH_BYTES */
 } clusten_status;
 
 /* Opaque stream handle: a hipStream_t.  NULL is the legacy default stream. */
@@ -112,6 +116,22 @@ int clusten_qk_backward(const void* d_attn,
                         const int64_t* nbhd_idx, void* d_query, void* d_key,
                         void* workspace, size_t workspace_bytes,
                         clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* clusten_qk_backward without a workspace argument and without any allocation, for callers that cannot call
+ * hipMalloc (code under HIP graph capture, tight serving loops, harnesses that forbid it).  It has no counterpart
+ * in the reference, whose backward allocates its outputs itself (clustenqk_cuda_kernel.cu:151-152).  Same
+ * arguments, results and kernels as clusten_qk_backward; the fp32 buffer in which the d_key of F16/BF16 data is
+ * summed is a device array of CLUSTEN_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until
+ * the process ends.  B*H*N*C*4 bytes of it are used (none for F32/F64): a larger problem is refused with
+ * CLUSTEN_ERR_TOO_LARGE.  The array's address on a device is looked up on the first call made with that device
+ * current.  Calls on one GPU share the array (each clears the part it uses on its own stream first), so calls that
+ * overlap in time on one GPU race: keep them on one stream or order them with events. */
+#define CLUSTEN_STATIC_SCRATCH_BYTES (32u << 20)
+int clusten_qk_backward_static(const void* d_attn,
+                               const void* query, clusten_strides query_strides,
+                               const void* key, clusten_strides key_strides,
+                               const int64_t* nbhd_idx, void* d_query, void* d_key,
+                               clusten_attn_shape shape, int dtype, clusten_stream stream);
 
 /* ---- AV:  feat[b,h,i,c] = sum_j attn[b,h,i,j] * value[b,h,nbhd_idx[b,i,j],c] ------------------ */
 

@@ -40,6 +40,7 @@ _PROTOTYPES = {
     "clusten_qk_backward_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
     "clusten_qk_backward": (ctypes.c_int, [_P, _P, Strides, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape,
                                            ctypes.c_int, _P]),
+    "clusten_qk_backward_static": (ctypes.c_int, [_P, _P, Strides, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_av_forward": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_av_backward_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
     "clusten_av_backward": (ctypes.c_int, [_P, Strides, _P, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape,
@@ -329,6 +330,34 @@ def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nb
                                        _ptr(d_query), _ptr(d_key), _ptr(ws), ws_bytes, shape, code, _stream(device)),
                "clusten_qk_backward")
     return d_query, d_key
+
+
+STATIC_SCRATCH_BYTES = 32 << 20   # CLUSTEN_STATIC_SCRATCH_BYTES of include/clusten_hip.h
+
+
+def qk_backward_static(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor,
+                       d_query: torch.Tensor, d_key: torch.Tensor) -> None:
+    """`clusten_qk_backward_static`: the QK backward into the caller's contiguous (b,h,n,c) tensors d_query and d_key,
+    through the entry point that allocates nothing (the fp32 sums of 16-bit data live in a fixed device array of
+    the library: at most STATIC_SCRATCH_BYTES / 4 elements of d_key, else RuntimeError).  Nothing is allocated here
+    either; calls that overlap in time on one GPU race on that array."""
+    lib = load()
+    device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
+    for name, t in (("d_attn", d_attn), ("d_query", d_query), ("d_key", d_key)):
+        _require_cuda(name, t, device)
+    if tuple(d_attn.shape) != (shape.B, shape.H, shape.N, shape.M) or d_attn.dtype != query.dtype:
+        raise RuntimeError("d_attn must be (b,h,n,m) with the dtype of query")
+    for name, t in (("d_query", d_query), ("d_key", d_key)):
+        if t.shape != query.shape or t.dtype != query.dtype or not t.is_contiguous():
+            raise RuntimeError("%s must be a contiguous (b,h,n,c) tensor with the dtype of query" % name)
+    if not d_attn.is_contiguous() or _rows(query) is not query or _rows(key) is not key or idx is not nbhd_idx:
+        raise RuntimeError("qk_backward_static copies nothing: d_attn and nbhd_idx contiguous, rows with channel stride 1")
+    if d_query.numel() == 0 or shape.M == 0:
+        raise RuntimeError("qk_backward_static: empty problem")
+    with torch.cuda.device(device):
+        _check(lib.clusten_qk_backward_static(_ptr(d_attn), _ptr(query), _strides(query), _ptr(key), _strides(key),
+                                              _ptr(idx), _ptr(d_query), _ptr(d_key), shape, code, _stream(device)),
+               "clusten_qk_backward_static")
 
 
 def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, token_major: bool = False) -> torch.Tensor:

@@ -37,6 +37,7 @@ const char* clusten_status_string(int status) {
         case CLUSTEN_ERR_WORKSPACE: return "workspace missing or too small";
         case CLUSTEN_ERR_LAUNCH: return "kernel launch failed";
         case CLUSTEN_ERR_UNALIGNED: return "pointer or stride is not aligned";
+        case CLUSTEN_ERR_TOO_LARGE: return "problem exceeds the fixed scratch of the allocation-free entry point";
         default: return "unknown status";
     }
 }

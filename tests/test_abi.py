@@ -33,7 +33,7 @@ def test_abi_version_and_status_strings():
     lib = _native.load()
     assert lib.clusten_abi_version() == _native.ABI_VERSION
     seen = set()
-    for code in range(0, 8):
+    for code in range(0, 9):
         s = lib.clusten_status_string(code).decode()
         assert s and s not in seen
         seen.add(s)
