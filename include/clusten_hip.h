@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define CLUSTEN_ABI_VERSION 1
+#define CLUSTEN_ABI_VERSION 2
 
 /* Element type of every floating-point tensor of a call.  The reference dispatches
  * double / float / half (AT_DISPATCH_FLOATING_TYPES_AND_HALF, clustenqk_cuda_kernel.cu:78);
@@ -107,8 +107,11 @@ int clusten_qk_forward(const void* query, clusten_strides query_strides,
 /* Replaces clustenqk_cuda.backward (clustenqk_cuda.cpp:35-45, clustenqk_cuda_kernel.cu:91-178):
  *   d_query[b,h,i,c] = sum_j key[b,h,idx[b,i,j],c] * d_attn[b,h,i,j]
  *   d_key[b,h,n,c]   = sum_{(i,j): idx[b,i,j]=n} query[b,h,i,c] * d_attn[b,h,i,j]
- * d_query, d_key are (B,H,N,C) contiguous, need not be zeroed.  For F16/BF16 the scatter is
- * accumulated in fp32 in `workspace` (clusten_qk_backward_workspace_bytes) and rounded once. */
+ * d_query, d_key are (B,H,N,C) contiguous, need not be zeroed.  `workspace` (clusten_qk_backward_workspace_bytes,
+ * 16-byte aligned) holds what the scatter needs: the pair lists of lists made of whole clusters (see
+ * clusten_cluster_pairs below: built on every call; such lists take a gather without atomics whose sums repeat bit
+ * for bit, chosen on the device — the host reads nothing back) and, for F16/BF16, the fp32 sums of the atomic
+ * kernels that any other list takes (rounded once). */
 size_t clusten_qk_backward_workspace_bytes(clusten_attn_shape shape, int dtype);
 int clusten_qk_backward(const void* d_attn,
                         const void* query, clusten_strides query_strides,
@@ -122,8 +125,8 @@ int clusten_qk_backward(const void* d_attn,
  * in the reference, whose backward allocates its outputs itself (clustenqk_cuda_kernel.cu:151-152).  Same
  * arguments, results and kernels as clusten_qk_backward; the fp32 buffer in which the d_key of F16/BF16 data is
  * summed is a device array of CLUSTEN_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until
- * the process ends.  B*H*N*C*4 bytes of it are used (none for F32/F64): a larger problem is refused with
- * CLUSTEN_ERR_TOO_LARGE.  The array's address on a device is looked up on the first call made with that device
+ * the process ends.  clusten_qk_backward_workspace_bytes(shape, dtype) bytes of it are used: a problem that needs more
+ * is refused with CLUSTEN_ERR_TOO_LARGE.  The array's address on a device is looked up on the first call made with that device
  * current.  Calls on one GPU share the array (each clears the part it uses on its own stream first), so calls that
  * overlap in time on one GPU race: keep them on one stream or order them with events. */
 #define CLUSTEN_STATIC_SCRATCH_BYTES (32u << 20)
@@ -242,42 +245,50 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
-/* The scatter of the two attention backward passes as a gather, for neighbour lists made of whole clusters
- * (nbhd_idx[b,i,8r+t] = 8 c(b,i,r) + t, the lists of models/aff_transformer.py:476-480):
+/* ---- lists made of whole clusters: the backward scatters as gathers (optional) ------------------------------ */
+
+/* The pair lists of neighbour lists made of whole clusters, built on the device without any read-back by the host.
+ * A list tensor nbhd_idx (B,rows,M) int64 that points into sequences of n_rows rows is "made of whole clusters" when
+ * every run of 8 slots holds the 8 rows of one cluster: nbhd_idx[b,i,8r+t] = 8 c(b,i,r) + t (the lists of
+ * models/aff_transformer.py:476-480); when n_rows % 8 != 0 the last cluster has n_rows % 8 rows and the slots past
+ * them hold row 0 (models/point_utils.py:203-206).  For such lists the block `pair_lists` receives, for every cluster
+ * (b,g), the pairs (i,r) with c(b,i,r) = g in ascending order — what clusten_scatter_rows_by_cluster and
+ * clusten_wf_backward_by_cluster read; it can serve every head and every layer that uses the same lists.  The block is
+ * opaque but for its first int32, the flag `not_whole`: 0 when the lists are made of whole clusters, 1 when some run is
+ * not (the rest of the block then means nothing, and the two consumers leave their outputs untouched).
+ * clusten_qk_backward, clusten_av_backward and clusten_wf_backward build the same lists in their workspace on every
+ * call and select their kernels through the same flag on the device.
+ *   clusten_cluster_pairs_bytes: size of the block; 0 when the shape is not supported (M % 8 != 0, M > 64, n_rows < 8,
+ *   or more than about 7000 clusters per image); pair_lists must be 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).
+ * rows = N for attention lists (n_rows = N too), Nout for a merge's lists (n_rows = N).  No counterpart in the
+ * reference's extension modules. */
+size_t clusten_cluster_pairs_bytes(int B, int rows, int M, int n_rows);
+int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair_lists_bytes, int B, int rows, int M,
+                          int n_rows, clusten_stream stream);
+
+/* The scatter of the two attention backward passes as a gather, for lists made of whole clusters:
  *   y[b,h, 8g+t, :] = sum over the pairs (i,r) with c(b,i,r) = g of  p[b,h,i,8r+t] * x[b,h,i,:]
  * which equals the d_key of clusten_qk_backward (p = d_attn, x = query) and the d_value of clusten_av_backward
- * (p = attn, x = d_feat) on such lists, without atomics, zero-fill or workspace, and with sums that do not depend on
- * the order of execution.  The caller lists the pairs of every cluster once (shared by the heads, and by every
- * layer that uses the same lists): pairs (B*N*M/8) int32 holds i*8 + r, grouped by (b, g) in any order inside a
- * group; pair_offsets (B*N/8 + 1) int32 holds the start of every group in it.
+ * (p = attn, x = d_feat) on such lists, without atomics, zero-fill or workspace, every sum in fp32 in a fixed order
+ * (results repeat bit for bit).  pair_lists: the block clusten_cluster_pairs filled for (B, N, M, N).
  * p (B,H,N,M) and y (B,H,N,C) contiguous, x strided (B,H,N,C), all of `dtype` (F32, F16 or BF16); every row of y is
- * written.  C = 32, N % 8 == 0, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the reference's
- * extension modules. */
-/* First step towards the pair lists clusten_scatter_rows_by_cluster and clusten_wf_backward_by_cluster read:
- * keys[(b*N+i)*M/8 + r] = b*n_rows/8 + c for every run of 8 list entries nbhd_idx[b,i,8r..8r+7] = 8c..8c+7 with
- * 0 <= 8c <= n_rows-8 (n_rows: the length of the sequence the lists point into; N for attention, the finer sequence
- * for WF); any other run sets *not_whole (which the caller clears first) to 1.  Sorting the keys gives `pairs` (the
- * position of each key: i*8 + r) and `pair_offsets` (the first position of every key value).  nbhd_idx (B,N,M)
- * int64, keys (B*N*M/8) int32; n_rows % 8 == M % 8 == 0 (else CLUSTEN_ERR_BAD_DIMS).  No counterpart in the
- * reference's extension modules. */
-int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int n_rows,
-                         clusten_stream stream);
+ * written — unless the block's flag says the lists are not made of whole clusters: then y is left untouched.
+ * C in {16,32,64}, N >= 8, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS); rows 16-byte aligned (else
+ * CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
+int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const void* pair_lists,
+                                    void* y, clusten_attn_shape shape, int dtype, clusten_stream stream);
 
 /* clusten_wf_backward for lists made of whole clusters, the feature gradient as a gather (no atomics, no workspace,
- * every row of d_feat written once):
+ * every row of d_feat written once from an fp32 sum in a fixed order):
  *   d_feat[b, 8g+t, :] = sum over the pairs (i,r) of cluster (b,g) of  sum_ic weights[b,i,8r+t,ic] * d_feat_new[b,i,ic,:]
- * with pair_offsets (B*N/8 + 1) and pairs (B*Nout*M/8) as for clusten_scatter_rows_by_cluster (i counts the output
- * tokens, g the clusters of the N feature rows); d_weights as clusten_wf_backward computes it.  IC = 4, C % 32 == 0,
- * N % 8 == 0, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS); dtype F32, F16 or BF16.  No counterpart in the
- * reference's extension modules. */
+ * pair_lists: the block clusten_cluster_pairs filled for (B, Nout, M, N) (i counts the output tokens, g the clusters
+ * of the N feature rows); d_weights as clusten_wf_backward computes it.  When the block's flag says the lists are not
+ * made of whole clusters d_feat is left untouched.  IC = 4, C % 32 == 0, N >= 8, M % 8 == 0, M <= 64 (else
+ * CLUSTEN_ERR_BAD_DIMS); dtype F32, F16 or BF16.  No counterpart in the reference's extension modules. */
 int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat,
-                                   const int64_t* nbhd_idx, const int32_t* pair_offsets, const int32_t* pairs,
+                                   const int64_t* nbhd_idx, const void* pair_lists,
                                    void* d_weights, void* d_feat, clusten_wf_shape shape, int dtype,
                                    clusten_stream stream);
-
-int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides,
-                                    const int32_t* pair_offsets, const int32_t* pairs, void* y,
-                                    clusten_attn_shape shape, int dtype, clusten_stream stream);
 
 /* Attention of every token over every token of a short sequence, fused: the branch the reference model takes in
  * a stage whose neighbourhood size reaches its number of tokens (models/aff_transformer.py:108-113 and :125-155:

@@ -2,7 +2,7 @@
 
 PyTorch is used for device memory and streams only: outputs and workspaces are allocated with
 `torch.empty` (stream-ordered caching allocator), kernels are enqueued on the tensor device's
-current stream, nothing synchronises.  There is no CPU path and no fallback: a missing library,
+current stream, nothing synchronises and nothing is remembered between calls.  There is no CPU path and no fallback: a missing library,
 a CPU tensor or a non-zero status raises RuntimeError.
 """
 from __future__ import annotations
@@ -14,7 +14,7 @@ import torch
 
 _LIB_PATH = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "lib", "libclusten_hip.so"))
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
 
@@ -55,9 +55,11 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
-    "clusten_cluster_keys": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
-    "clusten_wf_backward_by_cluster": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
-    "clusten_scatter_rows_by_cluster": (ctypes.c_int, [_P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_cluster_pairs_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "clusten_cluster_pairs": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                             ctypes.c_int, _P]),
+    "clusten_wf_backward_by_cluster": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
+    "clusten_scatter_rows_by_cluster": (ctypes.c_int, [_P, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
                                                       ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_linear_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -203,76 +205,39 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -
     return attn
 
 
-_PAIR_CACHE: "dict" = {}       # lists seen lately -> their pairs by cluster, or None when they are not whole clusters
-_PAIR_CACHE_SIZE = 8
-WF_BY_CLUSTER_MIN_ROWS = 1 << 14   # b*n (feature rows) from which WF's d_feat goes cluster by cluster: a merge's list
-                                   # tensor is used once, so its sort must pay within that one call
-_SEEN_ONCE = object()          # cache value of a list tensor met once, whose pair lists have not been made yet
-_PAD_ENTRY = 1 << 30           # flag of a pair listed under cluster 0 for the pad slots of the short last cluster
-BY_CLUSTER_MIN_ROWS = 1 << 12  # b*n from which the backward scatters go cluster by cluster, from the second use of a
-                               # list tensor on (the sort of the lists, 0.3-0.4 ms, is shared by the layers of a stage)
-
-
-def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None, on_second_sight: bool = False):
-    """For lists made of whole clusters (nbhd_idx[b,i,8r+t] = 8 c + t with c = c(b,i,r), every entry a row of the
-    sequence of `n_rows` rows the lists point into — n by default —, m a multiple of 8, m <= 64; the short last
-    cluster of a sequence whose length is not a multiple of 8 is followed by pad slots that hold row 0):
-    (pair_offsets, pairs), int32 tensors that list, for every cluster (b,g), the pairs (i,r) with c(b,i,r) = g as
-    i*8 + r — the form `scatter_rows_by_cluster` reads.  None for any other list.  One sort of the b*n*m/8 cluster
-    numbers and one look at the result from the host; the answer is kept for the lists seen lately (the layers of a
-    stage share theirs), keyed by the tensor's memory and version.  With `on_second_sight` a list tensor met for the
-    first time is only remembered (None is returned) and the pair lists are made when it comes again: lists used once
-    never pay for the sort."""
-    if nbhd_idx.dim() != 3 or not nbhd_idx.is_cuda or nbhd_idx.dtype != torch.int64:
+def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
+    """The pair lists of `nbhd_idx` (b,rows,m) int64, whose entries point into sequences of `n_rows` rows (rows by
+    default): an opaque uint8 block for `scatter_rows_by_cluster` / `wf_backward_by_cluster`, built on the device by
+    `clusten_cluster_pairs` (keys, then a stable counting sort per image); the host reads nothing back.  Its first
+    int32 (`pairs_not_whole`) is 1 when the lists are not made of whole clusters — the consumers then leave their
+    outputs untouched.  None when the shape is not supported (m not a multiple of 8 or above 64, n_rows < 8)."""
+    lib = load()
+    _require_cuda("nbhd_idx", nbhd_idx)
+    if nbhd_idx.dim() != 3 or nbhd_idx.dtype != torch.int64:
+        raise RuntimeError("nbhd_idx must be an int64 (b,rows,m) tensor")
+    B, rows, M = nbhd_idx.shape
+    D = rows if n_rows is None else int(n_rows)
+    nbytes = lib.clusten_cluster_pairs_bytes(B, rows, M, D) if B and rows and M else 0
+    if nbytes == 0:
         return None
-    B, N, M = nbhd_idx.shape
-    D = N if n_rows is None else int(n_rows)
-    if B == 0 or N == 0 or D < 8 or M % 8 or M == 0 or M > 64 or not nbhd_idx.is_contiguous():
-        return None
-    key = (nbhd_idx.data_ptr(), nbhd_idx._version, B, N, M, D, nbhd_idx.device.index)
-    hit = _PAIR_CACHE.get(key)
-    if hit is not None and hit[1] is not _SEEN_ONCE:
-        return hit[1]
-    if hit is None and on_second_sight:
-        if len(_PAIR_CACHE) >= _PAIR_CACHE_SIZE:
-            _PAIR_CACHE.pop(next(iter(_PAIR_CACHE)))
-        _PAIR_CACHE[key] = (nbhd_idx, _SEEN_ONCE)
-        return None
-    _PAIR_CACHE.pop(key, None)
-    R = M // 8
-    K = (D + 7) // 8
-    if B * K >= 1 << 30 or B * N * R >= 1 << 30 or N >= 1 << 26:
-        return None
-    device = nbhd_idx.device
-    keys = torch.empty(B * N * R, dtype=torch.int32, device=device)
-    not_whole = torch.zeros(1, dtype=torch.int32, device=device)
+    idx = nbhd_idx.contiguous()
+    device = idx.device
+    block = torch.empty(nbytes, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
-        _check(load().clusten_cluster_keys(_ptr(nbhd_idx), _ptr(keys), _ptr(not_whole), B, N, M, D, _stream(device)),
-               "clusten_cluster_keys")
-    result = None
-    if int(not_whole) == 0:                      # the one host synchronisation
-        where = torch.arange(B * N * R, dtype=torch.int32, device=device)
-        entries = ((where // R) % N) * 8 + where % R                       # i*8 + r
-        if D % 8:
-            # the pairs that name the short last cluster also feed row 0 with their pad slots: listed a second time,
-            # flagged, under cluster 0 of their image
-            short = (keys % K) == K - 1
-            keys = torch.cat([keys, keys[short] - (K - 1)])
-            entries = torch.cat([entries, entries[short] | _PAD_ENTRY])
-        ordered, order = torch.sort(keys)
-        pairs = entries[order].contiguous()
-        offsets = torch.searchsorted(ordered, torch.arange(B * K + 1, dtype=torch.int32, device=device),
-                                     out_int32=True)
-        result = (offsets, pairs)
-    if len(_PAIR_CACHE) >= _PAIR_CACHE_SIZE:
-        _PAIR_CACHE.pop(next(iter(_PAIR_CACHE)))
-    _PAIR_CACHE[key] = (nbhd_idx, result)        # the tensor is held: its address cannot be reused meanwhile
-    return result
+        _check(lib.clusten_cluster_pairs(_ptr(idx), _ptr(block), nbytes, B, rows, M, D, _stream(device)),
+               "clusten_cluster_pairs")
+    return block
 
 
-def scatter_rows_by_cluster(p: torch.Tensor, x: torch.Tensor, pair_lists) -> torch.Tensor:
-    """y (b,h,n,32) with y[b,h,8g+t] = sum over the pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i]: the d_key /
-    d_value of the attention backward passes for lists made of whole clusters, `pair_lists` from `cluster_pairs`."""
+def pairs_not_whole(pair_lists: torch.Tensor) -> torch.Tensor:
+    """The flag of a `cluster_pairs` block as a one-element int32 device tensor (reading it on the host synchronises)."""
+    return pair_lists[:4].view(torch.int32)
+
+
+def scatter_rows_by_cluster(p: torch.Tensor, x: torch.Tensor, pair_lists: torch.Tensor, out=None) -> torch.Tensor:
+    """y (b,h,n,c) with y[b,h,8g+t] = sum over the pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i]: the d_key /
+    d_value of the attention backward passes for lists made of whole clusters, `pair_lists` from `cluster_pairs`.
+    When the block's flag says the lists are not whole clusters `out` (new memory unless given) is left untouched."""
     lib = load()
     _require_cuda("p", p)
     device = p.device
@@ -281,28 +246,23 @@ def scatter_rows_by_cluster(p: torch.Tensor, x: torch.Tensor, pair_lists) -> tor
         raise RuntimeError("p must be (b,h,n,m) and x (b,h,n,c) of one dtype")
     B, H, N, C = x.shape
     M = p.shape[3]
-    offsets, pairs = pair_lists
-    if offsets.numel() != B * ((N + 7) // 8) + 1 or pairs.numel() < B * N * (M // 8) or C != 32 or N < 8 or M % 8:
-        raise RuntimeError("scatter_rows_by_cluster: head dim 32, m a multiple of 8, pair lists of these lists")
+    if pair_lists is None or pair_lists.numel() != lib.clusten_cluster_pairs_bytes(B, N, M, N):
+        raise RuntimeError("scatter_rows_by_cluster: pair lists of these lists (cluster_pairs)")
     code = _dtype_code(p, "p")
     p, x = p.contiguous(), _rows(x)
-    y = torch.empty((B, H, N, C), dtype=p.dtype, device=device)
+    y = torch.empty((B, H, N, C), dtype=p.dtype, device=device) if out is None else out
     if y.numel() == 0:
         return y
     shape = AttnShape(B, H, N, C, M)
     with torch.cuda.device(device):
-        _check(lib.clusten_scatter_rows_by_cluster(_ptr(p), _ptr(x), _strides(x), _ptr(offsets), _ptr(pairs), _ptr(y), shape,
+        _check(lib.clusten_scatter_rows_by_cluster(_ptr(p), _ptr(x), _strides(x), _ptr(pair_lists), _ptr(y), shape,
                                                    code, _stream(device)),
                "clusten_scatter_rows_by_cluster")
     return y
 
 
-def _pairs_for_backward(nbhd_idx: torch.Tensor, shape) -> "tuple | None":
-    """The pair lists when the backward scatter of this problem goes cluster by cluster: head dim 32, lists made of
-    whole clusters, and enough rows for the sort of the lists to pay."""
-    if shape.C != 32 or shape.B * shape.N < BY_CLUSTER_MIN_ROWS or torch.cuda.is_current_stream_capturing():
-        return None
-    return cluster_pairs(nbhd_idx, on_second_sight=BY_CLUSTER_MIN_ROWS > 0)
+def _workspace(nbytes: int, device):
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
 
 
 def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor):
@@ -313,18 +273,13 @@ def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nb
     if tuple(d_attn.shape) != (shape.B, shape.H, shape.N, shape.M) or d_attn.dtype != query.dtype:
         raise RuntimeError("d_attn must be (b,h,n,m) with the dtype of query")
     d_attn = d_attn.contiguous()
-    if d_attn.numel() != 0 and shape.M != 0:
-        lists = _pairs_for_backward(idx, shape)
-        if lists is not None:
-            # lists of whole clusters: d_query is the AV forward on (d_attn, key), d_key a gather cluster by cluster
-            return av_forward(d_attn, key, idx), scatter_rows_by_cluster(d_attn, query, lists)
     query, key = _rows(query), _rows(key)
     d_query = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=query.dtype, device=device)
     d_key = torch.empty_like(d_query)
     if d_query.numel() == 0 or shape.M == 0:
         return d_query.zero_(), d_key.zero_()
     ws_bytes = lib.clusten_qk_backward_workspace_bytes(shape, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    ws = _workspace(ws_bytes, device)
     with torch.cuda.device(device):
         _check(lib.clusten_qk_backward(_ptr(d_attn), _ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx),
                                        _ptr(d_query), _ptr(d_key), _ptr(ws), ws_bytes, shape, code, _stream(device)),
@@ -400,18 +355,13 @@ def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_
     if tuple(attn.shape) != (shape.B, shape.H, shape.N, shape.M) or attn.dtype != v.dtype:
         raise RuntimeError("attn must be (b,h,n,m) with the dtype of v")
     attn = attn.contiguous()
-    if attn.numel() != 0 and shape.M != 0:
-        lists = _pairs_for_backward(idx, shape)
-        if lists is not None:
-            # lists of whole clusters: d_attn is the QK forward on (d_feat, v), d_v a gather cluster by cluster
-            return qk_forward(d_feat, v, idx), scatter_rows_by_cluster(attn, d_feat, lists)
     d_feat, v = _rows(d_feat), _rows(v)
     d_attn = torch.empty((shape.B, shape.H, shape.N, shape.M), dtype=attn.dtype, device=device)
     d_v = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=attn.dtype, device=device)
     if d_v.numel() == 0 or shape.M == 0:
         return d_attn.zero_(), d_v.zero_()
     ws_bytes = lib.clusten_av_backward_workspace_bytes(shape, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    ws = _workspace(ws_bytes, device)
     with torch.cuda.device(device):
         _check(lib.clusten_av_backward(_ptr(d_feat), _strides(d_feat), _ptr(attn), _ptr(v), _strides(v), _ptr(idx),
                                        _ptr(d_attn), _ptr(d_v), _ptr(ws), ws_bytes, shape, code, _stream(device)),
@@ -463,24 +413,34 @@ def wf_backward(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Ten
     d_feat = torch.empty_like(feat)
     if d_weights.numel() == 0 or d_feat.numel() == 0:
         return d_weights.zero_(), d_feat.zero_()
-    if (shape.IC == 4 and shape.C % 32 == 0 and shape.B * shape.N >= WF_BY_CLUSTER_MIN_ROWS
-            and weights.dtype in (torch.float32, torch.float16, torch.bfloat16)
-            and not torch.cuda.is_current_stream_capturing()):
-        lists = cluster_pairs(idx, shape.N)
-        if lists is not None:
-            # lists of whole clusters: d_feat as a gather over the pairs of every cluster of the feature rows
-            with torch.cuda.device(device):
-                _check(lib.clusten_wf_backward_by_cluster(_ptr(d_feat_new), _ptr(weights), _ptr(feat), _ptr(idx),
-                                                          _ptr(lists[0]), _ptr(lists[1]), _ptr(d_weights), _ptr(d_feat),
-                                                          shape, code, _stream(device)),
-                       "clusten_wf_backward_by_cluster")
-            return d_weights, d_feat
     ws_bytes = lib.clusten_wf_backward_workspace_bytes(shape, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes else None
+    ws = _workspace(ws_bytes, device)
     with torch.cuda.device(device):
         _check(lib.clusten_wf_backward(_ptr(d_feat_new), _ptr(weights), _ptr(feat), _ptr(idx), _ptr(d_weights),
                                        _ptr(d_feat), _ptr(ws), ws_bytes, shape, code, _stream(device)),
                "clusten_wf_backward")
+    return d_weights, d_feat
+
+
+def wf_backward_by_cluster(d_feat_new: torch.Tensor, weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor,
+                           pair_lists: torch.Tensor, d_feat=None):
+    """(d_weights, d_feat) of the WF operator through `clusten_wf_backward_by_cluster`: the feature gradient as a gather
+    over `pair_lists` = `cluster_pairs(nbhd_idx, n)`.  When the block's flag says the lists are not whole clusters
+    `d_feat` (new memory unless given) is left untouched."""
+    lib = load()
+    device, code, idx, shape = _wf_problem(weights, feat, nbhd_idx)
+    _require_cuda("d_feat_new", d_feat_new, device)
+    if tuple(d_feat_new.shape) != (shape.B, shape.Nout, shape.IC, shape.C) or d_feat_new.dtype != weights.dtype:
+        raise RuntimeError("d_feat_new must be (b,n_,ic,c) with the dtype of weights")
+    if pair_lists is None or pair_lists.numel() != lib.clusten_cluster_pairs_bytes(shape.B, shape.Nout, shape.M, shape.N):
+        raise RuntimeError("wf_backward_by_cluster: pair lists of these lists (cluster_pairs(nbhd_idx, n))")
+    d_feat_new, weights, feat = d_feat_new.contiguous(), weights.contiguous(), feat.contiguous()
+    d_weights = torch.empty_like(weights)
+    d_feat = torch.empty_like(feat) if d_feat is None else d_feat
+    with torch.cuda.device(device):
+        _check(lib.clusten_wf_backward_by_cluster(_ptr(d_feat_new), _ptr(weights), _ptr(feat), _ptr(idx), _ptr(pair_lists),
+                                                  _ptr(d_weights), _ptr(d_feat), shape, code, _stream(device)),
+               "clusten_wf_backward_by_cluster")
     return d_weights, d_feat
 
 

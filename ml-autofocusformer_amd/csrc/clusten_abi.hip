@@ -188,37 +188,58 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     dtype, as_stream(stream));
 }
 
-int clusten_cluster_keys(const int64_t* nbhd_idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int n_rows,
-                         clusten_stream stream) {
-    if (!nbhd_idx || !keys || !not_whole) return CLUSTEN_ERR_NULL_POINTER;
-    if (B <= 0 || N <= 0 || M <= 0 || n_rows < 8 || M % 8 != 0) return CLUSTEN_ERR_BAD_DIMS;
-    if ((int64_t)B * ((n_rows + 7) / 8) >= ((int64_t)1 << 31) || ((int64_t)B * N * (M / 8) + 255) / 256 >= ((int64_t)1 << 31)) {
-        return CLUSTEN_ERR_BAD_DIMS;
-    }
-    return launch_cluster_keys(nbhd_idx, keys, not_whole, B, N, M, n_rows, as_stream(stream));
+size_t clusten_cluster_pairs_bytes(int B, int rows, int M, int n_rows) {
+    if (!cluster_pairs_supported(B, rows, M, n_rows)) return 0;
+    return cluster_pairs_layout(B, rows, M, n_rows).bytes;
+}
+
+int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair_lists_bytes, int B, int rows, int M,
+                          int n_rows, clusten_stream stream) {
+    if (!nbhd_idx || !pair_lists) return CLUSTEN_ERR_NULL_POINTER;
+    if (!cluster_pairs_supported(B, rows, M, n_rows)) return CLUSTEN_ERR_BAD_DIMS;
+    const ClusterPairsLayout l = cluster_pairs_layout(B, rows, M, n_rows);
+    if (pair_lists_bytes < l.bytes) return CLUSTEN_ERR_WORKSPACE;
+    if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
+    char* ws = static_cast<char*>(pair_lists);
+    return launch_cluster_pairs(nbhd_idx, reinterpret_cast<int32_t*>(ws + l.keys), reinterpret_cast<int32_t*>(ws + l.flag),
+                                reinterpret_cast<int32_t*>(ws + l.pairs), reinterpret_cast<int32_t*>(ws + l.starts),
+                                reinterpret_cast<int32_t*>(ws + l.ends), B, rows, M, n_rows, as_stream(stream));
 }
 
 int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat, const int64_t* nbhd_idx,
-                                   const int32_t* pair_offsets, const int32_t* pairs, void* d_weights, void* d_feat,
-                                   clusten_wf_shape shape, int dtype, clusten_stream stream) {
-    if (!d_feat_new || !weights || !feat || !nbhd_idx || !pair_offsets || !pairs || !d_weights || !d_feat) {
+                                   const void* pair_lists, void* d_weights, void* d_feat, clusten_wf_shape shape, int dtype,
+                                   clusten_stream stream) {
+    if (!d_feat_new || !weights || !feat || !nbhd_idx || !pair_lists || !d_weights || !d_feat) {
         return CLUSTEN_ERR_NULL_POINTER;
     }
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_wf_shape(shape)) return st;
+    if (!cluster_pairs_supported(shape.B, shape.Nout, shape.M, shape.N)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
     int st = launch_wf_dweights(d_feat_new, feat, nbhd_idx, d_weights, shape, dtype, as_stream(stream));
     if (st != CLUSTEN_OK) return st;
-    return launch_wf_dfeat_by_cluster(d_feat_new, weights, pair_offsets, pairs, d_feat, shape, dtype, as_stream(stream));
+    const ClusterPairsLayout l = cluster_pairs_layout(shape.B, shape.Nout, shape.M, shape.N);
+    const char* ws = static_cast<const char*>(pair_lists);
+    return launch_wf_dfeat_by_cluster(d_feat_new, weights, reinterpret_cast<const int32_t*>(ws + l.starts),
+                                      reinterpret_cast<const int32_t*>(ws + l.ends),
+                                      reinterpret_cast<const int32_t*>(ws + l.pairs),
+                                      reinterpret_cast<const int32_t*>(ws + l.flag), d_feat, shape, dtype, as_stream(stream));
 }
 
-int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const int32_t* pair_offsets,
-                                    const int32_t* pairs, void* y, clusten_attn_shape shape, int dtype,
-                                    clusten_stream stream) {
-    if (!p || !x || !pair_offsets || !pairs || !y) return CLUSTEN_ERR_NULL_POINTER;
+int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const void* pair_lists, void* y,
+                                    clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!p || !x || !pair_lists || !y) return CLUSTEN_ERR_NULL_POINTER;
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
     if (!strides_ok(x_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
-    return launch_scatter_by_cluster(p, x, x_strides, pair_offsets, pairs, y, shape, dtype, as_stream(stream));
+    if (!cluster_pairs_supported(shape.B, shape.N, shape.M, shape.N)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
+    const ClusterPairsLayout l = cluster_pairs_layout(shape.B, shape.N, shape.M, shape.N);
+    const char* ws = static_cast<const char*>(pair_lists);
+    return launch_scatter_by_cluster(p, x, x_strides, reinterpret_cast<const int32_t*>(ws + l.starts),
+                                     reinterpret_cast<const int32_t*>(ws + l.ends),
+                                     reinterpret_cast<const int32_t*>(ws + l.pairs),
+                                     reinterpret_cast<const int32_t*>(ws + l.flag), y, shape, dtype, as_stream(stream));
 }
 
 int clusten_dense_attention_forward(const void* query, clusten_strides query_strides, const void* key,

@@ -29,7 +29,8 @@ int launch_gather_sum_clusters(const void* p, const void* rows, clusten_strides 
 
 // out[b,h,idx[b,i,j],c] += p[b,h,i,j] * x[b,h,i,c]               (QK's d_key; AV's d_value)
 //   p : contiguous (B,H,N,M);  x : strided (B,H,N,C);  out : contiguous (B,H,N,C), zeroed here.
-//   For F16/BF16 the sum is built in fp32 in `workspace` and rounded once.
+//   Lists made of whole clusters (found out on the device) go through pair lists in `workspace` and a gather without
+//   atomics; for any other list the sum is built with fp32 atomics (for F16/BF16 in `workspace`, rounded once).
 size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype);
 int launch_scatter_rows(const void* p, const void* x, clusten_strides x_strides, const int64_t* idx, void* out,
                         void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream);
@@ -66,15 +67,32 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
                              hipStream_t stream);
 
+// The pair lists of lists made of whole clusters (cluster_pairs.hip), built on the device: for `rows` list rows per
+//   image of M slots that point into a sequence of D rows (K = ceil(D/8) clusters), pairs[starts[b*K+g] .. ends[b*K+g])
+//   holds the entries i*8 + r whose run r of list row i is cluster g of image b, ascending; *not_whole becomes 1 when
+//   some run is not a whole cluster (then the other outputs mean nothing), else 0.  `keys` is scratch.
+//   Sizes as cluster_pairs_layout() gives them (byte offsets into one 16-byte aligned block, `bytes` in all).
+struct ClusterPairsLayout {
+    size_t flag, keys, pairs, starts, ends, bytes;
+};
+bool cluster_pairs_supported(int B, int rows, int M, int D);
+ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D);
+int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* not_whole, int32_t* pairs, int32_t* starts,
+                         int32_t* ends, int B, int rows, int M, int D, hipStream_t stream);
 // y[b,h,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i,:]: see scatter_by_cluster.hip.
-int launch_cluster_keys(const int64_t* idx, int32_t* keys, int32_t* not_whole, int B, int N, int M, int D,
-                        hipStream_t stream);
+//   C in {16,32,64}.  `not_whole` (may be null): device flag; the kernel does nothing when it points to non-zero.
+bool scatter_by_cluster_supported(const void* p, const void* x, clusten_strides xs, const void* y,
+                                  const clusten_attn_shape& s, int dtype);
+int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* starts, const int32_t* ends,
+                              const int32_t* pairs, const int32_t* not_whole, void* y, clusten_attn_shape s, int dtype,
+                              hipStream_t stream);
 // d_feat[b,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of sum_ic w[b,i,8r+t,ic] * d_out[b,i,ic,:]: see
-//   wf_dfeat_by_cluster.hip.  IC = 4, C % 32 == 0, N % 8 == 0.
-int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
-                               clusten_wf_shape s, int dtype, hipStream_t stream);
-int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* offsets,
-                              const int32_t* pairs, void* y, clusten_attn_shape s, int dtype, hipStream_t stream);
+//   wf_dfeat_by_cluster.hip.  IC = 4, C % 32 == 0.  `not_whole` as above.
+bool wf_dfeat_by_cluster_supported(const void* d_out, const void* w, const void* d_feat, const clusten_wf_shape& s,
+                                   int dtype);
+int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* starts, const int32_t* ends,
+                               const int32_t* pairs, const int32_t* not_whole, void* d_feat, clusten_wf_shape s, int dtype,
+                               hipStream_t stream);
 
 // Attention of every token over every token (N <= 64) in one kernel: see dense_attention.hip.  q, k, v, out : strided
 //   (B,H,N,C) of T in {F16, BF16}, C = 32; table (rows,H) of T; pe_idx int64 (B,N,N); blank_k, blank_v : fp32 (H,C).
@@ -149,10 +167,12 @@ int launch_knn2d(const float* query, const float* database, int64_t* idx, float*
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 
 // Fill `count` fp32 / fp64 words with zero (a kernel, so that callers may capture it in a HIP graph).
-int launch_zero_f32(float* dst, size_t count, hipStream_t stream);
+//   `only_if` (may be null): a device flag; the kernel does nothing when it points to zero.
+int launch_zero_f32(float* dst, size_t count, hipStream_t stream, const int32_t* only_if = nullptr);
 int launch_zero_f64(double* dst, size_t count, hipStream_t stream);
 
-// dst[i] = round(src[i]) for i < count, T in {F16, BF16}.
-int launch_round_from_f32(const float* src, void* dst, size_t count, int dtype, hipStream_t stream);
+// dst[i] = round(src[i]) for i < count, T in {F16, BF16}.  `only_if` as above.
+int launch_round_from_f32(const float* src, void* dst, size_t count, int dtype, hipStream_t stream,
+                          const int32_t* only_if = nullptr);
 
 }  // namespace clusten

@@ -1,36 +1,80 @@
-// Storage-type dispatch for scatter_rows (see scatter_rows_impl.hpp): zeroes the fp32 accumulation
-// buffer, runs the scatter, and rounds to fp16/bf16 when the storage type is narrower than fp32.
+// Storage-type dispatch for scatter_rows (see scatter_rows_impl.hpp).  Two sets of kernels are enqueued and a device
+// flag decides which of them works: the pair lists and the cluster-by-cluster gather (cluster_pairs.hip,
+// scatter_by_cluster.hip) for lists made of whole clusters, the zero-fill, atomic scatter and rounding to fp16/bf16
+// for any other list.  The host never learns which: nothing is read back.
 #include "scatter_rows_impl.hpp"
 
 namespace clusten {
 
-int scatter_rows_f32(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t);
-int scatter_rows_f16(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t);
-int scatter_rows_bf16(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t);
+int scatter_rows_f32(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t,
+                     const int32_t*);
+int scatter_rows_f16(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t,
+                     const int32_t*);
+int scatter_rows_bf16(const void*, const void*, clusten_strides, const int64_t*, float*, const clusten_attn_shape&, hipStream_t,
+                      const int32_t*);
 
-size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype) {
-    if (dtype == CLUSTEN_F16 || dtype == CLUSTEN_BF16) return (size_t)s.B * s.H * s.N * s.C * sizeof(float);
-    return 0;
+namespace {
+
+// Workspace of one scatter: the pair lists of the cluster-by-cluster kernel when the shape admits it (whether the
+// lists are made of whole clusters is found out on the device), then the fp32 sums of 16-bit data for the atomic kernels.
+struct ScatterPlan {
+    bool by_cluster;
+    ClusterPairsLayout pairs;
+    size_t acc32;   // offset of the fp32 buffer
+    size_t bytes;
+};
+
+ScatterPlan scatter_plan(const clusten_attn_shape& s, int dtype) {
+    ScatterPlan plan;
+    plan.by_cluster = dtype != CLUSTEN_F64 && (s.C == 16 || s.C == 32 || s.C == 64) &&
+                      cluster_pairs_supported(s.B, s.N, s.M, s.N);
+    plan.pairs = plan.by_cluster ? cluster_pairs_layout(s.B, s.N, s.M, s.N) : ClusterPairsLayout{};
+    plan.acc32 = plan.by_cluster ? plan.pairs.bytes : 0;
+    const bool narrow = dtype == CLUSTEN_F16 || dtype == CLUSTEN_BF16;
+    plan.bytes = plan.acc32 + (narrow ? (size_t)s.B * s.H * s.N * s.C * sizeof(float) : 0);
+    return plan;
 }
+
+}  // namespace
+
+size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype) { return scatter_plan(s, dtype).bytes; }
 
 int launch_scatter_rows(const void* p, const void* x, clusten_strides xs, const int64_t* idx, void* out,
                         void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream) {
     const size_t count = (size_t)s.B * s.H * s.N * s.C;
+    const ScatterPlan plan = scatter_plan(s, dtype);
+    if (plan.bytes != 0 && !aligned16(workspace)) return CLUSTEN_ERR_UNALIGNED;
+    char* ws = static_cast<char*>(workspace);
     int st;
+    // lists made of whole clusters: a gather over sorted pair lists, chosen on the device through `flag`
+    const int32_t* flag = nullptr;
+    if (plan.by_cluster && scatter_by_cluster_supported(p, x, xs, out, s, dtype)) {
+        int32_t* not_whole = reinterpret_cast<int32_t*>(ws + plan.pairs.flag);
+        int32_t* keys = reinterpret_cast<int32_t*>(ws + plan.pairs.keys);
+        int32_t* pairs = reinterpret_cast<int32_t*>(ws + plan.pairs.pairs);
+        int32_t* starts = reinterpret_cast<int32_t*>(ws + plan.pairs.starts);
+        int32_t* ends = reinterpret_cast<int32_t*>(ws + plan.pairs.ends);
+        st = launch_cluster_pairs(idx, keys, not_whole, pairs, starts, ends, s.B, s.N, s.M, s.N, stream);
+        if (st != CLUSTEN_OK) return st;
+        st = launch_scatter_by_cluster(p, x, xs, starts, ends, pairs, not_whole, out, s, dtype, stream);
+        if (st != CLUSTEN_OK) return st;
+        flag = not_whole;
+    }
+    // any other list: atomics (these kernels return at once when the flag says the lists were whole clusters)
     switch (dtype) {
         case CLUSTEN_F32:
-            st = launch_zero_f32(static_cast<float*>(out), count, stream);
+            st = launch_zero_f32(static_cast<float*>(out), count, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            return scatter_rows_f32(p, x, xs, idx, static_cast<float*>(out), s, stream);
+            return scatter_rows_f32(p, x, xs, idx, static_cast<float*>(out), s, stream, flag);
         case CLUSTEN_F16:
         case CLUSTEN_BF16: {
-            float* acc32 = static_cast<float*>(workspace);
-            st = launch_zero_f32(acc32, count, stream);
+            float* acc32 = reinterpret_cast<float*>(ws + plan.acc32);
+            st = launch_zero_f32(acc32, count, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            st = dtype == CLUSTEN_F16 ? scatter_rows_f16(p, x, xs, idx, acc32, s, stream)
-                                      : scatter_rows_bf16(p, x, xs, idx, acc32, s, stream);
+            st = dtype == CLUSTEN_F16 ? scatter_rows_f16(p, x, xs, idx, acc32, s, stream, flag)
+                                      : scatter_rows_bf16(p, x, xs, idx, acc32, s, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            return launch_round_from_f32(acc32, out, count, dtype, stream);
+            return launch_round_from_f32(acc32, out, count, dtype, stream, flag);
         }
         case CLUSTEN_F64:
             st = launch_zero_f64(static_cast<double*>(out), count, stream);

@@ -35,13 +35,14 @@ namespace clusten {
 template <typename T, int C, int Q, bool GUARD>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void scatter_rows_tile_kernel(
     const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out, int H,
-    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles) {
+    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles, const int32_t* __restrict__ only_if) {
     constexpr int HPW = kWave / C;
     constexpr int SLOTS = 16 * Q;
     static_assert(C == 16 || C == 32 || C == 64, "a row of 16 lanes must stay inside one head");
     static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
     typedef typename Quad<T>::raw QuadRaw;
 
+    if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
     {
@@ -247,7 +248,8 @@ template <typename T, typename A>
 __global__ __launch_bounds__(256) void scatter_rows_elem_kernel(const T* __restrict__ p, const T* __restrict__ x,
                                                                 const int64_t* __restrict__ idx, A* __restrict__ out,
                                                                 int B, int H, int N, int C, int M,
-                                                                clusten_strides xs) {
+                                                                clusten_strides xs, const int32_t* __restrict__ only_if) {
+    if (only_if != nullptr && *only_if == 0) return;
     const int64_t total = (int64_t)B * H * N * C;
     for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (int64_t)gridDim.x * blockDim.x) {
         const int c = (int)(o % C);
@@ -266,48 +268,48 @@ __global__ __launch_bounds__(256) void scatter_rows_elem_kernel(const T* __restr
 
 template <typename T, int C, int Q, bool GUARD>
 int scatter_tile_q(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
-                   const clusten_attn_shape& s, hipStream_t stream) {
+                   const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int grid = xcd_grid(total);
     hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(x), idx, out, s.H, s.N, s.M, xs,
-                       tiles_per_batch, total);
+                       tiles_per_batch, total, only_if);
     return launch_status();
 }
 
 template <typename T, int C>
 int scatter_tile(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
-                 const clusten_attn_shape& s, hipStream_t stream) {
-    if (s.M == 48) return scatter_tile_q<T, C, 3, false>(p, x, xs, idx, out, s, stream);
-    return scatter_tile_q<T, C, 4, true>(p, x, xs, idx, out, s, stream);
+                 const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
+    if (s.M == 48) return scatter_tile_q<T, C, 3, false>(p, x, xs, idx, out, s, stream, only_if);
+    return scatter_tile_q<T, C, 4, true>(p, x, xs, idx, out, s, stream, only_if);
 }
 
 template <typename T, typename A>
 int scatter_elem(const void* p, const void* x, clusten_strides xs, const int64_t* idx, A* out,
-                 const clusten_attn_shape& s, hipStream_t stream) {
+                 const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if = nullptr) {
     const int64_t total = (int64_t)s.B * s.H * s.N * s.C;
     const int64_t want = (total + 255) / 256;
     const int grid = (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
     hipLaunchKernelGGL((scatter_rows_elem_kernel<T, A>), dim3(grid), dim3(256), 0, stream, static_cast<const T*>(p),
-                       static_cast<const T*>(x), idx, out, s.B, s.H, s.N, s.C, s.M, xs);
+                       static_cast<const T*>(x), idx, out, s.B, s.H, s.N, s.C, s.M, xs, only_if);
     return launch_status();
 }
 
 // Accumulate into the zeroed fp32 buffer `acc32` (which is `out` itself for fp32 storage).
 template <typename T>
 int scatter_rows_typed(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* acc32,
-                       const clusten_attn_shape& s, hipStream_t stream) {
+                       const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
     const bool quads_ok = s.M % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0;
     if (quads_ok) {
         switch (s.C) {
-            case 16: return scatter_tile<T, 16>(p, x, xs, idx, acc32, s, stream);
-            case 32: return scatter_tile<T, 32>(p, x, xs, idx, acc32, s, stream);
-            case 64: return scatter_tile<T, 64>(p, x, xs, idx, acc32, s, stream);
+            case 16: return scatter_tile<T, 16>(p, x, xs, idx, acc32, s, stream, only_if);
+            case 32: return scatter_tile<T, 32>(p, x, xs, idx, acc32, s, stream, only_if);
+            case 64: return scatter_tile<T, 64>(p, x, xs, idx, acc32, s, stream, only_if);
             default: break;
         }
     }
-    return scatter_elem<T, float>(p, x, xs, idx, acc32, s, stream);
+    return scatter_elem<T, float>(p, x, xs, idx, acc32, s, stream, only_if);
 }
 
 }  // namespace clusten

@@ -16,15 +16,18 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const Piece* __restrict__ 
     if (i < pieces) dst[i] = src[i];
 }
 
+// `only_if` (may be null): a device flag; the kernel does nothing when it points to zero.
 template <typename W>
-__global__ __launch_bounds__(kBlock) void zero_kernel(W* __restrict__ dst, size_t count) {
+__global__ __launch_bounds__(kBlock) void zero_kernel(W* __restrict__ dst, size_t count, const int32_t* only_if) {
+    if (only_if != nullptr && *only_if == 0) return;
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) dst[i] = W(0);
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void round_kernel(const float* __restrict__ src, T* __restrict__ dst,
-                                                      size_t count) {
+                                                      size_t count, const int32_t* only_if) {
+    if (only_if != nullptr && *only_if == 0) return;
     const size_t stride = (size_t)gridDim.x * kBlock;
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) dst[i] = from_acc<T>(src[i]);
 }
@@ -45,29 +48,31 @@ int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
     return launch_status();
 }
 
-int launch_zero_f32(float* dst, size_t count, hipStream_t stream) {
+int launch_zero_f32(float* dst, size_t count, hipStream_t stream, const int32_t* only_if) {
     // whole 16-byte pieces when the buffer allows it
     if (aligned16(dst) && count % 4 == 0) {
         hipLaunchKernelGGL((zero_kernel<Piece>), dim3(grid_for(count / 4)), dim3(kBlock), 0, stream,
-                           reinterpret_cast<Piece*>(dst), count / 4);
+                           reinterpret_cast<Piece*>(dst), count / 4, only_if);
     } else {
-        hipLaunchKernelGGL((zero_kernel<float>), dim3(grid_for(count)), dim3(kBlock), 0, stream, dst, count);
+        hipLaunchKernelGGL((zero_kernel<float>), dim3(grid_for(count)), dim3(kBlock), 0, stream, dst, count, only_if);
     }
     return launch_status();
 }
 
 int launch_zero_f64(double* dst, size_t count, hipStream_t stream) {
-    hipLaunchKernelGGL((zero_kernel<double>), dim3(grid_for(count)), dim3(kBlock), 0, stream, dst, count);
+    hipLaunchKernelGGL((zero_kernel<double>), dim3(grid_for(count)), dim3(kBlock), 0, stream, dst, count,
+                       static_cast<const int32_t*>(nullptr));
     return launch_status();
 }
 
-int launch_round_from_f32(const float* src, void* dst, size_t count, int dtype, hipStream_t stream) {
+int launch_round_from_f32(const float* src, void* dst, size_t count, int dtype, hipStream_t stream,
+                          const int32_t* only_if) {
     if (dtype == CLUSTEN_F16) {
         hipLaunchKernelGGL((round_kernel<f16_t>), dim3(grid_for(count)), dim3(kBlock), 0, stream, src,
-                           static_cast<f16_t*>(dst), count);
+                           static_cast<f16_t*>(dst), count, only_if);
     } else if (dtype == CLUSTEN_BF16) {
         hipLaunchKernelGGL((round_kernel<bf16_t>), dim3(grid_for(count)), dim3(kBlock), 0, stream, src,
-                           static_cast<bf16_t*>(dst), count);
+                           static_cast<bf16_t*>(dst), count, only_if);
     } else {
         return CLUSTEN_ERR_BAD_DTYPE;
     }

@@ -29,34 +29,71 @@ int launch_wf_dweights(const void* d_out, const void* feat, const int64_t* idx, 
     }
 }
 
-size_t wf_dfeat_workspace_bytes(clusten_wf_shape s, int dtype) {
-    if (dtype == CLUSTEN_F16 || dtype == CLUSTEN_BF16) return (size_t)s.B * s.N * s.C * sizeof(float);
-    return 0;
+namespace {
+
+// See ScatterPlan in scatter_rows.hip: pair lists first (when the shape admits the cluster-by-cluster kernel), then
+// the fp32 sums of 16-bit data.
+struct DfeatPlan {
+    bool by_cluster;
+    ClusterPairsLayout pairs;
+    size_t acc32;
+    size_t bytes;
+};
+
+DfeatPlan dfeat_plan(const clusten_wf_shape& s, int dtype) {
+    DfeatPlan plan;
+    plan.by_cluster = dtype != CLUSTEN_F64 && s.IC == 4 && s.C % 32 == 0 && cluster_pairs_supported(s.B, s.Nout, s.M, s.N);
+    plan.pairs = plan.by_cluster ? cluster_pairs_layout(s.B, s.Nout, s.M, s.N) : ClusterPairsLayout{};
+    plan.acc32 = plan.by_cluster ? plan.pairs.bytes : 0;
+    const bool narrow = dtype == CLUSTEN_F16 || dtype == CLUSTEN_BF16;
+    plan.bytes = plan.acc32 + (narrow ? (size_t)s.B * s.N * s.C * sizeof(float) : 0);
+    return plan;
 }
+
+}  // namespace
+
+size_t wf_dfeat_workspace_bytes(clusten_wf_shape s, int dtype) { return dfeat_plan(s, dtype).bytes; }
 
 int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* d_feat, void* workspace,
                     clusten_wf_shape s, int dtype, hipStream_t stream) {
     const size_t count = (size_t)s.B * s.N * s.C;
+    const DfeatPlan plan = dfeat_plan(s, dtype);
+    if (plan.bytes != 0 && !aligned16(workspace)) return CLUSTEN_ERR_UNALIGNED;
+    char* ws = static_cast<char*>(workspace);
     int st;
+    // lists made of whole clusters: a gather over sorted pair lists, chosen on the device through `flag`
+    const int32_t* flag = nullptr;
+    if (plan.by_cluster && wf_dfeat_by_cluster_supported(d_out, w, d_feat, s, dtype)) {
+        int32_t* not_whole = reinterpret_cast<int32_t*>(ws + plan.pairs.flag);
+        int32_t* keys = reinterpret_cast<int32_t*>(ws + plan.pairs.keys);
+        int32_t* pairs = reinterpret_cast<int32_t*>(ws + plan.pairs.pairs);
+        int32_t* starts = reinterpret_cast<int32_t*>(ws + plan.pairs.starts);
+        int32_t* ends = reinterpret_cast<int32_t*>(ws + plan.pairs.ends);
+        st = launch_cluster_pairs(idx, keys, not_whole, pairs, starts, ends, s.B, s.Nout, s.M, s.N, stream);
+        if (st != CLUSTEN_OK) return st;
+        st = launch_wf_dfeat_by_cluster(d_out, w, starts, ends, pairs, not_whole, d_feat, s, dtype, stream);
+        if (st != CLUSTEN_OK) return st;
+        flag = not_whole;
+    }
     switch (dtype) {
         case CLUSTEN_F32:
-            st = launch_zero_f32(static_cast<float*>(d_feat), count, stream);
+            st = launch_zero_f32(static_cast<float*>(d_feat), count, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            return wf_dfeat_typed<float, float>(d_out, w, idx, static_cast<float*>(d_feat), s, stream);
+            return wf_dfeat_typed<float, float>(d_out, w, idx, static_cast<float*>(d_feat), s, stream, flag);
         case CLUSTEN_F16:
         case CLUSTEN_BF16: {
-            float* acc32 = static_cast<float*>(workspace);
-            st = launch_zero_f32(acc32, count, stream);
+            float* acc32 = reinterpret_cast<float*>(ws + plan.acc32);
+            st = launch_zero_f32(acc32, count, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            st = dtype == CLUSTEN_F16 ? wf_dfeat_typed<f16_t, float>(d_out, w, idx, acc32, s, stream)
-                                      : wf_dfeat_typed<bf16_t, float>(d_out, w, idx, acc32, s, stream);
+            st = dtype == CLUSTEN_F16 ? wf_dfeat_typed<f16_t, float>(d_out, w, idx, acc32, s, stream, flag)
+                                      : wf_dfeat_typed<bf16_t, float>(d_out, w, idx, acc32, s, stream, flag);
             if (st != CLUSTEN_OK) return st;
-            return launch_round_from_f32(acc32, d_feat, count, dtype, stream);
+            return launch_round_from_f32(acc32, d_feat, count, dtype, stream, flag);
         }
         case CLUSTEN_F64:
             st = launch_zero_f64(static_cast<double*>(d_feat), count, stream);
             if (st != CLUSTEN_OK) return st;
-            return wf_dfeat_typed<double, double>(d_out, w, idx, static_cast<double*>(d_feat), s, stream);
+            return wf_dfeat_typed<double, double>(d_out, w, idx, static_cast<double*>(d_feat), s, stream, nullptr);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }

@@ -8,12 +8,12 @@
 //
 //   d_feat[b, 8g + t, :] = sum over the pairs (i, r) with c(b,i,r) = g of  sum_ic w[b,i,8r+t,ic] * d_out[b,i,ic,:]
 //
-// With the pairs of every cluster listed once (see scatter_by_cluster.hip: the same sorted pair lists) a pair is one
+// With the pairs of every cluster listed once (cluster_pairs.hip: the same sorted pair lists) a pair is one
 // `v_mfma_f32_16x16x4_f32` per 16 channels: A = the pair's 8 x 4 block of weights (32 contiguous elements), B = the
 // four d_out rows of its output token, k = the inner channel.  One wave per cluster takes the channels 32 at a time;
 // d_out rows and weight blocks of 8 pairs at a time travel to LDS by LDS-direct loads (16-bit data is widened when the
-// operands are read).  Every row of d_feat is written exactly once: no atomics, no zero-fill, no workspace.  It has
-// no counterpart in the reference's extension modules.
+// operands are read).  Every row of d_feat is written exactly once, from fp32 sums over all its pairs: no atomics, no
+// zero-fill, no fp32 workspace.  It has no counterpart in the reference's extension modules.
 #include "launch.hpp"
 #include "mfma.hpp"
 
@@ -29,8 +29,10 @@ constexpr int kEntryMask = kPadEntry - 1;
 
 template <typename T>
 __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __restrict__ d_out, const T* __restrict__ w,
-                                                                    const int32_t* __restrict__ offsets,
+                                                                    const int32_t* __restrict__ starts,
+                                                                    const int32_t* __restrict__ ends,
                                                                     const int32_t* __restrict__ pairs,
+                                                                    const int32_t* __restrict__ not_whole,
                                                                     T* __restrict__ d_feat, int N, int Nout, int C, int M,
                                                                     int clusters_per_image, int total_clusters) {
     constexpr int EB = (int)sizeof(T);
@@ -49,14 +51,15 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
     constexpr int LDS_BYTES = L_BASE + kListMax * 4;
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
+    if (not_whole != nullptr && *not_whole != 0) return;   // not lists of whole clusters: the atomic kernel runs instead
     const int unit = xcd_tile(blockIdx.x, total_clusters);
     if (unit < 0) return;
     const int b = unit / clusters_per_image;
     const int g = unit - b * clusters_per_image;
     const int lane = threadIdx.x;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int first = offsets[unit];
-    const int count = offsets[unit + 1] - first;
+    const int first = starts[unit];
+    const int count = ends[unit] - first;
     int* list = reinterpret_cast<int*>(stage + L_BASE);
     const char* d_out_b = reinterpret_cast<const char*>(d_out + (int64_t)b * Nout * kIC * C);
     const char* w_b = reinterpret_cast<const char*>(w + (int64_t)b * Nout * M * kIC);
@@ -64,17 +67,23 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
     const int rows_here = min(8, N - 8 * g);   // the last cluster of a sequence may be short
     const int pad_from = N & 7;                // ... and the lists that name it hold row 0 in slots pad_from .. 7
 
-    // a cluster listed by more than kListMax pairs is taken in segments; the later segments add to what is stored
-    for (int seg = 0; seg == 0 || seg < count; seg += kListMax) {
-        const int n = min(kListMax, count - seg);   // <= 0 only for a cluster nobody lists: its rows become zero
-        lds_sync();
-        for (int e = lane; e < n; e += kWave) list[e] = pairs[first + seg + e];
-        lds_sync();
-        for (int c0 = 0; c0 < C; c0 += kChunk) {
-            F32x4 acc[2] = {F32x4{0.f, 0.f, 0.f, 0.f}, F32x4{0.f, 0.f, 0.f, 0.f}};
+    // a cluster listed by more than kListMax pairs is taken in segments, every channel chunk walking all of them
+    // before it writes its rows; the usual cluster's list is read once for all chunks
+    const bool one_segment = count <= kListMax;
+    if (one_segment) {
+        for (int e = lane; e < count; e += kWave) list[e] = pairs[first + e];
+    }
+    for (int c0 = 0; c0 < C; c0 += kChunk) {
+        F32x4 acc[2] = {F32x4{0.f, 0.f, 0.f, 0.f}, F32x4{0.f, 0.f, 0.f, 0.f}};
+        for (int seg = 0; seg < count; seg += kListMax) {
+            const int n = min(kListMax, count - seg);
+            if (!one_segment) {
+                lds_sync();
+                for (int e = lane; e < n; e += kWave) list[e] = pairs[first + seg + e];
+            }
             for (int base = 0; base < n; base += kPass) {
                 const int here = min(kPass, n - base);
-                lds_sync();  // the previous pass has been read
+                lds_sync();  // the previous pass has been read (and the list is in place)
 #pragma unroll
                 for (int a = 0; a < X_DMA; ++a) {
                     // lane -> (pair, inner channel, 16-byte piece of the row)
@@ -110,61 +119,64 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
                     }
                 }
             }
-            // rows 4*kq + j of the result (kq < 2: the cluster's 8 rows), channels c0 + 16*cb + r16
-            lds_sync();
-            if (kq < 2) {
+        }
+        // rows 4*kq + j of the result (kq < 2: the cluster's 8 rows), channels c0 + 16*cb + r16
+        lds_sync();
+        if (kq < 2) {
 #pragma unroll
-                for (int cb = 0; cb < 2; ++cb) {
+            for (int cb = 0; cb < 2; ++cb) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        reinterpret_cast<float*>(stage + O_BASE)[(4 * kq + j) * kChunk + 16 * cb + r16] = acc[cb][j];
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    reinterpret_cast<float*>(stage + O_BASE)[(4 * kq + j) * kChunk + 16 * cb + r16] = acc[cb][j];
                 }
             }
-            lds_sync();
-            {
-                // 8 rows x 32 channels: four consecutive channels per lane
-                const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
-                float v[4] = {o[0], o[1], o[2], o[3]};
-                T* dst = rows_out + (int64_t)(lane >> 3) * C + c0 + (lane & 7) * 4;
-                if (seg > 0 && (lane >> 3) < rows_here) {
-                    float old[4];
-                    Quad<T>::unpack(*reinterpret_cast<const typename Quad<T>::raw*>(dst), old);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += old[e];
-                }
-                if ((lane >> 3) < rows_here) *reinterpret_cast<typename Quad<T>::raw*>(dst) = Quad<T>::pack(v);
-            }
+        }
+        lds_sync();
+        {
+            // 8 rows x 32 channels: four consecutive channels per lane
+            const F32x4 o = *reinterpret_cast<const F32x4*>(stage + O_BASE + lane * 16);
+            const float v[4] = {o[0], o[1], o[2], o[3]};
+            T* dst = rows_out + (int64_t)(lane >> 3) * C + c0 + (lane & 7) * 4;
+            if ((lane >> 3) < rows_here) *reinterpret_cast<typename Quad<T>::raw*>(dst) = Quad<T>::pack(v);
         }
     }
 }
 
 template <typename T>
-int launch_typed(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
-                 const clusten_wf_shape& s, hipStream_t stream) {
+int launch_typed(const void* d_out, const void* w, const int32_t* starts, const int32_t* ends, const int32_t* pairs,
+                 const int32_t* not_whole, void* d_feat, const clusten_wf_shape& s, hipStream_t stream) {
     const int per_image = (s.N + 7) / 8;
     const int64_t total = (int64_t)s.B * per_image;
     if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
     hipLaunchKernelGGL((wf_dfeat_by_cluster_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWave), 0, stream,
-                       static_cast<const T*>(d_out), static_cast<const T*>(w), offsets, pairs, static_cast<T*>(d_feat), s.N,
+                       static_cast<const T*>(d_out), static_cast<const T*>(w), starts, ends, pairs, not_whole,
+                       static_cast<T*>(d_feat), s.N,
                        s.Nout, s.C, s.M, per_image, (int)total);
     return launch_status();
 }
 
 }  // namespace
 
-int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* offsets, const int32_t* pairs, void* d_feat,
-                               clusten_wf_shape s, int dtype, hipStream_t stream) {
-    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+bool wf_dfeat_by_cluster_supported(const void* d_out, const void* w, const void* d_feat, const clusten_wf_shape& s,
+                                   int dtype) {
+    if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return false;
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M <= 0) return false;
     const int64_t eb = (int64_t)dtype_size(dtype);
     if ((int64_t)s.Nout * kIC * s.C * eb >= ((int64_t)1 << 31) || (int64_t)s.Nout * s.M * kIC * eb >= ((int64_t)1 << 31)) {
-        return CLUSTEN_ERR_BAD_DIMS;
+        return false;
     }
-    if (!aligned16(d_out) || !aligned16(w) || !aligned16(d_feat)) return CLUSTEN_ERR_UNALIGNED;
+    return aligned16(d_out) && aligned16(w) && aligned16(d_feat);
+}
+
+int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* starts, const int32_t* ends,
+                               const int32_t* pairs, const int32_t* not_whole, void* d_feat, clusten_wf_shape s, int dtype,
+                               hipStream_t stream) {
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (!wf_dfeat_by_cluster_supported(d_out, w, d_feat, s, dtype)) return CLUSTEN_ERR_UNALIGNED;
     switch (dtype) {
-        case CLUSTEN_F32: return launch_typed<float>(d_out, w, offsets, pairs, d_feat, s, stream);
-        case CLUSTEN_F16: return launch_typed<f16_t>(d_out, w, offsets, pairs, d_feat, s, stream);
-        case CLUSTEN_BF16: return launch_typed<bf16_t>(d_out, w, offsets, pairs, d_feat, s, stream);
+        case CLUSTEN_F32: return launch_typed<float>(d_out, w, starts, ends, pairs, not_whole, d_feat, s, stream);
+        case CLUSTEN_F16: return launch_typed<f16_t>(d_out, w, starts, ends, pairs, not_whole, d_feat, s, stream);
+        case CLUSTEN_BF16: return launch_typed<bf16_t>(d_out, w, starts, ends, pairs, not_whole, d_feat, s, stream);
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
 }

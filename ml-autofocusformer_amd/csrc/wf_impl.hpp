@@ -309,7 +309,9 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
 template <typename T, typename A>
 __global__ __launch_bounds__(256) void wf_dfeat_kernel(const T* __restrict__ d_out, const T* __restrict__ w,
                                                        const int64_t* __restrict__ idx, A* __restrict__ d_feat, int N,
-                                                       int Nout, int C, int M, int IC, int total_tokens) {
+                                                       int Nout, int C, int M, int IC, int total_tokens,
+                                                       const int32_t* __restrict__ only_if) {
+    if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
     const int token = xcd_tile(blockIdx.x, total_tokens);
     if (token < 0) return;
     {
@@ -412,12 +414,12 @@ int wf_dweights_typed(const void* d_out, const void* feat, const int64_t* idx, v
 
 template <typename T, typename A>
 int wf_dfeat_typed(const void* d_out, const void* w, const int64_t* idx, A* acc, const clusten_wf_shape& s,
-                   hipStream_t stream) {
+                   hipStream_t stream, const int32_t* only_if) {
     const int total = s.B * s.Nout;
     const int threads = s.C >= 256 ? 256 : (s.C > 64 ? 128 : 64);
     hipLaunchKernelGGL((wf_dfeat_kernel<T, A>), dim3(xcd_grid(total)), dim3(threads), 0, stream,
                        static_cast<const T*>(d_out), static_cast<const T*>(w), idx, acc, s.N, s.Nout, s.C, s.M, s.IC,
-                       total);
+                       total, only_if);
     return launch_status();
 }
 

@@ -99,17 +99,24 @@ def test_bad_strides_are_rejected():
 def test_workspace_contract():
     lib = _native.load()
     s = _shape(B=2, H=2, N=16, C=32, M=8)
-    assert lib.clusten_qk_backward_workspace_bytes(s, 0) == 0          # fp32 accumulates in place
-    assert lib.clusten_qk_backward_workspace_bytes(s, 3) == 0
+    assert lib.clusten_qk_backward_workspace_bytes(s, 3) == 0          # fp64: atomics straight into d_key
+    pairs = lib.clusten_cluster_pairs_bytes(2, 16, 8, 16)              # the pair lists of (B,N,M) lists over N rows
+    assert pairs > 0 and pairs % 256 == 0
+    assert lib.clusten_qk_backward_workspace_bytes(s, 0) == pairs      # fp32 accumulates in place
     need = lib.clusten_qk_backward_workspace_bytes(s, 1)
-    assert need == 2 * 2 * 16 * 32 * 4                                  # one fp32 per d_key element
+    assert need == pairs + 2 * 2 * 16 * 32 * 4                          # ... plus one fp32 per d_key element
     assert lib.clusten_av_backward_workspace_bytes(s, 2) == need
+    odd = _shape(B=2, H=2, N=16, C=32, M=5)                            # no runs of 8: no pair lists
+    assert lib.clusten_qk_backward_workspace_bytes(odd, 0) == 0
+    assert lib.clusten_qk_backward_workspace_bytes(odd, 1) == 2 * 2 * 16 * 32 * 4
+    assert lib.clusten_cluster_pairs_bytes(2, 16, 5, 16) == 0 and lib.clusten_cluster_pairs_bytes(2, 16, 8, 4) == 0
     rows = _native.Strides(2 * 16 * 32, 16 * 32, 32)
     assert lib.clusten_qk_backward(FAKE, FAKE, rows, FAKE, rows, FAKE, FAKE, FAKE, P(0), 0, s, 1, P(0)) == 5
     assert lib.clusten_qk_backward(FAKE, FAKE, rows, FAKE, rows, FAKE, FAKE, FAKE, FAKE, need - 1, s, 1, P(0)) == 5
     w = _wshape(B=2, N=16, Nout=4, C=64, M=8, IC=4)
-    assert lib.clusten_wf_backward_workspace_bytes(w, 0) == 0
-    assert lib.clusten_wf_backward_workspace_bytes(w, 2) == 2 * 16 * 64 * 4
+    wpairs = lib.clusten_cluster_pairs_bytes(2, 4, 8, 16)
+    assert lib.clusten_wf_backward_workspace_bytes(w, 0) == wpairs
+    assert lib.clusten_wf_backward_workspace_bytes(w, 2) == wpairs + 2 * 16 * 64 * 4
     assert lib.clusten_wf_backward(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, P(0), 0, w, 2, P(0)) == 5
 
 

@@ -191,30 +191,39 @@ def test_logits_equal_with_hip_operators_and_with_the_oracle(device, amp):
 
 
 @pytest.mark.gpu
-def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkeypatch):
+@pytest.mark.parametrize("embed_dim", [(32, 64, 128, 256), (64, 128, 256, 512)])
+def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkeypatch, embed_dim):
     """A training step of the model with the backward scatters (d_key, d_value, WF d_feat) running as gathers over
-    sorted pair lists — the model's own lists are made of whole clusters — against the same step on the oracle."""
+    sorted pair lists — the model's own lists are made of whole clusters — against the same step on the oracle,
+    at head dim 16 and 32."""
     from aff.model import default_ops
     from clusten import _native
-    monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
-    monkeypatch.setattr(_native, "WF_BY_CLUSTER_MIN_ROWS", 0)
-    _native._PAIR_CACHE.clear()
-    seen = []
-    real = _native.cluster_pairs
-    monkeypatch.setattr(_native, "cluster_pairs", lambda *a: (seen.append(real(*a) is not None), real(*a))[1])
-    hip = small_model(default_ops(), img_size=128, num_classes=16).to(device).train()
-    ref = small_model(oracle_ops(), img_size=128, num_classes=16).to(device).train()
+    seen = {"qk": [], "av": [], "wf": []}
+
+    def watched(name, fn, n_rows):
+        def call(*a):
+            block = _native.cluster_pairs(a[3], n_rows(a))
+            seen[name].append(block is not None and int(_native.pairs_not_whole(block)) == 0)
+            return fn(*a)
+        return call
+
+    monkeypatch.setattr(_native, "qk_backward", watched("qk", _native.qk_backward, lambda a: None))
+    monkeypatch.setattr(_native, "av_backward", watched("av", _native.av_backward, lambda a: None))
+    monkeypatch.setattr(_native, "wf_backward", watched("wf", _native.wf_backward, lambda a: a[2].shape[1]))
+    hip = small_model(default_ops(), img_size=128, num_classes=16, embed_dim=embed_dim).to(device).train()
+    ref = small_model(oracle_ops(), img_size=128, num_classes=16, embed_dim=embed_dim).to(device).train()
     ref.load_state_dict(hip.state_dict())
     x = torch.randn(4, 3, 128, 128, generator=torch.Generator().manual_seed(8)).to(device)
     target = torch.randn(4, 16, generator=torch.Generator().manual_seed(9)).to(device)
     for model in (hip, ref):
         ((model(x) - target) ** 2).mean().backward()
-    assert any(seen), "no list of the model took the cluster-by-cluster path"
+    # every local attention layer and every merge handed over lists made of whole clusters
+    for name, flags in seen.items():
+        assert flags and all(flags), "%s: %s" % (name, flags)
     for (name, p), (_, q) in zip(hip.named_parameters(), ref.named_parameters()):
         assert p.grad is not None and torch.isfinite(p.grad).all(), name
         # 1e-7: the bias ahead of the BatchNorm has a gradient of zero, both sides hold rounding noise there
         assert float((p.grad - q.grad).abs().max()) <= 1e-3 * float(q.grad.abs().max()) + 1e-7, name
-    _native._PAIR_CACHE.clear()
 
 
 @pytest.mark.gpu

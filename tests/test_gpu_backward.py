@@ -78,24 +78,21 @@ def test_attn_backward_lists_made_of_runs(device, kind, dtype):
         _check_attn_backward(wl.attn_case("runs", 77, B=2, H=h, N=396, C=c, M=m, lists="runs:" + kind), device, dtype)
 
 
-@pytest.fixture
-def by_cluster(monkeypatch):
-    """The cluster-by-cluster scatter for problems of any size (in production it starts at 65536 rows)."""
-    monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 0)
-    monkeypatch.setattr(_native, "WF_BY_CLUSTER_MIN_ROWS", 0)
-    _native._PAIR_CACHE.clear()
-    yield
-    _native._PAIR_CACHE.clear()
+def _whole(idx, device, n_rows=None):
+    """True when the library finds `idx` to be lists made of whole clusters (reads the device flag: test only)."""
+    block = _native.cluster_pairs(idx.to(device), n_rows)
+    return block is not None and int(_native.pairs_not_whole(block)) == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-def test_attn_backward_cluster_by_cluster(device, dtype, by_cluster):
+def test_attn_backward_cluster_by_cluster(device, dtype):
     """Lists made of whole clusters: d_key / d_value as a gather over the pairs of every cluster (no atomics)."""
     g = torch.Generator().manual_seed(79)
-    for B, H, N, nnc in ((2, 3, 200, 6), (1, 2, 392, 6), (3, 1, 64, 8), (2, 2, 24, 3)):
+    for B, H, N, nnc, C in ((2, 3, 200, 6, 32), (1, 2, 392, 6, 32), (3, 1, 64, 8, 32), (2, 2, 24, 3, 32), (2, 2, 200, 6, 16),
+                            (1, 3, 136, 6, 64)):
         idx = wl.model_like_lists(B, N, g, nnc=min(nnc, N // 8))
-        assert _native.cluster_pairs(idx.to(device)) is not None
-        case = wl.attn_case("model", 80, B=B, H=H, N=N, C=32, M=idx.shape[-1])
+        assert _whole(idx, device)
+        case = wl.attn_case("model", 80, B=B, H=H, N=N, C=C, M=idx.shape[-1])
         case.nbhd_idx = idx
         _check_attn_backward(case, device, dtype)
 
@@ -110,14 +107,14 @@ def _padded_model_lists(B, N, nnc, gen):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-def test_backward_cluster_by_cluster_with_a_short_last_cluster(device, dtype, by_cluster):
+def test_backward_cluster_by_cluster_with_a_short_last_cluster(device, dtype):
     """196 tokens = 24 clusters and one of 4: the lists that name it hold row 0 in their last slots, and those slots'
     contributions must reach row 0 (attention scatters and the WF feature gradient)."""
     g = torch.Generator().manual_seed(88)
     for B, H, N in ((2, 2, 196), (1, 3, 100), (2, 1, 13)):
         idx = _padded_model_lists(B, N, min(6, (N + 7) // 8), g)
         assert (idx == 0).sum() > B * N // 8
-        assert _native.cluster_pairs(idx.to(device)) is not None
+        assert _whole(idx, device)
         case = wl.attn_case("padded", 89, B=B, H=H, N=N, C=32, M=idx.shape[-1], lists="random")
         case.nbhd_idx = idx
         _check_attn_backward(case, device, dtype)
@@ -126,21 +123,19 @@ def test_backward_cluster_by_cluster_with_a_short_last_cluster(device, dtype, by
     pick = torch.rand(B, Nout, K, generator=g).argsort(dim=2)[:, :, :6]
     rows = pick.unsqueeze(3) * 8 + torch.arange(8)
     idx = torch.where(rows < N, rows, torch.zeros_like(rows)).reshape(B, Nout, 48)
-    assert _native.cluster_pairs(idx.to(device), N) is not None
+    assert _whole(idx, device, N)
     case = wl.wf_case("padded", 90, B=B, N=N, C=C, IC=4, M=48, Nout=Nout)
     case.nbhd_idx = idx
     _check_wf_backward(case, device, dtype)
 
 
-def test_cluster_by_cluster_scatter_properties(device, by_cluster):
+def test_cluster_by_cluster_scatter_properties(device):
     g = torch.Generator().manual_seed(81)
     B, H, N, C = 2, 3, 200, 32
     idx = wl.model_like_lists(B, N, g).to(device)
     M = idx.shape[-1]
     lists = _native.cluster_pairs(idx)
-    offsets, pairs = lists
-    assert offsets.dtype == torch.int32 and offsets.numel() == B * N // 8 + 1 and int(offsets[-1]) == B * N * M // 8
-    assert _native.cluster_pairs(idx) is lists                       # kept for the lists seen lately
+    assert lists.dtype == torch.uint8 and int(_native.pairs_not_whole(lists)) == 0
     # integer-valued data: every product and sum exact, so the result equals the oracle's bit for bit
     q = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
     k = torch.randint(-4, 5, (B, H, N, C), generator=g).float()
@@ -148,31 +143,85 @@ def test_cluster_by_cluster_scatter_properties(device, by_cluster):
     dq_ref, dk_ref = oracle.qk_gather_backward(d_attn, q, k, idx.cpu())
     dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx)
     assert torch.equal(dq.cpu(), dq_ref) and torch.equal(dk.cpu(), dk_ref)
-    # no atomics: two runs on random data give the same bits
+    # no atomics: two runs on random data give the same bits, through the optional entry point and through the
+    # drop-in backward (whose first call takes the same kernels as every later one)
     x = torch.randn(B, H, N, C, generator=g).to(device)
     p = torch.randn(B, H, N, M, generator=g).to(device)
-    assert torch.equal(_native.scatter_rows_by_cluster(p, x, lists), _native.scatter_rows_by_cluster(p, x, lists))
+    first = _native.scatter_rows_by_cluster(p, x, lists)
+    assert torch.equal(first, _native.scatter_rows_by_cluster(p, x, lists))
+    assert torch.equal(first, _native.scatter_rows_by_cluster(p, x, _native.cluster_pairs(idx)))   # a stable sort
+    assert torch.equal(first, _native.qk_backward(p, x, x, idx)[1])
+    assert torch.equal(first, _native.qk_backward(p, x, x, idx)[1])
     # a cluster nobody lists receives zeros; one listed by more pairs than a wave holds at once is taken in segments
+    # (16-bit data too: the sum over all segments is rounded once)
     lone = torch.zeros(1, 2400, 48, dtype=torch.int64)
     lone[:] = (torch.arange(48) % 8) + 8 * (torch.arange(48) // 8 + 1)          # everybody lists clusters 1..6
     lone = lone.to(device)
     lists2 = _native.cluster_pairs(lone)
     x2 = torch.randn(1, 2, 2400, C, generator=g)
     p2 = torch.randn(1, 2, 2400, 48, generator=g)
-    want = oracle.qk_gather_backward(p2, x2, x2, lone.cpu())[1]
-    got = _native.scatter_rows_by_cluster(p2.to(device), x2.to(device), lists2)
-    assert oracle.rel_err(got, want) <= TOL_SCATTER_F32 and float(got[:, :, :8].abs().max()) == 0.0
-    # in production a list tensor is only remembered when it is first met; its pair lists are made when it comes again
-    _native._PAIR_CACHE.clear()
-    assert _native.cluster_pairs(idx, on_second_sight=True) is None
-    again = _native.cluster_pairs(idx, on_second_sight=True)
-    assert again is not None and torch.equal(again[1], pairs) and _native.cluster_pairs(idx, on_second_sight=True) is again
-    # lists that are not whole clusters keep the atomic path
-    assert _native.cluster_pairs(torch.randint(N, (B, N, M), generator=g).to(device)) is None
-    shifted = idx.clone()
-    shifted[0, 0, :8] += 1
-    assert _native.cluster_pairs(shifted.clamp_(max=N - 1)) is None
+    for dtype, tol in ((torch.float32, TOL_SCATTER_F32), (torch.float16, TOL[torch.float16]),
+                       (torch.bfloat16, TOL[torch.bfloat16])):
+        xs, ps = x2.to(dtype), p2.to(dtype)
+        want = oracle.qk_gather_backward(ps.float(), xs.float(), xs.float(), lone.cpu())[1]
+        got = _native.scatter_rows_by_cluster(ps.to(device), xs.to(device), lists2)
+        assert oracle.rel_err(got, want) <= tol and float(got[:, :, :8].float().abs().max()) == 0.0
+        if dtype != torch.float32:
+            # one rounding of the fp32 sum: at most half a unit in the last place from the oracle's fp32 result
+            assert oracle.rel_err(got, want.to(dtype).float()) <= (2e-3 if dtype == torch.float16 else 1.6e-2) * 0.51
+    # lists that are not whole clusters: the flag is up, the optional entry point leaves its output alone, the drop-in
+    # backward takes the atomic kernels
+    for other in (torch.randint(N, (B, N, M), generator=g).to(device),
+                  (idx + (torch.arange(M, device=device) < 8)).clamp_(max=N - 1)):
+        block = _native.cluster_pairs(other)
+        assert int(_native.pairs_not_whole(block)) == 1
+        marker = torch.full((B, H, N, C), 7.0, device=device)
+        _native.scatter_rows_by_cluster(p, x, block, out=marker)
+        assert bool((marker == 7.0).all())
+        want = oracle.qk_gather_backward(p.cpu(), x.cpu(), x.cpu(), other.cpu())[1]
+        assert oracle.rel_err(_native.qk_backward(p, x, x, other)[1], want) <= TOL_SCATTER_F32
     assert _native.cluster_pairs(idx[:, :, :44].contiguous()) is None
+
+
+def test_backward_never_reads_the_device_from_the_host(device):
+    """The drop-in backward of the three operators recorded into a HIP graph (a capture fails on any synchronisation or
+    read-back) and replayed with eager work between the replays: every replay equals the eager result bit for bit on
+    lists made of whole clusters."""
+    g = torch.Generator().manual_seed(93)
+    B, H, N, C = 2, 2, 200, 32
+    idx = wl.model_like_lists(B, N, g).to(device)
+    M = idx.shape[-1]
+    q, k = (torch.randn(B, H, N, C, generator=g).to(device) for _ in range(2))
+    d_attn = torch.randn(B, H, N, M, generator=g).to(device)
+    widx = _wf_cluster_lists(B, N, 50, 6, g).to(device)
+    w = torch.randn(B, 50, 48, 4, generator=g).to(device)
+    f = torch.randn(B, N, 64, generator=g).to(device)
+    d_out = torch.randn(B, 50, 4, 64, generator=g).to(device)
+
+    def step():
+        return (_native.qk_backward(d_attn, q, k, idx) + _native.av_backward(q, d_attn, k, idx)
+                + _native.wf_backward(d_out, w, f, widx))
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for _ in range(3):
+        for t in outs:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got, want)
+        again = step()                           # eager work between the replays
+        for got, want in zip(again, eager):
+            assert torch.equal(got, want)
 
 
 def _wf_cluster_lists(B, N, Nout, nnc, gen):
@@ -183,18 +232,18 @@ def _wf_cluster_lists(B, N, Nout, nnc, gen):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-def test_wf_backward_cluster_by_cluster(device, dtype, by_cluster):
+def test_wf_backward_cluster_by_cluster(device, dtype):
     """WF lists made of whole clusters: d_feat as a gather over the pairs of every cluster (no atomics)."""
     g = torch.Generator().manual_seed(83)
     for B, N, Nout, C, nnc in ((2, 200, 50, 64, 6), (1, 392, 98, 128, 6), (2, 64, 16, 32, 8), (1, 48, 12, 96, 3)):
         idx = _wf_cluster_lists(B, N, Nout, nnc, g)
-        assert _native.cluster_pairs(idx.to(device), N) is not None
+        assert _whole(idx, device, N)
         case = wl.wf_case("clusters", 84, B=B, N=N, C=C, IC=4, M=idx.shape[-1], Nout=Nout)
         case.nbhd_idx = idx
         _check_wf_backward(case, device, dtype)
 
 
-def test_wf_cluster_by_cluster_properties(device, by_cluster):
+def test_wf_cluster_by_cluster_properties(device):
     g = torch.Generator().manual_seed(85)
     B, N, Nout, C, IC = 2, 200, 50, 64, 4
     idx = _wf_cluster_lists(B, N, Nout, 6, g)
@@ -215,9 +264,16 @@ def test_wf_cluster_by_cluster_properties(device, by_cluster):
     want = oracle.wf_gather_backward(d2, w2, f2, many)[1]
     got = _native.wf_backward(d2.to(device), w2.to(device), f2.to(device), many.to(device))[1]
     assert oracle.rel_err(got, want) <= TOL_SCATTER_F32 and float(got[:, 48:].abs().max()) == 0.0
+    got16 = _native.wf_backward(d2.half().to(device), w2.half().to(device), f2.half().to(device), many.to(device))[1]
+    want16 = oracle.wf_gather_backward(d2.half().float(), w2.half().float(), f2.half().float(), many)[1]
+    assert oracle.rel_err(got16, want16.half().float()) <= 2e-3 * 0.51          # the fp32 sum rounded once
+    # the optional entry point on the same pair lists gives the same bits as the drop-in backward
+    block = _native.cluster_pairs(many.to(device), 160)
+    assert torch.equal(_native.wf_backward_by_cluster(d2.to(device), w2.to(device), f2.to(device), many.to(device),
+                                                      block)[1], got)
     # other inner channel counts and lists that are not whole clusters keep the atomic kernel
     case = wl.wf_case("knn", 86, B=2, N=200, C=64, IC=4)
-    assert _native.cluster_pairs(case.nbhd_idx.to(device), 200) is None
+    assert not _whole(case.nbhd_idx, device, 200)
     _check_wf_backward(case, device, torch.float32)
     case1 = wl.wf_case("ic1", 87, B=1, N=64, C=64, IC=1, M=48, Nout=16)
     case1.nbhd_idx = _wf_cluster_lists(1, 64, 16, 6, g)

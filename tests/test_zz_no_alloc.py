@@ -41,17 +41,13 @@ def _both(device, d_attn, q, k, idx):
     return (got_q, got_k), (want_q, want_k)
 
 
-@pytest.fixture(autouse=True)
-def _atomic_kernels(monkeypatch):
-    # compare against the kernels the static entry point shares, not the cluster-by-cluster path of the bindings
-    monkeypatch.setattr(_native, "BY_CLUSTER_MIN_ROWS", 1 << 62)
-
-
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_two_calls_in_a_row_the_second_smaller(device, dtype):
     tol = TOL_SCATTER_F32 if dtype == torch.float32 else TOL[dtype]
-    # first call: 2*3*392*32 sums in the scratch; second: a smaller problem that reuses its first part
-    for step, (B, H, N, C, M, lists) in enumerate(((2, 3, 392, 32, 48, "windowed"), (1, 2, 104, 32, 48, "random"))):
+    # first call: pair-list scratch and 2*3*392*32 sums in the scratch; second: a smaller problem that reuses its first
+    # part; third: lists made of whole clusters (the cluster-by-cluster kernel, its pair lists in the scratch)
+    for step, (B, H, N, C, M, lists) in enumerate(((2, 3, 392, 32, 48, "windowed"), (1, 2, 104, 32, 48, "random"),
+                                                   (1, 2, 64, 32, 48, "model"))):
         for integer in (True, False):
             d_attn, q, k, idx = _inputs(300 + step, B, H, N, C, M, dtype, lists, integer)
             (got_q, got_k), (want_q, want_k) = _both(device, d_attn, q, k, idx)
@@ -68,7 +64,7 @@ def test_two_calls_in_a_row_the_second_smaller(device, dtype):
 
 def test_a_problem_beyond_the_scratch_is_refused(device):
     lib = _native.load()
-    # 16-bit data: 4 bytes of scratch per d_key element
+    # 16-bit data: at least 4 bytes of scratch per d_key element
     elems = _native.STATIC_SCRATCH_BYTES // 4
     shape = _native.AttnShape(1, 1, elems // 32 + 8, 32, 8)
     rows = _native.Strides(shape.N * 32, shape.N * 32, 32)
