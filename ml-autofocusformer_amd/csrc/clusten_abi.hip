@@ -201,7 +201,8 @@ int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair
     if (pair_lists_bytes < l.bytes) return CLUSTEN_ERR_WORKSPACE;
     if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
     char* ws = static_cast<char*>(pair_lists);
-    return launch_cluster_pairs(nbhd_idx, reinterpret_cast<int32_t*>(ws + l.keys), reinterpret_cast<int32_t*>(ws + l.flag),
+    return launch_cluster_pairs(nbhd_idx, reinterpret_cast<int32_t*>(ws + l.keys), reinterpret_cast<int32_t*>(ws + l.wg_bad),
+                                reinterpret_cast<int32_t*>(ws + l.flag),
                                 reinterpret_cast<int32_t*>(ws + l.pairs), reinterpret_cast<int32_t*>(ws + l.starts),
                                 reinterpret_cast<int32_t*>(ws + l.ends), B, rows, M, n_rows, as_stream(stream));
 }

@@ -25,25 +25,48 @@ namespace {
 constexpr int kPadEntry = 1 << 30;
 constexpr int kSortLdsBytes = 60000;
 
-__global__ __launch_bounds__(64) void clear_flag_kernel(int32_t* flag) {
-    if (threadIdx.x == 0) *flag = 0;
-}
-
-// One thread per run: 64 bytes of the list.  Workgroups that start after the flag is up have nothing left to find.
-__global__ __launch_bounds__(256) void cluster_keys_kernel(const int64_t* __restrict__ idx, int32_t* __restrict__ keys,
-                                                           int32_t* not_whole, int D, int64_t runs) {
-    if (*static_cast<volatile int32_t*>(not_whole) != 0) return;
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (e >= runs) return;
-    const int64_t* run = idx + e * 8;
-    const int64_t head = run[0];
-    // a whole cluster, or the short last one (D % 8 rows) followed by pad slots that hold row 0
-    const int own = (head == D - (D & 7)) ? (D & 7) : 8;
-    bool ok = (head & 7) == 0 && head >= 0 && head < D;
+// Four lanes per run of 8 entries, 16 bytes (two entries) each, so that a wave reads 1 KiB of the lists per access;
+// every thread takes kKeysPerThread such pieces, all requested before the first is looked at.
+// Every workgroup reports what it found in a word of its own (`wg_bad`), and the sort kernel that follows adds the
+// words up: one flag for all would be one address, served by one channel of the L2, and waves that polled it in order
+// to leave early, raised it with an atomic each or even just stored to it spent their time queueing at that channel
+// (250 us instead of 45 on lists that are not whole clusters).
+constexpr int kKeysBlock = 256;
+constexpr int kKeysPerThread = 4;
+__global__ __launch_bounds__(kKeysBlock) void cluster_keys_kernel(const int64_t* __restrict__ idx,
+                                                                  int32_t* __restrict__ keys,
+                                                                  int32_t* __restrict__ wg_bad, int D, int64_t runs) {
+    typedef long long I64x2 __attribute__((ext_vector_type(2)));
+    const int lane = threadIdx.x & 63;
+    const int64_t first = (int64_t)blockIdx.x * (kKeysBlock * kKeysPerThread) + threadIdx.x;
+    I64x2 two[kKeysPerThread];
 #pragma unroll
-    for (int t = 1; t < 8; ++t) ok = ok && run[t] == (t < own ? head + t : 0);
-    keys[e] = ok ? (int32_t)(head >> 3) : 0;
-    if (!ok) atomicOr(not_whole, 1);
+    for (int u = 0; u < kKeysPerThread; ++u) {
+        const int64_t piece = first + u * kKeysBlock;                // two entries
+        two[u] = (piece >> 2) < runs ? *reinterpret_cast<const I64x2*>(idx + piece * 2) : I64x2{0, 0};
+    }
+    bool any_bad = false;
+#pragma unroll
+    for (int u = 0; u < kKeysPerThread; ++u) {
+        const int64_t piece = first + u * kKeysBlock;
+        const int64_t e = piece >> 2;                                // the run
+        const int q = (int)(piece & 3);                              // which quarter of it
+        const bool live = e < runs;
+        // the run's first entry, from the first lane of the quad (64-bit shuffle as two halves)
+        const int lo = __shfl((int)(two[u][0] & 0xffffffffll), lane & ~3);
+        const int hi = __shfl((int)(two[u][0] >> 32), lane & ~3);
+        const int64_t head = ((int64_t)hi << 32) | (uint32_t)lo;
+        // a whole cluster, or the short last one (D % 8 rows) followed by pad slots that hold row 0
+        const int own = (head == D - (D & 7)) ? (D & 7) : 8;
+        bool ok = (head & 7) == 0 && head >= 0 && head < D;
+        ok = ok && two[u][0] == (2 * q < own ? head + 2 * q : 0) && two[u][1] == (2 * q + 1 < own ? head + 2 * q + 1 : 0);
+        const uint64_t bad = __ballot(live && !ok);
+        const bool run_ok = ((bad >> (lane & ~3)) & 0xf) == 0;
+        if (live && q == 0) keys[e] = run_ok ? (int32_t)(head >> 3) : 0;
+        any_bad = any_bad || bad != 0;
+    }
+    const int found = __syncthreads_or(any_bad);
+    if (threadIdx.x == 0) wg_bad[blockIdx.x] = found ? 1 : 0;
 }
 
 // Exclusive scan of one value per thread over the workgroup; `scratch` holds one int per wave.  Returns the sum of
@@ -72,11 +95,20 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* scratch, int* to
 // One workgroup per image.  E entries (i, r) of the image in the order e = i*R + r; K clusters; `cap` entries of
 // `pairs` per image (2E when the sequence ends in a short cluster, else E).
 __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __restrict__ keys,
-                                                            const int32_t* __restrict__ not_whole,
+                                                            const int32_t* __restrict__ wg_bad, int n_wg_bad,
+                                                            int32_t* __restrict__ not_whole,
                                                             int32_t* __restrict__ pairs, int32_t* __restrict__ starts,
                                                             int32_t* __restrict__ ends, int E, int R, int K, int cap,
-                                                            int pad) {
-    if (*not_whole != 0) return;
+                                                            int pad, int key_bits) {
+    {
+        // what the workgroups of the keys kernel found, added up by every workgroup here for itself; the first one
+        // writes the flag the later kernels read
+        int bad = 0;
+        for (int z = threadIdx.x; z < n_wg_bad; z += blockDim.x) bad |= wg_bad[z];
+        bad = __syncthreads_or(bad);
+        if (blockIdx.x == 0 && threadIdx.x == 0) *not_whole = bad ? 1 : 0;
+        if (bad) return;
+    }
     extern __shared__ int32_t lds[];
     const int W = blockDim.x >> 6, w = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int* hist = lds;              // [W][K]: count, then the start inside the key's list, of wave w's entries of key k
@@ -89,7 +121,15 @@ __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __res
 
     for (int z = threadIdx.x; z < W * K; z += blockDim.x) hist[z] = 0;
     __syncthreads();
-    for (int e = lo + lane; e < hi; e += 64) atomicAdd(&hist[w * K + my_keys[e]], 1);
+    for (int e0 = lo; e0 < hi; e0 += 4 * 64) {
+        int k4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) k4[u] = e0 + 64 * u + lane < hi ? my_keys[e0 + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (k4[u] >= 0) atomicAdd(&hist[w * K + k4[u]], 1);
+        }
+    }
     __syncthreads();
     for (int k = threadIdx.x; k < K; k += blockDim.x) {
         int run = 0;
@@ -121,31 +161,45 @@ __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __res
     __syncthreads();
     int32_t* out = pairs + (int64_t)b * cap;
     const int again_at = base[0] + regular0;       // where the flagged copies go
-    for (int e0 = lo; e0 < hi; e0 += 64) {
-        const int e = e0 + lane;
-        const bool valid = e < hi;
-        const int k = valid ? my_keys[e] : -1;
-        const int entry = (e / R) * 8 + e % R;
-        uint64_t remaining = __ballot(valid);
-        while (remaining != 0) {
-            const int sl = __builtin_ctzll(remaining);
-            const int ks = __builtin_amdgcn_readlane(k, sl);
-            const bool hit = k == ks;
-            const uint64_t match = __ballot(hit);
-            const int rank = __popcll(match & ((1ull << lane) - 1));
-            const int cur = hist[w * K + ks];
-            if (hit) {
-                out[base[ks] + cur + rank] = entry;
-                if (pad && ks == K - 1) out[again_at + cur + rank] = entry | kPadEntry;
+    for (int e00 = lo; e00 < hi; e00 += 4 * 64) {
+        int k4[4];    // four steps' keys requested together
+#pragma unroll
+        for (int u = 0; u < 4; ++u) k4[u] = e00 + 64 * u + lane < hi ? my_keys[e00 + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e00 + 64 * u + lane;
+            const int k = k4[u];
+            const bool valid = k >= 0;
+            const int entry = (e / R) * 8 + e % R;
+            // the lanes of this step that hold the lane's key: one ballot per bit of the key
+            uint64_t same = __ballot(valid);
+            for (int bit = 0; bit < key_bits; ++bit) {
+                const bool one = (k >> bit) & 1;
+                const uint64_t ones = __ballot(one);
+                same &= one ? ones : ~ones;
             }
-            lds_sync();
-            if (lane == sl) hist[w * K + ks] = cur + __popcll(match);
-            lds_sync();
-            remaining &= ~match;
+            const int rank = __popcll(same & ((1ull << lane) - 1));
+            const int group = __popcll(same);
+            const int leader = valid ? __builtin_ctzll(same) : lane;
+            // the first lane of every group moves its key's cursor (distinct keys: distinct addresses) and tells the others
+            int cur = 0;
+            if (valid && rank == 0) cur = atomicAdd(&hist[w * K + k], group);
+            cur = __shfl(cur, leader);
+            if (valid) {
+                out[base[k] + cur + rank] = entry;
+                if (pad && k == K - 1) out[again_at + cur + rank] = entry | kPadEntry;
+            }
         }
     }
 }
 
+}  // namespace
+
+namespace {
+inline size_t keys_workgroups(int64_t runs) {
+    const int64_t per = (int64_t)kKeysBlock * kKeysPerThread;
+    return (size_t)((4 * runs + per - 1) / per);
+}
 }  // namespace
 
 bool cluster_pairs_supported(int B, int rows, int M, int D) {
@@ -162,7 +216,8 @@ ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D) {
     const size_t cap = (D % 8) ? 2 * E : E;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     l.flag = 0;
-    l.keys = 256;
+    l.wg_bad = 256;
+    l.keys = l.wg_bad + up(keys_workgroups((int64_t)B * (int64_t)E) * 4);
     l.pairs = l.keys + up((size_t)B * E * 4);
     l.starts = l.pairs + up((size_t)B * cap * 4);
     l.ends = l.starts + up((size_t)B * K * 4);
@@ -170,23 +225,24 @@ ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D) {
     return l;
 }
 
-int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* not_whole, int32_t* pairs, int32_t* starts,
-                         int32_t* ends, int B, int rows, int M, int D, hipStream_t stream) {
+int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int32_t* not_whole, int32_t* pairs,
+                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream) {
     const int R = M / 8, K = (D + 7) / 8;
     const int64_t E = (int64_t)rows * R;
     const int64_t runs = (int64_t)B * E;
     const int cap = (int)((D % 8) ? 2 * E : E);
-    hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(64), 0, stream, not_whole);
-    hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)((runs + 255) / 256)), dim3(256), 0, stream, idx, keys, not_whole,
-                       D, runs);
+    const int n_wg = (int)keys_workgroups(runs);
+    hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)n_wg), dim3(kKeysBlock), 0, stream, idx, keys, wg_bad, D, runs);
     int waves = (kSortLdsBytes / 4 - 16) / K - 1;    // (waves + 1) * K + waves ints of LDS
     waves = waves > 16 ? 16 : waves;
     const int64_t steps = (E + 63) / 64;
     if (waves > steps) waves = (int)steps;
     if (waves < 1) waves = 1;
     const size_t lds = ((size_t)(waves + 1) * K + 16) * 4;
-    hipLaunchKernelGGL(cluster_sort_kernel, dim3(B), dim3(64 * waves), lds, stream, keys, not_whole, pairs, starts, ends,
-                       (int)E, R, K, cap, (D % 8) ? 1 : 0);
+    int key_bits = 0;
+    while ((1 << key_bits) < K) ++key_bits;
+    hipLaunchKernelGGL(cluster_sort_kernel, dim3(B), dim3(64 * waves), lds, stream, keys, wg_bad, n_wg, not_whole, pairs,
+                       starts, ends, (int)E, R, K, cap, (D % 8) ? 1 : 0, key_bits);
     return launch_status();
 }
 

@@ -70,15 +70,15 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
 // The pair lists of lists made of whole clusters (cluster_pairs.hip), built on the device: for `rows` list rows per
 //   image of M slots that point into a sequence of D rows (K = ceil(D/8) clusters), pairs[starts[b*K+g] .. ends[b*K+g])
 //   holds the entries i*8 + r whose run r of list row i is cluster g of image b, ascending; *not_whole becomes 1 when
-//   some run is not a whole cluster (then the other outputs mean nothing), else 0.  `keys` is scratch.
+//   some run is not a whole cluster (then the other outputs mean nothing), else 0.  `keys` and `wg_bad` are scratch.
 //   Sizes as cluster_pairs_layout() gives them (byte offsets into one 16-byte aligned block, `bytes` in all).
 struct ClusterPairsLayout {
-    size_t flag, keys, pairs, starts, ends, bytes;
+    size_t flag, wg_bad, keys, pairs, starts, ends, bytes;
 };
 bool cluster_pairs_supported(int B, int rows, int M, int D);
 ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D);
-int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* not_whole, int32_t* pairs, int32_t* starts,
-                         int32_t* ends, int B, int rows, int M, int D, hipStream_t stream);
+int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int32_t* not_whole, int32_t* pairs,
+                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream);
 // y[b,h,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i,:]: see scatter_by_cluster.hip.
 //   C in {16,32,64}.  `not_whole` (may be null): device flag; the kernel does nothing when it points to non-zero.
 bool scatter_by_cluster_supported(const void* p, const void* x, clusten_strides xs, const void* y,

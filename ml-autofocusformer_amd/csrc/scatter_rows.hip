@@ -51,10 +51,11 @@ int launch_scatter_rows(const void* p, const void* x, clusten_strides xs, const 
     if (plan.by_cluster && scatter_by_cluster_supported(p, x, xs, out, s, dtype)) {
         int32_t* not_whole = reinterpret_cast<int32_t*>(ws + plan.pairs.flag);
         int32_t* keys = reinterpret_cast<int32_t*>(ws + plan.pairs.keys);
+        int32_t* wg_bad = reinterpret_cast<int32_t*>(ws + plan.pairs.wg_bad);
         int32_t* pairs = reinterpret_cast<int32_t*>(ws + plan.pairs.pairs);
         int32_t* starts = reinterpret_cast<int32_t*>(ws + plan.pairs.starts);
         int32_t* ends = reinterpret_cast<int32_t*>(ws + plan.pairs.ends);
-        st = launch_cluster_pairs(idx, keys, not_whole, pairs, starts, ends, s.B, s.N, s.M, s.N, stream);
+        st = launch_cluster_pairs(idx, keys, wg_bad, not_whole, pairs, starts, ends, s.B, s.N, s.M, s.N, stream);
         if (st != CLUSTEN_OK) return st;
         st = launch_scatter_by_cluster(p, x, xs, starts, ends, pairs, not_whole, out, s, dtype, stream);
         if (st != CLUSTEN_OK) return st;

@@ -66,10 +66,11 @@ int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* 
     if (plan.by_cluster && wf_dfeat_by_cluster_supported(d_out, w, d_feat, s, dtype)) {
         int32_t* not_whole = reinterpret_cast<int32_t*>(ws + plan.pairs.flag);
         int32_t* keys = reinterpret_cast<int32_t*>(ws + plan.pairs.keys);
+        int32_t* wg_bad = reinterpret_cast<int32_t*>(ws + plan.pairs.wg_bad);
         int32_t* pairs = reinterpret_cast<int32_t*>(ws + plan.pairs.pairs);
         int32_t* starts = reinterpret_cast<int32_t*>(ws + plan.pairs.starts);
         int32_t* ends = reinterpret_cast<int32_t*>(ws + plan.pairs.ends);
-        st = launch_cluster_pairs(idx, keys, not_whole, pairs, starts, ends, s.B, s.Nout, s.M, s.N, stream);
+        st = launch_cluster_pairs(idx, keys, wg_bad, not_whole, pairs, starts, ends, s.B, s.Nout, s.M, s.N, stream);
         if (st != CLUSTEN_OK) return st;
         st = launch_wf_dfeat_by_cluster(d_out, w, starts, ends, pairs, not_whole, d_feat, s, dtype, stream);
         if (st != CLUSTEN_OK) return st;
