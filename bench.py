@@ -6,13 +6,17 @@ stage-1 shape (BASELINE.json configs[2], stage 1: B128, H2, N3136, head dim 32, 
 fp32; WF 3136 -> 784 tokens, 64 channels, 4 inner channels): one QK launch, one AV launch, one WF
 launch through the C ABI, inputs resident in HBM.  `value` is the algorithmic bytes of the three ops
 (every input read once, every output written once, int64 neighbour lists) divided by the time of a
-step.  The `roofline` object prices the slowest of the three kernels against the 8 TB/s HBM peak
-from per-launch HIP-event timings taken inside the timed region; `cpu_baseline` is the PyTorch
-gather oracle timed on the host cores on a batch slice of the same workload.
+step.  The three kernels take a third of the step each; the `roofline` object prices the one furthest
+below the 8 TB/s HBM peak among those tied for the longest (per-launch HIP-event timings taken inside
+the timed region) and carries the step's own fraction beside it; `replay_probe` times the same three
+kernels compiled without their arithmetic (same loads, LDS traffic and stores) in the same interleaved
+pass; `cpu_baseline` is the PyTorch gather oracle timed on the host cores on a batch slice of the same
+workload, `config0_cpu` the reference's own CPU-runnable configuration timed in full on both sides.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
 
-`--full` adds the other stages and configurations to the JSON line under "other_configs".
+The other stages and configurations are timed too and land under "other_configs"; `--quick` leaves
+them (and the images/s leg's GEMM tuning) out.
 """
 import argparse
 import json
@@ -29,8 +33,10 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch at the headline workload, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of `bench.py --only {qk,av,wf}`, each counter scaled by what it reads for the copy probe of known
-# size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md.
+# size; see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md, which names the source revision the
+# counters were read at.  A constant of that run, not a measurement of this one: TRAFFIC_MEASURED says when.
 MEASURED_TRAFFIC_BYTES = {"qk": 359.56e6 + 154.14e6, "av": 410.98e6 + 102.76e6, "wf": 219.18e6 + 102.76e6}
+TRAFFIC_MEASURED = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md"
 
 
 def _time_kernels(fns, steps, warmup):
@@ -106,6 +112,69 @@ def _cpu_baseline(attn_case, wf_case, full_bytes, full_batch, slice_b=32, budget
                   "tensors), median of %d passes, %.2f s per pass, %.1f s in all; a baseline, not the target"
                   % (slice_b, full_batch, reps, med, sum(times)),
     }
+
+
+def _config0(steps=200):
+    """Configuration 0 (the reference's CPU-runnable case: QK forward, B2 H2 N1024 C32 M48 fp32) timed in full on the
+    host cores (gather oracle, 3 untimed + 10 timed calls, median) and through the HIP kernel on the same tensors."""
+    import torch
+    import workloads as wl
+    from clusten import _native
+    from oracle import clusten_oracle as oracle
+
+    case = wl.config0()
+    B, H, N, C = case.query.shape
+    M = case.nbhd_idx.shape[-1]
+    nbytes = wl.attn_bytes(B, H, N, C, M, 4)
+    torch.set_num_threads(os.cpu_count() or 1)
+    times = []
+    for i in range(13):
+        t0 = time.perf_counter()
+        ref = oracle.qk_gather(case.query, case.key, case.nbhd_idx)
+        if i >= 3:
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    cpu_s = times[len(times) // 2]
+    d = case.to("cuda")
+    got = _native.qk_forward(d.query, d.key, d.nbhd_idx)
+    err = oracle.rel_err(got, ref)
+    _, per, _ = _time_kernels([lambda: _native.qk_forward(d.query, d.key, d.nbhd_idx)], steps, 10)
+    return {"shape": "QK forward B%d H%d N%d C%d M%d fp32" % (B, H, N, C, M), "algorithmic_bytes": nbytes,
+            "cpu_ms": round(cpu_s * 1e3, 3), "cpu_GBps": round(nbytes / cpu_s / 1e9, 3),
+            "cpu_cores": torch.get_num_threads(), "cpu_calls": "3 untimed + 10 timed, median",
+            "gpu_us": round(per[0] * 1e3, 2), "gpu_GBps": round(nbytes / per[0] / 1e6, 1),
+            "gpu_note": "2.6 MB: the launch, not the memory system, is what this size measures",
+            "rel_err_gpu_vs_cpu": float("%.3g" % err)}
+
+
+def _stream_gather_interference(tiles=50176, gathers=24, reps=20):
+    """How far the device overlaps an operator's two kinds of traffic: streams from / to memory (5 KiB in, 3 KiB out per
+    tile) and gathers that hit the L2 (24 KiB per tile inside 800 KB windows shared by 392 tiles — the QK shape), alone
+    and together, without arithmetic.  The streams rotate over four buffers so that they come from memory."""
+    import torch
+    from clusten import _native
+
+    sets = 4
+    ins = [torch.empty(tiles * 5120, dtype=torch.uint8, device="cuda").random_(0, 255) for _ in range(sets)]
+    outs = [torch.empty(tiles * 3072, dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    rows = torch.empty((tiles + 391) // 392 * 3136 * 256, dtype=torch.uint8, device="cuda").random_(0, 255)
+    res = {}
+    for name, mode in (("streams_us", 1), ("gathers_us", 2), ("both_us", 3)):
+        turn = [0]
+
+        def one():
+            i = turn[0] % sets
+            turn[0] += 1
+            _native.stream_gather_probe(ins[i], outs[i], rows, tiles, gathers, 3136, 392, mode)
+
+        _, per, _ = _time_kernels([one], reps, 4)
+        res[name] = round(per[0] * 1e3, 1)
+    res["stream_bytes"] = tiles * 8192
+    res["gather_bytes"] = tiles * gathers * 1024
+    res["streams_GBps"] = round(res["stream_bytes"] / res["streams_us"] / 1e3, 1)
+    res["gathers_GBps"] = round(res["gather_bytes"] / res["gathers_us"] / 1e3, 1)
+    res["both_over_sum"] = round(res["both_us"] / (res["streams_us"] + res["gathers_us"]), 3)
+    return res
 
 
 def _copy_bandwidth(nbytes=1 << 30, reps=20):
@@ -330,13 +399,17 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--full", action="store_true", help="also time the other stages and configurations")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--full", action="store_true", help="(default now) also time the other stages and configurations")
+    ap.add_argument("--quick", action="store_true",
+                    help="headline only: leave out the other configurations and the GEMM tuning of the images/s leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (the baseline and configuration 0)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the AFF-Tiny images/s leg")
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
-    ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model"), default=None,
+    ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model", "replay-qk", "replay-av", "replay-wf",
+                                       "interference"),
+                    default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -355,6 +428,9 @@ def main():
         print(json.dumps({"aff_tiny_224": _aff_tiny_throughput(tune_gemms=not args.no_gemm_tuning)}), flush=True)
         return
 
+    if args.only == "interference":
+        print(json.dumps({"only": "interference", **_stream_gather_interference()}), flush=True)
+        return
     B = 128
     acase = wl.config2_attn(1, B=B)
     wcase = wl.config2_wf(1, IC=4, B=B)
@@ -369,6 +445,10 @@ def main():
     fns = [lambda: _native.qk_forward(q, k, idx),
            lambda: _native.av_forward(attn, v, idx),
            lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
+    # the same kernels without their arithmetic (same loads, LDS traffic and stores): see include/clusten_hip.h
+    replay_fns = [lambda: _native.qk_forward(q, k, idx, replay=True),
+                  lambda: _native.av_forward(attn, v, idx, replay=True),
+                  lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx, replay=True)]
     torch.cuda.synchronize()
     if args.only == "bwd-model":  # the same on lists as the model builds them (whole clusters, nearest first)
         mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model")
@@ -384,6 +464,15 @@ def main():
             src = torch.empty(qk_bytes // 8, dtype=torch.float32, device="cuda").normal_()
             dst = torch.empty_like(src)
             one, nbytes = (lambda: _native.copy_probe(src, dst)), 2 * src.numel() * 4
+        elif args.only.startswith("replay-"):
+            # interleaved with the other two real kernels, as in the default pass: the probe's inputs come from HBM
+            i = ("qk", "av", "wf").index(args.only[7:])
+            trio = list(fns)
+            trio[i] = replay_fns[i]
+            _, per3, _ = _time_kernels(trio, args.steps, args.warmup)
+            print(json.dumps({"only": args.only, "launches": args.steps + args.warmup,
+                              "avg_us": round(per3[i] * 1e3, 2)}), flush=True)
+            return
         else:
             i = ("qk", "av", "wf").index(args.only)
             one, nbytes = fns[i], (qk_bytes, qk_bytes, wf_bytes)[i]
@@ -393,6 +482,8 @@ def main():
         return
     ms_per_step, per, wall_ms = _time_kernels(fns, args.steps, args.warmup)
     torch.cuda.synchronize()
+    _, per_replay, _ = _time_kernels(replay_fns, args.steps, args.warmup)
+    torch.cuda.synchronize()
 
     names = ("gather_dot_tile_kernel (QK)", "gather_sum_tile_kernel (AV)", "wf_forward_row_kernel (WF)")
     kbytes = (qk_bytes, qk_bytes, wf_bytes)
@@ -401,10 +492,10 @@ def main():
                for n, t, nb in zip(names, per, kbytes)]
     # The three kernels take a third of the step each (within 2 us of one another, less than the run-to-run spread of
     # the event timings), so "the longest" alone would name a different kernel from run to run: kernels within 2 % of
-    # the longest count as tied, and of those the one that moves the most algorithmic bytes is reported (AV, which
-    # is also the longest in the rocprofv3 summary); `kernels` lists all three either way.
+    # the longest count as tied, and of those the one furthest below the roofline is reported; `kernels` lists all three
+    # and `step_frac` is the whole step's fraction.
     longest = max(per)
-    dom = max((i for i in range(3) if per[i] >= 0.98 * longest), key=lambda i: (kbytes[i], per[i]))
+    dom = min((i for i in range(3) if per[i] >= 0.98 * longest), key=lambda i: kbytes[i] / per[i])
     value = total_bytes / ms_per_step / 1e6
     out = {
         "metric": "CLUSTEN QK+AV+WF forward, algorithmic GB/s (AFF-Tiny stage-1 shape)",
@@ -425,12 +516,22 @@ def main():
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "roofline": {"bound": "hbm", "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": kernels[dom]["frac_of_hbm_peak"],
-                     "traffic": MEASURED_TRAFFIC_BYTES[("qk", "av", "wf")[dom]], "kernel": names[dom]},
+                     "traffic": MEASURED_TRAFFIC_BYTES[("qk", "av", "wf")[dom]], "traffic_source": TRAFFIC_MEASURED,
+                     "kernel": names[dom], "step_frac": round(value / HBM_PEAK_GBPS, 4),
+                     "step_traffic": sum(MEASURED_TRAFFIC_BYTES.values())},
         "kernels": kernels,
+        "replay_probe": {"what": "the same kernels compiled without their matrix instructions (same global loads, LDS "
+                                 "accesses and stores), timed in the same interleaved pass",
+                         "kernels": [{"kernel": n, "replay_us": round(r * 1e3, 2), "kernel_us": round(t * 1e3, 2),
+                                      "kernel_over_replay": round(t / r, 3)}
+                                     for n, t, r in zip(names, per, per_replay)]},
         "host_wall_ms_per_step": round(wall_ms, 4),
         "copy_probe_GBps": round(_copy_bandwidth(), 1),
+        "stream_gather_interference": _stream_gather_interference(),
     }
-    if args.full:
+    if not args.no_cpu:
+        out["config0_cpu"] = _config0()
+    if not args.quick:
         other = {}
         for s in (2, 3, 4):
             other["cfg2_s%d_attn" % s] = _bench_attn(wl.config2_attn(s, B=B), args.steps, args.warmup)
@@ -479,7 +580,7 @@ def main():
         out["other_configs"] = other
     if not args.no_e2e:
         try:
-            out["aff_tiny_224"] = _aff_tiny_throughput(tune_gemms=not args.no_gemm_tuning)
+            out["aff_tiny_224"] = _aff_tiny_throughput(tune_gemms=not (args.no_gemm_tuning or args.quick))
         except Exception as exc:  # noqa: BLE001 - a secondary figure must not cost the line its headline
             out["aff_tiny_224"] = {"error": "%s: %s" % (type(exc).__name__, exc)}
     if not args.no_cpu:

@@ -88,6 +88,11 @@ _PROTOTYPES = {
                                             ctypes.c_int, ctypes.c_float, ctypes.c_float, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
+    "clusten_stream_gather_probe": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_int, _P]),
+    "clusten_qk_forward_replay": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_av_forward_replay": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
+    "clusten_wf_forward_replay": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
 }
 
 EXPORTS = tuple(_PROTOTYPES)
@@ -191,8 +196,9 @@ def _attn_problem(a: torch.Tensor, rows: torch.Tensor, nbhd_idx: torch.Tensor, n
     return device, _dtype_code(a, names[0]), idx, AttnShape(B, H, N, C, idx.shape[2])
 
 
-def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
-    """attn (b,h,n,m) = query · key[nbhd_idx]; query/key (b,h,n,c) may be strided views."""
+def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor, replay: bool = False) -> torch.Tensor:
+    """attn (b,h,n,m) = query · key[nbhd_idx]; query/key (b,h,n,c) may be strided views.  `replay` (a measurement aid,
+    fp32): the same kernels without their arithmetic — the result holds no meaningful values."""
     lib = load()
     device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
     query, key = _rows(query), _rows(key)
@@ -200,8 +206,9 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor) -
     if attn.numel() == 0:
         return attn
     with torch.cuda.device(device):
-        _check(lib.clusten_qk_forward(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx), _ptr(attn),
-                                      shape, code, _stream(device)), "clusten_qk_forward")
+        fn = lib.clusten_qk_forward_replay if replay else lib.clusten_qk_forward
+        _check(fn(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx), _ptr(attn), shape, code,
+                  _stream(device)), "clusten_qk_forward")
     return attn
 
 
@@ -315,9 +322,10 @@ def qk_backward_static(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Ten
                "clusten_qk_backward_static")
 
 
-def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, token_major: bool = False) -> torch.Tensor:
+def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, token_major: bool = False,
+               replay: bool = False) -> torch.Tensor:
     """feat (b,h,n,c) = attn · v[nbhd_idx].  With token_major=True the result is a (b,h,n,c) view of
-    (b,n,h,c) storage, so that `.permute(0,2,1,3).reshape(b,n,h*c)` needs no copy."""
+    (b,n,h,c) storage, so that `.permute(0,2,1,3).reshape(b,n,h*c)` needs no copy.  `replay`: see qk_forward."""
     lib = load()
     _require_cuda("attn", attn)
     device = attn.device
@@ -342,8 +350,9 @@ def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, toke
     if shape.M == 0:
         return feat.zero_()
     with torch.cuda.device(device):
-        _check(lib.clusten_av_forward(_ptr(attn), _ptr(v), _strides(v), _ptr(idx), _ptr(feat), _strides(feat), shape,
-                                      code, _stream(device)), "clusten_av_forward")
+        fn = lib.clusten_av_forward_replay if replay else lib.clusten_av_forward
+        _check(fn(_ptr(attn), _ptr(v), _strides(v), _ptr(idx), _ptr(feat), _strides(feat), shape, code, _stream(device)),
+               "clusten_av_forward")
     return feat
 
 
@@ -385,8 +394,8 @@ def _wf_problem(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tenso
     return device, _dtype_code(weights, "weights"), idx, WfShape(B, N, Nout, C, M, IC)
 
 
-def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
-    """feat_new (b,n_,ic,c) = weightsᵀ · feat[nbhd_idx]."""
+def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor, replay: bool = False) -> torch.Tensor:
+    """feat_new (b,n_,ic,c) = weightsᵀ · feat[nbhd_idx].  `replay`: see qk_forward."""
     lib = load()
     device, code, idx, shape = _wf_problem(weights, feat, nbhd_idx)
     weights, feat = weights.contiguous(), feat.contiguous()
@@ -396,8 +405,8 @@ def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor
     if shape.M == 0 or shape.N == 0:
         return out.zero_()
     with torch.cuda.device(device):
-        _check(lib.clusten_wf_forward(_ptr(weights), _ptr(feat), _ptr(idx), _ptr(out), shape, code, _stream(device)),
-               "clusten_wf_forward")
+        fn = lib.clusten_wf_forward_replay if replay else lib.clusten_wf_forward
+        _check(fn(_ptr(weights), _ptr(feat), _ptr(idx), _ptr(out), shape, code, _stream(device)), "clusten_wf_forward")
     return out
 
 
@@ -1107,3 +1116,22 @@ def copy_probe(src: torch.Tensor, dst: torch.Tensor) -> None:
         raise RuntimeError("copy_probe needs contiguous tensors of equal byte size")
     with torch.cuda.device(src.device):
         _check(lib.clusten_copy_probe(_ptr(src), _ptr(dst), nbytes, _stream(src.device)), "clusten_copy_probe")
+
+
+def stream_gather_probe(stream_in: torch.Tensor, stream_out: torch.Tensor, rows: torch.Tensor, tiles: int, gathers: int,
+                        window_rows: int, tiles_per_window: int, mode: int) -> None:
+    """`clusten_stream_gather_probe` (measurement aid): per tile, mode bit 0 = read 5 KiB of `stream_in` and write 3 KiB
+    of `stream_out`, bit 1 = gather `gathers` x 1 KiB of random 256-byte rows inside the tile's window of `rows`."""
+    lib = load()
+    _require_cuda("stream_in", stream_in)
+    device = stream_in.device
+    _require_cuda("stream_out", stream_out, device)
+    _require_cuda("rows", rows, device)
+    nbytes = lambda t: t.numel() * t.element_size()
+    windows = (tiles + tiles_per_window - 1) // tiles_per_window
+    if (nbytes(stream_in) < tiles * 5120 or nbytes(stream_out) < tiles * 3072
+            or nbytes(rows) < windows * window_rows * 256):
+        raise RuntimeError("stream_gather_probe: a buffer is too small for %d tiles" % tiles)
+    with torch.cuda.device(device):
+        _check(lib.clusten_stream_gather_probe(_ptr(stream_in), _ptr(stream_out), _ptr(rows), tiles, gathers, window_rows,
+                                               tiles_per_window, mode, _stream(device)), "clusten_stream_gather_probe")

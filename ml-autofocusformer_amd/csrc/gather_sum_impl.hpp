@@ -380,7 +380,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                                     ChIO::unpack(g_raw[ss], g);
 #pragma unroll
                                     for (int e = 0; e < S::ECH; ++e) {
-                                        d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[ss], g[e], d[e], 0, 0, 0);
+                                        d[e] = mfma_16x16x4(a4[ss], g[e], d[e]);
                                     }
                                 }
                             }
@@ -572,7 +572,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                                 }
 #pragma unroll
                                 for (int e = 0; e < S::ECH; ++e) {
-                                    d[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(aop, g[e], d[e], 0, 0, 0);
+                                    d[e] = mfma_16x16x4(aop, g[e], d[e]);
                                 }
                             }
                         }

@@ -166,6 +166,11 @@ int launch_knn2d(const float* query, const float* database, int64_t* idx, float*
 // dst[0:bytes) = src[0:bytes), 16 bytes per lane per step.
 int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 
+// A wave per tile: mode bit 0 = read 5 KiB of `in` and write 3 KiB of `out` per tile, bit 1 = gather `gathers` x 1 KiB
+//   of 256-byte rows at random inside the tile's window of `rows` (window = tile / tiles_per_window).  See util.hip.
+int launch_stream_gather_probe(const void* in, void* out, const void* rows, int tiles, int gathers, int window_rows,
+                               int tiles_per_window, int mode, hipStream_t stream);
+
 // Fill `count` fp32 / fp64 words with zero (a kernel, so that callers may capture it in a HIP graph).
 //   `only_if` (may be null): a device flag; the kernel does nothing when it points to zero.
 int launch_zero_f32(float* dst, size_t count, hipStream_t stream, const int32_t* only_if = nullptr);

@@ -9,6 +9,37 @@ namespace clusten {
 
 typedef float F32x4 __attribute__((ext_vector_type(4)));
 
+// CLUSTEN_REPLAY = 1 (set by replay_probe.hip alone, which compiles the forward kernels a second time under another
+// namespace) turns every matrix instruction of the kernels into one integer operation on its operands: every global
+// load, LDS access and store stays exactly where it is and the arithmetic goes.  What such a kernel takes is what the
+// memory instruction stream of the real kernel costs on its own.
+#ifndef CLUSTEN_REPLAY
+#define CLUSTEN_REPLAY 0
+#endif
+
+__device__ __forceinline__ F32x4 replay_touch(uint32_t a, uint32_t b, F32x4 d) {
+    d[0] = __uint_as_float(__float_as_uint(d[0]) ^ a ^ b);
+    return d;
+}
+
+// D (16x16) += A (16x4) * B (4x16), fp32: `v_mfma_f32_16x16x4_f32`.
+__device__ __forceinline__ F32x4 mfma_16x16x4(float a, float b, F32x4 d) {
+    if constexpr (CLUSTEN_REPLAY != 0) {
+        return replay_touch(__float_as_uint(a), __float_as_uint(b), d);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, d, 0, 0, 0);
+    }
+}
+
+// Sixteen independent 4x4 blocks, D += A (4x1) * B (1x4), fp32: `v_mfma_f32_4x4x1_16b_f32`.
+__device__ __forceinline__ F32x4 mfma_4x4x1(float a, float b, F32x4 d) {
+    if constexpr (CLUSTEN_REPLAY != 0) {
+        return replay_touch(__float_as_uint(a), __float_as_uint(b), d);
+    } else {
+        return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, d, 0, 0, 0);
+    }
+}
+
 // s_waitcnt immediate (gfx9 encoding) that waits until at most `vm` vector-memory operations are
 // outstanding and leaves the LDS/scalar and export counters alone.
 constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (15 << 8); }
@@ -53,11 +84,10 @@ __device__ __forceinline__ F32x4 tile_mfma(const Raw& a, const Raw& b, F32x4 d) 
     if constexpr (sizeof(T) == 4) {
         constexpr int VEC = (int)sizeof(Raw) / 4;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            d = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(raw_word(a, e)), __uint_as_float(raw_word(b, e)), d,
-                                                     0, 0, 0);
-        }
+        for (int e = 0; e < VEC; ++e) d = mfma_16x16x4(__uint_as_float(raw_word(a, e)), __uint_as_float(raw_word(b, e)), d);
         return d;
+    } else if constexpr (CLUSTEN_REPLAY != 0) {
+        return replay_touch(raw_word(a, 0) ^ raw_word(a, 1), raw_word(b, 0) ^ raw_word(b, 1), d);
     } else if constexpr (sizeof(Raw) == 16) {
         typedef _Float16 H8 __attribute__((ext_vector_type(8)));
         typedef __bf16 B8 __attribute__((ext_vector_type(8)));

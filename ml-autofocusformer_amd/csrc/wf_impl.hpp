@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         const float bop = (!GUARD || j < mc) ? x[e] : 0.f;
-                        acc[e] = __builtin_amdgcn_mfma_f32_4x4x1f32(aop, bop, acc[e], 0, 0, 0);
+                        acc[e] = mfma_4x4x1(aop, bop, acc[e]);
                     }
                 });
         }
