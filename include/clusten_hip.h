@@ -147,6 +147,18 @@ int clusten_av_forward(const void* attn,
                        void* feat, clusten_strides feat_strides,
                        clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* clusten_av_forward for fp32 attention weights over 16-bit values — what mixed precision hands the operator: the
+ * softmax that precedes it returns fp32, the value projection fp16 or bf16, and the reference's wrapper casts the
+ * values up first (clusten/clusten.py:52-53).  Here the 16-bit rows are read in place and widened on the way to the
+ * staging buffer: the same values and arithmetic as clusten_av_forward on a cast copy (bit-identical results),
+ * without that pass over the value tensor.  attn (B,H,N,M) and feat (strided (B,H,N,C)) fp32; value strided (B,H,N,C)
+ * of value_dtype, F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE). */
+int clusten_av_forward_mixed(const void* attn,
+                             const void* value, clusten_strides value_strides, int value_dtype,
+                             const int64_t* nbhd_idx,
+                             void* feat, clusten_strides feat_strides,
+                             clusten_attn_shape shape, clusten_stream stream);
+
 /* Replaces clustenav_cuda.backward (clustenav_cuda.cpp:35-45, clustenav_cuda_kernel.cu:93-218):
  *   d_attn[b,h,i,j]  = sum_c value[b,h,idx[b,i,j],c] * d_feat[b,h,i,c]
  *   d_value[b,h,n,c] = sum_{(i,j): idx[b,i,j]=n} attn[b,h,i,j] * d_feat[b,h,i,c]
@@ -165,6 +177,12 @@ int clusten_av_backward(const void* d_feat, clusten_strides d_feat_strides,
  * clustenwf_cuda_kernel.cu:18-93). */
 int clusten_wf_forward(const void* weights, const void* feat, const int64_t* nbhd_idx,
                        void* feat_new, clusten_wf_shape shape, int dtype, clusten_stream stream);
+
+/* clusten_wf_forward for fp32 weights over 16-bit features, read in place (the reference's wrapper casts the features
+ * up first, clusten/clusten.py:78-79); bit-identical to clusten_wf_forward on a cast copy.  weights (B,Nout,M,IC) and
+ * feat_new (B,Nout,IC,C) fp32; feat (B,N,C) of feat_dtype, F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE). */
+int clusten_wf_forward_mixed(const void* weights, const void* feat, int feat_dtype, const int64_t* nbhd_idx,
+                             void* feat_new, clusten_wf_shape shape, clusten_stream stream);
 
 /* Replaces clustenwf_cuda.backward (clustenwf_cuda.cpp:35-45, clustenwf_cuda_kernel.cu:96-229):
  *   d_weights[b,i,j,ic] = sum_c feat[b,idx[b,i,j],c] * d_feat_new[b,i,ic,c]

@@ -42,10 +42,12 @@ _PROTOTYPES = {
                                            ctypes.c_int, _P]),
     "clusten_qk_backward_static": (ctypes.c_int, [_P, _P, Strides, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_av_forward": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
+    "clusten_av_forward_mixed": (ctypes.c_int, [_P, _P, Strides, ctypes.c_int, _P, _P, Strides, AttnShape, _P]),
     "clusten_av_backward_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
     "clusten_av_backward": (ctypes.c_int, [_P, Strides, _P, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape,
                                            ctypes.c_int, _P]),
     "clusten_wf_forward": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
+    "clusten_wf_forward_mixed": (ctypes.c_int, [_P, _P, ctypes.c_int, _P, _P, WfShape, _P]),
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
     "clusten_qk_forward_clusters": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
@@ -356,6 +358,40 @@ def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, toke
     return feat
 
 
+def mixed_supported(first: torch.Tensor, second: torch.Tensor) -> bool:
+    """True for the operand pair mixed precision hands AV and WF: an fp32 first operand (attention weights, merge
+    weights) and an fp16 / bf16 second one (values, features), both on the GPU."""
+    return (first.is_cuda and second.is_cuda and first.dtype == torch.float32
+            and second.dtype in (torch.float16, torch.bfloat16))
+
+
+def av_forward_mixed(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
+    """feat (b,h,n,c) fp32 = attn (fp32) · v[nbhd_idx] with v fp16 / bf16 read in place: bit-identical to
+    `av_forward(attn, v.float(), nbhd_idx)` (the cast clusten/clusten.py:52-53 makes) without the copy."""
+    lib = load()
+    if not mixed_supported(attn, v):
+        raise RuntimeError("av_forward_mixed takes fp32 attn and fp16 / bf16 v on the GPU")
+    device = attn.device
+    _require_cuda("v", v, device)
+    if attn.dim() != 4 or v.dim() != 4 or nbhd_idx.dim() != 3 or attn.shape[:3] != v.shape[:3]:
+        raise RuntimeError("attn must be (b,h,n,m), v (b,h,n,c) and nbhd_idx (b,n,m)")
+    B, H, N, C = v.shape
+    idx = _idx(nbhd_idx, (B, N), device)
+    if idx.shape[2] != attn.shape[3]:
+        raise RuntimeError("attn has %d slots per token, nbhd_idx %d" % (attn.shape[3], idx.shape[2]))
+    shape = AttnShape(B, H, N, C, idx.shape[2])
+    attn, v = attn.contiguous(), _rows(v)
+    feat = torch.empty((B, H, N, C), dtype=torch.float32, device=device)
+    if feat.numel() == 0:
+        return feat
+    if shape.M == 0:
+        return feat.zero_()
+    with torch.cuda.device(device):
+        _check(lib.clusten_av_forward_mixed(_ptr(attn), _ptr(v), _strides(v), _DTYPE_CODE[v.dtype], _ptr(idx), _ptr(feat),
+                                            _strides(feat), shape, _stream(device)), "clusten_av_forward_mixed")
+    return feat
+
+
 def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor):
     """(d_attn (b,h,n,m), d_v (b,h,n,c)), both contiguous."""
     lib = load()
@@ -407,6 +443,34 @@ def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor
     with torch.cuda.device(device):
         fn = lib.clusten_wf_forward_replay if replay else lib.clusten_wf_forward
         _check(fn(_ptr(weights), _ptr(feat), _ptr(idx), _ptr(out), shape, code, _stream(device)), "clusten_wf_forward")
+    return out
+
+
+def wf_forward_mixed(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
+    """feat_new (b,n_,ic,c) fp32 = weights (fp32)ᵀ · feat[nbhd_idx] with feat fp16 / bf16 read in place: bit-identical to
+    `wf_forward(weights, feat.float(), nbhd_idx)` (the cast clusten/clusten.py:78-79 makes) without the copy."""
+    lib = load()
+    if not mixed_supported(weights, feat):
+        raise RuntimeError("wf_forward_mixed takes fp32 weights and fp16 / bf16 feat on the GPU")
+    device = weights.device
+    _require_cuda("feat", feat, device)
+    if weights.dim() != 4 or feat.dim() != 3 or nbhd_idx.dim() != 3 or weights.shape[0] != feat.shape[0]:
+        raise RuntimeError("weights must be (b,n_,m,ic), feat (b,n,c) and nbhd_idx (b,n_,m)")
+    B, Nout, M, IC = weights.shape
+    N, C = feat.shape[1], feat.shape[2]
+    idx = _idx(nbhd_idx, (B, Nout), device)
+    if idx.shape[2] != M:
+        raise RuntimeError("weights has %d slots per token, nbhd_idx %d" % (M, idx.shape[2]))
+    shape = WfShape(B, N, Nout, C, M, IC)
+    weights, feat = weights.contiguous(), feat.contiguous()
+    out = torch.empty((B, Nout, IC, C), dtype=torch.float32, device=device)
+    if out.numel() == 0:
+        return out
+    if M == 0 or N == 0:
+        return out.zero_()
+    with torch.cuda.device(device):
+        _check(lib.clusten_wf_forward_mixed(_ptr(weights), _ptr(feat), _DTYPE_CODE[feat.dtype], _ptr(idx), _ptr(out), shape,
+                                            _stream(device)), "clusten_wf_forward_mixed")
     return out
 
 

@@ -14,6 +14,8 @@ Same behaviour as the reference:
 Differences, none visible in results:
   * strided query / key / value views whose channel stride is 1 are read in place instead of being
     copied by `.contiguous()`, and key is not transposed;
+  * fp32 attn with fp16 / bf16 v, and fp32 weights with fp16 / bf16 feat (what mixed precision produces), are
+    computed from the 16-bit operand in place: bit-identical to the reference's cast-first forward, one pass less;
   * fp16 / bf16 sums are accumulated in fp32 and rounded once (the reference accumulates in half);
   * bfloat16 is accepted.
 """
@@ -51,15 +53,21 @@ class CLUSTENAVFunction(Function):
 
     @staticmethod
     def forward(ctx, attn, v, nbhd_idx):
-        if attn.dtype != v.dtype:
-            v = v.to(attn.dtype)
-        feat = _native.av_forward(attn, v, nbhd_idx)
+        if _native.mixed_supported(attn, v):
+            # fp32 weights over 16-bit values (mixed precision): the values are read in place; same result as the cast
+            feat = _native.av_forward_mixed(attn, v, nbhd_idx)
+        else:
+            if attn.dtype != v.dtype:
+                v = v.to(attn.dtype)
+            feat = _native.av_forward(attn, v, nbhd_idx)
         ctx.save_for_backward(attn, v, nbhd_idx)
         return feat
 
     @staticmethod
     def backward(ctx, grad_feat):
         attn, v, nbhd_idx = ctx.saved_tensors
+        if v.dtype != attn.dtype:
+            v = v.to(attn.dtype)
         d_attn, d_v = _native.av_backward(grad_feat, attn, v, nbhd_idx)
         return d_attn, d_v, None
 
@@ -71,14 +79,20 @@ class CLUSTENWFFunction(Function):
 
     @staticmethod
     def forward(ctx, weights, feat, nbhd_idx):
-        if feat.dtype != weights.dtype:
-            feat = feat.to(weights.dtype)
-        feat_new = _native.wf_forward(weights, feat, nbhd_idx)
+        if _native.mixed_supported(weights, feat):
+            # fp32 weights over 16-bit features: the features are read in place; same result as the cast
+            feat_new = _native.wf_forward_mixed(weights, feat, nbhd_idx)
+        else:
+            if feat.dtype != weights.dtype:
+                feat = feat.to(weights.dtype)
+            feat_new = _native.wf_forward(weights, feat, nbhd_idx)
         ctx.save_for_backward(weights, feat, nbhd_idx)
         return feat_new
 
     @staticmethod
     def backward(ctx, grad_feat_new):
         weights, feat, nbhd_idx = ctx.saved_tensors
+        if feat.dtype != weights.dtype:
+            feat = feat.to(weights.dtype)
         d_weights, d_feat = _native.wf_backward(grad_feat_new, weights, feat, nbhd_idx)
         return d_weights, d_feat, None

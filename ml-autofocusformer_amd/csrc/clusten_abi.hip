@@ -84,6 +84,17 @@ int clusten_av_forward(const void* attn, const void* value, clusten_strides valu
                              as_stream(stream));
 }
 
+int clusten_av_forward_mixed(const void* attn, const void* value, clusten_strides value_strides, int value_dtype,
+                             const int64_t* nbhd_idx, void* feat, clusten_strides feat_strides, clusten_attn_shape shape,
+                             clusten_stream stream) {
+    if (!attn || !value || !nbhd_idx || !feat) return CLUSTEN_ERR_NULL_POINTER;
+    if (value_dtype != CLUSTEN_F16 && value_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(value_strides, shape.C) || !strides_ok(feat_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    return launch_gather_sum_mixed(attn, value, value_strides, nbhd_idx, feat, feat_strides, shape, value_dtype,
+                                   as_stream(stream));
+}
+
 size_t clusten_av_backward_workspace_bytes(clusten_attn_shape shape, int dtype) {
     if (!dtype_ok(dtype) || check_attn_shape(shape) != CLUSTEN_OK) return 0;
     return scatter_rows_workspace_bytes(shape, dtype);
@@ -113,6 +124,14 @@ int clusten_wf_forward(const void* weights, const void* feat, const int64_t* nbh
     if (!dtype_ok(dtype)) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_wf_shape(shape)) return st;
     return launch_wf_forward(weights, feat, nbhd_idx, feat_new, shape, dtype, as_stream(stream));
+}
+
+int clusten_wf_forward_mixed(const void* weights, const void* feat, int feat_dtype, const int64_t* nbhd_idx, void* feat_new,
+                             clusten_wf_shape shape, clusten_stream stream) {
+    if (!weights || !feat || !nbhd_idx || !feat_new) return CLUSTEN_ERR_NULL_POINTER;
+    if (feat_dtype != CLUSTEN_F16 && feat_dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_wf_shape(shape)) return st;
+    return launch_wf_forward_mixed(weights, feat, nbhd_idx, feat_new, shape, feat_dtype, as_stream(stream));
 }
 
 size_t clusten_wf_backward_workspace_bytes(clusten_wf_shape shape, int dtype) {

@@ -94,8 +94,12 @@ struct SumStaging {
 // EXACT = the list has exactly 16*Q slots (no slot of the chunk is missing).
 // CLUSTERS (FAST kernels only) = the lists arrive as int32 cluster numbers, M/8 per token: slot j of a token is row
 // 8*g + j%8 of its cluster g = number j/8 (row 0 where that is past the last row); `idx` then points to (B, N, M/8) int32.
-template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false>
-__global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const T* __restrict__ rows,
+// TR = storage type of the gathered rows when it differs from T, the type of p and out: fp32 p with fp16 / bf16 rows
+// (attention weights straight from a softmax times 16-bit values under mixed precision).  The rows are then read in
+// place, eight bytes per lane, widened and written to the staging buffer in the layout the fp32 kernel keeps there:
+// the same values and the same arithmetic as a cast of the rows to fp32 ahead of the call, without that pass.
+template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false, typename TR = T>
+__global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restrict__ p, const TR* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx,
                                                                 T* __restrict__ out, int H_all, int N, int M,
                                                                 clusten_strides rs, clusten_strides os,
@@ -105,8 +109,23 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
     typedef VecIO<T, S::SPP> PieceIO;
     static_assert(C == 16 || C == 32 || C == 64, "channel blocks of 16");
     static_assert(FAST || Q == 4, "long lists are taken 64 slots at a time");
+    static_assert(sizeof(TR) == sizeof(T) || (sizeof(T) == 4 && sizeof(TR) == 2), "rows of T, or 16-bit rows under fp32");
+    constexpr int NARROW = (int)(sizeof(T) / sizeof(TR));   // 1, or 2 for 16-bit rows under fp32 p
 
     __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
+
+    // One access of a gather: every lane brings 16 bytes of staging — its piece of a row — to `dst` + 16 * lane.
+    // `off` is the byte offset of the piece inside (b, h) as if the rows were stored as T.
+    auto stage_rows = [&](const char* rows_bh, uint32_t off, char* dst) {
+        if constexpr (NARROW == 1) {
+            CLUSTEN_LDS_DMA16(rows_bh + off, dst);
+        } else {
+            const U32x2 raw = *reinterpret_cast<const U32x2*>(rows_bh + lane_offset(off >> 1));
+            float x[4];
+            VecIO<TR, 4>::unpack(raw, x);
+            *reinterpret_cast<F32x4*>(dst + threadIdx.x * 16) = F32x4{x[0], x[1], x[2], x[3]};
+        }
+    };
 
     // a workgroup serves the heads [h0, h0 + H) of its tile: short sequences with many heads are launched with
     // several head groups per tile (neighbours in the grid, so the later ones find the tile's lists in the L2)
@@ -321,7 +340,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 const float* pm_lane = pm + (kq * kTileTokens + (n & 7)) * S::PM_STRIDE;
 
                 for (int h = 0; h < H; ++h) {
-                    const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+                    const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(TR);
                     if (h >= 1 && h + 1 < H) {
 #pragma unroll
                         for (int k = 0; k < S::NI_P; ++k) {
@@ -343,7 +362,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                         for (int i = 0; i < S::NI_G; ++i) {
                             if (i * S::RPI < rows_batched) {  // rows past the last one repeat it (their p is zero)
                                 const uint32_t urow = (uint32_t)ulist[min(base + i * S::RPI + g_sub, total_rows - 1)];
-                                CLUSTEN_LDS_DMA16(rows_bh + (urow * row_pitch + (uint32_t)(g_pos * 16)), stage + i * 1024);
+                                stage_rows(rows_bh, urow * row_pitch + (uint32_t)(g_pos * 16), stage + i * 1024);
                             }
                         }
                         // clear the re-indexed p of this pass, then add this pass's pieces
@@ -424,7 +443,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
             }
         }
         for (int h = 0; h < H; ++h) {
-            const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+            const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(TR);
             F32x4 d[S::ECH];
 #pragma unroll
             for (int e = 0; e < S::ECH; ++e) d[e] = F32x4{0.f, 0.f, 0.f, 0.f};
@@ -436,7 +455,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                 // gather: rows of this chunk -> LDS (and the p pieces when they were not prefetched)
                 if constexpr (FAST) {
 #pragma unroll
-                    for (int i = 0; i < S::NI_G; ++i) CLUSTEN_LDS_DMA16(rows_bh + g_off[i], stage + i * 1024);
+                    for (int i = 0; i < S::NI_G; ++i) stage_rows(rows_bh, g_off[i], stage + i * 1024);
                 } else {
                     // this pass's list of the chunk
                     int mine;
@@ -452,7 +471,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                     for (int i = 0; i < S::NI_G; ++i) {
                         const int srow = min(i * S::RPI + g_sub, mc - 1);
                         const uint32_t off = (uint32_t)__shfl(mine, srow) * row_pitch + (uint32_t)(g_pos * 16);
-                        CLUSTEN_LDS_DMA16(rows_bh + off, stage + i * 1024);
+                        stage_rows(rows_bh, off, stage + i * 1024);
                     }
                 }
                 const int ps = FAST ? (h & 1) : 0;
@@ -608,26 +627,26 @@ __global__ __launch_bounds__(256) void gather_sum_elem_kernel(const T* __restric
     }
 }
 
-template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false>
+template <typename T, int C, int Q, bool FAST, bool EXACT, bool CLUSTERS = false, typename TR = T>
 int launch_tile_q(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
                   clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int groups = head_groups_for(total, s.H);
     const int grid = xcd_grid(total * groups);
-    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT, CLUSTERS>), dim3(grid), dim3(kWave), 0, stream,
-                       static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N,
+    hipLaunchKernelGGL((gather_sum_tile_kernel<T, C, Q, FAST, EXACT, CLUSTERS, TR>), dim3(grid), dim3(kWave), 0, stream,
+                       static_cast<const T*>(p), static_cast<const TR*>(rows), idx, static_cast<T*>(out), s.H, s.N,
                        s.M, rs, os, tiles_per_batch, total, groups);
     return launch_status();
 }
 
-template <typename T, int C>
+template <typename T, int C, typename TR = T>
 int launch_tile(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out, clusten_strides os,
                 const clusten_attn_shape& s, hipStream_t stream) {
     // 48 slots is the neighbourhood size of every 224x224 model: three slot blocks, no range checks
-    if (s.M == 48) return launch_tile_q<T, C, 3, true, true>(p, rows, rs, idx, out, os, s, stream);
-    if (s.M <= 64) return launch_tile_q<T, C, 4, true, false>(p, rows, rs, idx, out, os, s, stream);
-    return launch_tile_q<T, C, 4, false, false>(p, rows, rs, idx, out, os, s, stream);
+    if (s.M == 48) return launch_tile_q<T, C, 3, true, true, false, TR>(p, rows, rs, idx, out, os, s, stream);
+    if (s.M <= 64) return launch_tile_q<T, C, 4, true, false, false, TR>(p, rows, rs, idx, out, os, s, stream);
+    return launch_tile_q<T, C, 4, false, false, false, TR>(p, rows, rs, idx, out, os, s, stream);
 }
 
 template <typename T>
@@ -683,5 +702,53 @@ int gather_sum_typed(const void* p, const void* rows, clusten_strides rs, const 
     return launch_elem<T>(p, rows, rs, idx, out, os, s, stream);
 }
 
+// One thread per output element, rows of another storage type than p and out.
+template <typename T, typename TR>
+__global__ __launch_bounds__(256) void gather_sum_mixed_elem_kernel(const T* __restrict__ p, const TR* __restrict__ rows,
+                                                                    const int64_t* __restrict__ idx, T* __restrict__ out,
+                                                                    int B, int H, int N, int C, int M, clusten_strides rs,
+                                                                    clusten_strides os) {
+    const int64_t total = (int64_t)B * H * N * C;
+    for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(o % C);
+        const int64_t q1 = o / C;
+        const int i = (int)(q1 % N);
+        const int64_t q2 = q1 / N;
+        const int h = (int)(q2 % H);
+        const int b = (int)(q2 / H);
+        const int64_t* list = idx + ((int64_t)b * N + i) * M;
+        const T* prow = p + (((int64_t)b * H + h) * N + i) * M;
+        const TR* base = rows + b * rs.b + h * rs.h + c;
+        float acc = 0.f;
+        for (int j = 0; j < M; ++j) acc += to_acc(prow[j]) * to_acc(base[list[j] * rs.n]);
+        out[b * os.b + h * os.h + i * os.n + c] = from_acc<T>(acc);
+    }
+}
+
+// fp32 p and out with rows of TR = fp16 / bf16, read in place (see the TR parameter of the tile kernel).
+template <typename TR>
+int gather_sum_mixed_typed(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
+                           clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
+    // p rows are whole 16-byte pieces, out rows 16-byte groups, a lane's piece of a gathered row 8 bytes
+    const bool rows8 = (reinterpret_cast<uintptr_t>(rows) & 7u) == 0 && (rs.b * 2) % 8 == 0 && (rs.h * 2) % 8 == 0 &&
+                       (rs.n * 2) % 8 == 0;
+    const bool quads_ok = ((int64_t)s.M * 4) % 16 == 0 && aligned16(p) && rows8 && rows_aligned16(out, os, 4) &&
+                          slice_fits_int32(rs, s.H, s.N, s.C);
+    if (quads_ok) {
+        switch (s.C) {
+            case 16: return launch_tile<float, 16, TR>(p, rows, rs, idx, out, os, s, stream);
+            case 32: return launch_tile<float, 32, TR>(p, rows, rs, idx, out, os, s, stream);
+            case 64: return launch_tile<float, 64, TR>(p, rows, rs, idx, out, os, s, stream);
+            default: break;
+        }
+    }
+    const int64_t total = (int64_t)s.B * s.H * s.N * s.C;
+    const int64_t want = (total + 255) / 256;
+    const int grid = (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
+    hipLaunchKernelGGL((gather_sum_mixed_elem_kernel<float, TR>), dim3(grid), dim3(256), 0, stream,
+                       static_cast<const float*>(p), static_cast<const TR*>(rows), idx, static_cast<float*>(out), s.B, s.H,
+                       s.N, s.C, s.M, rs, os);
+    return launch_status();
+}
 
 }  // namespace clusten

@@ -22,6 +22,10 @@ int launch_gather_dot_clusters(const void* a, clusten_strides a_strides, const v
 int launch_gather_sum(const void* p, const void* rows, clusten_strides rows_strides, const int64_t* idx, void* out,
                       clusten_strides out_strides, clusten_attn_shape s, int dtype, hipStream_t stream);
 
+// The same for fp32 p and out over rows of rows_dtype = F16 / BF16, read in place (equal to a cast of the rows first).
+int launch_gather_sum_mixed(const void* p, const void* rows, clusten_strides rows_strides, const int64_t* idx, void* out,
+                            clusten_strides out_strides, clusten_attn_shape s, int rows_dtype, hipStream_t stream);
+
 // The same with the lists given as cluster numbers (see launch_gather_dot_clusters).
 int launch_gather_sum_clusters(const void* p, const void* rows, clusten_strides rows_strides, const int32_t* cluster_idx,
                                void* out, clusten_strides out_strides, clusten_attn_shape s, int dtype,
@@ -38,6 +42,10 @@ int launch_scatter_rows(const void* p, const void* x, clusten_strides x_strides,
 // out[b,i,ic,c] = sum_j w[b,i,j,ic] * feat[b,idx[b,i,j],c]      (WF forward)
 int launch_wf_forward(const void* w, const void* feat, const int64_t* idx, void* out, clusten_wf_shape s, int dtype,
                       hipStream_t stream);
+
+// The same for fp32 w and out over feat of feat_dtype = F16 / BF16, read in place (equal to a cast of feat first).
+int launch_wf_forward_mixed(const void* w, const void* feat, const int64_t* idx, void* out, clusten_wf_shape s,
+                            int feat_dtype, hipStream_t stream);
 
 // d_w[b,i,j,ic] = sum_c feat[b,idx[b,i,j],c] * d_out[b,i,ic,c]  (WF backward, weights)
 int launch_wf_dweights(const void* d_out, const void* feat, const int64_t* idx, void* d_w, clusten_wf_shape s,

@@ -18,6 +18,18 @@ int launch_wf_forward(const void* w, const void* feat, const int64_t* idx, void*
     }
 }
 
+int wf_forward_mixed_f16(const void*, const void*, const int64_t*, void*, const clusten_wf_shape&, hipStream_t);
+int wf_forward_mixed_bf16(const void*, const void*, const int64_t*, void*, const clusten_wf_shape&, hipStream_t);
+
+int launch_wf_forward_mixed(const void* w, const void* feat, const int64_t* idx, void* out, clusten_wf_shape s,
+                            int feat_dtype, hipStream_t stream) {
+    switch (feat_dtype) {
+        case CLUSTEN_F16: return wf_forward_mixed_f16(w, feat, idx, out, s, stream);
+        case CLUSTEN_BF16: return wf_forward_mixed_bf16(w, feat, idx, out, s, stream);
+        default: return CLUSTEN_ERR_BAD_DTYPE;
+    }
+}
+
 int launch_wf_dweights(const void* d_out, const void* feat, const int64_t* idx, void* d_w, clusten_wf_shape s,
                        int dtype, hipStream_t stream) {
     switch (dtype) {

@@ -42,10 +42,14 @@ namespace clusten {
 
 // LPT = lanes per token (16, 32 or 64).  GUARD = false: the list has exactly 16*Q slots;
 // GUARD = true: any length, taken 64 slots at a time (Q = 4) with every slot range-checked.
-template <typename T, int LPT, int Q, bool GUARD>
+// TF = storage type of feat when it differs from T, the type of w and out: fp32 weights over fp16 / bf16 features, read
+// in place (a lane takes its VEC channels of a row as 8 bytes and widens them): the same values and arithmetic as a cast
+// of feat to fp32 ahead of the call, without that pass.
+template <typename T, int LPT, int Q, bool GUARD, typename TF = T>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void wf_forward_row_kernel(
-    const T* __restrict__ w, const T* __restrict__ feat, const int64_t* __restrict__ idx, T* __restrict__ out, int N,
+    const T* __restrict__ w, const TF* __restrict__ feat, const int64_t* __restrict__ idx, T* __restrict__ out, int N,
     int Nout, int C, int M, int IC, int total_tokens, int total_groups) {
+    typedef typename VecIO<TF, 16 / (int)sizeof(T)>::raw FeatRaw;   // the lane's channels of a gathered row
     constexpr int TPW = kWave / LPT;               // output tokens per wave
     constexpr int VEC = 16 / (int)sizeof(T);       // channels per lane and column block
     constexpr int SLOTS = 16 * Q;
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     const int64_t* list_p = idx + (int64_t)token * M;
     const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
     T* out_tok = out + (int64_t)token * IC * C;
-    const uint32_t row_bytes = (uint32_t)C * sizeof(T);
+    const uint32_t row_bytes = (uint32_t)C * sizeof(TF);
     // weights: the wave's tokens are consecutive, so their rows are one contiguous run
     const char* w_wave = reinterpret_cast<const char*>(w + (int64_t)token0 * M * IC);
     const int w_tok_bytes = M * IC * (int)sizeof(T);
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
         F32x4 acc[VEC];  // acc[e][ic] = out[ic][c0 + col + e]
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = F32x4{0.f, 0.f, 0.f, 0.f};
-        const uint32_t lane_bytes = (uint32_t)(c0 + col) * sizeof(T);
+        const uint32_t lane_bytes = (uint32_t)(c0 + col) * sizeof(TF);
 
         for (int j0 = 0; j0 < M; j0 += kWave) {
             const int mc = min(kWave, M - j0);
@@ -120,7 +124,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
             // IC read the last one: the rows of the 4x4 blocks they feed are never stored.
             const char* w_lane = wbuf + min(tl, ntok - 1) * w_chunk_bytes + min(ic_lane, IC - 1) * (int)sizeof(T);
 
-            Piece fv[SLOTS];
+            FeatRaw fv[SLOTS];
             T wv[SLOTS];
             slot_pipeline<SLOTS, GS>(
                 [&](auto ji) {
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                     // one 24-bit multiply-add, and the access is encoded as uniform base + lane offset.
                     const int row = rowlane_bcast<j % 16>(lst[j / 16]);
                     const uint32_t off = __umul24((uint32_t)((GUARD && j >= mc) ? 0 : row), row_bytes) + lane_bytes;
-                    fv[j] = *reinterpret_cast<const Piece*>(feat_b + lane_offset(off));
+                    fv[j] = *reinterpret_cast<const FeatRaw*>(feat_b + lane_offset(off));
                     // the weight of the slot comes from LDS with the group's rows, a pipeline group ahead of its use
                     wv[j] = *reinterpret_cast<const T*>(w_lane + (GUARD ? min(j, mc - 1) : j) * IC * (int)sizeof(T));
                 },
@@ -138,7 +142,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                     constexpr int j = decltype(ji)::value;
                     const float aop = (!GUARD || j < mc) ? to_acc(wv[j]) : 0.f;
                     float x[VEC];
-                    VecIO<T, VEC>::unpack(fv[j], x);
+                    VecIO<TF, VEC>::unpack(fv[j], x);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         const float bop = (!GUARD || j < mc) ? x[e] : 0.f;
@@ -335,31 +339,31 @@ inline int elem_grid(int64_t total) {
     return (int)(want < (int64_t)1 << 20 ? want : (int64_t)1 << 20);
 }
 
-template <typename T, int LPT>
+template <typename T, int LPT, typename TF = T>
 int wf_forward_row(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
     const int total = s.B * s.Nout;
     const int groups = (total + kWave / LPT - 1) / (kWave / LPT);
     if (s.M == 48) {  // the neighbourhood size of every 224x224 model: no range checks
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 3, false>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
-                           static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 3, false, TF>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
+                           static_cast<const T*>(w), static_cast<const TF*>(feat), idx, static_cast<T*>(out), s.N,
                            s.Nout, s.C, s.M, s.IC, total, groups);
     } else {
-        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 4, true>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
-                           static_cast<const T*>(w), static_cast<const T*>(feat), idx, static_cast<T*>(out), s.N,
+        hipLaunchKernelGGL((wf_forward_row_kernel<T, LPT, 4, true, TF>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
+                           static_cast<const T*>(w), static_cast<const TF*>(feat), idx, static_cast<T*>(out), s.N,
                            s.Nout, s.C, s.M, s.IC, total, groups);
     }
     return launch_status();
 }
 
-template <typename T>
+template <typename T, typename TF = T>
 int wf_forward_vec(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
                    hipStream_t stream) {
-    // lanes per token: the widest of 64, 32, 16 whose 16-byte accesses tile the row
+    // lanes per token: the widest of 64, 32, 16 whose 16-byte accesses (of T) tile the row
     const int row_bytes = s.C * (int)sizeof(T);
-    if (row_bytes % 1024 == 0) return wf_forward_row<T, 64>(w, feat, idx, out, s, stream);
-    if (row_bytes % 512 == 0) return wf_forward_row<T, 32>(w, feat, idx, out, s, stream);
-    return wf_forward_row<T, 16>(w, feat, idx, out, s, stream);
+    if (row_bytes % 1024 == 0) return wf_forward_row<T, 64, TF>(w, feat, idx, out, s, stream);
+    if (row_bytes % 512 == 0) return wf_forward_row<T, 32, TF>(w, feat, idx, out, s, stream);
+    return wf_forward_row<T, 16, TF>(w, feat, idx, out, s, stream);
 }
 
 template <typename T>
@@ -383,6 +387,42 @@ int wf_forward_typed(const void* w, const void* feat, const int64_t* idx, void* 
                       (s.M <= 64 || (64 * s.IC * (int)sizeof(T)) % 16 == 0);
     if (rows_ok && w_ok) return wf_forward_vec<T>(w, feat, idx, out, s, stream);
     return wf_forward_elem<T>(w, feat, idx, out, s, stream);
+}
+
+// One thread per output element, feat of another storage type than w and out.
+template <typename T, typename TF>
+__global__ __launch_bounds__(256) void wf_forward_mixed_elem_kernel(const T* __restrict__ w, const TF* __restrict__ feat,
+                                                                    const int64_t* __restrict__ idx, T* __restrict__ out,
+                                                                    int B, int N, int Nout, int C, int M, int IC) {
+    const int64_t total = (int64_t)B * Nout * IC * C;
+    for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(o % C);
+        const int64_t q1 = o / C;
+        const int ic = (int)(q1 % IC);
+        const int64_t token = q1 / IC;  // b*Nout + i
+        const int b = (int)(token / Nout);
+        const int64_t* list = idx + token * M;
+        const T* wrow = w + token * M * IC + ic;
+        const TF* base = feat + (int64_t)b * N * C + c;
+        float acc = 0.f;
+        for (int j = 0; j < M; ++j) acc += to_acc(wrow[(int64_t)j * IC]) * to_acc(base[list[j] * C]);
+        out[o] = from_acc<T>(acc);
+    }
+}
+
+// fp32 weights and output with features of TF = fp16 / bf16, read in place (see the TF parameter of the row kernel).
+template <typename TF>
+int wf_forward_mixed_typed(const void* w, const void* feat, const int64_t* idx, void* out, const clusten_wf_shape& s,
+                           hipStream_t stream) {
+    const bool rows_ok = (s.C * 4) % 256 == 0 && (reinterpret_cast<uintptr_t>(feat) & 7u) == 0 && aligned16(out) &&
+                         (int64_t)s.N * s.C * 2 < ((int64_t)1 << 31);
+    const bool w_ok = s.IC <= 4 && ((int64_t)s.M * s.IC * 4) % 16 == 0 && aligned16(w) && (s.M <= 64 || (64 * s.IC * 4) % 16 == 0);
+    if (rows_ok && w_ok) return wf_forward_vec<float, TF>(w, feat, idx, out, s, stream);
+    const int64_t total = (int64_t)s.B * s.Nout * s.IC * s.C;
+    hipLaunchKernelGGL((wf_forward_mixed_elem_kernel<float, TF>), dim3(elem_grid(total)), dim3(256), 0, stream,
+                       static_cast<const float*>(w), static_cast<const TF*>(feat), idx, static_cast<float*>(out), s.B, s.N,
+                       s.Nout, s.C, s.M, s.IC);
+    return launch_status();
 }
 
 template <typename T>
