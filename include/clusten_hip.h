@@ -459,12 +459,32 @@ int clusten_merge_weights_forward(const float* table_weights, const int64_t* pe_
  * rank = position of the token's anchor cell on the row-by-row walk (alternating direction) over a rows x cols
  * grid of cells of cell_w x cell_h, ratio = squared distance to the previous anchor of the walk over (squared
  * distance to the next + 1e-5); every float operation rounded as the reference's tensor expressions round it.
- *   pos (B,N,2) fp32 as (x, y), inside the canvas; ranking (B,N) int64; N <= 4096, rows * cols >= 2 (else
- *   CLUSTEN_ERR_BAD_DIMS); workspace: clusten_scanline_rank_workspace_bytes(B, N) bytes, 16-byte aligned.
+ *   pos (B,N,2) fp32 as (x, y), inside the canvas; ranking (B,N) int64; N <= clusten_scanline_rank_max_tokens()
+ *   (the sort of an image runs in the LDS of one compute unit: 16384 tokens on an MI355X, which covers the 9216
+ *   tokens of the first stage of a 384 x 384 model), rows * cols >= 2 (else CLUSTEN_ERR_BAD_DIMS); workspace:
+ *   clusten_scanline_rank_workspace_bytes(B, N) bytes, 16-byte aligned.
  * No counterpart in the reference's extension modules. */
+int clusten_scanline_rank_max_tokens(void);
 size_t clusten_scanline_rank_workspace_bytes(int B, int N);
 int clusten_scanline_rank(const float* pos, int64_t* ranking, void* workspace, size_t workspace_bytes,
                           int B, int N, int rows, int cols, float cell_w, float cell_h, clusten_stream stream);
+
+/* What `space_filling_cluster` does with the ranking (models/point_utils.py:161-208): the positions in cluster order
+ * and the mean position of every cluster of m consecutive tokens of that order,
+ *   pos_sorted[b,i] = pos[b, ranking[b,i]]          centres[b,g] = mean of pos_sorted[b, g*m .. min(g*m+m, N))
+ * (a short last cluster is averaged over the tokens it has, as the reference's masked mean does).  pos, pos_sorted
+ * (B,N,2), centres (B,ceil(N/m),2): fp32, 8-byte aligned; ranking (B,N) int64, a permutation per image — unchecked;
+ * pos_sorted may be NULL.  No counterpart in the reference's extension modules. */
+int clusten_cluster_centres(const float* pos, const int64_t* ranking, float* pos_sorted, float* centres,
+                            int B, int N, int m, clusten_stream stream);
+
+/* Rows of a (B,N,.) tensor in a given order, out[b,i,:] = x[b, order[b,i], :]: the reordering of the tokens into
+ * cluster order at the start of a stage (`feat.gather(index=ranking.expand(...), dim=1)`,
+ * models/aff_transformer.py:465-466) without an index per element.  Rows of row_bytes bytes (a multiple of 16, else
+ * CLUSTEN_ERR_BAD_DIMS), x and out 16-byte aligned; order (B,N) int64 with values in [0,N) — unchecked —, or (N) for
+ * every image when order_shared != 0.  No counterpart in the reference's extension modules. */
+int clusten_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes,
+                        int order_shared, clusten_stream stream);
 
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 

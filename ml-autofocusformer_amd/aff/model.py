@@ -50,7 +50,8 @@ def default_ops():
                            bias_table_grad=_native.bias_table_grad,
                            attn_softmax_backward=_native.attn_softmax_backward,
                            neighbour_lists=_native.neighbour_lists,
-                           neighbour_lists_supported=_native.neighbour_lists_supported)
+                           neighbour_lists_supported=_native.neighbour_lists_supported,
+                           gather_rows=_native.gather_rows, gather_rows_supported=_native.gather_rows_supported)
 
 
 def _cast_params(lin, dt):
@@ -545,7 +546,11 @@ class BasicLayer(nn.Module):
             else:
                 pos, ranking, member_idx, mask, pe_idx, cluster_idx = self.neighbourhoods(pos, h, w, radius, table_width)
                 if ranking is not None:
-                    feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
+                    rows_op = getattr(self.ops, "gather_rows", None)
+                    if rows_op is not None and not torch.is_grad_enabled() and self.ops.gather_rows_supported(feat):
+                        feat = rows_op(feat, ranking[:, :, 0])          # inference: one row-gather kernel
+                    else:
+                        feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
 
         carry = None
         for blk in self.blocks:

@@ -137,17 +137,25 @@ def space_filling_cluster(pos, m, h, w, no_reorder=False):
         if ranking is None:
             ranking = _scanline_ranking(pos, m, h, w)
 
-        pos = pos.gather(1, ranking.unsqueeze(2).expand(-1, -1, d))
-        if k * m == n:
+        if pos.is_cuda and d == 2:
+            # the positions in cluster order and the cluster centres from one kernel of the HIP library
+            from clusten import _native
+            pos, cluster_centres = _native.cluster_centres(pos, ranking, m)
             mask = None
-            cluster_centres = pos.reshape(b, k, m, d).mean(2)
+            if k * m != n:
+                mask = (torch.arange(k * m, device=pos.device) < n).to(torch.int64).reshape(1, k, m).expand(b, -1, -1)
         else:
-            padded = pos.new_zeros(b, k * m, d)
-            padded[:, :n] = pos
-            mask = torch.zeros(b, k * m, dtype=torch.int64, device=pos.device)
-            mask[:, :n] = 1
-            mask = mask.reshape(b, k, m)
-            cluster_centres = padded.reshape(b, k, m, d).sum(2) / mask.sum(2, keepdim=True)
+            pos = pos.gather(1, ranking.unsqueeze(2).expand(-1, -1, d))
+            if k * m == n:
+                mask = None
+                cluster_centres = pos.reshape(b, k, m, d).mean(2)
+            else:
+                padded = pos.new_zeros(b, k * m, d)
+                padded[:, :n] = pos
+                mask = torch.zeros(b, k * m, dtype=torch.int64, device=pos.device)
+                mask[:, :n] = 1
+                mask = mask.reshape(b, k, m)
+                cluster_centres = padded.reshape(b, k, m, d).sum(2) / mask.sum(2, keepdim=True)
 
         if no_reorder:
             member_idx = torch.zeros(b, k * m, dtype=torch.int64, device=pos.device)

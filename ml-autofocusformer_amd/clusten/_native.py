@@ -85,6 +85,9 @@ _PROTOTYPES = {
                                               ctypes.c_int, ctypes.c_int, _P]),
     "clusten_merge_weights_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                     ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_scanline_rank_max_tokens": (ctypes.c_int, []),
+    "clusten_cluster_centres": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_gather_rows": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "clusten_scanline_rank": (ctypes.c_int, [_P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                             ctypes.c_int, ctypes.c_float, ctypes.c_float, _P]),
@@ -1116,8 +1119,61 @@ def merge_weights(table_weights: torch.Tensor, pe_idx: torch.Tensor, nbhd_idx: t
 
 
 def scanline_rank_supported(pos: torch.Tensor, rows: int, cols: int) -> bool:
-    """True when `scanline_rank` takes this case: CUDA (B,N,2) positions, N <= 4096, at least two anchor cells."""
-    return pos.is_cuda and pos.dim() == 3 and pos.shape[2] == 2 and 0 < pos.shape[1] <= 4096 and rows * cols >= 2
+    """True when `scanline_rank` takes this case: CUDA (B,N,2) positions, at least two anchor cells, and a sequence
+    that one compute unit's LDS sorts (16384 tokens on an MI355X)."""
+    if not (pos.is_cuda and pos.dim() == 3 and pos.shape[2] == 2 and pos.shape[1] > 0 and rows * cols >= 2):
+        return False
+    with torch.cuda.device(pos.device):
+        return pos.shape[1] <= load().clusten_scanline_rank_max_tokens()
+
+
+def cluster_centres(pos: torch.Tensor, ranking: torch.Tensor, m: int):
+    """(pos in ranking order (B,N,2), mean position of every cluster of m consecutive tokens of that order
+    (B,ceil(N/m),2)): what `space_filling_cluster` derives from its ranking (point_utils.py:161-208), in one kernel."""
+    lib = load()
+    _require_cuda("pos", pos)
+    device = pos.device
+    _require_cuda("ranking", ranking, device)
+    if pos.dim() != 3 or pos.shape[2] != 2 or ranking.shape != pos.shape[:2] or ranking.dtype != torch.int64:
+        raise RuntimeError("pos must be (B,N,2) and ranking an int64 (B,N) tensor")
+    pos = pos.detach().float().contiguous()
+    ranking = ranking.contiguous()
+    b, n, _ = pos.shape
+    k = (n + m - 1) // m
+    pos_sorted = torch.empty_like(pos)
+    centres = torch.empty(b, k, 2, dtype=torch.float32, device=device)
+    if pos.numel():
+        with torch.cuda.device(device):
+            _check(lib.clusten_cluster_centres(_ptr(pos), _ptr(ranking), _ptr(pos_sorted), _ptr(centres), b, n, m,
+                                               _stream(device)), "clusten_cluster_centres")
+    return pos_sorted, centres
+
+
+def gather_rows_supported(x: torch.Tensor) -> bool:
+    """True when `gather_rows` takes this case: a CUDA (B,N,C) tensor whose rows are whole 16-byte pieces."""
+    return x.is_cuda and x.dim() == 3 and x.numel() > 0 and (x.shape[2] * x.element_size()) % 16 == 0
+
+
+def gather_rows(x: torch.Tensor, order: torch.Tensor) -> torch.Tensor:
+    """out[b,i,:] = x[b, order[b,i], :] for x (B,N,C) and order (B,N) int64 — or (N,), one order for every image:
+    `x.gather(1, order.unsqueeze(2).expand(-1, -1, C))` without an index per element.  No autograd."""
+    lib = load()
+    _require_cuda("x", x)
+    device = x.device
+    _require_cuda("order", order, device)
+    if not gather_rows_supported(x) or order.dtype != torch.int64:
+        raise RuntimeError("gather_rows takes (B,N,C) rows of whole 16-byte pieces and an int64 order")
+    b, n, c = x.shape
+    shared = order.dim() == 1
+    if tuple(order.shape) != ((n,) if shared else (b, n)):
+        raise RuntimeError("order must be (B,N) or (N,)")
+    x = x.detach().contiguous()
+    order = order.contiguous()
+    out = torch.empty_like(x)
+    with torch.cuda.device(device):
+        _check(lib.clusten_gather_rows(_ptr(x), _ptr(order), _ptr(out), b, n, c * x.element_size(), int(shared),
+                                       _stream(device)), "clusten_gather_rows")
+    return out
 
 
 def scanline_rank(pos: torch.Tensor, rows: int, cols: int, cell_w: float, cell_h: float) -> torch.Tensor:

@@ -405,13 +405,35 @@ size_t clusten_scanline_rank_workspace_bytes(int B, int N) {
 int clusten_scanline_rank(const float* pos, int64_t* ranking, void* workspace, size_t workspace_bytes, int B, int N,
                           int rows, int cols, float cell_w, float cell_h, clusten_stream stream) {
     if (!pos || !ranking || !workspace) return CLUSTEN_ERR_NULL_POINTER;
-    if (B <= 0 || N <= 0 || N > 4096 || rows <= 0 || cols <= 0 || (int64_t)rows * cols < 2 ||
+    if (B <= 0 || N <= 0 || N > scanline_rank_max_tokens() || rows <= 0 || cols <= 0 || (int64_t)rows * cols < 2 ||
         (int64_t)rows * cols >= ((int64_t)1 << 24) || !(cell_w > 0.f) || !(cell_h > 0.f)) {
         return CLUSTEN_ERR_BAD_DIMS;
     }
     if (workspace_bytes < scanline_rank_workspace_bytes(B, N)) return CLUSTEN_ERR_WORKSPACE;
     if (!aligned16(workspace) || (reinterpret_cast<uintptr_t>(pos) & 7u) != 0) return CLUSTEN_ERR_UNALIGNED;
     return launch_scanline_rank(pos, ranking, workspace, B, N, rows, cols, cell_w, cell_h, as_stream(stream));
+}
+
+int clusten_scanline_rank_max_tokens(void) { return scanline_rank_max_tokens(); }
+
+int clusten_cluster_centres(const float* pos, const int64_t* ranking, float* pos_sorted, float* centres, int B, int N, int m,
+                            clusten_stream stream) {
+    if (!pos || !ranking || !centres) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || m <= 0 || (int64_t)B * ((N + m - 1) / m) >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if ((reinterpret_cast<uintptr_t>(pos) & 7u) != 0 || (reinterpret_cast<uintptr_t>(centres) & 7u) != 0 ||
+        (reinterpret_cast<uintptr_t>(pos_sorted) & 7u) != 0) {
+        return CLUSTEN_ERR_UNALIGNED;
+    }
+    return launch_cluster_centres(pos, ranking, pos_sorted, centres, B, N, m, as_stream(stream));
+}
+
+int clusten_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes, int order_shared,
+                        clusten_stream stream) {
+    if (!x || !order || !out) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || row_bytes <= 0 || row_bytes % 16 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((B * N * (row_bytes / 16) + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (!aligned16(x) || !aligned16(out)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_gather_rows(x, order, out, B, N, row_bytes, order_shared, as_stream(stream));
 }
 
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,

@@ -162,6 +162,17 @@ int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int6
 //   cells of cell_w x cell_h (see scanline_rank.hip).  pos (B,N,2) fp32 as (x, y); ranking (B,N) int64; N <= 4096,
 //   rows * cols >= 2; workspace of scanline_rank_workspace_bytes(B, N) bytes.
 size_t scanline_rank_workspace_bytes(int B, int N);
+int scanline_rank_max_tokens();   // the longest sequence the LDS of the current device sorts (a power of two)
+
+// pos_sorted[b,i] = pos[b, ranking[b,i]] (may be null) and centres[b,g] = mean of the positions of tokens
+//   ranking[b, g*m .. g*m+m-1] (the last cluster may be short): pos, pos_sorted (B,N,2), centres (B,ceil(N/m),2) fp32.
+int launch_cluster_centres(const float* pos, const int64_t* ranking, float* pos_sorted, float* centres, int B, int N, int m,
+                           hipStream_t stream);
+
+// out[b,i,:] = x[b, order[b,i], :] for rows of row_bytes bytes (a multiple of 16); order (B,N) int64, or (N) for
+//   every b when order_shared.
+int launch_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes, int order_shared,
+                       hipStream_t stream);
 int launch_scanline_rank(const float* pos, int64_t* ranking, void* workspace, int B, int N, int rows, int cols,
                          float cell_w, float cell_h, hipStream_t stream);
 

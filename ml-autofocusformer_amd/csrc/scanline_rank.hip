@@ -25,6 +25,8 @@ namespace clusten {
 namespace {
 
 constexpr int kRankBlock = 256;
+// threads of the sorting workgroup: 1024 for long sequences (every step of the network touches P/2 pairs)
+inline int kRankThreads(int P) { return P > 4096 ? 1024 : kRankBlock; }
 
 struct Anchors {
     int rows, cols;
@@ -79,13 +81,13 @@ __global__ __launch_bounds__(kRankBlock) void rank_ratio_kernel(const float2* __
 }
 
 // one workgroup per image: (key bits, token index) pairs sorted in LDS; padding pairs sort last
-__global__ __launch_bounds__(kRankBlock) void rank_sort_kernel(const int* __restrict__ rank, const float* __restrict__ ratio,
+__global__ __launch_bounds__(1024) void rank_sort_kernel(const int* __restrict__ rank, const float* __restrict__ ratio,
                                                                const int* __restrict__ max_bits,
                                                                int64_t* __restrict__ ranking, int N, int P) {
     extern __shared__ uint64_t pairs[];
     const int b = blockIdx.x;
     const float scale = __int_as_float(*max_bits) + 1.f;
-    for (int i = threadIdx.x; i < P; i += kRankBlock) {
+    for (int i = threadIdx.x; i < P; i += blockDim.x) {
         uint64_t v = ~0ull;
         if (i < N) {
             const int64_t e = (int64_t)b * N + i;
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(kRankBlock) void rank_sort_kernel(const int* __rest
     __syncthreads();
     for (int k = 2; k <= P; k <<= 1) {
         for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int t = threadIdx.x; t < P / 2; t += kRankBlock) {
+            for (int t = threadIdx.x; t < P / 2; t += blockDim.x) {
                 const int i = (t / j) * 2 * j + (t % j), l = i + j;
                 const bool up = (i & k) == 0;
                 const uint64_t x = pairs[i], y = pairs[l];
@@ -109,7 +111,7 @@ __global__ __launch_bounds__(kRankBlock) void rank_sort_kernel(const int* __rest
             __syncthreads();
         }
     }
-    for (int i = threadIdx.x; i < N; i += kRankBlock) ranking[(int64_t)b * N + i] = (int64_t)(pairs[i] & 0xffffffffu);
+    for (int i = threadIdx.x; i < N; i += blockDim.x) ranking[(int64_t)b * N + i] = (int64_t)(pairs[i] & 0xffffffffu);
 }
 
 }  // namespace
@@ -129,8 +131,89 @@ int launch_scanline_rank(const float* pos, int64_t* ranking, void* workspace, in
     if (int st = launch_status()) return st;
     int P = 2;
     while (P < N) P <<= 1;
-    hipLaunchKernelGGL(rank_sort_kernel, dim3((unsigned)B), dim3(kRankBlock), (size_t)P * 8, stream, rank, ratio, max_bits,
+    const size_t lds = (size_t)P * 8;
+    if (lds > 48 * 1024) {
+        // more LDS than a workgroup gets without asking (a CU of this device holds 160 KB): 9216 tokens need 128 KB
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(rank_sort_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return CLUSTEN_ERR_BAD_DIMS;
+        }
+    }
+    hipLaunchKernelGGL(rank_sort_kernel, dim3((unsigned)B), dim3(kRankThreads(P)), lds, stream, rank, ratio, max_bits,
                        ranking, N, P);
+    return launch_status();
+}
+
+int scanline_rank_max_tokens() {
+    int dev = 0, bytes = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 4096;
+    }
+    int P = 2;
+    while ((size_t)P * 2 * 8 <= (size_t)bytes) P <<= 1;
+    return P;
+}
+
+// ---- reordered positions and cluster centres --------------------------------------------------------------------
+
+namespace {
+
+// one thread per cluster: its members' positions in ranking order, and their mean
+__global__ __launch_bounds__(256) void cluster_centres_kernel(const float2* __restrict__ pos,
+                                                              const int64_t* __restrict__ ranking,
+                                                              float2* __restrict__ pos_sorted, float2* __restrict__ centres,
+                                                              int N, int m, int K, int64_t clusters) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= clusters) return;
+    const int64_t b = e / K;
+    const int g = (int)(e - b * K);
+    const int first = g * m, count = min(m, N - first);
+    float sx = 0.f, sy = 0.f;
+    for (int t = 0; t < count; ++t) {
+        const float2 p = pos[b * N + ranking[b * N + first + t]];
+        if (pos_sorted != nullptr) pos_sorted[b * N + first + t] = p;
+        sx += p.x;
+        sy += p.y;
+    }
+    centres[e] = make_float2(sx / (float)count, sy / (float)count);
+}
+
+// out[b,i,:] = x[b, order[b,i], :], 16 bytes per lane
+__global__ __launch_bounds__(256) void gather_rows_kernel(const Piece* __restrict__ x, const int64_t* __restrict__ order,
+                                                          Piece* __restrict__ out, int N, int pieces_per_row,
+                                                          int64_t order_batch_stride, int64_t total_pieces) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total_pieces) return;
+    const int64_t row = e / pieces_per_row;
+    const int piece = (int)(e - row * pieces_per_row);
+    const int64_t b = row / N;
+    const int i = (int)(row - b * N);
+    const int64_t src = b * N + order[b * order_batch_stride + i];
+    out[e] = x[src * pieces_per_row + piece];
+}
+
+}  // namespace
+
+int launch_cluster_centres(const float* pos, const int64_t* ranking, float* pos_sorted, float* centres, int B, int N, int m,
+                           hipStream_t stream) {
+    const int K = (N + m - 1) / m;
+    const int64_t clusters = (int64_t)B * K;
+    hipLaunchKernelGGL(cluster_centres_kernel, dim3((unsigned)((clusters + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const float2*>(pos), ranking, reinterpret_cast<float2*>(pos_sorted),
+                       reinterpret_cast<float2*>(centres), N, m, K, clusters);
+    return launch_status();
+}
+
+int launch_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes, int order_shared,
+                       hipStream_t stream) {
+    const int ppr = row_bytes / 16;
+    const int64_t total = B * N * ppr;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<const Piece*>(x), order, static_cast<Piece*>(out), N, ppr,
+                       order_shared ? (int64_t)0 : (int64_t)N, total);
     return launch_status();
 }
 

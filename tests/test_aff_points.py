@@ -145,17 +145,54 @@ def test_ranking_kernel_equals_the_tensor_formulation(device, name):
         p = p.float()
         ref = _scanline_ranking(p, m, h, w)                                  # CPU tensors: the tensor formulation
         rows, cols = _anchor_grid(p.shape[1], m, h, w)
-        if p.shape[1] <= 4096:
-            assert _native.scanline_rank_supported(p.to(device), rows, cols)
-            got = _native.scanline_rank(p.to(device), rows, cols, w / cols, h / rows)
-            assert got.dtype == torch.int64 and torch.equal(got.cpu(), ref)
-        else:   # longer sequences keep the tensor formulation on the GPU
-            assert not _native.scanline_rank_supported(p.to(device), rows, cols)
-        # and through the public function: same clusters on both devices
+        assert _native.scanline_rank_supported(p.to(device), rows, cols)
+        got = _native.scanline_rank(p.to(device), rows, cols, w / cols, h / rows)
+        assert got.dtype == torch.int64 and torch.equal(got.cpu(), ref)
+        # and through the public function: same clusters on both devices (positions in cluster order and cluster
+        # centres come from one kernel on the GPU; the centres of integer positions are exact on both)
         cpu = space_filling_cluster(p, m, h, w)
         gpu = space_filling_cluster(p.to(device), m, h, w)
         assert torch.equal(gpu[4].cpu(), cpu[4]) and torch.equal(gpu[0].cpu(), cpu[0])
         assert torch.allclose(gpu[1].cpu(), cpu[1], rtol=1e-6, atol=1e-6)
-    assert not _native.scanline_rank_supported(torch.zeros(1, 5000, 2, device=device), 10, 10)
+        if float((p - p.round()).abs().max()) == 0.0:
+            assert torch.equal(gpu[1].cpu(), cpu[1])
+        assert (gpu[3] is None) == (cpu[3] is None) and (cpu[3] is None or torch.equal(gpu[3].cpu(), cpu[3]))
+    assert _native.load().clusten_scanline_rank_max_tokens() >= 16384
+    assert not _native.scanline_rank_supported(torch.zeros(1, 40000, 2, device=device), 10, 10)
     with pytest.raises(RuntimeError):
         _native.scanline_rank(pos.float(), 4, 4, 1.0, 1.0)
+
+
+@pytest.mark.gpu
+def test_ranking_kernel_on_the_first_stage_of_a_384_model(device):
+    """9216 tokens on a 96 x 96 grid, clusters of 24 (configs/aff_base_22kto1k_384.yaml:10): the sort of an image takes
+    128 KB of LDS; same order as the tensor formulation, on the grid and on scattered fractional positions."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(24)
+    ys, xs = torch.meshgrid(torch.arange(96), torch.arange(96), indexing="ij")
+    grid = torch.stack([xs, ys], dim=2).reshape(1, -1, 2).float().expand(2, -1, -1).contiguous()
+    scattered = torch.rand(2, 9216, 2, generator=gen) * 95.99
+    for p in (grid, scattered):
+        ref = _scanline_ranking(p, 24, 96, 96)
+        rows, cols = _anchor_grid(9216, 24, 96, 96)
+        assert _native.scanline_rank_supported(p.to(device), rows, cols)
+        got = _native.scanline_rank(p.to(device), rows, cols, 96 / cols, 96 / rows)
+        assert torch.equal(got.cpu(), ref)
+        cpu = space_filling_cluster(p, 24, 96, 96)
+        gpu = space_filling_cluster(p.to(device), 24, 96, 96)
+        assert torch.equal(gpu[0].cpu(), cpu[0]) and torch.allclose(gpu[1].cpu(), cpu[1], rtol=1e-6, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_row_gather_kernel(device, dtype):
+    from clusten import _native
+    gen = torch.Generator().manual_seed(25)
+    for b, n, c in ((3, 196, 256), (2, 784, 128), (1, 50, 8 if dtype == torch.float16 else 4)):
+        x = torch.randn(b, n, c, generator=gen).to(dtype).to(device)
+        order = torch.stack([torch.randperm(n, generator=gen) for _ in range(b)]).to(device)
+        assert _native.gather_rows_supported(x)
+        want = x.gather(1, order.unsqueeze(2).expand(-1, -1, c))
+        assert torch.equal(_native.gather_rows(x, order), want)
+        assert torch.equal(_native.gather_rows(x, order[0]), x[:, order[0]])
+    assert not _native.gather_rows_supported(torch.zeros(1, 4, 3, device=device))
