@@ -152,7 +152,9 @@ int clusten_av_forward(const void* attn,
  * values up first (clusten/clusten.py:52-53).  Here the 16-bit rows are read in place and widened on the way to the
  * staging buffer: the same values and arithmetic as clusten_av_forward on a cast copy (bit-identical results),
  * without that pass over the value tensor.  attn (B,H,N,M) and feat (strided (B,H,N,C)) fp32; value strided (B,H,N,C)
- * of value_dtype, F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE). */
+ * of value_dtype, F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE).  Lists of more than 64 slots that clusten_av_forward hands
+ * to its kernels for long runs (M a multiple of 24, 32 or 16 with at most 8 runs) are turned down with
+ * CLUSTEN_ERR_BAD_DIMS: cast the values and call clusten_av_forward. */
 int clusten_av_forward_mixed(const void* attn,
                              const void* value, clusten_strides value_strides, int value_dtype,
                              const int64_t* nbhd_idx,

@@ -361,19 +361,21 @@ def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, toke
     return feat
 
 
-def mixed_supported(first: torch.Tensor, second: torch.Tensor) -> bool:
+def mixed_supported(first: torch.Tensor, second: torch.Tensor, attention: bool = False) -> bool:
     """True for the operand pair mixed precision hands AV and WF: an fp32 first operand (attention weights, merge
-    weights) and an fp16 / bf16 second one (values, features), both on the GPU."""
+    weights) and an fp16 / bf16 second one (values, features), both on the GPU.  For attention (`attention=True`) lists
+    of more than 64 slots are left to the cast-first path: they have kernels of their own (long runs), and only the
+    same kernel gives the same bits."""
     return (first.is_cuda and second.is_cuda and first.dtype == torch.float32
-            and second.dtype in (torch.float16, torch.bfloat16))
+            and second.dtype in (torch.float16, torch.bfloat16) and (not attention or first.shape[-1] <= 64))
 
 
 def av_forward_mixed(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor) -> torch.Tensor:
     """feat (b,h,n,c) fp32 = attn (fp32) · v[nbhd_idx] with v fp16 / bf16 read in place: bit-identical to
     `av_forward(attn, v.float(), nbhd_idx)` (the cast clusten/clusten.py:52-53 makes) without the copy."""
     lib = load()
-    if not mixed_supported(attn, v):
-        raise RuntimeError("av_forward_mixed takes fp32 attn and fp16 / bf16 v on the GPU")
+    if not mixed_supported(attn, v, attention=True):
+        raise RuntimeError("av_forward_mixed takes fp32 attn of at most 64 slots and fp16 / bf16 v on the GPU")
     device = attn.device
     _require_cuda("v", v, device)
     if attn.dim() != 4 or v.dim() != 4 or nbhd_idx.dim() != 3 or attn.shape[:3] != v.shape[:3]:

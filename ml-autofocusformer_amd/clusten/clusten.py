@@ -53,7 +53,7 @@ class CLUSTENAVFunction(Function):
 
     @staticmethod
     def forward(ctx, attn, v, nbhd_idx):
-        if _native.mixed_supported(attn, v):
+        if _native.mixed_supported(attn, v, attention=True):
             # fp32 weights over 16-bit values (mixed precision): the values are read in place; same result as the cast
             feat = _native.av_forward_mixed(attn, v, nbhd_idx)
         else:

@@ -53,6 +53,7 @@
 
 #include "launch.hpp"
 #include "mfma.hpp"
+#include "gather_runs_impl.hpp"
 
 namespace clusten {
 
@@ -622,6 +623,10 @@ int gather_dot_typed(const void* a, clusten_strides as, const void* rows, cluste
     const bool vec_ok = rows_aligned16(rows, rs, sizeof(T)) && rows_aligned16(a, as, sizeof(T)) && aligned16(out) &&
                         slice_fits_int32(rs, s.H, s.N, s.C) && slice_fits_int32(as, s.H, s.N, s.C);
     if (vec_ok) {
+        // long lists made of long runs (the 384 x 384 models: 6 clusters of 24 tokens)
+        if (const int L = runs_length_for(s.M); L != 0 && runs_head_dim_ok<T>(s.C)) {
+            return launch_gather_dot_runs<T>(a, as, rows, rs, idx, out, s, L, stream);
+        }
         switch (s.C) {
             case 16: return launch_tile<T, 16>(a, as, rows, rs, idx, out, s, stream);
             case 32: return launch_tile<T, 32>(a, as, rows, rs, idx, out, s, stream);

@@ -49,6 +49,7 @@
 
 #include "launch.hpp"
 #include "mfma.hpp"
+#include "gather_runs_impl.hpp"
 
 namespace clusten {
 
@@ -692,6 +693,10 @@ int gather_sum_typed(const void* p, const void* rows, clusten_strides rs, const 
     const bool quads_ok = ((int64_t)s.M * sizeof(T)) % 16 == 0 && aligned16(p) && rows_aligned16(rows, rs, sizeof(T)) &&
                           rows_aligned16(out, os, sizeof(T)) && slice_fits_int32(rs, s.H, s.N, s.C);
     if (quads_ok) {
+        // long lists made of long runs (the 384 x 384 models: 6 clusters of 24 tokens)
+        if (const int L = runs_length_for(s.M); L != 0 && runs_head_dim_ok<T>(s.C)) {
+            return launch_gather_sum_runs<T>(p, rows, rs, idx, out, os, s, L, stream);
+        }
         switch (s.C) {
             case 16: return launch_tile<T, 16>(p, rows, rs, idx, out, os, s, stream);
             case 32: return launch_tile<T, 32>(p, rows, rs, idx, out, os, s, stream);
@@ -734,6 +739,9 @@ int gather_sum_mixed_typed(const void* p, const void* rows, clusten_strides rs, 
                        (rs.n * 2) % 8 == 0;
     const bool quads_ok = ((int64_t)s.M * 4) % 16 == 0 && aligned16(p) && rows8 && rows_aligned16(out, os, 4) &&
                           slice_fits_int32(rs, s.H, s.N, s.C);
+    // long lists made of long runs have kernels of their own for rows of the weights' type only: a result that equals
+    // the cast-first path bit for bit needs the same kernel, so such a call is turned down (the caller casts)
+    if (runs_length_for(s.M) != 0 && runs_head_dim_ok<float>(s.C)) return CLUSTEN_ERR_BAD_DIMS;
     if (quads_ok) {
         switch (s.C) {
             case 16: return launch_tile<float, 16, TR>(p, rows, rs, idx, out, os, s, stream);

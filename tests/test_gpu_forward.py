@@ -105,6 +105,60 @@ def test_list_lengths(device, m):
     _check_attn(wl.attn_case("m%d" % m, 55, B=2, H=2, N=320, C=32, M=m), device, torch.float32)
 
 
+def _cluster_lists(B, N, cluster, nnc, gen, kind="model"):
+    """Lists of nnc runs of `cluster` slots: the members of a token's nearest clusters ("model", nearest first, as the
+    reference builds them), with the short last cluster padded by row 0 ("padded"), with runs of other rows mixed in
+    ("irregular": some runs are not consecutive rows, one token repeats a run), or runs scattered over the whole sequence
+    so that a tile holds more distinct runs than the kernel keeps ("scattered")."""
+    if kind == "model":
+        return wl.model_like_lists(B, N, gen, cluster=cluster, nnc=nnc)
+    K = (N + cluster - 1) // cluster
+    own = torch.arange(N) // cluster
+    if kind == "scattered":
+        pick = torch.rand(B, N, K, generator=gen).argsort(dim=2)[:, :, :nnc]
+    else:
+        lo = (own - 4).clamp(min=0, max=max(K - 9, 0))
+        pick = torch.rand(B, N, min(9, K), generator=gen).argsort(dim=2)[:, :, :nnc] + lo.view(1, N, 1)
+    rows = pick.unsqueeze(3) * cluster + torch.arange(cluster)
+    idx = torch.where(rows < N, rows, torch.zeros_like(rows)).reshape(B, N, nnc * cluster)
+    if kind == "irregular":
+        idx[:, 5::7, cluster:2 * cluster] = torch.randint(N, (B, len(range(5, N, 7)), cluster), generator=gen)
+        idx[:, 3::11, 2 * cluster:3 * cluster] = idx[:, 3::11, :cluster]            # a run held twice by one token
+        idx[:, 2::13, 0] = idx[:, 2::13, 1]                                         # a duplicate inside a run
+    return idx
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["model", "padded", "irregular", "scattered"])
+def test_long_lists_made_of_long_runs(device, dtype, kind):
+    """The neighbourhoods of the 384 x 384 models (configs/aff_base_22kto1k_384.yaml:10-11): 6 clusters of 24 tokens, 144
+    slots — and other run lengths the kernels for long runs take (32, 16)."""
+    g = torch.Generator().manual_seed(57)
+    for N, cluster, nnc, C, H in ((2304, 24, 6, 32, 2), (600, 24, 6, 64, 1), (400, 32, 4, 32, 3), (328, 16, 5, 32, 2)):
+        if kind == "model" and N % cluster:
+            N -= N % cluster
+        if kind != "padded" and kind != "model":
+            N -= N % 8
+        idx = _cluster_lists(1 if N > 1000 else 2, N, cluster, nnc, g, kind)
+        case = wl.attn_case("runs%d" % cluster, 58, B=idx.shape[0], H=H, N=N, C=C, M=idx.shape[-1], lists="random")
+        case.nbhd_idx = idx
+        _check_attn(case, device, dtype)
+
+
+def test_long_runs_integer_valued_data_is_bit_exact(device):
+    g = torch.Generator().manual_seed(59)
+    N, H, C = 960, 2, 32
+    for kind in ("model", "padded", "irregular", "scattered"):
+        idx = _cluster_lists(2, N, 24, 6, g, kind)
+        q = torch.randint(-4, 5, (2, H, N, C), generator=g).float()
+        k = torch.randint(-4, 5, (2, H, N, C), generator=g).float()
+        p = torch.randint(-3, 4, (2, H, N, 144), generator=g).float()
+        assert torch.equal(_native.qk_forward(q.to(device), k.to(device), idx.to(device)).cpu(),
+                           oracle.qk_gather_chunked(q, k, idx)), kind
+        assert torch.equal(_native.av_forward(p.to(device), k.to(device), idx.to(device)).cpu(),
+                           oracle.av_gather_chunked(p, k, idx)), kind
+
+
 @pytest.mark.parametrize("h", [1, 3, 5, 16])
 def test_head_counts(device, h):
     _check_attn(wl.attn_case("h%d" % h, 56, B=2, H=h, N=104, C=32), device, torch.float32)

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("lists", ["windowed", "model", "random", "runs:padded", "runs:repeated"])
 def test_av_mixed_equals_the_cast_first_path(device, dtype, lists):
     g = torch.Generator().manual_seed(40)
-    for B, H, N, C, M in ((2, 2, 200, 32, 48), (1, 3, 104, 16, 48), (2, 2, 136, 64, 32), (1, 2, 77, 32, 20), (1, 2, 160, 32, 144),
+    for B, H, N, C, M in ((2, 2, 200, 32, 48), (1, 3, 104, 16, 48), (2, 2, 136, 64, 32), (1, 2, 77, 32, 20), (1, 2, 160, 32, 64),
                           (2, 1, 50, 24, 8)):
         if lists == "model" and (M != 48 or N % 8):
             continue
@@ -34,6 +34,19 @@ def test_av_mixed_equals_the_cast_first_path(device, dtype, lists):
         assert torch.equal(got, want), (lists, B, H, N, C, M)
         ref = oracle.av_gather(attn.cpu(), v.float().cpu(), case.nbhd_idx)
         assert oracle.rel_err(got, ref) <= TOL[torch.float32]
+
+
+def test_av_mixed_leaves_long_lists_to_the_cast_first_path(device):
+    from clusten import CLUSTENAVFunction
+    g = torch.Generator().manual_seed(48)
+    case = wl.attn_case("mixed", 49, B=1, H=2, N=160, C=32, M=144)
+    v = case.value.half().to(device)
+    attn = torch.softmax(torch.randn(1, 2, 160, 144, generator=g), dim=-1).to(device)
+    idx = case.nbhd_idx.to(device)
+    assert not _native.mixed_supported(attn, v, attention=True)
+    with pytest.raises(RuntimeError):
+        _native.av_forward_mixed(attn, v, idx)
+    assert torch.equal(CLUSTENAVFunction.apply(attn, v, idx), _native.av_forward(attn, v.float(), idx))
 
 
 def test_av_mixed_reads_strided_values_in_place(device):
