@@ -92,30 +92,32 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* scratch, int* to
     return before + inc - v;
 }
 
-// One workgroup per image.  E entries (i, r) of the image in the order e = i*R + r; K clusters; `cap` entries of
-// `pairs` per image (2E when the sequence ends in a short cluster, else E).
-__global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __restrict__ keys,
-                                                            const int32_t* __restrict__ wg_bad, int n_wg_bad,
-                                                            int32_t* __restrict__ not_whole,
-                                                            int32_t* __restrict__ pairs, int32_t* __restrict__ starts,
-                                                            int32_t* __restrict__ ends, int E, int R, int K, int cap,
-                                                            int pad, int key_bits) {
-    {
-        // what the workgroups of the keys kernel found, added up by every workgroup here for itself; the first one
-        // writes the flag the later kernels read
-        int bad = 0;
-        for (int z = threadIdx.x; z < n_wg_bad; z += blockDim.x) bad |= wg_bad[z];
-        bad = __syncthreads_or(bad);
-        if (blockIdx.x == 0 && threadIdx.x == 0) *not_whole = bad ? 1 : 0;
-        if (bad) return;
-    }
+// The stable counting sort of one image by one workgroup.  E entries in the order e = 0 .. E-1, K keys; the sorted
+// entries go to `pairs` (cap per image), the bounds of every key's list to starts / ends.
+//   ROWS = false: keys[e] = cluster number of run e = i*R + r, entry = i*8 + r; `pad`: the pairs of the short last
+//                 cluster are listed again, flagged, under cluster 0;
+//   ROWS = true:  keys64[e] = destination row of list entry e (any row: entries outside [0, K) are left out),
+//                 entry = e.
+template <bool ROWS>
+__device__ __forceinline__ void sort_image(const void* __restrict__ keys_any, int32_t* __restrict__ pairs,
+                                           int32_t* __restrict__ starts, int32_t* __restrict__ ends, int E, int R, int K,
+                                           int cap, int pad, int key_bits) {
     extern __shared__ int32_t lds[];
     const int W = blockDim.x >> 6, w = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int* hist = lds;              // [W][K]: count, then the start inside the key's list, of wave w's entries of key k
     int* base = lds + W * K;      // [K]: the key's total, then the start of its list inside the image
     int* scratch = base + K;      // [W]
     const int b = blockIdx.x;
-    const int32_t* my_keys = keys + (int64_t)b * E;
+    const int32_t* keys32 = static_cast<const int32_t*>(keys_any) + (int64_t)b * E;
+    const int64_t* keys64 = static_cast<const int64_t*>(keys_any) + (int64_t)b * E;
+    auto key_of = [&](int e) -> int {
+        if constexpr (ROWS) {
+            const int64_t row = keys64[e];
+            return (row >= 0 && row < K) ? (int)row : -1;
+        } else {
+            return keys32[e];
+        }
+    };
     const int share = (((E + W - 1) / W + 63) / 64) * 64;   // entries per wave, in whole steps of 64
     const int lo = min(E, w * share), hi = min(E, lo + share);
 
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __res
     for (int e0 = lo; e0 < hi; e0 += 4 * 64) {
         int k4[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) k4[u] = e0 + 64 * u + lane < hi ? my_keys[e0 + 64 * u + lane] : -1;
+        for (int u = 0; u < 4; ++u) k4[u] = e0 + 64 * u + lane < hi ? key_of(e0 + 64 * u + lane) : -1;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             if (k4[u] >= 0) atomicAdd(&hist[w * K + k4[u]], 1);
@@ -164,13 +166,13 @@ __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __res
     for (int e00 = lo; e00 < hi; e00 += 4 * 64) {
         int k4[4];    // four steps' keys requested together
 #pragma unroll
-        for (int u = 0; u < 4; ++u) k4[u] = e00 + 64 * u + lane < hi ? my_keys[e00 + 64 * u + lane] : -1;
+        for (int u = 0; u < 4; ++u) k4[u] = e00 + 64 * u + lane < hi ? key_of(e00 + 64 * u + lane) : -1;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = e00 + 64 * u + lane;
             const int k = k4[u];
             const bool valid = k >= 0;
-            const int entry = (e / R) * 8 + e % R;
+            const int entry = ROWS ? e : (e / R) * 8 + e % R;
             // the lanes of this step that hold the lane's key: one ballot per bit of the key
             uint64_t same = __ballot(valid);
             for (int bit = 0; bit < key_bits; ++bit) {
@@ -191,6 +193,34 @@ __global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __res
             }
         }
     }
+}
+
+// One workgroup per image: the pair lists of lists made of whole clusters.
+__global__ __launch_bounds__(1024) void cluster_sort_kernel(const int32_t* __restrict__ keys,
+                                                            const int32_t* __restrict__ wg_bad, int n_wg_bad,
+                                                            int32_t* __restrict__ not_whole,
+                                                            int32_t* __restrict__ pairs, int32_t* __restrict__ starts,
+                                                            int32_t* __restrict__ ends, int E, int R, int K, int cap,
+                                                            int pad, int key_bits) {
+    {
+        // what the workgroups of the keys kernel found, added up by every workgroup here for itself; the first one
+        // writes the flag the later kernels read
+        int bad = 0;
+        for (int z = threadIdx.x; z < n_wg_bad; z += blockDim.x) bad |= wg_bad[z];
+        bad = __syncthreads_or(bad);
+        if (blockIdx.x == 0 && threadIdx.x == 0) *not_whole = bad ? 1 : 0;
+        if (bad) return;
+    }
+    sort_image<false>(keys, pairs, starts, ends, E, R, K, cap, pad, key_bits);
+}
+
+// One workgroup per image: the entries (i, j) of any list tensor by destination row, for the lists that are not made
+// of whole clusters (`only_if`, may be null: a device flag; nothing happens when it points to zero).
+__global__ __launch_bounds__(1024) void row_sort_kernel(const int64_t* __restrict__ idx, const int32_t* __restrict__ only_if,
+                                                        int32_t* __restrict__ entries, int32_t* __restrict__ starts,
+                                                        int32_t* __restrict__ ends, int E, int K, int key_bits) {
+    if (only_if != nullptr && *only_if == 0) return;
+    sort_image<true>(idx, entries, starts, ends, E, 1, K, E, 0, key_bits);
 }
 
 }  // namespace
@@ -243,6 +273,55 @@ int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int
     while ((1 << key_bits) < K) ++key_bits;
     hipLaunchKernelGGL(cluster_sort_kernel, dim3(B), dim3(64 * waves), lds, stream, keys, wg_bad, n_wg, not_whole, pairs,
                        starts, ends, (int)E, R, K, cap, (D % 8) ? 1 : 0, key_bits);
+    return launch_status();
+}
+
+// ---- entries of any list tensor by destination row ---------------------------------------------------------------
+
+namespace {
+constexpr int kRowSortLdsBytes = 150 * 1024;   // of the 160 KB of a compute unit
+inline int row_sort_waves(int K, int64_t E) {
+    int waves = (kRowSortLdsBytes / 4 - 16) / K - 1;
+    waves = waves > 16 ? 16 : waves;
+    const int64_t steps = (E + 63) / 64;
+    if (waves > steps) waves = (int)steps;
+    return waves;
+}
+}  // namespace
+
+bool row_entries_supported(int B, int rows, int M, int D) {
+    if (B <= 0 || rows <= 0 || M <= 0 || D <= 0) return false;
+    const int64_t E = (int64_t)rows * M;
+    if (E >= ((int64_t)1 << 30) || E * B >= ((int64_t)1 << 31) || (int64_t)B * D >= ((int64_t)1 << 30)) return false;
+    return row_sort_waves(D, E) >= 1;
+}
+
+RowEntriesLayout row_entries_layout(int B, int rows, int M, int D) {
+    RowEntriesLayout l;
+    auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+    l.entries = 0;
+    l.starts = up((size_t)B * rows * M * 4);
+    l.ends = l.starts + up((size_t)B * D * 4);
+    l.bytes = l.ends + up((size_t)B * D * 4);
+    return l;
+}
+
+int launch_row_entries(const int64_t* idx, const int32_t* only_if, int32_t* entries, int32_t* starts, int32_t* ends, int B,
+                       int rows, int M, int D, hipStream_t stream) {
+    const int64_t E = (int64_t)rows * M;
+    const int waves = row_sort_waves(D, E);
+    const size_t lds = ((size_t)(waves + 1) * D + 16) * 4;
+    int key_bits = 0;
+    while ((1 << key_bits) < D) ++key_bits;
+    if (lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(row_sort_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return CLUSTEN_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(row_sort_kernel, dim3(B), dim3(64 * waves), lds, stream, idx, only_if, entries, starts, ends, (int)E, D,
+                       key_bits);
     return launch_status();
 }
 

@@ -87,6 +87,23 @@ bool cluster_pairs_supported(int B, int rows, int M, int D);
 ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D);
 int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int32_t* not_whole, int32_t* pairs,
                          int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream);
+// The entries (i, j) of a list tensor (B, rows, M) by the row of the D-row sequence they name, built on the device
+//   (cluster_pairs.hip): entries[starts[b*D+n] .. ends[b*D+n]) holds e = i*M + j for every idx[b,i,j] = n, ascending.
+//   `only_if` (may be null): device flag; nothing is done when it points to zero.  Sizes as row_entries_layout() gives
+//   them (byte offsets into one 16-byte aligned block).
+struct RowEntriesLayout {
+    size_t entries, starts, ends, bytes;
+};
+bool row_entries_supported(int B, int rows, int M, int D);
+RowEntriesLayout row_entries_layout(int B, int rows, int M, int D);
+int launch_row_entries(const int64_t* idx, const int32_t* only_if, int32_t* entries, int32_t* starts, int32_t* ends, int B,
+                       int rows, int M, int D, hipStream_t stream);
+// d_feat[b,n,:] = sum over the entries (i,j) of row (b,n) of sum_ic w[b,i,j,ic] * d_out[b,i,ic,:]: see wf_dfeat_rows.hip.
+bool wf_dfeat_rows_supported(const void* d_out, const void* d_feat, const clusten_wf_shape& s, int dtype);
+int launch_wf_dfeat_rows(const void* d_out, const void* w, const int32_t* starts, const int32_t* ends,
+                         const int32_t* entries, const int32_t* only_if, void* d_feat, clusten_wf_shape s, int dtype,
+                         hipStream_t stream);
+
 // y[b,h,8g+t,:] = sum over the listed pairs (i,r) of cluster (b,g) of p[b,h,i,8r+t] * x[b,h,i,:]: see scatter_by_cluster.hip.
 //   C in {16,32,64}.  `not_whole` (may be null): device flag; the kernel does nothing when it points to non-zero.
 bool scatter_by_cluster_supported(const void* p, const void* x, clusten_strides xs, const void* y,

@@ -46,17 +46,23 @@ namespace {
 // See ScatterPlan in scatter_rows.hip: pair lists first (when the shape admits the cluster-by-cluster kernel), then
 // the fp32 sums of 16-bit data.
 struct DfeatPlan {
-    bool by_cluster;
+    bool by_cluster;            // lists made of whole clusters (found out on the device): gather over sorted pair lists
+    bool by_row;                // any other list: gather over the entries sorted by destination row
     ClusterPairsLayout pairs;
-    size_t acc32;
+    RowEntriesLayout rows;
+    size_t rows_at;             // offset of the row entries block
+    size_t acc32;               // offset of the fp32 buffer of the atomic kernels (16-bit data, shapes by_row does not take)
     size_t bytes;
 };
 
 DfeatPlan dfeat_plan(const clusten_wf_shape& s, int dtype) {
     DfeatPlan plan;
     plan.by_cluster = dtype != CLUSTEN_F64 && s.IC == 4 && s.C % 32 == 0 && cluster_pairs_supported(s.B, s.Nout, s.M, s.N);
+    plan.by_row = dtype != CLUSTEN_F64 && s.IC <= 4 && s.C % 4 == 0 && row_entries_supported(s.B, s.Nout, s.M, s.N);
     plan.pairs = plan.by_cluster ? cluster_pairs_layout(s.B, s.Nout, s.M, s.N) : ClusterPairsLayout{};
-    plan.acc32 = plan.by_cluster ? plan.pairs.bytes : 0;
+    plan.rows = plan.by_row ? row_entries_layout(s.B, s.Nout, s.M, s.N) : RowEntriesLayout{};
+    plan.rows_at = plan.by_cluster ? plan.pairs.bytes : 0;
+    plan.acc32 = plan.rows_at + (plan.by_row ? plan.rows.bytes : 0);
     const bool narrow = dtype == CLUSTEN_F16 || dtype == CLUSTEN_BF16;
     plan.bytes = plan.acc32 + (narrow ? (size_t)s.B * s.N * s.C * sizeof(float) : 0);
     return plan;
@@ -88,6 +94,17 @@ int launch_wf_dfeat(const void* d_out, const void* w, const int64_t* idx, void* 
         if (st != CLUSTEN_OK) return st;
         flag = not_whole;
     }
+    // any other list: the entries sorted by destination row, one wave per row (these kernels return at once when the
+    // flag says the lists were whole clusters)
+    if (plan.by_row && wf_dfeat_rows_supported(d_out, d_feat, s, dtype)) {
+        int32_t* entries = reinterpret_cast<int32_t*>(ws + plan.rows_at + plan.rows.entries);
+        int32_t* rstarts = reinterpret_cast<int32_t*>(ws + plan.rows_at + plan.rows.starts);
+        int32_t* rends = reinterpret_cast<int32_t*>(ws + plan.rows_at + plan.rows.ends);
+        st = launch_row_entries(idx, flag, entries, rstarts, rends, s.B, s.Nout, s.M, s.N, stream);
+        if (st != CLUSTEN_OK) return st;
+        return launch_wf_dfeat_rows(d_out, w, rstarts, rends, entries, flag, d_feat, s, dtype, stream);
+    }
+    // shapes neither takes (and fp64): atomics
     switch (dtype) {
         case CLUSTEN_F32:
             st = launch_zero_f32(static_cast<float*>(d_feat), count, stream, flag);

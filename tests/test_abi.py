@@ -115,8 +115,10 @@ def test_workspace_contract():
     assert lib.clusten_qk_backward(FAKE, FAKE, rows, FAKE, rows, FAKE, FAKE, FAKE, FAKE, need - 1, s, 1, P(0)) == 5
     w = _wshape(B=2, N=16, Nout=4, C=64, M=8, IC=4)
     wpairs = lib.clusten_cluster_pairs_bytes(2, 4, 8, 16)
-    assert lib.clusten_wf_backward_workspace_bytes(w, 0) == wpairs
-    assert lib.clusten_wf_backward_workspace_bytes(w, 2) == wpairs + 2 * 16 * 64 * 4
+    wf32 = lib.clusten_wf_backward_workspace_bytes(w, 0)
+    assert wf32 >= wpairs + 2 * 4 * 8 * 4 + 2 * 2 * 16 * 4              # pair lists, then the entries by destination row
+    assert lib.clusten_wf_backward_workspace_bytes(w, 2) == wf32 + 2 * 16 * 64 * 4
+    assert lib.clusten_wf_backward_workspace_bytes(w, 3) == 0          # fp64: atomics straight into d_feat
     assert lib.clusten_wf_backward(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, P(0), 0, w, 2, P(0)) == 5
 
 

@@ -280,6 +280,37 @@ def test_wf_cluster_by_cluster_properties(device):
     _check_wf_backward(case1, device, torch.float32)
 
 
+def test_wf_feature_gradient_on_any_list_is_a_gather_in_a_fixed_order(device):
+    """Lists that are not made of whole clusters (nearest-neighbour lists, random lists): the entries are sorted by the
+    row they name on the device and every row is summed by one wave in ascending entry order — two runs give the same
+    bits, integer-valued data the oracle's bits, rows nobody lists zeros, and a row half the entries name the right sum."""
+    g = torch.Generator().manual_seed(94)
+    case = wl.wf_case("knn", 95, B=3, N=200, C=64, IC=4)
+    d_out = torch.randn(3, 50, 4, 64, generator=g)
+    args = [t.to(device) for t in (d_out, case.weights, case.feat, case.nbhd_idx)]
+    first = _native.wf_backward(*args)[1]
+    for _ in range(3):
+        assert torch.equal(_native.wf_backward(*args)[1], first)
+    assert oracle.rel_err(first, oracle.wf_gather_backward(d_out, case.weights, case.feat, case.nbhd_idx)[1]) <= 1e-5
+    # integer-valued data, random lists with repeats, odd sizes, fewer inner channels
+    for B, N, Nout, C, IC, M in ((2, 77, 19, 32, 4, 20), (1, 130, 40, 96, 3, 48), (2, 64, 16, 128, 1, 7)):
+        idx = torch.randint(N, (B, Nout, M), generator=g)
+        idx[:, :, 0] = 5                                               # every output token names row 5
+        w = torch.randint(-3, 4, (B, Nout, M, IC), generator=g).float()
+        f = torch.randint(-3, 4, (B, N, C), generator=g).float()
+        d2 = torch.randint(-3, 4, (B, Nout, IC, C), generator=g).float()
+        dw_ref, df_ref = oracle.wf_gather_backward(d2, w, f, idx)
+        dw, df = _native.wf_backward(d2.to(device), w.to(device), f.to(device), idx.to(device))
+        assert torch.equal(dw.cpu(), dw_ref) and torch.equal(df.cpu(), df_ref), (B, N, Nout, C, IC, M)
+    # rows nobody lists are zero; 16-bit data is summed in fp32 and rounded once
+    idx = torch.randint(100, 200, (2, 50, 48), generator=g)
+    w16, f16, d16 = case.weights[:2].half(), case.feat[:2].half(), d_out[:2].half()
+    got = _native.wf_backward(d16.to(device), w16.to(device), f16.to(device), idx.to(device))[1]
+    want = oracle.wf_gather_backward(d16.float(), w16.float(), f16.float(), idx)[1]
+    assert float(got[:, :100].float().abs().max()) == 0.0
+    assert oracle.rel_err(got, want.half().float()) <= 2e-3 * 0.51
+
+
 def test_scatter_union_path_is_bit_exact_on_integer_data(device):
     g = torch.Generator().manual_seed(78)
     B, H, N, C = 2, 3, 200, 32
