@@ -574,6 +574,14 @@ def main():
             "one_kernel_us": round(per_a[0] * 1e3, 1), "three_kernels_us": round(per_a[1] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
         del mcase, cidx, mattn, q16, k16, v16, pe_idx
+        # the first stage of the 384 x 384 models as the reference model builds its lists there: clusters of 24 tokens,
+        # the members of the 6 nearest clusters = 144 slots (configs/aff_base_22kto1k_384.yaml:10-11), B = 16
+        for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            gen384 = wl.generator(31)
+            c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
+            c384.nbhd_idx = wl.model_like_lists(16, 9216, gen384, cluster=24, nnc=6)
+            other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
+        del c384
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
         other["cfg2_s1_backward_fp32_model_like_lists"] = _bench_backward(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), wcase, max(args.steps // 5, 5), 3)
