@@ -388,7 +388,7 @@ def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
             "batch": batch, "warmup": warmup, "timed": timed,
             "dtype": "fp16 autocast (attention: one fp16 kernel per layer, fp32 sums; WF fp32)",
             "inference_path": "16-bit weight copies, position-bias tables and merge-weight tables kept between "
-                              "forwards; layer norm (with the residual addition ahead of it), merge weights, kNN, token "
+                              "forwards; layer norm (with the residual addition ahead of it), merge centres and the rows at them, merge weights, kNN, token "
                               "ranking, neighbour lists, local and global attention, the small Linear layers of stage 1 "
                               "and the patch embedding's epilogues through the HIP library's optional entry points",
             "share_of_forward": share}

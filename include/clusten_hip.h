@@ -488,6 +488,35 @@ int clusten_cluster_centres(const float* pos, const int64_t* ranking, float* pos
 int clusten_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes,
                         int order_shared, clusten_stream stream);
 
+/* The merge centres of the adaptive down-sampling (`ClusterMerging.forward`, models/aff_transformer.py:296-334):
+ *   prior   = 1 where both coordinates of the token are multiples of its grid spacing, else 0; the spacing is
+ *             `stride` when min_dist is NULL (:297), else 2^(ceil(log2(min_dist)) + 1) per token (:299-303)
+ *   score   = prior + learned_prob * alpha (product rounded in prob_dtype, :306-309; skipped when learned_prob is NULL)
+ *             + (-100 where both coordinates are multiples of 2*stride, when reserve_on, :312-315)
+ *   centre[b, 0 .. sample_num)                = the sample_num tokens of image b with the highest score (:320)
+ *   centre[b, sample_num .. +reserve_num)     = with reserve_on, the tokens on that coarse grid, ascending index (:323)
+ * `topk(sorted=False)` leaves the order of the sampled tokens open; here it is fixed: the tokens whose score is above
+ * the sample_num-th highest by ascending index, then as many of those equal to it as are needed, by ascending index.
+ * pos (B,N,2) fp32, 8-byte aligned; min_dist (B,N) fp32 or NULL; learned_prob (B,N) of prob_dtype or NULL; centre
+ * (B, sample_num + (reserve_on ? reserve_num : 0)) int64.  An image must hold at least reserve_num tokens on the coarse
+ * grid (the reference's reshape demands exactly that many); further ones are left out.  0 < sample_num, sample_num
+ * [+ reserve_num] <= N <= clusten_merge_centres_max_tokens(), else CLUSTEN_ERR_BAD_DIMS.  No counterpart in the
+ * reference's extension modules. */
+int clusten_merge_centres_max_tokens(void);
+int clusten_merge_centres(const float* pos, const float* min_dist, const void* learned_prob, int prob_dtype,
+                          int64_t* centre, int B, int N, int sample_num, int reserve_num, int reserve_on, float alpha,
+                          int stride, clusten_stream stream);
+
+/* The rows of up to four per-token tensors at the merge centres in one launch (the `gather` calls of
+ * models/aff_transformer.py:337-344 on pos, member_idx, pe_idx and cluster_mask):
+ *   dst[t][b,i,:] = src[t][b, centre[b,i], :]      t < count, 1 <= count <= 4
+ * src[t] (B,N,.) and dst[t] (B,n_out,.) contiguous with rows of row_bytes[t] bytes, a multiple of 8 (else
+ * CLUSTEN_ERR_BAD_DIMS), 8-byte aligned (else CLUSTEN_ERR_UNALIGNED); src, dst and row_bytes are host arrays of
+ * `count` entries; centre (B,n_out) int64 with values in [0,N) — unchecked.  No counterpart in the reference's
+ * extension modules. */
+int clusten_merge_rows(const void* const* src, void* const* dst, const int* row_bytes, int count,
+                       const int64_t* centre, int64_t B, int N, int n_out, clusten_stream stream);
+
 /* ---- producer of the neighbourhood lists (optional) ------------------------------------------- */
 
 /* K nearest neighbours of 2-D points inside each batch element: for query point q of batch element b,

@@ -51,7 +51,9 @@ def default_ops():
                            attn_softmax_backward=_native.attn_softmax_backward,
                            neighbour_lists=_native.neighbour_lists,
                            neighbour_lists_supported=_native.neighbour_lists_supported,
-                           gather_rows=_native.gather_rows, gather_rows_supported=_native.gather_rows_supported)
+                           gather_rows=_native.gather_rows, gather_rows_supported=_native.gather_rows_supported,
+                           merge_centres=_native.merge_centres, merge_centres_supported=_native.merge_centres_supported,
+                           merge_rows=_native.merge_rows, merge_rows_supported=_native.merge_rows_supported)
 
 
 def _cast_params(lin, dt):
@@ -392,6 +394,12 @@ class ClusterMerging(nn.Module):
         """Indices (b, n') of the tokens kept as merge centres (aff_transformer.py:296-334)."""
         b, n, _ = pos.shape
         keep = int(n * self.ds_rate)
+        one_pass = getattr(self.ops, "merge_centres", None)
+        if one_pass is not None and self.ops.merge_centres_supported(pos, learned_prob):
+            # scores, selection and the reserved tokens in one kernel; among equal scores at the cut the lower index
+            dist = None if stride == 2 else knn(pos, pos, 2, return_dist=True)[1][:, :, 1]
+            return one_pass(pos, dist, learned_prob, float(self.alpha), stride,
+                            keep - reserve_num if self.reserve_on else keep, reserve_num, self.reserve_on)
         if stride == 2:                      # tokens still fill the grid: every other row and column
             prior = ((pos % stride).sum(-1) == 0).float()
         else:                                # adaptive grid: spacing from the distance to the nearest other token
@@ -418,23 +426,34 @@ class ClusterMerging(nn.Module):
         centre = self.select(pos, learned_prob, stride, reserve_num)                     # (b, n')
         n_out = centre.shape[1]
         assert n_out == int(n * self.ds_rate), "number of merge centres"
-        pos = pos.gather(1, centre.unsqueeze(2).expand(-1, -1, pos.shape[2]))
-        rows = centre.unsqueeze(2).expand(-1, -1, m)
-        member_idx = member_idx.gather(1, rows)                                          # (b, n', m)
-        pe_idx = pe_idx.gather(1, rows)
+        rows_op = getattr(self.ops, "merge_rows", None)
+        mask_rows = None
+        if rows_op is not None and self.ops.merge_rows_supported(pos, member_idx, pe_idx):
+            # the rows of the per-token tensors at the centres in one launch
+            if cluster_mask is not None and self.ops.merge_rows_supported(cluster_mask):
+                pos, member_idx, pe_idx, mask_rows = rows_op(centre, pos, member_idx, pe_idx, cluster_mask)
+            else:
+                pos, member_idx, pe_idx = rows_op(centre, pos, member_idx, pe_idx)
+            rows = centre.unsqueeze(2).expand(-1, -1, m)
+        else:
+            pos = pos.gather(1, centre.unsqueeze(2).expand(-1, -1, pos.shape[2]))
+            rows = centre.unsqueeze(2).expand(-1, -1, m)
+            member_idx = member_idx.gather(1, rows)                                      # (b, n', m)
+            pe_idx = pe_idx.gather(1, rows)
+        if cluster_mask is not None and mask_rows is None:
+            mask_rows = cluster_mask.gather(1, rows)
         table_w = _table_function(self, "_weight_table_cache", self.weight_net, table,
                                   lambda: self.weight_net(table))                         # (rows, 4)
         one_pass = getattr(self.ops, "merge_weights", None)
         if one_pass is not None and not torch.is_grad_enabled() and self.ops.merge_weights_supported(table_w):
             # inference: lookup, importance of each neighbour and mask in one kernel
-            weights = one_pass(table_w, pe_idx, member_idx, learned_prob,
-                               None if cluster_mask is None else cluster_mask.gather(1, rows))
+            weights = one_pass(table_w, pe_idx, member_idx, learned_prob, mask_rows)
         else:
             weights = _table_rows(table_w, pe_idx)                                       # (b, n', m, 4)
             if learned_prob is not None:
                 weights = weights * learned_prob.gather(1, member_idx.reshape(b, -1, 1)).reshape(b, n_out, m, 1)
             if cluster_mask is not None:
-                weights = weights * cluster_mask.gather(1, rows).unsqueeze(3)
+                weights = weights * mask_rows.unsqueeze(3)
         merged = self.ops.wf(weights, feat, member_idx).reshape(b, n_out, -1)            # channel = ic * c + c'
         return pos, _linear(self.linear, _layer_norm(self.norm, merged, self.ops, True), self.ops)
 

@@ -88,6 +88,10 @@ _PROTOTYPES = {
     "clusten_scanline_rank_max_tokens": (ctypes.c_int, []),
     "clusten_cluster_centres": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_gather_rows": (ctypes.c_int, [_P, _P, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_merge_centres_max_tokens": (ctypes.c_int, []),
+    "clusten_merge_centres": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_int, _P]),
+    "clusten_merge_rows": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, _P, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _P]),
     "clusten_scanline_rank_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
     "clusten_scanline_rank": (ctypes.c_int, [_P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                             ctypes.c_int, ctypes.c_float, ctypes.c_float, _P]),
@@ -1176,6 +1180,87 @@ def gather_rows(x: torch.Tensor, order: torch.Tensor) -> torch.Tensor:
         _check(lib.clusten_gather_rows(_ptr(x), _ptr(order), _ptr(out), b, n, c * x.element_size(), int(shared),
                                        _stream(device)), "clusten_gather_rows")
     return out
+
+
+def merge_centres_supported(pos: torch.Tensor, learned_prob=None) -> bool:
+    """True when `merge_centres` takes this case: CUDA (B,N,2) positions of a sequence the selecting workgroup holds
+    in LDS, importance scores (if any) in fp32 / fp16 / bf16."""
+    if not (pos.is_cuda and pos.dim() == 3 and pos.shape[2] == 2 and pos.numel() > 0):
+        return False
+    if learned_prob is not None and not (learned_prob.is_cuda and learned_prob.dtype in _DTYPE_CODES
+                                         and learned_prob.numel() == pos.shape[0] * pos.shape[1]):
+        return False
+    return pos.shape[1] <= load().clusten_merge_centres_max_tokens()
+
+
+def merge_centres(pos: torch.Tensor, min_dist, learned_prob, alpha: float, stride: int, sample_num: int,
+                  reserve_num: int, reserve_on: bool) -> torch.Tensor:
+    """(B, sample_num [+ reserve_num]) int64: the tokens `ClusterMerging` keeps (aff_transformer.py:296-334) — the
+    sample_num tokens of highest score (grid prior + learned_prob * alpha, - 100 on the reserved coarse grid), those
+    above the sample_num-th score by ascending index and then those equal to it, followed, with reserve_on, by the
+    reserve_num tokens of the coarse grid by ascending index.  `min_dist` (B,N): distance of every token to its
+    nearest other token, or None while the tokens still fill the grid of `stride`."""
+    lib = load()
+    _require_cuda("pos", pos)
+    device = pos.device
+    if not merge_centres_supported(pos, learned_prob):
+        raise RuntimeError("merge_centres: unsupported positions or importance scores")
+    b, n, _ = pos.shape
+    pos = pos.detach().float().contiguous()
+    if min_dist is not None:
+        _require_cuda("min_dist", min_dist, device)
+        if min_dist.numel() != b * n:
+            raise RuntimeError("min_dist must be (B,N)")
+        min_dist = min_dist.detach().float().contiguous()
+    code = 0
+    if learned_prob is not None:
+        _require_cuda("learned_prob", learned_prob, device)
+        learned_prob = learned_prob.detach().contiguous()
+        code = _DTYPE_CODES[learned_prob.dtype]
+    centre = torch.empty(b, sample_num + (reserve_num if reserve_on else 0), dtype=torch.int64, device=device)
+    with torch.cuda.device(device):
+        _check(lib.clusten_merge_centres(_ptr(pos), _ptr(min_dist), _ptr(learned_prob), code, _ptr(centre), b, n,
+                                         sample_num, reserve_num, int(bool(reserve_on)), ctypes.c_float(alpha),
+                                         stride, _stream(device)), "clusten_merge_centres")
+    return centre
+
+
+def merge_rows_supported(*tensors) -> bool:
+    """True when `merge_rows` takes these tensors: CUDA (B,N,.) with rows of whole 8-byte words, at most four."""
+    return 1 <= len(tensors) <= 4 and all(
+        t.is_cuda and t.dim() == 3 and t.numel() > 0 and (t.shape[2] * t.element_size()) % 8 == 0 for t in tensors)
+
+
+def merge_rows(centre: torch.Tensor, *tensors):
+    """The rows of up to four (B,N,.) tensors at centre (B,n') int64, in one launch:
+    `t.gather(1, centre.unsqueeze(2).expand(-1, -1, t.shape[2]))` for each (aff_transformer.py:337-344)."""
+    lib = load()
+    if not merge_rows_supported(*tensors):
+        raise RuntimeError("merge_rows takes one to four CUDA (B,N,.) tensors with rows of whole 8-byte words")
+    device = tensors[0].device
+    _require_cuda("centre", centre, device)
+    b, n = tensors[0].shape[:2]
+    if centre.dtype != torch.int64 or centre.dim() != 2 or centre.shape[0] != b:
+        raise RuntimeError("centre must be (B,n') int64")
+    centre = centre.contiguous()
+    n_out = centre.shape[1]
+    src, dst = [], []
+    for t in tensors:
+        _require_cuda("tensor", t, device)
+        if tuple(t.shape[:2]) != (b, n):
+            raise RuntimeError("every tensor must be (B,N,.)")
+        src.append(t.detach().contiguous())
+        dst.append(torch.empty(b, n_out, t.shape[2], dtype=t.dtype, device=device))
+    if n_out == 0:
+        return tuple(dst)
+    k = len(src)
+    srcs = (ctypes.c_void_p * k)(*[t.data_ptr() for t in src])
+    dsts = (ctypes.c_void_p * k)(*[t.data_ptr() for t in dst])
+    sizes = (ctypes.c_int * k)(*[t.shape[2] * t.element_size() for t in src])
+    with torch.cuda.device(device):
+        _check(lib.clusten_merge_rows(srcs, dsts, sizes, k, _ptr(centre), b, n, n_out, _stream(device)),
+               "clusten_merge_rows")
+    return tuple(dst)
 
 
 def scanline_rank(pos: torch.Tensor, rows: int, cols: int, cell_w: float, cell_h: float) -> torch.Tensor:

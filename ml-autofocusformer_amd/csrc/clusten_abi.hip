@@ -436,6 +436,29 @@ int clusten_gather_rows(const void* x, const int64_t* order, void* out, int64_t 
     return launch_gather_rows(x, order, out, B, N, row_bytes, order_shared, as_stream(stream));
 }
 
+int clusten_merge_centres_max_tokens(void) { return merge_centres_max_tokens(); }
+
+int clusten_merge_centres(const float* pos, const float* min_dist, const void* learned_prob, int prob_dtype,
+                          int64_t* centre, int B, int N, int sample_num, int reserve_num, int reserve_on, float alpha,
+                          int stride, clusten_stream stream) {
+    if (!pos || !centre) return CLUSTEN_ERR_NULL_POINTER;
+    if (learned_prob && prob_dtype != CLUSTEN_F32 && prob_dtype != CLUSTEN_F16 && prob_dtype != CLUSTEN_BF16)
+        return CLUSTEN_ERR_BAD_DTYPE;
+    if (!(reinterpret_cast<uintptr_t>(pos) % 8 == 0)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_merge_centres(pos, min_dist, learned_prob, learned_prob ? prob_dtype : CLUSTEN_F32, centre, B, N,
+                                sample_num, reserve_num, reserve_on, alpha, stride, as_stream(stream));
+}
+
+int clusten_merge_rows(const void* const* src, void* const* dst, const int* row_bytes, int count, const int64_t* centre,
+                       int64_t B, int N, int n_out, clusten_stream stream) {
+    if (!src || !dst || !row_bytes || !centre) return CLUSTEN_ERR_NULL_POINTER;
+    if (count < 1 || count > 4 || B <= 0 || N <= 0 || n_out <= 0) return CLUSTEN_ERR_BAD_DIMS;
+    int64_t words = 0;
+    for (int t = 0; t < count; ++t) words += row_bytes[t] / 8;
+    if ((B * n_out * words + 255) / 256 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    return launch_merge_rows(src, dst, row_bytes, count, centre, B, N, n_out, as_stream(stream));
+}
+
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
                   clusten_stream stream) {
     if (!query || !database || !idx) return CLUSTEN_ERR_NULL_POINTER;

@@ -190,6 +190,19 @@ int launch_cluster_centres(const float* pos, const int64_t* ranking, float* pos_
 //   every b when order_shared.
 int launch_gather_rows(const void* x, const int64_t* order, void* out, int64_t B, int N, int row_bytes, int order_shared,
                        hipStream_t stream);
+// centre[b, :] = the tokens the adaptive down-sampling keeps (models/aff_transformer.py:296-334): the sample_num tokens
+//   of highest score = grid prior + prob * alpha [- 100 on the reserved grid], ascending index among those above the
+//   sample_num-th score, then those equal to it; then, with reserve_on, the reserve_num reserved tokens by ascending
+//   index.  pos (B,N,2) fp32; min_dist (B,N) fp32 distance to the nearest other token, or null for the regular grid of
+//   `stride`; prob (B,N) of prob_dtype or null; centre (B, sample_num [+ reserve_num]) int64.
+int merge_centres_max_tokens();
+int launch_merge_centres(const float* pos, const float* min_dist, const void* prob, int prob_dtype, int64_t* centre, int B,
+                         int N, int sample_num, int reserve_num, int reserve_on, float alpha, int stride,
+                         hipStream_t stream);
+// dst[t][b,i,:] = src[t][b, centre[b,i], :] for t < count <= 4 tensors (B,N,.) with rows of row_bytes[t] bytes
+//   (multiples of 8); centre (B,n_out) int64.
+int launch_merge_rows(const void* const* src, void* const* dst, const int* row_bytes, int count, const int64_t* centre,
+                      int64_t B, int N, int n_out, hipStream_t stream);
 int launch_scanline_rank(const float* pos, int64_t* ranking, void* workspace, int B, int N, int rows, int cols,
                          float cell_w, float cell_h, hipStream_t stream);
 
