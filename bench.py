@@ -451,7 +451,7 @@ def main():
                   lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx, replay=True)]
     torch.cuda.synchronize()
     if args.only == "bwd-model":  # the same on lists as the model builds them (whole clusters, nearest first)
-        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model")
+        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built")
         print(json.dumps({"only": "bwd-model", "launches": args.steps + args.warmup,
                           **_bench_backward(mcase, wcase, args.steps, args.warmup)}), flush=True)
         return
@@ -541,16 +541,20 @@ def main():
         other["cfg1_fp16"] = _bench_attn(wl.config1(torch.float16), args.steps, args.warmup)
         other["cfg3_bf16_attn"] = _bench_attn(wl.config3_attn(), args.steps, args.warmup)
         other["cfg3_bf16_wf_ic4"] = _bench_wf(wl.config3_wf(), args.steps, args.warmup)
+        # lists built by the model's own clustering of adaptively kept tokens (`workloads.model_built_lists`), and the
+        # strips of a regular grid used before that generator existed (fewer distinct clusters per tile: faster)
+        other["cfg2_s1_model_built_lists"] = _bench_attn(
+            wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built"), args.steps, args.warmup)
         other["cfg2_s1_model_like_lists"] = _bench_attn(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
-        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model").to("cuda")
+        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built").to("cuda")
         cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()   # the same lists as cluster numbers
         mattn = torch.softmax(_native.qk_forward(mcase.query, mcase.key, mcase.nbhd_idx), dim=-1)
         _, per_c, _ = _time_kernels([lambda: _native.qk_forward_clusters(mcase.query, mcase.key, cidx),
                                      lambda: _native.av_forward_clusters(mattn, mcase.value, cidx)],
                                     args.steps, args.warmup)
-        other["cfg2_s1_model_like_lists_as_cluster_numbers"] = {"qk_us": round(per_c[0] * 1e3, 1),
-                                                                 "av_us": round(per_c[1] * 1e3, 1)}
+        other["cfg2_s1_model_built_lists_as_cluster_numbers"] = {"qk_us": round(per_c[0] * 1e3, 1),
+                                                                  "av_us": round(per_c[1] * 1e3, 1)}
         # local attention of one block at the same shape under mixed precision: one kernel against the three
         # operators' kernels with the softmax kernel between them (what the model ran before)
         h16 = lambda t: t.to(torch.float16)
@@ -570,7 +574,7 @@ def main():
                                                                        blank_k, blank_v), three_kernels],
                                     args.steps, args.warmup)
         fused_bytes = 4 * q16.numel() * 2 + cidx.numel() * 4 + pe_idx.numel() * 8
-        other["cfg2_s1_local_attention_fp16_model_like_lists"] = {
+        other["cfg2_s1_local_attention_fp16_model_built_lists"] = {
             "one_kernel_us": round(per_a[0] * 1e3, 1), "three_kernels_us": round(per_a[1] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
         del mcase, cidx, mattn, q16, k16, v16, pe_idx
@@ -579,12 +583,12 @@ def main():
         for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             gen384 = wl.generator(31)
             c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
-            c384.nbhd_idx = wl.model_like_lists(16, 9216, gen384, cluster=24, nnc=6)
+            c384.nbhd_idx = wl.model_built_lists(16, 9216, gen384, cluster=24, nnc=6)
             other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
         del c384
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
-        other["cfg2_s1_backward_fp32_model_like_lists"] = _bench_backward(
-            wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), wcase, max(args.steps // 5, 5), 3)
+        other["cfg2_s1_backward_fp32_model_built_lists"] = _bench_backward(
+            wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built"), wcase, max(args.steps // 5, 5), 3)
         out["other_configs"] = other
     if not args.no_e2e:
         try:

@@ -89,7 +89,13 @@ struct Staging {
     static constexpr int OA_BYTES = A_SLOT_BYTES > OUT_PIECES ? A_SLOT_BYTES : OUT_PIECES;  // a-rows, then output chunk
     static constexpr int ULIST_BASE = A_BASE + 2 * OA_BYTES;
     static constexpr int USLOT_BASE = ULIST_BASE + (UNION ? U_MAX * 8 * 4 : 0);
-    static constexpr int BYTES = USLOT_BASE + (UNION ? kWave * 4 : 0);
+    // union path: the score matrix of a pass lives outside the row area, so that the rows of the next pass can be
+    // requested while it is picked from: in the a-row slot of the head where that is large enough (fp32 data: the
+    // scores of a pass are as many bytes as the head's output chunk), else in an area of its own
+    static constexpr bool SCORES_IN_A = OA_BYTES >= kTileTokens * 16 * QU * 4;
+    static constexpr int SSTR = SCORES_IN_A ? 16 * QU : SROW;  // floats per token row of the score matrix
+    static constexpr int SCORE_BASE = SCORES_IN_A ? A_BASE : USLOT_BASE + (UNION ? kWave * 4 : 0);
+    static constexpr int BYTES = USLOT_BASE + (UNION ? kWave * 4 : 0) + (UNION && !SCORES_IN_A ? kTileTokens * SROW * 4 : 0);
     static constexpr int EL = C / 4;                            // channels per lane (a quarter row)
     static constexpr int QB = RB / 4;                           // bytes per lane
     static constexpr int UNIT = QB < 16 ? QB : 16;              // bytes per LDS read
@@ -292,29 +298,42 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                 }
 
                 const int total_rows = 8 * U;
-                for (int h = 0; h < H; ++h) {
+                // Passes of UROWS union rows, heads outside.  The rows of the next pass (of this head or the next) are
+                // requested as soon as the operands of the current one are in registers, so they travel while the
+                // current pass is multiplied and picked; the stores of a head are issued after the first request of
+                // the next head, and the wait for those rows leaves them in flight.
+                auto gather_pass = [&](int h, int base) {
                     const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+                    const int rows_here = min(UROWS, total_rows - base);
+#pragma unroll
+                    for (int i = 0; i < S::NI_U; ++i) {
+                        if (i * S::RPI < rows_here) {
+                            const int srow = i * S::RPI + g_sub;
+                            const uint32_t urow = (uint32_t)ulist[min(base + srow, total_rows - 1)];
+                            CLUSTEN_LDS_DMA16(rows_bh + (urow * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
+                                              stage + i * 1024);
+                        }
+                    }
+                };
+                // store instructions of a head that have an active lane: all of them on a full tile
+                bool all_stores = true;
+#pragma unroll
+                for (int k = 0; k < NQD; ++k) all_stores = all_stores && (4 * kWave * k < nt * M);
+                gather_pass(0, 0);
+                for (int h = 0; h < H; ++h) {
                     F32x4 val[NQD];
 #pragma unroll
                     for (int k = 0; k < NQD; ++k) val[k] = F32x4{0.f, 0.f, 0.f, 0.f};
+                    typename RunIO::raw a_raw[S::NU];
+                    char* score = stage + S::SCORE_BASE + (S::SCORES_IN_A ? (h & 1) * S::OA_BYTES : 0);
                     for (int base = 0; base < total_rows; base += UROWS) {
                         const int rows_here = min(UROWS, total_rows - base);
-                        __syncthreads();  // the previous pass has picked its scores
-#pragma unroll
-                        for (int i = 0; i < S::NI_U; ++i) {
-                            if (i * S::RPI < rows_here) {
-                                const int srow = i * S::RPI + g_sub;
-                                const uint32_t urow = (uint32_t)ulist[min(base + srow, total_rows - 1)];
-                                CLUSTEN_LDS_DMA16(rows_bh + (urow * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
-                                                  stage + i * 1024);
-                            }
+                        if (base == 0 && h > 0 && all_stores) {
+                            lds_sync_vm<NQD>();  // everything but the stores of the previous head
+                        } else {
+                            lds_sync_vm<0>();
                         }
-                        if (h >= 2 && base == 0) fetch_a(h);
-                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-                        __syncthreads();
-
                         typename RunIO::raw g_raw[QU][S::NU];
-                        typename RunIO::raw a_raw[S::NU];
 #pragma unroll
                         for (int u = 0; u < S::NU; ++u) {
 #pragma unroll
@@ -324,11 +343,19 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                                                                                                   blk * 16 * S::RB);
                                 }
                             }
-                            a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] +
-                                                                                     (h & 1) * S::OA_BYTES);
+                            if (base == 0) {
+                                a_raw[u] = *reinterpret_cast<const typename RunIO::raw*>(stage + lds_a[u] +
+                                                                                         (h & 1) * S::OA_BYTES);
+                            }
                         }
-                        __syncthreads();  // operands are in registers: the rows make room for the scores
-
+                        lds_sync();  // operands are in registers: the row area is free for the next pass
+                        const bool last = base + UROWS >= total_rows;
+                        if (base == 0 && h >= 1 && h + 1 < H) fetch_a(h + 1);  // into the slot head h-1 has left
+                        if (!last) {
+                            gather_pass(h, base + UROWS);
+                        } else if (h + 1 < H) {
+                            gather_pass(h + 1, 0);
+                        }
 #pragma unroll
                         for (int blk = 0; blk < QU; ++blk) {
                             if (blk * 16 < rows_here) {
@@ -337,16 +364,16 @@ __global__ __launch_bounds__(kWave) void gather_dot_tile_kernel(const T* __restr
                                 for (int u = 0; u < S::NU; ++u) d = tile_mfma<T>(g_raw[blk][u], a_raw[u], d);
                                 // lane (r, kq): union rows 16*blk + 4*kq .. +3 of token r
                                 if (r < kTileTokens) {
-                                    *reinterpret_cast<F32x4*>(stage + (r * S::SROW + 16 * blk + 4 * kq) * 4) = d;
+                                    *reinterpret_cast<F32x4*>(score + (r * S::SSTR + 16 * blk + 4 * kq) * 4) = d;
                                 }
                             }
                         }
-                        __syncthreads();
+                        lds_sync();
 #pragma unroll
                         for (int k = 0; k < NQD; ++k) {
                             const int sl = sidx[k] - base;
                             if (sl >= 0 && sl < UROWS) {
-                                val[k] = *reinterpret_cast<const F32x4*>(stage + (qtok[k] * S::SROW + sl) * 4);
+                                val[k] = *reinterpret_cast<const F32x4*>(score + (qtok[k] * S::SSTR + sl) * 4);
                             }
                         }
                     }

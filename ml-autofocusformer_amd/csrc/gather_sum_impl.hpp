@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                     for (int base = 0, pass = 0; base < total_rows; base += PROWS, ++pass) {
                         const int rows_here = min(PROWS, total_rows - base);
                         const int rows_batched = (rows_here + 15) & ~15;  // MFMA batches cover 16 rows
-                        __syncthreads();  // the previous pass (or head) has read its operands
+                        lds_sync();  // the previous pass (or head) has read its operands
 #pragma unroll
                         for (int i = 0; i < S::NI_G; ++i) {
                             if (i * S::RPI < rows_batched) {  // rows past the last one repeat it (their p is zero)
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                         for (int z = lane * 16; z < S::PM_BYTES; z += kWave * 16) {
                             *reinterpret_cast<F32x4*>(stage + S::PM_BASE + z) = F32x4{0.f, 0.f, 0.f, 0.f};
                         }
-                        __syncthreads();
+                        lds_sync();
 #pragma unroll
                         for (int k = 0; k < S::NI_P; ++k) {
                             if (ppass[k] == pass) {
@@ -381,8 +381,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_tile_kernel(const T* __restr
                                 }
                             }
                         }
-                        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-                        __syncthreads();
+                        lds_sync_vm<0>();
 
                         // batches of 4 steps (16 union rows = 2 runs); batches past the last row are skipped
 #pragma unroll

@@ -64,7 +64,7 @@ def test_attn_backward_cluster_shared(device, dtype):
     _check_attn_backward(wl.attn_case("shared", 72, B=2, H=2, N=200, C=32), device, dtype)
 
 
-@pytest.mark.parametrize("lists", ["random", "model"])
+@pytest.mark.parametrize("lists", ["random", "model", "model_built"])
 def test_attn_backward_per_token_lists(device, lists):
     _check_attn_backward(wl.attn_case(lists, 73, B=2, H=4, N=392, C=32, lists=lists), device, torch.float32)
 

@@ -57,7 +57,7 @@ def test_cluster_shared_lists_all_dtypes(device, dtype):
     _check_attn(wl.attn_case("shared", 50, B=3, H=2, N=392, C=32), device, dtype)
 
 
-@pytest.mark.parametrize("lists", ["random", "model", "model_canonical"])
+@pytest.mark.parametrize("lists", ["random", "model", "model_canonical", "model_built"])
 def test_per_token_lists(device, lists):
     # random lists hold duplicates, like the reference's own test scripts (torch.randint)
     _check_attn(wl.attn_case(lists, 51, B=2, H=4, N=784 if lists != "random" else 196, C=32, lists=lists), device,
