@@ -278,7 +278,7 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
  * not (the rest of the block then means nothing, and the two consumers leave their outputs untouched).
  * clusten_qk_backward, clusten_av_backward and clusten_wf_backward build the same lists in their workspace on every
  * call and select their kernels through the same flag on the device.
- *   clusten_cluster_pairs_bytes: size of the block; 0 when the shape is not supported (M % 8 != 0, M > 64, n_rows < 8,
+ *   clusten_cluster_pairs_bytes: size of the block; 0 when the shape is not supported (M % 8 != 0, M > 256, n_rows < 8,
  *   or more than about 7000 clusters per image); pair_lists must be 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).
  * rows = N for attention lists (n_rows = N too), Nout for a merge's lists (n_rows = N).  No counterpart in the
  * reference's extension modules. */
@@ -293,7 +293,7 @@ int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair
  * (results repeat bit for bit).  pair_lists: the block clusten_cluster_pairs filled for (B, N, M, N).
  * p (B,H,N,M) and y (B,H,N,C) contiguous, x strided (B,H,N,C), all of `dtype` (F32, F16 or BF16); every row of y is
  * written — unless the block's flag says the lists are not made of whole clusters: then y is left untouched.
- * C in {16,32,64}, N >= 8, M % 8 == 0, M <= 64 (else CLUSTEN_ERR_BAD_DIMS); rows 16-byte aligned (else
+ * C in {16,32,64}, N >= 8, M % 8 == 0, M <= 256 (else CLUSTEN_ERR_BAD_DIMS); rows 16-byte aligned (else
  * CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
 int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const void* pair_lists,
                                     void* y, clusten_attn_shape shape, int dtype, clusten_stream stream);
@@ -303,7 +303,7 @@ int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_stride
  *   d_feat[b, 8g+t, :] = sum over the pairs (i,r) of cluster (b,g) of  sum_ic weights[b,i,8r+t,ic] * d_feat_new[b,i,ic,:]
  * pair_lists: the block clusten_cluster_pairs filled for (B, Nout, M, N) (i counts the output tokens, g the clusters
  * of the N feature rows); d_weights as clusten_wf_backward computes it.  When the block's flag says the lists are not
- * made of whole clusters d_feat is left untouched.  IC = 4, C % 32 == 0, N >= 8, M % 8 == 0, M <= 64 (else
+ * made of whole clusters d_feat is left untouched.  IC = 4, C % 32 == 0, N >= 8, M % 8 == 0, M <= 256 (else
  * CLUSTEN_ERR_BAD_DIMS); dtype F32, F16 or BF16.  No counterpart in the reference's extension modules. */
 int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat,
                                    const int64_t* nbhd_idx, const void* pair_lists,

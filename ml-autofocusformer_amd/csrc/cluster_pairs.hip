@@ -6,7 +6,7 @@
 // models/aff_transformer.py:476-480; the short last cluster of a sequence whose length is not a multiple of 8 is
 // followed by pad slots that hold row 0, models/point_utils.py:203-206).  For such lists
 //   keys[(b*N + i)*R + r] = c(b,i,r)                                       (cluster_keys_kernel; R = M/8)
-//   pairs[starts[b*K+g] .. ends[b*K+g]) = the entries i*8 + r with c(b,i,r) = g, ascending   (cluster_sort_kernel)
+//   pairs[starts[b*K+g] .. ends[b*K+g]) = the entries i*32 + r with c(b,i,r) = g, ascending  (cluster_sort_kernel)
 // Any other run sets *not_whole, which the consumers read on the device: the cluster-by-cluster kernels return at
 // once when it is set, the atomic kernels when it is clear.
 //
@@ -94,7 +94,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* scratch, int* to
 
 // The stable counting sort of one image by one workgroup.  E entries in the order e = 0 .. E-1, K keys; the sorted
 // entries go to `pairs` (cap per image), the bounds of every key's list to starts / ends.
-//   ROWS = false: keys[e] = cluster number of run e = i*R + r, entry = i*8 + r; `pad`: the pairs of the short last
+//   ROWS = false: keys[e] = cluster number of run e = i*R + r, entry = i*32 + r; `pad`: the pairs of the short last
 //                 cluster are listed again, flagged, under cluster 0;
 //   ROWS = true:  keys64[e] = destination row of list entry e (any row: entries outside [0, K) are left out),
 //                 entry = e.
@@ -172,7 +172,7 @@ __device__ __forceinline__ void sort_image(const void* __restrict__ keys_any, in
             const int e = e00 + 64 * u + lane;
             const int k = k4[u];
             const bool valid = k >= 0;
-            const int entry = ROWS ? e : (e / R) * 8 + e % R;
+            const int entry = ROWS ? e : ((e / R) << kPairRunBits) + e % R;
             // the lanes of this step that hold the lane's key: one ballot per bit of the key
             uint64_t same = __ballot(valid);
             for (int bit = 0; bit < key_bits; ++bit) {
@@ -233,10 +233,10 @@ inline size_t keys_workgroups(int64_t runs) {
 }  // namespace
 
 bool cluster_pairs_supported(int B, int rows, int M, int D) {
-    if (B <= 0 || rows <= 0 || M <= 0 || M % 8 != 0 || M > 64 || D < 8) return false;
+    if (B <= 0 || rows <= 0 || M <= 0 || M % 8 != 0 || M > kPairMaxSlots || D < 8) return false;
     const int64_t R = M / 8, K = (D + 7) / 8;
     const int64_t E = (int64_t)rows * R;
-    if (rows >= (1 << 26) || 2 * E * B >= ((int64_t)1 << 31) || K * B >= ((int64_t)1 << 30)) return false;
+    if (rows >= (1 << (30 - kPairRunBits)) || 2 * E * B >= ((int64_t)1 << 31) || K * B >= ((int64_t)1 << 30)) return false;
     return (2 * K + 16) * 4 + 64 <= kSortLdsBytes;   // at least one wave's histogram fits
 }
 

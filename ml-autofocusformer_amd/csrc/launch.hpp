@@ -6,6 +6,13 @@
 
 namespace clusten {
 
+// An entry of a pair list (cluster_pairs.hip) names run r of token i of its image as i << kPairRunBits | r: lists of
+// up to 256 slots, i.e. 32 runs of 8.  Bit 30 flags the second listing of a pair that names a short last cluster.
+constexpr int kPairRunBits = 5;
+constexpr int kPairRunMask = (1 << kPairRunBits) - 1;
+constexpr int kPairMaxSlots = 8 << kPairRunBits;
+
+
 // out[b,h,i,j] = sum_c a[b,h,i,c] * rows[b,h,idx[b,i,j],c]      (QK forward; AV's d_attn)
 //   a, rows : strided (B,H,N,C);  out : contiguous (B,H,N,M)
 int launch_gather_dot(const void* a, clusten_strides a_strides, const void* rows, clusten_strides rows_strides,

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
 #pragma unroll
                 for (int a = 0; a < X_DMA; ++a) {
                     const int e = list[base + min(ROWS_PER_DMA * a + lane / LANES_PER_ROW, here - 1)] & kEntryMask;
-                    CLUSTEN_LDS_DMA16(x_bh + lane_offset((uint32_t)(e >> 3) * (uint32_t)xs.n * EB +
+                    CLUSTEN_LDS_DMA16(x_bh + lane_offset((uint32_t)(e >> kPairRunBits) * (uint32_t)xs.n * EB +
                                                          (uint32_t)(lane % LANES_PER_ROW) * 16),
                                       stage + X_BASE + a * 1024);
                 }
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
                     constexpr int LANES_PER_PIECE = PIECE_B / 16;
                     if (lane < kPass * LANES_PER_PIECE) {
                         const int e = list[base + min(lane / LANES_PER_PIECE, here - 1)] & kEntryMask;
-                        CLUSTEN_LDS_DMA16(p_bh + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * EB +
+                        CLUSTEN_LDS_DMA16(p_bh + lane_offset(((uint32_t)(e >> kPairRunBits) * (uint32_t)M + (uint32_t)(e & kPairRunMask) * 8) * EB +
                                                              (uint32_t)(lane % LANES_PER_PIECE) * 16),
                                           stage + P_BASE);
                     }
@@ -187,7 +187,7 @@ int launch_typed(const void* p, const void* x, clusten_strides xs, const int32_t
 bool scatter_by_cluster_supported(const void* p, const void* x, clusten_strides xs, const void* y,
                                   const clusten_attn_shape& s, int dtype) {
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return false;
-    if ((s.C != 16 && s.C != 32 && s.C != 64) || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M <= 0) return false;
+    if ((s.C != 16 && s.C != 32 && s.C != 64) || s.N < 8 || s.M % 8 != 0 || s.M > kPairMaxSlots || s.M <= 0) return false;
     const size_t eb = dtype_size(dtype);
     return rows_aligned16(x, xs, (int)eb) && aligned16(p) && aligned16(y) && slice_fits_int32(xs, s.H, s.N, s.C) &&
            (int64_t)s.N * s.M * (int64_t)eb < ((int64_t)1 << 31);
@@ -196,7 +196,7 @@ bool scatter_by_cluster_supported(const void* p, const void* x, clusten_strides 
 int launch_scatter_by_cluster(const void* p, const void* x, clusten_strides xs, const int32_t* starts, const int32_t* ends,
                               const int32_t* pairs, const int32_t* not_whole, void* y, clusten_attn_shape s, int dtype,
                               hipStream_t stream) {
-    if ((s.C != 16 && s.C != 32 && s.C != 64) || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if ((s.C != 16 && s.C != 32 && s.C != 64) || s.N < 8 || s.M % 8 != 0 || s.M > kPairMaxSlots || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
     if (!scatter_by_cluster_supported(p, x, xs, y, s, dtype)) return CLUSTEN_ERR_UNALIGNED;
     switch (dtype) {
         case CLUSTEN_F32: return launch_typed<float>(p, x, xs, starts, ends, pairs, not_whole, y, s, stream);

@@ -90,13 +90,13 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
                     const int slot = a * 64 + lane;
                     const int e = list[base + min(slot / LANES_PER_PAIR, here - 1)] & kEntryMask;
                     const int ic = (slot / LANES_PER_ROW) % kIC;
-                    CLUSTEN_LDS_DMA16(d_out_b + lane_offset((((uint32_t)(e >> 3) * kIC + (uint32_t)ic) * (uint32_t)C +
+                    CLUSTEN_LDS_DMA16(d_out_b + lane_offset((((uint32_t)(e >> kPairRunBits) * kIC + (uint32_t)ic) * (uint32_t)C +
                                                              (uint32_t)c0) * EB + (uint32_t)(lane % LANES_PER_ROW) * 16),
                                       stage + X_BASE + a * 1024);
                 }
                 if (lane < kPass * LANES_PER_W) {
                     const int e = list[base + min(lane / LANES_PER_W, here - 1)] & kEntryMask;
-                    CLUSTEN_LDS_DMA16(w_b + lane_offset(((uint32_t)(e >> 3) * (uint32_t)M + (uint32_t)(e & 7) * 8) * (kIC * EB) +
+                    CLUSTEN_LDS_DMA16(w_b + lane_offset(((uint32_t)(e >> kPairRunBits) * (uint32_t)M + (uint32_t)(e & kPairRunMask) * 8) * (kIC * EB) +
                                                         (uint32_t)(lane % LANES_PER_W) * 16),
                                       stage + W_BASE);
                 }
@@ -160,7 +160,7 @@ int launch_typed(const void* d_out, const void* w, const int32_t* starts, const 
 bool wf_dfeat_by_cluster_supported(const void* d_out, const void* w, const void* d_feat, const clusten_wf_shape& s,
                                    int dtype) {
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return false;
-    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M <= 0) return false;
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > kPairMaxSlots || s.M <= 0) return false;
     const int64_t eb = (int64_t)dtype_size(dtype);
     if ((int64_t)s.Nout * kIC * s.C * eb >= ((int64_t)1 << 31) || (int64_t)s.Nout * s.M * kIC * eb >= ((int64_t)1 << 31)) {
         return false;
@@ -171,7 +171,7 @@ bool wf_dfeat_by_cluster_supported(const void* d_out, const void* w, const void*
 int launch_wf_dfeat_by_cluster(const void* d_out, const void* w, const int32_t* starts, const int32_t* ends,
                                const int32_t* pairs, const int32_t* not_whole, void* d_feat, clusten_wf_shape s, int dtype,
                                hipStream_t stream) {
-    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > 64 || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (s.IC != kIC || s.C % kChunk != 0 || s.N < 8 || s.M % 8 != 0 || s.M > kPairMaxSlots || s.M == 0) return CLUSTEN_ERR_BAD_DIMS;
     if (!wf_dfeat_by_cluster_supported(d_out, w, d_feat, s, dtype)) return CLUSTEN_ERR_UNALIGNED;
     switch (dtype) {
         case CLUSTEN_F32: return launch_typed<float>(d_out, w, starts, ends, pairs, not_whole, d_feat, s, stream);

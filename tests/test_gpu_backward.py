@@ -97,6 +97,26 @@ def test_attn_backward_cluster_by_cluster(device, dtype):
         _check_attn_backward(case, device, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attn_backward_cluster_by_cluster_on_the_long_lists_of_the_384_models(device, dtype):
+    """Clusters of 24 tokens, the members of the 6 nearest = 144 slots (configs/aff_base_22kto1k_384.yaml:10-11): every
+    run of 8 slots of such a list is a whole cluster of 8 rows too, 18 runs per token, so the scatters run as gathers;
+    a sequence that does not end on a cluster of 24 has runs of pad slots only and keeps the atomic kernels."""
+    g = torch.Generator().manual_seed(83)
+    for B, H, N, whole in ((2, 2, 240, True), (1, 4, 576, True), (2, 2, 250, False)):
+        idx = wl.model_built_lists(B, N, g, cluster=24, nnc=6)
+        assert idx.shape[-1] == 144 and _whole(idx, device) == whole
+        case = wl.attn_case("long", 84, B=B, H=H, N=N, C=32, M=144, lists="random")
+        case.nbhd_idx = idx
+        _check_attn_backward(case, device, dtype)
+    # the same lists for a merge: WF feature gradient by cluster
+    idx = wl.model_built_lists(2, 240, g, cluster=24, nnc=6)[:, ::4].contiguous()
+    wcase = wl.wf_case("long_wf", 85, B=2, N=240, C=64, M=144)
+    wcase.nbhd_idx = idx
+    assert _whole(idx, device, n_rows=240)
+    _check_wf_backward(wcase, device, dtype)
+
+
 def _padded_model_lists(B, N, nnc, gen):
     """Lists over a sequence whose last cluster is short: (B,N,8*nnc), clusters chosen at random per token, the
     slots past the last row hold index 0 (as the model pads them)."""
