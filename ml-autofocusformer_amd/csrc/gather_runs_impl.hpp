@@ -74,11 +74,23 @@ __device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_token
     const int own = (v0 + L > N && v0 < N) ? N - v0 : L;
     bool regular = v0 >= 0 && v0 < N;
     bool same = true;
-    for (int t = 0; t < L; t += 2) {
-        const I64x2 two = *reinterpret_cast<const I64x2*>(run + t);
-        const int x = (int)two[0], y = (int)two[1];
-        regular = regular && x == (t < own ? v0 + t : 0) && y == (t + 1 < own ? v0 + t + 1 : 0);
-        same = same && x == __shfl(x, rho % R) && y == __shfl(y, rho % R);
+    // the run's entries, 8 loads of two at a time in flight (one after the other they would be L / 2 round trips to
+    // memory before the tile's first gather)
+    for (int t0 = 0; t0 < L; t0 += 16) {
+        I64x2 two[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            two[u] = *reinterpret_cast<const I64x2*>(run + min(t0 + 2 * u, L - 2));
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = t0 + 2 * u;
+            if (t < L) {   // uniform
+                const int x = (int)two[u][0], y = (int)two[u][1];
+                regular = regular && x == (t < own ? v0 + t : 0) && y == (t + 1 < own ? v0 + t + 1 : 0);
+                same = same && x == __shfl(x, rho % R) && y == __shfl(y, rho % R);
+            }
+        }
     }
     const bool shared = __all((lane >= nruns || same) ? 1 : 0) != 0;
     const int key = regular ? v0 : (shared ? ~(rho % R) : ~lane);   // other runs never merge
@@ -97,10 +109,20 @@ __device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_token
     }
     if (remaining != 0) return -1;
     if (first && lane < nruns) {
-        for (int t = 0; t < L; t += 2) {   // the rows of a distinct run, read again by the lane that stands for it
-            const I64x2 two = *reinterpret_cast<const I64x2*>(run + t);
-            ulist[uslot * L + t] = (int)two[0];
-            ulist[uslot * L + t + 1] = (int)two[1];
+        for (int t0 = 0; t0 < L; t0 += 16) {   // the rows of a distinct run, read again by the lane that stands for it
+            I64x2 two[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                two[u] = *reinterpret_cast<const I64x2*>(run + min(t0 + 2 * u, L - 2));
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int t = t0 + 2 * u;
+                if (t < L) {
+                    ulist[uslot * L + t] = (int)two[u][0];
+                    ulist[uslot * L + t + 1] = (int)two[u][1];
+                }
+            }
         }
     }
     if (lane < nruns) uslots[lane] = uslot;
