@@ -132,7 +132,7 @@ __device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_token
 // ---- gather_dot ----------------------------------------------------------------------------------------------------
 
 template <typename T, int C>
-__global__ __launch_bounds__(kWave) void gather_dot_runs_kernel(const T* __restrict__ a, const T* __restrict__ rows,
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ? 3 : 1))) void gather_dot_runs_kernel(const T* __restrict__ a, const T* __restrict__ rows,
                                                                 const int64_t* __restrict__ idx, T* __restrict__ out,
                                                                 int H, int N, int M, int L, clusten_strides as,
                                                                 clusten_strides rs, int tiles_per_batch, int total_tiles) {
@@ -181,47 +181,91 @@ __global__ __launch_bounds__(kWave) void gather_dot_runs_kernel(const T* __restr
         const int total_rows = U * L;
         const char* a_part = reinterpret_cast<const char*>(a + (int64_t)b * as.b + (int64_t)(i0 + t0) * as.n);
         char* out_part = reinterpret_cast<char*>(out + (((int64_t)b * H) * N + i0 + t0) * M);
-        for (int h = 0; h < H; ++h) {
-            const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
-            lds_sync();  // the previous head's operands have been read
+        // Heads outside, passes of UROWS union rows inside.  The rows of the next pass (of this head or the next one,
+        // whose a-rows go along into the other a-row slot) are requested as soon as the operands of the current pass
+        // are in registers, and the stores of a head are issued after the first request of the next head, whose wait
+        // leaves them in flight: a tile's chain of passes is long (heads x 4 passes at 144 slots), and each link
+        // would otherwise be a full trip to memory.
+        auto fetch_a = [&](int h) {
 #pragma unroll
             for (int i = 0; i < S::NI_A; ++i) {
                 const int srow = i * S::RPI + g_sub;
                 CLUSTEN_LDS_DMA16(a_part + (int64_t)h * as.h * sizeof(T) +
                                       lane_offset((uint32_t)min(srow, ntok - 1) * (uint32_t)as.n * sizeof(T) +
                                                   (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
-                                  stage + S::A_BASE + i * 1024);
+                                  stage + S::A_BASE + (h & 1) * S::A_SLOT + i * 1024);
             }
+        };
+        auto gather_pass = [&](int h, int base) {
+            const char* rows_bh = rows_b + (int64_t)h * rs.h * sizeof(T);
+            const int rows_here = min(S::UROWS, total_rows - base);
+#pragma unroll
+            for (int i = 0; i < S::NI_U; ++i) {
+                if (i * S::RPI < rows_here) {
+                    const int srow = i * S::RPI + g_sub;
+                    const uint32_t urow = (uint32_t)ulist[min(base + srow, total_rows - 1)];
+                    CLUSTEN_LDS_DMA16(rows_bh + lane_offset(urow * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
+                                      stage + i * 1024);
+                }
+            }
+        };
+        const int n_stores = (ntok * M + 4 * kWave - 1) / (4 * kWave);   // store instructions of a head, <= NQD_MAX
+        lds_sync();  // the previous group of tokens has read its operands
+        fetch_a(0);
+        gather_pass(0, 0);
+        for (int h = 0; h < H; ++h) {
             F32x4 val[NQD_MAX];
 #pragma unroll
             for (int k = 0; k < NQD_MAX; ++k) val[k] = F32x4{0.f, 0.f, 0.f, 0.f};
             for (int base = 0; base < total_rows; base += S::UROWS) {
                 const int rows_here = min(S::UROWS, total_rows - base);
-                lds_sync();  // the previous pass has picked its scores and read its rows
-#pragma unroll
-                for (int i = 0; i < S::NI_U; ++i) {
-                    if (i * S::RPI < rows_here) {
-                        const int srow = i * S::RPI + g_sub;
-                        const uint32_t urow = (uint32_t)ulist[min(base + srow, total_rows - 1)];
-                        CLUSTEN_LDS_DMA16(rows_bh + lane_offset(urow * row_pitch + (uint32_t)((g_pos ^ S::swz(srow)) * 16)),
-                                          stage + i * 1024);
+                Piece a_raw[S::NU];
+                if (base == 0 && h > 0) {
+                    // everything but the stores of the previous head
+                    switch (n_stores) {
+                        case 1: lds_sync_vm<1>(); break;
+                        case 2: lds_sync_vm<2>(); break;
+                        case 3: lds_sync_vm<3>(); break;
+                        case 4: lds_sync_vm<4>(); break;
+                        case 5: lds_sync_vm<5>(); break;
+                        case 6: lds_sync_vm<6>(); break;
+                        case 7: lds_sync_vm<7>(); break;
+                        case 8: lds_sync_vm<8>(); break;
+                        default: lds_sync_vm<0>(); break;
                     }
+                } else {
+                    lds_sync_vm<0>();
                 }
-                lds_sync_vm<0>();
+                Piece g_raw[S::UROWS / 16][S::NU];
+#pragma unroll
+                for (int u = 0; u < S::NU; ++u) {
+                    const int piece = kq * S::NU + u;
+#pragma unroll
+                    for (int blk = 0; blk < S::UROWS / 16; ++blk) {
+                        if (blk * 16 < rows_here) {
+                            const int grow = 16 * blk + r;
+                            g_raw[blk][u] = *reinterpret_cast<const Piece*>(stage + grow * S::RB + ((piece ^ S::swz(grow)) * 16));
+                        }
+                    }
+                    a_raw[u] = *reinterpret_cast<const Piece*>(stage + S::A_BASE + (h & 1) * S::A_SLOT + (r & 7) * S::RB +
+                                                               ((piece ^ S::swz(r & 7)) * 16));
+                }
+                lds_sync();  // operands are in registers: the row area is free for the next pass
+                if (base + S::UROWS < total_rows) {
+                    gather_pass(h, base + S::UROWS);
+                } else if (h + 1 < H) {
+                    fetch_a(h + 1);
+                    gather_pass(h + 1, 0);
+                }
 #pragma unroll
                 for (int blk = 0; blk < S::UROWS / 16; ++blk) {
                     if (blk * 16 < rows_here) {
                         F32x4 d = F32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int u = 0; u < S::NU; ++u) {
-                            const int piece = kq * S::NU + u;
-                            const int grow = 16 * blk + r;
-                            const Piece gp = *reinterpret_cast<const Piece*>(stage + grow * S::RB + ((piece ^ S::swz(grow)) * 16));
-                            const Piece ap = *reinterpret_cast<const Piece*>(stage + S::A_BASE + (r & 7) * S::RB +
-                                                                           ((piece ^ S::swz(r & 7)) * 16));
                             float gx[S::VEC], ax[S::VEC];
-                            PieceIO::unpack(gp, gx);
-                            PieceIO::unpack(ap, ax);
+                            PieceIO::unpack(g_raw[blk][u], gx);
+                            PieceIO::unpack(a_raw[u], ax);
 #pragma unroll
                             for (int e = 0; e < S::VEC; ++e) d = mfma_16x16x4(gx[e], ax[e], d);
                         }
@@ -246,6 +290,8 @@ __global__ __launch_bounds__(kWave) void gather_dot_runs_kernel(const T* __restr
                 }
             }
         }
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // the next group's tables go over areas the stores do not touch, but
+                                                      // its first wait counts from zero
         t0 += ntok;
     }
 }
