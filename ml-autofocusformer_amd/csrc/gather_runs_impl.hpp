@@ -131,22 +131,16 @@ __device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_token
 
 // ---- gather_dot ----------------------------------------------------------------------------------------------------
 
+// Tokens [i0, i0 + nt) (nt <= 8) of batch element b, all heads; `stage`: RunsStaging<T, C>::BYTES bytes of LDS.
 template <typename T, int C>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ? 3 : 1))) void gather_dot_runs_kernel(const T* __restrict__ a, const T* __restrict__ rows,
-                                                                const int64_t* __restrict__ idx, T* __restrict__ out,
-                                                                int H, int N, int M, int L, clusten_strides as,
-                                                                clusten_strides rs, int tiles_per_batch, int total_tiles) {
+__device__ __forceinline__ void gather_dot_runs_tokens(char* stage, const T* __restrict__ a, const T* __restrict__ rows,
+                                                       const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
+                                                       int M, int L, clusten_strides as, clusten_strides rs, int b, int i0,
+                                                       int nt) {
     typedef RunsStaging<T, C> S;
     typedef VecIO<T, S::VEC> PieceIO;
     typedef VecIO<T, 4> OutIO;
-    __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
     constexpr int NQD_MAX = (kTileTokens * 256 / 4 + kWave - 1) / kWave;   // output groups of 4 per lane, M <= 256
-
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
-    const int b = tile / tiles_per_batch;
-    const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
-    const int nt = min(kTileTokens, N - i0);
     const int lane = threadIdx.x;
     const int r = lane & 15, kq = lane >> 4;
     const int g_sub = lane / S::PPR, g_pos = lane % S::PPR;
@@ -296,23 +290,29 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ?
     }
 }
 
-// ---- gather_sum ----------------------------------------------------------------------------------------------------
-
 template <typename T, int C>
-__global__ __launch_bounds__(kWave) void gather_sum_runs_kernel(const T* __restrict__ p, const T* __restrict__ rows,
-                                                                const int64_t* __restrict__ idx, T* __restrict__ out,
-                                                                int H, int N, int M, int L, clusten_strides rs,
-                                                                clusten_strides os, int tiles_per_batch, int total_tiles) {
-    typedef RunsStaging<T, C> S;
-    typedef VecIO<T, 4> OutIO;
-    __shared__ __attribute__((aligned(1024))) char stage[S::BYTES];
-    constexpr int CB = C / 16;   // channel blocks of 16
-
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ? 3 : 1))) void gather_dot_runs_kernel(
+    const T* __restrict__ a, const T* __restrict__ rows, const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
+    int M, int L, clusten_strides as, clusten_strides rs, int tiles_per_batch, int total_tiles) {
+    __shared__ __attribute__((aligned(1024))) char stage[RunsStaging<T, C>::BYTES];
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
-    const int nt = min(kTileTokens, N - i0);
+    gather_dot_runs_tokens<T, C>(stage, a, rows, idx, out, H, N, M, L, as, rs, b, i0, min(kTileTokens, N - i0));
+}
+
+// ---- gather_sum ----------------------------------------------------------------------------------------------------
+
+// Tokens [i0, i0 + nt) (nt <= 8) of batch element b, all heads; `stage`: RunsStaging<T, C>::BYTES bytes of LDS.
+template <typename T, int C>
+__device__ __forceinline__ void gather_sum_runs_tokens(char* stage, const T* __restrict__ p, const T* __restrict__ rows,
+                                                       const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
+                                                       int M, int L, clusten_strides rs, clusten_strides os, int b, int i0,
+                                                       int nt) {
+    typedef RunsStaging<T, C> S;
+    typedef VecIO<T, 4> OutIO;
+    constexpr int CB = C / 16;   // channel blocks of 16
     const int lane = threadIdx.x;
     const int n16 = lane & 15, kq = lane >> 4;
     const int g_sub = lane / S::PPR, g_pos = lane % S::PPR;
@@ -425,6 +425,19 @@ __global__ __launch_bounds__(kWave) void gather_sum_runs_kernel(const T* __restr
         }
         t0 += ntok;
     }
+}
+
+template <typename T, int C>
+__global__ __launch_bounds__(kWave) void gather_sum_runs_kernel(const T* __restrict__ p, const T* __restrict__ rows,
+                                                                const int64_t* __restrict__ idx, T* __restrict__ out,
+                                                                int H, int N, int M, int L, clusten_strides rs,
+                                                                clusten_strides os, int tiles_per_batch, int total_tiles) {
+    __shared__ __attribute__((aligned(1024))) char stage[RunsStaging<T, C>::BYTES];
+    const int tile = xcd_tile(blockIdx.x, total_tiles);
+    if (tile < 0) return;
+    const int b = tile / tiles_per_batch;
+    const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
+    gather_sum_runs_tokens<T, C>(stage, p, rows, idx, out, H, N, M, L, rs, os, b, i0, min(kTileTokens, N - i0));
 }
 
 // ---- launch ----------------------------------------------------------------------------------------------------------

@@ -49,7 +49,7 @@
 
 #include "launch.hpp"
 #include "mfma.hpp"
-#include "gather_runs_impl.hpp"
+#include "gather_runs24_impl.hpp"
 
 namespace clusten {
 
@@ -694,6 +694,7 @@ int gather_sum_typed(const void* p, const void* rows, clusten_strides rs, const 
     if (quads_ok) {
         // long lists made of long runs (the 384 x 384 models: 6 clusters of 24 tokens)
         if (const int L = runs_length_for(s.M); L != 0 && runs_head_dim_ok<T>(s.C)) {
+            if (L == kRun24) return launch_gather_sum_runs24<T>(p, rows, rs, idx, out, os, s, stream);
             return launch_gather_sum_runs<T>(p, rows, rs, idx, out, os, s, L, stream);
         }
         switch (s.C) {
