@@ -585,6 +585,13 @@ def main():
             c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
             c384.nbhd_idx = wl.model_built_lists(16, 9216, gen384, cluster=24, nnc=6)
             other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
+            if dt == torch.float32:
+                # merge lists of the same stage: the 144-slot lists of every fourth token, 9216 -> 2304 tokens, C = 128
+                w384 = wl.wf_case("aff_base_384_wf", 32, B=16, N=9216, C=128, M=144)
+                w384.nbhd_idx = c384.nbhd_idx[:, ::4].contiguous()
+                other["aff_base_384_stage1_wf_fp32_model_lists"] = _bench_wf(w384, max(args.steps // 2, 5), 5)
+                other["aff_base_384_stage1_backward_fp32_model_lists"] = _bench_backward(c384, w384, 5, 2)
+                del w384
         del c384
         other["cfg2_s1_backward_fp32"] = _bench_backward(acase, wcase, max(args.steps // 5, 5), 3)
         other["cfg2_s1_backward_fp32_model_built_lists"] = _bench_backward(

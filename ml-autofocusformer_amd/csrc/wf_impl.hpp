@@ -235,16 +235,19 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
     const int r = lane & 15, kq = lane >> 4;      // MFMA row / k index: the lane holds quarter kq of row r
     const int g_sub = lane >> 4, g_pos = lane & 15;  // gather side: piece g_pos of staging row 4*i + g_sub
 
-    const int mine = (int)idx[(int64_t)token * M + min(lane, M - 1)];
     const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
     const char* g_tok = reinterpret_cast<const char*>(d_out + (int64_t)token * IC * C);
     const uint32_t row_pitch = (uint32_t)C * sizeof(T);
+    // lists of more than 16*Q slots go 16*Q slots at a time
+    for (int j0 = 0; j0 < M; j0 += ROWS) {
+    const int mc = min(ROWS, M - j0);
+    const int mine = (int)idx[(int64_t)token * M + j0 + min(lane, mc - 1)];
 
     uint32_t g_off[NI_G];
 #pragma unroll
     for (int i = 0; i < NI_G; ++i) {
         const int srow = 4 * i + g_sub;
-        g_off[i] = (uint32_t)__shfl(mine, min(srow, M - 1)) * row_pitch + (uint32_t)((g_pos ^ (srow & 15)) * 16);
+        g_off[i] = (uint32_t)__shfl(mine, min(srow, mc - 1)) * row_pitch + (uint32_t)((g_pos ^ (srow & 15)) * 16);
     }
     uint32_t a_off[2];
 #pragma unroll
@@ -296,15 +299,17 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int slot = 16 * blk + 4 * kq + e;
-                if (slot < M) reinterpret_cast<T*>(stage)[slot * IC + r] = from_acc<T>(d[blk][e]);
+                if (slot < mc) reinterpret_cast<T*>(stage)[slot * IC + r] = from_acc<T>(d[blk][e]);
             }
         }
     }
     __syncthreads();
-    const int out_bytes = M * IC * (int)sizeof(T);
-    char* dst = reinterpret_cast<char*>(d_w + (int64_t)token * M * IC);
+    const int out_bytes = mc * IC * (int)sizeof(T);
+    char* dst = reinterpret_cast<char*>(d_w + ((int64_t)token * M + j0) * IC);
     for (int off = lane * 16; off < out_bytes; off += kWave * 16) {
         store_streaming(reinterpret_cast<Piece*>(dst + off), *reinterpret_cast<const Piece*>(stage + off));
+    }
+    __syncthreads();  // the chunk has left LDS before the next one's rows arrive
     }
 }
 
@@ -430,8 +435,9 @@ int wf_dweights_typed(const void* d_out, const void* feat, const int64_t* idx, v
                       hipStream_t stream) {
     // whole 256-byte row blocks, 32-bit byte offsets inside one batch element of feat, d_w rows in 16-byte pieces
     const bool tile_ok = (s.C * (int)sizeof(T)) % 256 == 0 && aligned16(feat) && aligned16(d_out) && aligned16(d_w) &&
-                         (int64_t)s.N * s.C * (int64_t)sizeof(T) < ((int64_t)1 << 31) && s.M <= 64 && s.IC <= 8 &&
-                         ((int64_t)s.M * s.IC * sizeof(T)) % 16 == 0;
+                         (int64_t)s.N * s.C * (int64_t)sizeof(T) < ((int64_t)1 << 31) && s.IC <= 8 &&
+                         ((int64_t)s.M * s.IC * sizeof(T)) % 16 == 0 &&
+                         (s.M <= 64 || (64 * s.IC * (int)sizeof(T)) % 16 == 0);
     if constexpr (sizeof(T) <= 4) if (tile_ok) {
         const int total_tokens = s.B * s.Nout;
         if (s.M <= 48) {
