@@ -231,7 +231,7 @@ int clusten_av_forward_clusters(const void* attn, const void* value, clusten_str
  * blank_logit may be NULL when query (strided (B,H,N,C) like clusten_qk_forward's, `dtype`) and blank_key
  * ((H,C), fp32, contiguous) are given: the logit is then their dot product per token and head
  * (`(q * blank_k).sum(-1)`, models/aff_transformer.py:144), computed in fp32 inside the same pass.
- * M <= 64 and M % 4 == 0, else CLUSTEN_ERR_BAD_DIMS; attn and probs 16-byte aligned, else
+ * M <= 256 and M % 4 == 0, else CLUSTEN_ERR_BAD_DIMS; attn and probs 16-byte aligned, else
  * CLUSTEN_ERR_UNALIGNED. */
 int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const int64_t* pe_idx,
                                  const int64_t* mask, const float* blank_logit, const void* query,
@@ -427,7 +427,7 @@ int clusten_add_row_score_forward(const void* x, int x_dtype, const void* branch
  * for the `rows` = B*H*N rows of M neighbours.  d_logit is the gradient of the attention logits, and, through
  * clusten_bias_table_grad, of the bias table (both enter the softmax as a sum; the mask is a constant).  probs,
  * d_probs (rows,M), blank_prob, d_blank_prob, d_blank_logit (rows) fp32; d_logit (rows,M) of `dtype` (F32, F16 or
- * BF16); M <= 64, M % 4 == 0 (else CLUSTEN_ERR_BAD_DIMS); 16-byte aligned.  No counterpart in the reference's
+ * BF16); M <= 256, M % 4 == 0 (else CLUSTEN_ERR_BAD_DIMS); 16-byte aligned.  No counterpart in the reference's
  * extension modules. */
 int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
                                   const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,

@@ -584,8 +584,8 @@ def av_forward_clusters(attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.
 
 
 def attn_softmax_supported(attn: torch.Tensor, m: int) -> bool:
-    """True when `attn_softmax` takes this case: a CUDA tensor of a 16/32-bit float type, M <= 64, M % 4 == 0."""
-    return attn.is_cuda and attn.dtype in (torch.float32, torch.float16, torch.bfloat16) and m <= 64 and m % 4 == 0
+    """True when `attn_softmax` takes this case: a CUDA tensor of a 16/32-bit float type, M <= 256, M % 4 == 0."""
+    return attn.is_cuda and attn.dtype in (torch.float32, torch.float16, torch.bfloat16) and m <= 256 and m % 4 == 0
 
 
 def attn_softmax(attn: torch.Tensor, bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_logit=None,
@@ -656,8 +656,8 @@ def attn_softmax_backward(probs: torch.Tensor, blank_prob: torch.Tensor, d_probs
     if probs.dim() != 4 or probs.dtype != torch.float32 or logit_dtype not in _DTYPE_CODES:
         raise RuntimeError("probs must be fp32 (B,H,N,M); logits fp32, fp16 or bf16")
     b, h, n, m = probs.shape
-    if m > 64 or m % 4:
-        raise RuntimeError("attn_softmax_backward: M <= 64, M % 4 == 0")
+    if m > 256 or m % 4:
+        raise RuntimeError("attn_softmax_backward: M <= 256, M % 4 == 0")
     probs = probs.contiguous()
     d_probs = d_probs.to(torch.float32).expand_as(probs).contiguous()
     blank_prob = blank_prob.reshape(b, h, n).float().contiguous()

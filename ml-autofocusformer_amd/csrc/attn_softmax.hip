@@ -9,25 +9,28 @@
 // (B,H,N,M).  Here a token's M logits are read once and its probabilities written once; pe_idx and mask,
 // which the heads share, are read once per token.
 //
-// 16 lanes per token, 4 consecutive neighbours per lane (M <= 64, M % 4 == 0); a 256-thread workgroup takes 16
-// tokens.  Row maxima and sums are reduced inside the 16-lane rows with xor shuffles.  All arithmetic is fp32.
+// LPT = 16 lanes per token (M <= 64) or a whole wave (M <= 256: the 144 neighbours of the 384 x 384 models), 4
+// consecutive neighbours per lane (M % 4 == 0); a 256-thread workgroup takes 256 / LPT tokens.  Row maxima and sums
+// are reduced inside the LPT-lane rows with xor shuffles.  All arithmetic is fp32.
 #include "launch.hpp"
 
 namespace clusten {
 namespace {
 
-__device__ __forceinline__ float row16_max(float v) {
+template <int LPT>
+__device__ __forceinline__ float row_max(float v) {
 #pragma unroll
-    for (int m = 1; m < 16; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
+    for (int m = 1; m < LPT; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
     return v;
 }
-__device__ __forceinline__ float row16_sum(float v) {
+template <int LPT>
+__device__ __forceinline__ float row_sum(float v) {
 #pragma unroll
-    for (int m = 1; m < 16; m <<= 1) v += __shfl_xor(v, m);
+    for (int m = 1; m < LPT; m <<= 1) v += __shfl_xor(v, m);
     return v;
 }
 
-template <typename T>
+template <typename T, int LPT>
 __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__ attn, const T* __restrict__ table,
                                                            const int64_t* __restrict__ pe_idx,
                                                            const int64_t* __restrict__ mask,
@@ -37,10 +40,10 @@ __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__
                                                            float* __restrict__ blank_prob, int H, int N, int M,
                                                            int64_t tokens) {
     typedef Quad<T> Q4;
-    const int64_t tok_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int64_t tok_raw = (int64_t)blockIdx.x * (256 / LPT) + threadIdx.x / LPT;
     const bool tok_live = tok_raw < tokens;
     const int64_t tok = tok_live ? tok_raw : tokens - 1;  // every lane stays in the shuffles
-    const int sub = threadIdx.x & 15;
+    const int sub = threadIdx.x % LPT;
     const int j0 = sub * 4;
     const bool live = j0 < M;
     const int jc = live ? j0 : 0;
@@ -67,17 +70,17 @@ __global__ __launch_bounds__(256) void attn_softmax_kernel(const T* __restrict__
         if (q) {  // the blank token's logit: this token's query against the blank key of the head
             const T* qrow = q + b * qs.b + h * qs.h + i * qs.n;
             float part = 0.f;
-            for (int c = sub; c < C; c += 16) part += to_acc(qrow[c]) * blank_k[h * C + c];
-            bl = row16_sum(part);
+            for (int c = sub; c < C; c += LPT) part += to_acc(qrow[c]) * blank_k[h * C + c];
+            bl = row_sum<LPT>(part);
         } else {
             bl = blank[row];
         }
-        const float mx = fmaxf(row16_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]))), bl);
+        const float mx = fmaxf(row_max<LPT>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]))), bl);
         float ex[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) ex[e] = live ? expf(v[e] - mx) : 0.f;
         const float eb = expf(bl - mx);
-        const float inv = 1.f / (row16_sum((ex[0] + ex[1]) + (ex[2] + ex[3])) + eb);
+        const float inv = 1.f / (row_sum<LPT>((ex[0] + ex[1]) + (ex[2] + ex[3])) + eb);
         if (tok_live && live) {
             float4 o = make_float4(ex[0] * inv, ex[1] * inv, ex[2] * inv, ex[3] * inv);
             *reinterpret_cast<float4*>(probs + row * M + j0) = o;
@@ -91,10 +94,15 @@ int launch_typed(const void* attn, const void* table, const int64_t* pe_idx, con
                  const void* q, clusten_strides qs, const float* blank_k, float* probs, float* blank_prob,
                  const clusten_attn_shape& s, hipStream_t stream) {
     const int64_t tokens = (int64_t)s.B * s.N;
-    const int64_t blocks = (tokens + 15) / 16;
-    hipLaunchKernelGGL((attn_softmax_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                       static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank,
-                       static_cast<const T*>(q), qs, blank_k, s.C, probs, blank_prob, s.H, s.N, s.M, tokens);
+    if (s.M <= 64) {
+        hipLaunchKernelGGL((attn_softmax_kernel<T, 16>), dim3((unsigned)((tokens + 15) / 16)), dim3(256), 0, stream,
+                           static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank,
+                           static_cast<const T*>(q), qs, blank_k, s.C, probs, blank_prob, s.H, s.N, s.M, tokens);
+    } else {
+        hipLaunchKernelGGL((attn_softmax_kernel<T, 64>), dim3((unsigned)((tokens + 3) / 4)), dim3(256), 0, stream,
+                           static_cast<const T*>(attn), static_cast<const T*>(table), pe_idx, mask, blank,
+                           static_cast<const T*>(q), qs, blank_k, s.C, probs, blank_prob, s.H, s.N, s.M, tokens);
+    }
     return launch_status();
 }
 
@@ -114,18 +122,19 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
 // Backward of the softmax over the M neighbours and the blank token:
 //   s = sum_j p_j dp_j + p_blank dp_blank;   d_logit_j = p_j (dp_j - s);   d_blank_logit = p_blank (dp_blank - s)
 // (the bias, the mask and the logits enter the softmax as a sum, so d_logit is the gradient of each of them).
-// One row per 16 lanes, four consecutive neighbours per lane; probs, d_probs fp32, d_logit of the logits' type.
+// One row per 16 lanes (M <= 64) or per wave (M <= 256), four consecutive neighbours per lane; probs, d_probs fp32,
+// d_logit of the logits' type.
 namespace {
 
-template <typename T>
+template <typename T, int LPT>
 __global__ __launch_bounds__(256) void attn_softmax_backward_kernel(const float* __restrict__ probs,
                                                                     const float* __restrict__ blank_prob,
                                                                     const float* __restrict__ d_probs,
                                                                     const float* __restrict__ d_blank_prob,
                                                                     T* __restrict__ d_logit, float* __restrict__ d_blank_logit,
                                                                     int64_t rows, int M) {
-    const int sub = threadIdx.x & 15;
-    const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int sub = threadIdx.x % LPT;
+    const int64_t row_raw = (int64_t)blockIdx.x * (256 / LPT) + threadIdx.x / LPT;
     const bool live = row_raw < rows;
     const int64_t row = live ? row_raw : rows - 1;  // every lane stays in the shuffles
     const bool mine = 4 * sub < M;
@@ -136,8 +145,7 @@ __global__ __launch_bounds__(256) void attn_softmax_backward_kernel(const float*
     }
     const float pb = blank_prob[row], dpb = d_blank_prob[row];
     float s = (p.x * dp.x + p.y * dp.y) + (p.z * dp.z + p.w * dp.w);
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) s += __shfl_xor(s, m);
+    s = row_sum<LPT>(s);
     s += pb * dpb;
     if (!live) return;
     if (mine) {
@@ -152,20 +160,20 @@ __global__ __launch_bounds__(256) void attn_softmax_backward_kernel(const float*
 int launch_attn_softmax_backward(const float* probs, const float* blank_prob, const float* d_probs,
                                  const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
                                  int dtype, hipStream_t stream) {
-    const unsigned blocks = (unsigned)((rows + 15) / 16);
+    auto launch = [&](auto tag) {
+        typedef decltype(tag) T;
+        if (M <= 64) {
+            hipLaunchKernelGGL((attn_softmax_backward_kernel<T, 16>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream,
+                               probs, blank_prob, d_probs, d_blank_prob, static_cast<T*>(d_logit), d_blank_logit, rows, M);
+        } else {
+            hipLaunchKernelGGL((attn_softmax_backward_kernel<T, 64>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream,
+                               probs, blank_prob, d_probs, d_blank_prob, static_cast<T*>(d_logit), d_blank_logit, rows, M);
+        }
+    };
     switch (dtype) {
-        case CLUSTEN_F32:
-            hipLaunchKernelGGL(attn_softmax_backward_kernel<float>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
-                               d_probs, d_blank_prob, static_cast<float*>(d_logit), d_blank_logit, rows, M);
-            break;
-        case CLUSTEN_F16:
-            hipLaunchKernelGGL(attn_softmax_backward_kernel<f16_t>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
-                               d_probs, d_blank_prob, static_cast<f16_t*>(d_logit), d_blank_logit, rows, M);
-            break;
-        case CLUSTEN_BF16:
-            hipLaunchKernelGGL(attn_softmax_backward_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, probs, blank_prob,
-                               d_probs, d_blank_prob, static_cast<bf16_t*>(d_logit), d_blank_logit, rows, M);
-            break;
+        case CLUSTEN_F32: launch(float()); break;
+        case CLUSTEN_F16: launch(f16_t()); break;
+        case CLUSTEN_BF16: launch(bf16_t()); break;
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
     return launch_status();

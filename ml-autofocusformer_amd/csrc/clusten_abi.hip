@@ -181,7 +181,7 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
     if (query && !strides_ok(query_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
-    if (shape.M > 64 || shape.M % 4 != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (shape.M > 256 || shape.M % 4 != 0) return CLUSTEN_ERR_BAD_DIMS;
     if (!aligned16(attn) || !aligned16(probs)) return CLUSTEN_ERR_UNALIGNED;
     return launch_attn_softmax(attn, bias_table, pe_idx, mask, blank_logit, blank_logit ? nullptr : query, query_strides,
                                blank_key, probs, blank_prob, shape, dtype, as_stream(stream));
@@ -372,7 +372,7 @@ int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, c
                                   int dtype, clusten_stream stream) {
     if (!probs || !blank_prob || !d_probs || !d_blank_prob || !d_logit || !d_blank_logit) return CLUSTEN_ERR_NULL_POINTER;
     if (dtype != CLUSTEN_F32 && dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
-    if (rows <= 0 || M <= 0 || M > 64 || M % 4 != 0 || (rows + 15) / 16 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
+    if (rows <= 0 || M <= 0 || M > 256 || M % 4 != 0 || (rows + 3) / 4 >= ((int64_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
     if (!aligned16(probs) || !aligned16(d_probs) || !aligned16(d_logit)) return CLUSTEN_ERR_UNALIGNED;
     return launch_attn_softmax_backward(probs, blank_prob, d_probs, d_blank_prob, d_logit, d_blank_logit, rows, M, dtype,
                                         as_stream(stream));

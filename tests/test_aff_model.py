@@ -191,6 +191,34 @@ def test_logits_equal_with_hip_operators_and_with_the_oracle(device, amp):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("amp", [False, True])
+def test_clusters_of_24_with_144_neighbours_as_in_the_384_models(device, amp):
+    """configs/aff_base_22kto1k_384.yaml:10-11: CLUSTER_SIZE 24, NBHD_SIZE 144.  A 192 x 192 image gives 2304 and 576
+    tokens in the first two stages (local attention over 144-slot lists: the kernels for long runs, the softmax kernel
+    with a wave per token) and 144 / 36 in the last two (global attention).  Logits and parameter gradients against the
+    same model on the oracle."""
+    from aff.model import default_ops
+    kw = dict(img_size=192, num_classes=12, embed_dim=(64, 128, 256, 512), cluster_size=24, nbhd_size=(144, 144, 144, 144))
+    hip = small_model(default_ops(), **kw).to(device)
+    ref = small_model(oracle_ops(), **kw).to(device)
+    ref.load_state_dict(hip.state_dict())
+    x = torch.randn(2, 3, 192, 192, generator=torch.Generator().manual_seed(17)).to(device)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16, enabled=amp):
+        y_hip, y_ref = hip(x), ref(x)
+    assert torch.isfinite(y_hip).all()
+    assert oracle.rel_err(y_hip.float(), y_ref.float()) < (2e-2 if amp else 1e-4)
+    if amp:
+        return
+    hip.train(), ref.train()
+    target = torch.randn(2, 12, generator=torch.Generator().manual_seed(18)).to(device)
+    for model in (hip, ref):
+        ((model(x) - target) ** 2).mean().backward()
+    for (name, p), (_, q) in zip(hip.named_parameters(), ref.named_parameters()):
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        assert float((p.grad - q.grad).abs().max()) <= 1e-3 * float(q.grad.abs().max()) + 1e-7, name
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("embed_dim", [(32, 64, 128, 256), (64, 128, 256, 512)])
 def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkeypatch, embed_dim):
     """A training step of the model with the backward scatters (d_key, d_value, WF d_feat) running as gathers over
@@ -260,13 +288,31 @@ def test_fused_bias_mask_blank_softmax_equals_the_tensor_expressions(device, dty
     blank_ref = (query.float() * blank_key.reshape(1, h, 1, c)).sum(-1, keepdim=True)
     ref_q = torch.softmax(torch.cat([logits, blank_ref], dim=-1), dim=-1)
     assert oracle.rel_err(probs_q, ref_q[..., :-1]) < 1e-5 and oracle.rel_err(blank_q, ref_q[..., -1:]) < 1e-5
+    # the 144 neighbours of the 384 x 384 models (configs/aff_base_22kto1k_384.yaml:11): a wave per token
+    m3 = 144
+    attn3 = (torch.randn(2, h, 50, m3, generator=gen) * 2).to(dtype).to(device)
+    pe3 = torch.randint(rows, (2, 50, m3), generator=gen).to(device)
+    mask3 = (torch.rand(2, 50, m3, generator=gen) > 0.2).long().to(device) if with_mask else None
+    q3 = (torch.randn(2, 50, h, c, generator=gen) * 0.3).to(dtype).to(device).permute(0, 2, 1, 3)
+    p3, b3 = _native.attn_softmax(attn3, table, pe3, mask3, query=q3, blank_key=blank_key)
+    logits3 = attn3.float() + table.float()[pe3].permute(0, 3, 1, 2)
+    if mask3 is not None:
+        logits3 = logits3 + (1 - mask3.reshape(2, 1, 50, m3)) * (-100)
+    ref3 = torch.softmax(torch.cat([logits3, (q3.float() * blank_key.reshape(1, h, 1, c)).sum(-1, keepdim=True)], -1), -1)
+    assert oracle.rel_err(p3, ref3[..., :-1]) < 1e-5 and oracle.rel_err(b3, ref3[..., -1:]) < 1e-5
+    # ... and the backward of the softmax at that length
+    dp, dpb = torch.randn_like(p3), torch.randn_like(b3)
+    d_logit, d_blank = _native.attn_softmax_backward(p3, b3, dp, dpb, dtype)
+    s3 = (p3 * dp).sum(-1, keepdim=True) + b3 * dpb
+    assert oracle.rel_err(d_logit.float(), p3 * (dp - s3)) < (1e-5 if dtype == torch.float32 else 1e-2)
+    assert oracle.rel_err(d_blank, b3 * (dpb - s3)) < 1e-5
     # other list lengths, and the refusals
-    for m2 in (4, 16, 64):
+    for m2 in (4, 16, 64, 256):
         p2, b2 = _native.attn_softmax(attn[..., :1].expand(-1, -1, -1, m2).contiguous(), table,
                                       pe_idx[..., :1].expand(-1, -1, m2).contiguous(), None, blank)
         assert torch.allclose(p2.sum(-1, keepdim=True) + b2, torch.ones_like(b2), atol=1e-5)
         assert torch.allclose(p2, p2[..., :1].expand_as(p2))
-    assert not _native.attn_softmax_supported(attn, 72) and not _native.attn_softmax_supported(attn, 50)
+    assert not _native.attn_softmax_supported(attn, 260) and not _native.attn_softmax_supported(attn, 50)
     with pytest.raises(RuntimeError):
         _native.attn_softmax(attn.cpu(), table, pe_idx, mask, blank)
 
