@@ -56,15 +56,19 @@ __global__ __launch_bounds__(kWave) void scatter_by_cluster_kernel(const T* __re
     static_assert(X_BYTES % 1024 == 0 && 1024 % ROW_B == 0, "whole LDS-direct loads, whole rows per load");
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
-    if (not_whole != nullptr && *not_whole != 0) return;   // not lists of whole clusters: the atomic kernels run instead
     const int unit = xcd_tile(blockIdx.x, total_clusters);
     if (unit < 0) return;
+    // the flag and the bounds of the cluster's list are requested together (one trip to memory, not two); the bounds
+    // mean nothing when the flag is set, and are not used then
+    const int flagged = not_whole != nullptr ? *not_whole : 0;
+    const int first = starts[unit];
+    const int last = ends[unit];
+    if (flagged != 0) return;   // not lists of whole clusters: the atomic kernels run instead
     const int b = unit / clusters_per_image;
     const int g = unit - b * clusters_per_image;
     const int lane = threadIdx.x;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int first = starts[unit];
-    const int count = ends[unit] - first;
+    const int count = last - first;
     int* list = reinterpret_cast<int*>(stage + L_BASE);
     const int rows_here = min(8, N - 8 * g);   // the last cluster of a sequence may be short
     const int pad_from = N & 7;                // ... and the lists that name it hold row 0 in slots pad_from .. 7

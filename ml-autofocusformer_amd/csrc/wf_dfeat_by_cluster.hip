@@ -51,15 +51,19 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_by_cluster_kernel(const T* __r
     constexpr int LDS_BYTES = L_BASE + kListMax * 4;
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
-    if (not_whole != nullptr && *not_whole != 0) return;   // not lists of whole clusters: the atomic kernel runs instead
     const int unit = xcd_tile(blockIdx.x, total_clusters);
     if (unit < 0) return;
+    // the flag and the bounds of the cluster's list are requested together (one trip to memory, not two); the bounds
+    // mean nothing when the flag is set, and are not used then
+    const int flagged = not_whole != nullptr ? *not_whole : 0;
+    const int first = starts[unit];
+    const int last = ends[unit];
+    if (flagged != 0) return;   // not lists of whole clusters: the atomic kernel runs instead
     const int b = unit / clusters_per_image;
     const int g = unit - b * clusters_per_image;
     const int lane = threadIdx.x;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int first = starts[unit];
-    const int count = ends[unit] - first;
+    const int count = last - first;
     int* list = reinterpret_cast<int*>(stage + L_BASE);
     const char* d_out_b = reinterpret_cast<const char*>(d_out + (int64_t)b * Nout * kIC * C);
     const char* w_b = reinterpret_cast<const char*>(w + (int64_t)b * Nout * M * kIC);

@@ -28,15 +28,19 @@ __global__ __launch_bounds__(kWave) void wf_dfeat_rows_kernel(const T* __restric
                                                               const int32_t* __restrict__ only_if, T* __restrict__ d_feat,
                                                               int N, int Nout, int C, int M, int IC, int total_rows) {
     typedef VecIO<T, 4> Quad4;
-    if (only_if != nullptr && *only_if == 0) return;   // lists made of whole clusters: the other kernel has them
     const int row = xcd_tile(blockIdx.x, total_rows);
     if (row < 0) return;
+    // the flag and the bounds of the row's entries are requested together (one trip to memory, not two); the bounds
+    // mean nothing when the other kernel has the lists, and are not used then
+    const int wanted = only_if != nullptr ? *only_if : 1;
+    const int first = starts[row];
+    const int last = ends[row];
+    if (wanted == 0) return;   // lists made of whole clusters: the other kernel has them
     const int b = row / N;
     const int lane = threadIdx.x;
     const int ic = lane >> 4, c4 = lane & 15;
     const bool ic_ok = ic < IC;
-    const int first = starts[row];
-    const int count = ends[row] - first;
+    const int count = last - first;
     const T* d_out_b = d_out + (int64_t)b * Nout * IC * C;
     const T* w_b = w + (int64_t)b * Nout * M * IC;
     T* dst = d_feat + (int64_t)row * C;
