@@ -72,6 +72,28 @@ def test_model_like_lists_are_six_aligned_runs_of_eight():
     assert (canon.reshape(2, 784, 6, 8)[..., 0].diff(dim=-1) > 0).all()      # cluster ids ascending
 
 
+def test_model_built_lists_are_whole_clusters_of_neighbouring_tokens():
+    """Lists built by the balanced clustering itself: runs of whole clusters, the token's own cluster first, and
+    neighbouring clusters of the sequence sharing their neighbours (what the strips of `model_like_lists` lack)."""
+    for cluster, n in ((8, 784), (24, 600)):
+        idx = wl.model_built_lists(2, n, wl.generator(4), cluster=cluster, nnc=6)
+        assert idx.shape == (2, n, 6 * cluster) and int(idx.min()) >= 0 and int(idx.max()) < n
+        runs = idx.reshape(2, n, 6, cluster)
+        assert (runs[..., 0] % cluster == 0).all()
+        assert (runs == runs[..., :1] + torch.arange(cluster)).all()
+        own = torch.arange(n) // cluster
+        assert ((runs[..., 0] // cluster == own.view(1, n, 1)).any(dim=-1)).float().mean() > 0.95   # a token lists its own cluster
+        ids = runs[..., 0] // cluster                                      # (2, n, 6) cluster numbers
+        per_tile = ids[:, :n // cluster * cluster].reshape(2, -1, cluster * 6)
+        distinct = torch.tensor([[len(set(r.tolist())) for r in b] for b in per_tile]).float().mean()
+        assert 6 < float(distinct) < 14                                    # the tokens of a cluster pick from the same dozen
+    # a sequence that does not end on a cluster: pad slots hold row 0
+    idx = wl.model_built_lists(1, 100, wl.generator(5), cluster=8, nnc=4)
+    last = idx.reshape(1, 100, 4, 8)
+    short = last[last[..., 0] == 96]
+    assert short.numel() > 0 and (short[:, 4:] == 0).all() and (short[:, :4] == torch.arange(96, 100)).all()
+
+
 def test_algorithmic_bytes_match_the_published_table():
     # AFF-Tiny stage 1, fp32: QK = AV = 513.8 MB, WF IC4 = 321.1 MB, IC1 = 186.3 MB
     assert round(wl.attn_bytes(128, 2, 3136, 32, 48, 4) / 1e6, 1) == 513.8
