@@ -265,6 +265,29 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                       void* out, clusten_strides out_strides, float scale,
                                       clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* The same kernel with what it works out from cluster_idx, pe_idx and mask before its first head — the distinct
+ * clusters of every tile of 8 tokens, the bias-table row and mask bit of every slot, the runs a token repeats —
+ * handed over as a plan: the lists of a stage serve all its layers (models/aff_transformer.py:454-487 builds them once
+ * per stage, :505-507 runs the blocks on them), so the plan is built once per stage and read by every layer.
+ *   clusten_cluster_attention_plan_bytes(B, N): size of the plan for index tensors of B batch elements (B = 1 when
+ *   the lists are shared by every image);
+ *   clusten_cluster_attention_plan: fills it from cluster_idx (B,N,6) int32, pe_idx (B,N,48) int64 and mask (B,N,48)
+ *   int64 or NULL; plan 16-byte aligned (else CLUSTEN_ERR_UNALIGNED), plan_bytes at least the size above (else
+ *   CLUSTEN_ERR_WORKSPACE);
+ *   clusten_cluster_attention_forward_planned: clusten_cluster_attention_forward with `plan` in the place of the three
+ *   index tensors; same results bit for bit.
+ * No counterpart in the reference's extension modules. */
+size_t clusten_cluster_attention_plan_bytes(int B, int N);
+int clusten_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
+                                   size_t plan_bytes, int B, int N, clusten_stream stream);
+int clusten_cluster_attention_forward_planned(const void* query, clusten_strides query_strides,
+                                              const void* key, clusten_strides key_strides,
+                                              const void* value, clusten_strides value_strides,
+                                              const void* plan, const void* bias_table, int lists_shared,
+                                              const float* blank_key, const float* blank_value,
+                                              void* out, clusten_strides out_strides, float scale,
+                                              clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* ---- lists made of whole clusters: the backward scatters as gathers (optional) ------------------------------ */
 
 /* The pair lists of neighbour lists made of whole clusters, built on the device without any read-back by the host.

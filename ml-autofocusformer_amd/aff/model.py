@@ -37,6 +37,7 @@ def default_ops():
                            qk_clusters=_native.qk_forward_clusters, av_clusters=_native.av_forward_clusters,
                            clusters_supported=_native.clusters_supported,
                            cluster_attention=_native.cluster_attention,
+                           cluster_attention_plan=_native.cluster_attention_plan,
                            cluster_attention_supported=_native.cluster_attention_supported,
                            dense_attention=_native.dense_attention,
                            dense_attention_supported=_native.dense_attention_supported,
@@ -297,8 +298,10 @@ class ClusterAttention(nn.Module):
             # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
             # the values in one kernel; the query scale is applied to the scores inside it
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
+            plan = lists[3] if len(lists) > 3 else None     # what the kernel makes of the lists, once per stage
             out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], self.bias_table(table),
-                             lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale)
+                             lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale,
+                             **({"plan": plan} if plan is not None else {}))
             return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
         if (global_attn and dense is not None and not torch.is_grad_enabled()
@@ -558,6 +561,11 @@ class BasicLayer(nn.Module):
                                                   None if cluster_idx is None else cluster_idx.expand(b, -1, -1).contiguous())
                 if cluster_idx is not None:
                     grid_lists = (cluster_idx, pe_idx, mask)           # one image's lists, for the one-kernel attention
+                    planner = getattr(self.ops, "cluster_attention_plan", None)
+                    if planner is not None and not torch.is_grad_enabled() and cluster_idx.shape[2] == 6 and pe_idx.is_cuda:
+                        if (key, "plan") not in self._grid_cache:      # what that kernel makes of them, kept with them
+                            self._grid_cache[(key, "plan")] = planner(cluster_idx, pe_idx, mask)
+                        grid_lists = grid_lists + (self._grid_cache[(key, "plan")],)
                 member_idx, pe_idx, mask, cluster_idx = self._grid_cache[(key, b)]
                 pos = pos1.expand(b, -1, -1)
                 if ranking is not None and not feat_ordered:
@@ -571,6 +579,12 @@ class BasicLayer(nn.Module):
                     else:
                         feat = feat.gather(1, ranking.expand(-1, -1, feat.shape[2]))
 
+        planner = getattr(self.ops, "cluster_attention_plan", None)
+        if (grid_lists is None and cluster_idx is not None and planner is not None and not torch.is_grad_enabled()
+                and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda and feat.dtype != torch.float64
+                and torch.is_autocast_enabled("cuda")):
+            # the one-kernel attention of every block reads what it makes of the lists from a plan built once
+            grid_lists = (cluster_idx, pe_idx, mask, planner(cluster_idx, pe_idx, mask))
         carry = None
         for blk in self.blocks:
             feat, carry = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists, carry)

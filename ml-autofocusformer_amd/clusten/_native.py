@@ -57,6 +57,11 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
+    "clusten_cluster_attention_plan_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
+    "clusten_cluster_attention_plan": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_cluster_attention_forward_planned": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P,
+                                                                ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float,
+                                                                AttnShape, ctypes.c_int, _P]),
     "clusten_cluster_pairs_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "clusten_cluster_pairs": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                              ctypes.c_int, _P]),
@@ -680,9 +685,39 @@ def cluster_attention_supported(query: torch.Tensor, nnc: int) -> bool:
             and query.shape[3] == 32 and nnc == 6)
 
 
+def cluster_attention_plan(cluster_idx: torch.Tensor, pe_idx: torch.Tensor, mask) -> torch.Tensor:
+    """What `cluster_attention` works out from its three index tensors before its first head, for every tile of 8
+    tokens: a uint8 tensor to hand to every call that uses these lists (`plan=`), e.g. all layers of a stage.
+    cluster_idx (B,N,6) int32, pe_idx (B,N,48) int64, mask (B,N,48) of 0/1 or None — B = 1 for lists shared by every
+    image."""
+    lib = load()
+    _require_cuda("cluster_idx", cluster_idx)
+    device = cluster_idx.device
+    _require_cuda("pe_idx", pe_idx, device)
+    if cluster_idx.dim() != 3 or cluster_idx.shape[2] != 6:
+        raise RuntimeError("cluster_idx must be (B,N,6)")
+    lb, n = cluster_idx.shape[:2]
+    cidx = _cluster_idx(cluster_idx, (lb, n), device)
+    if pe_idx.shape != (lb, n, 48) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,48) like cluster_idx")
+    pe_idx = pe_idx.contiguous()
+    if mask is not None:
+        _require_cuda("mask", mask, device)
+        if mask.shape != (lb, n, 48):
+            raise RuntimeError("mask must have shape (B,N,48) like cluster_idx")
+        mask = mask.to(torch.int64).contiguous()
+    nbytes = lib.clusten_cluster_attention_plan_bytes(lb, n)
+    plan = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    if nbytes:
+        with torch.cuda.device(device):
+            _check(lib.clusten_cluster_attention_plan(_ptr(cidx), _ptr(pe_idx), _ptr(mask), _ptr(plan), nbytes, lb, n,
+                                                      _stream(device)), "clusten_cluster_attention_plan")
+    return plan
+
+
 def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cluster_idx: torch.Tensor,
                       bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_key: torch.Tensor,
-                      blank_value: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+                      blank_value: torch.Tensor, scale: float = 1.0, plan=None) -> torch.Tensor:
     """Local attention over the members of each token's clusters plus one blank token, in one kernel.
 
     query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
@@ -691,22 +726,35 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     Returns softmax(scale * q.k + bias - 100 * (1 - mask) | scale * q.blank_key) applied to the gathered values and
     the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the layout the output
     projection takes).  No autograd: for inference.  The fused form of models/aff_transformer.py:120-155.
+    `plan`: what `cluster_attention_plan` made of the same three index tensors; they are then not read (and may be
+    None), the result is the same.
     """
     lib = load()
     _require_cuda("query", query)
     device = query.device
     for name, t in (("key", key), ("value", value), ("bias_table", bias_table), ("pe_idx", pe_idx),
                     ("blank_key", blank_key), ("blank_value", blank_value)):
-        _require_cuda(name, t, device)
+        if not (plan is not None and t is None):
+            _require_cuda(name, t, device)
     if query.dim() != 4 or key.shape != query.shape or value.shape != query.shape:
         raise RuntimeError("query, key and value must be (B,H,N,C) tensors of one shape")
     b, h, n, c = query.shape
-    shared = b != 1 and cluster_idx.dim() == 3 and cluster_idx.shape[0] == 1
-    lb = 1 if shared else b
-    cidx = _cluster_idx(cluster_idx, (lb, n), device)
-    m = 8 * cidx.shape[2]
-    if pe_idx.shape != (lb, n, m) or pe_idx.dtype != torch.int64:
-        raise RuntimeError("pe_idx must be int64 of shape (B,N,M), or (1,N,M) like cluster_idx")
+    if plan is not None:
+        _require_cuda("plan", plan, device)
+        lb = b if plan.numel() == lib.clusten_cluster_attention_plan_bytes(b, n) else 1
+        if plan.dtype != torch.uint8 or plan.numel() != lib.clusten_cluster_attention_plan_bytes(lb, n):
+            raise RuntimeError("plan does not belong to lists of this shape")
+        shared = b != 1 and lb == 1
+        m = 48
+        cidx = pe_idx = mask = None
+    else:
+        shared = b != 1 and cluster_idx.dim() == 3 and cluster_idx.shape[0] == 1
+        lb = 1 if shared else b
+        cidx = _cluster_idx(cluster_idx, (lb, n), device)
+        m = 8 * cidx.shape[2]
+        if pe_idx.shape != (lb, n, m) or pe_idx.dtype != torch.int64:
+            raise RuntimeError("pe_idx must be int64 of shape (B,N,M), or (1,N,M) like cluster_idx")
+        pe_idx = pe_idx.contiguous()
     if bias_table.dim() != 2 or bias_table.shape[1] != h:
         raise RuntimeError("bias_table must have shape (rows, H)")
     if blank_key.numel() != h * c or blank_value.numel() != h * c:
@@ -715,7 +763,6 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     dtype = query.dtype
     query, key, value = _rows(query), _rows(key.to(dtype)), _rows(value.to(dtype))
     bias_table = bias_table.detach().to(dtype).contiguous()
-    pe_idx = pe_idx.contiguous()
     if mask is not None:
         _require_cuda("mask", mask, device)
         if mask.shape != (lb, n, m):
@@ -728,6 +775,15 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
         return out.reshape(b, n, h * c)
     out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
     shape = AttnShape(b, h, n, c, m)
+    if plan is not None:
+        with torch.cuda.device(device):
+            _check(lib.clusten_cluster_attention_forward_planned(_ptr(query), _strides(query), _ptr(key), _strides(key),
+                                                                 _ptr(value), _strides(value), _ptr(plan), _ptr(bias_table),
+                                                                 int(shared), _ptr(blank_key), _ptr(blank_value), _ptr(out),
+                                                                 _strides(out_view), ctypes.c_float(scale), shape, code,
+                                                                 _stream(device)),
+                   "clusten_cluster_attention_forward_planned")
+        return out.reshape(b, n, h * c)
     with torch.cuda.device(device):
         _check(lib.clusten_cluster_attention_forward(_ptr(query), _strides(query), _ptr(key), _strides(key),
                                                      _ptr(value), _strides(value), _ptr(cidx), _ptr(bias_table),

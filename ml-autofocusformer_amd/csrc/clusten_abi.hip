@@ -203,8 +203,43 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
         return CLUSTEN_ERR_BAD_STRIDE;
     }
     return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, cluster_idx, bias_table,
-                                    pe_idx, mask, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, shape,
-                                    dtype, as_stream(stream));
+                                    pe_idx, mask, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, nullptr,
+                                    shape, dtype, as_stream(stream));
+}
+
+size_t clusten_cluster_attention_plan_bytes(int B, int N) {
+    if (B <= 0 || N <= 0) return 0;
+    return cluster_attention_plan_bytes(B, N);
+}
+
+int clusten_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
+                                   size_t plan_bytes, int B, int N, clusten_stream stream) {
+    if (!cluster_idx || !pe_idx || !plan) return CLUSTEN_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (plan_bytes < cluster_attention_plan_bytes(B, N)) return CLUSTEN_ERR_WORKSPACE;
+    if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_cluster_attention_plan(cluster_idx, pe_idx, mask, plan, B, N, as_stream(stream));
+}
+
+int clusten_cluster_attention_forward_planned(const void* query, clusten_strides query_strides, const void* key,
+                                              clusten_strides key_strides, const void* value,
+                                              clusten_strides value_strides, const void* plan, const void* bias_table,
+                                              int lists_shared, const float* blank_key, const float* blank_value, void* out,
+                                              clusten_strides out_strides, float scale, clusten_attn_shape shape, int dtype,
+                                              clusten_stream stream) {
+    if (!query || !key || !value || !plan || !bias_table || !blank_key || !blank_value || !out) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
+        !strides_ok(out_strides, shape.C)) {
+        return CLUSTEN_ERR_BAD_STRIDE;
+    }
+    if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, nullptr, bias_table,
+                                    nullptr, nullptr, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, plan,
+                                    shape, dtype, as_stream(stream));
 }
 
 size_t clusten_cluster_pairs_bytes(int B, int rows, int M, int n_rows) {

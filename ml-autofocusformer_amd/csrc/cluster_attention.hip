@@ -69,6 +69,16 @@ static_assert(P_BYTES % 16 == 0 && P_BYTES <= kPassRows * kRB, "the probabilitie
 static_assert(kTileTokens * kSRow * 4 <= kPassRows * kRB, "the scores fit the K area");
 static_assert(kPassRows % 32 == 0 && Q_BASE % 16 == 0, "whole 32-row steps");
 
+// A tile's plan: what the kernel works out from the index tensors before its first head — the distinct clusters of
+// the tile, and per lane the bias-table rows (sign bit: masked slot), the distinct-cluster number of each run of its
+// token and the runs that repeat an earlier one.  The lists of a stage serve all its layers, so the plan is built once
+// per stage (cluster_attention_plan_kernel) and read back by every layer in two 16-byte loads per lane:
+//   [0, 16)            U, the number of distinct clusters
+//   [16, 16 + 192)     their cluster numbers
+//   [256, 256 + 2048)  per lane: pe[6] (24 bytes), us[6] (6 bytes), repeats (1 byte), 1 byte unused
+constexpr int kPlanLane = 256;
+constexpr int kPlanBytes = kPlanLane + kWave * 32;
+
 // Reductions over the 8 lanes of a token (lanes 8t .. 8t+7) with data-parallel-primitive moves: neighbours in a
 // quad, the other pair of the quad, then the mirrored lane of the other quad.  Every lane ends with the same value.
 template <int CTRL>
@@ -86,13 +96,90 @@ __device__ __forceinline__ float oct_sum(float v) {
     return v + dpp_move<0x141>(v);
 }
 
+// What a tile works out from the index tensors: `tok` = row of the lane's token (lane / 8) in them, `list_b` their
+// batch element.  Lane (t, i) = member i of the runs of token t.
+__device__ __forceinline__ void tile_setup(const int32_t* __restrict__ cluster_idx, const int64_t* __restrict__ pe_idx,
+                                           const int64_t* __restrict__ mask, int64_t list_b, int N, int i0, int nt,
+                                           int64_t tok, int (&pe)[kR], int (&us)[kR], int& repeats, int& U, int* ulist) {
+    const int lane = threadIdx.x;
+    const int t = lane >> 3, i = lane & 7;
+    // cluster numbers: lane rho < 48 owns run rho = token * 6 + run of the tile
+    const int rho = min(lane, kTileTokens * kR - 1);
+    const int cid = cluster_idx[(list_b * N + i0 + min(rho / kR, nt - 1)) * kR + rho % kR];
+    {
+        int64_t wide[kR];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) wide[r] = pe_idx[tok * kM + 8 * r + i];
+#pragma unroll
+        for (int r = 0; r < kR; ++r) pe[r] = (int)wide[r] & 0x7fffffff;
+        if (mask) {
+#pragma unroll
+            for (int r = 0; r < kR; ++r) wide[r] = mask[tok * kM + 8 * r + i];
+#pragma unroll
+            for (int r = 0; r < kR; ++r) pe[r] |= wide[r] == 0 ? (int)0x80000000 : 0;
+        }
+    }
+    // number the distinct cluster numbers in order of first appearance
+    uint64_t remaining = (1ull << (kTileTokens * kR)) - 1;
+    int uslot = 0;
+    bool first = false;
+    U = 0;
+    while (remaining != 0) {
+        const int s = __builtin_ctzll(remaining);
+        const int cs = __builtin_amdgcn_readlane(cid, s);
+        const bool hit = cid == cs;
+        const uint64_t match = __ballot(hit) & remaining;
+        if (hit) uslot = U;
+        first = first || lane == s;
+        remaining &= ~match;
+        ++U;
+    }
+    if (first) ulist[uslot] = cid;
+#pragma unroll
+    for (int r = 0; r < kR; ++r) us[r] = __shfl(uslot, t * kR + r);
+    // does a token of the tile list a cluster twice?  Bit r: run r repeats an earlier run of the token; its
+    // probability is then added to that run's before the probabilities are laid out by distinct cluster.
+    repeats = 0;
+#pragma unroll
+    for (int r = 1; r < kR; ++r) {
+#pragma unroll
+        for (int r2 = 0; r2 < r; ++r2) repeats |= us[r] == us[r2] ? 1 << r : 0;
+    }
+}
+
+// One wave per tile: the plan of every tile of the index tensors (B_lists batch elements).
+__global__ __launch_bounds__(kWave) void cluster_attention_plan_kernel(const int32_t* __restrict__ cluster_idx,
+                                                                       const int64_t* __restrict__ pe_idx,
+                                                                       const int64_t* __restrict__ mask,
+                                                                       char* __restrict__ plan, int N, int tiles_per_batch,
+                                                                       int total_tiles) {
+    __shared__ int ulist[kTileTokens * kR];
+    const int tile = blockIdx.x;
+    if (tile >= total_tiles) return;
+    const int b = tile / tiles_per_batch;
+    const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
+    const int nt = min(kTileTokens, N - i0);
+    const int lane = threadIdx.x;
+    const int64_t tok = (int64_t)b * N + i0 + min(lane >> 3, nt - 1);
+    int pe[kR], us[kR], repeats, U;
+    tile_setup(cluster_idx, pe_idx, mask, b, N, i0, nt, tok, pe, us, repeats, U, ulist);
+    lds_sync();
+    char* mine = plan + (int64_t)tile * kPlanBytes;
+    if (lane == 0) *reinterpret_cast<int*>(mine) = U;
+    if (lane < kTileTokens * kR) *reinterpret_cast<int*>(mine + 16 + lane * 4) = lane < U ? ulist[lane] : 0;
+    const uint32_t w2 = (uint32_t)us[0] | ((uint32_t)us[1] << 8) | ((uint32_t)us[2] << 16) | ((uint32_t)us[3] << 24);
+    const uint32_t w3 = (uint32_t)us[4] | ((uint32_t)us[5] << 8) | ((uint32_t)repeats << 16);
+    *reinterpret_cast<Piece*>(mine + kPlanLane + lane * 32) = Piece{(uint32_t)pe[0], (uint32_t)pe[1], (uint32_t)pe[2], (uint32_t)pe[3]};
+    *reinterpret_cast<Piece*>(mine + kPlanLane + lane * 32 + 16) = Piece{(uint32_t)pe[4], (uint32_t)pe[5], w2, w3};
+}
+
 template <typename T>
 __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const T* __restrict__ q, clusten_strides qs, const T* __restrict__ k, clusten_strides ks, const T* __restrict__ v,
     clusten_strides vs, const int32_t* __restrict__ cluster_idx, const T* __restrict__ table,
     const int64_t* __restrict__ pe_idx, const int64_t* __restrict__ mask, const float* __restrict__ blank_k,
     const float* __restrict__ blank_v, T* __restrict__ out, clusten_strides os, int H_all, int N, float scale,
-    int tiles_per_batch, int total_tiles, int lists_shared, int head_groups) {
+    int tiles_per_batch, int total_tiles, int lists_shared, int head_groups, const char* __restrict__ plan) {
     typedef short S4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) S4* LdsS4;
 
@@ -132,52 +219,25 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     fetch_q(0);
     if (H > 1) fetch_q(1);
 
-    // cluster numbers: lane rho < 48 owns run rho = token * 6 + run of the tile
-    const int rho = min(lane, kTileTokens * kR - 1);
-    const int cid = cluster_idx[(list_b * N + i0 + min(rho / kR, nt - 1)) * kR + rho % kR];
-
-    // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
-    int pe[kR];
-    {
-        int64_t wide[kR];
-#pragma unroll
-        for (int r = 0; r < kR; ++r) wide[r] = pe_idx[tok * kM + 8 * r + i];
-#pragma unroll
-        for (int r = 0; r < kR; ++r) pe[r] = (int)wide[r] & 0x7fffffff;
-        if (mask) {
-#pragma unroll
-            for (int r = 0; r < kR; ++r) wide[r] = mask[tok * kM + 8 * r + i];
-#pragma unroll
-            for (int r = 0; r < kR; ++r) pe[r] |= wide[r] == 0 ? (int)0x80000000 : 0;
-        }
-    }
-
-    // number the distinct cluster numbers in order of first appearance
-    uint64_t remaining = (1ull << (kTileTokens * kR)) - 1;
-    int uslot = 0, U = 0;
-    bool first = false;
-    while (remaining != 0) {
-        const int s = __builtin_ctzll(remaining);
-        const int cs = __builtin_amdgcn_readlane(cid, s);
-        const bool hit = cid == cs;
-        const uint64_t match = __ballot(hit) & remaining;
-        if (hit) uslot = U;
-        first = first || lane == s;
-        remaining &= ~match;
-        ++U;
-    }
+    int pe[kR];      // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
+    int us[kR];      // distinct-cluster number of this lane's token's runs
+    int repeats = 0; // bit r: run r repeats an earlier run of the token; its probability is added to that run's
+    int U = 0;
     int* ulist = reinterpret_cast<int*>(stage + UL_BASE);
-    if (first) ulist[uslot] = cid;
-    int us[kR];  // distinct-cluster number of this lane's token's runs
-#pragma unroll
-    for (int r = 0; r < kR; ++r) us[r] = __shfl(uslot, t * kR + r);
-    // does a token of the tile list a cluster twice?  Bit r: run r repeats an earlier run of the token; its
-    // probability is then added to that run's before the probabilities are laid out by distinct cluster.
-    int repeats = 0;
-#pragma unroll
-    for (int r = 1; r < kR; ++r) {
-#pragma unroll
-        for (int r2 = 0; r2 < r; ++r2) repeats |= us[r] == us[r2] ? 1 << r : 0;
+    if (plan != nullptr) {
+        // the tile's plan, built once for all layers that use these lists
+        const char* mine = plan + (list_b * tiles_per_batch + (tile - b * tiles_per_batch)) * (int64_t)kPlanBytes;
+        const Piece lo = *reinterpret_cast<const Piece*>(mine + kPlanLane + lane * 32);
+        const Piece hi = *reinterpret_cast<const Piece*>(mine + kPlanLane + lane * 32 + 16);
+        U = *reinterpret_cast<const int*>(mine);
+        if (lane < kTileTokens * kR) ulist[lane] = *reinterpret_cast<const int*>(mine + 16 + lane * 4);
+        pe[0] = (int)lo[0]; pe[1] = (int)lo[1]; pe[2] = (int)lo[2]; pe[3] = (int)lo[3];
+        pe[4] = (int)hi[0]; pe[5] = (int)hi[1];
+        us[0] = hi[2] & 0xff; us[1] = (hi[2] >> 8) & 0xff; us[2] = (hi[2] >> 16) & 0xff; us[3] = hi[2] >> 24;
+        us[4] = hi[3] & 0xff; us[5] = (hi[3] >> 8) & 0xff;
+        repeats = (hi[3] >> 16) & 0xff;
+    } else {
+        tile_setup(cluster_idx, pe_idx, mask, list_b, N, i0, nt, tok, pe, us, repeats, U, ulist);
     }
     const bool twice = __any(repeats) != 0;
     lds_sync();
@@ -395,24 +455,38 @@ template <typename T>
 int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out, clusten_strides os,
-                 float scale, int lists_shared, const clusten_attn_shape& s, hipStream_t stream) {
+                 float scale, int lists_shared, const void* plan, const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int groups = head_groups_for(total, s.H);  // 196 tokens x 8 heads, B = 128: 69.6 -> 63.9 us
     hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total * groups)), dim3(kWave), 0, stream,
                        static_cast<const T*>(q), qs, static_cast<const T*>(k), ks, static_cast<const T*>(v), vs,
                        cluster_idx, static_cast<const T*>(table), pe_idx, mask, blank_k, blank_v, static_cast<T*>(out),
-                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups);
+                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups, static_cast<const char*>(plan));
     return launch_status();
 }
 
 }  // namespace
 
+size_t cluster_attention_plan_bytes(int B, int N) {
+    return (size_t)B * ((N + kTileTokens - 1) / kTileTokens) * kPlanBytes;
+}
+
+int launch_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
+                                  int B, int N, hipStream_t stream) {
+    const int tiles_per_batch = (N + kTileTokens - 1) / kTileTokens;
+    const int64_t total = (int64_t)B * tiles_per_batch;
+    if (total <= 0 || total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
+    hipLaunchKernelGGL(cluster_attention_plan_kernel, dim3((unsigned)total), dim3(kWave), 0, stream, cluster_idx, pe_idx, mask,
+                       static_cast<char*>(plan), N, tiles_per_batch, (int)total);
+    return launch_status();
+}
+
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
-                             hipStream_t stream) {
+                             clusten_strides os, float scale, int lists_shared, const void* plan, clusten_attn_shape s,
+                             int dtype, hipStream_t stream) {
     if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
     if (s.C != kC || s.M != kM) return CLUSTEN_ERR_BAD_DIMS;
     const bool ok = rows_aligned16(q, qs, 2) && rows_aligned16(k, ks, 2) && rows_aligned16(v, vs, 2) &&
@@ -421,10 +495,10 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
     if (!ok) return CLUSTEN_ERR_UNALIGNED;
     if (dtype == CLUSTEN_F16) {
         return launch_typed<f16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                   lists_shared, s, stream);
+                                   lists_shared, plan, s, stream);
     }
     return launch_typed<bf16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                lists_shared, s, stream);
+                                lists_shared, plan, s, stream);
 }
 
 }  // namespace clusten

@@ -79,8 +79,13 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, int lists_shared, clusten_attn_shape s, int dtype,
-                             hipStream_t stream);
+                             clusten_strides os, float scale, int lists_shared, const void* plan, clusten_attn_shape s,
+                             int dtype, hipStream_t stream);
+// The per-tile plan the kernel above reads instead of cluster_idx, pe_idx and mask when it is given one (what it
+// would work out from them before its first head): B = batch elements of the index tensors.
+size_t cluster_attention_plan_bytes(int B, int N);
+int launch_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
+                                  int B, int N, hipStream_t stream);
 
 // The pair lists of lists made of whole clusters (cluster_pairs.hip), built on the device: for `rows` list rows per
 //   image of M slots that point into a sequence of D rows (K = ceil(D/8) clusters), pairs[starts[b*K+g] .. ends[b*K+g])

@@ -169,3 +169,34 @@ def test_cluster_numbers_out_of_range_read_row_zero(device):
     d = lambda x: x.to(device)
     out = _native.cluster_attention(d(q), d(k), d(v), d(wild), d(table), d(pe_idx), None, d(blank_k), d(blank_v), scale=0.2)
     assert oracle.rel_err(out, ref) <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
+def test_plan_built_once_gives_the_same_bits(device, kind):
+    """What the kernel works out from the index tensors, handed over as a plan (one per stage, read by every layer):
+    the result is bit-equal to the call that reads the tensors, for every kind of list, with and without a mask, on
+    partial tiles, and for lists shared by the batch."""
+    gen = torch.Generator().manual_seed(87)
+    d = lambda x: None if x is None else x.to(device)
+    for b, h, n in ((2, 3, 396), (1, 1, 64), (3, 4, 200)):
+        for with_mask in (False, True):
+            q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, torch.float16, with_mask)
+            plain = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k),
+                                              d(blank_v), scale=0.2)
+            plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+            assert plan.dtype == torch.uint8 and plan.numel() == _native.load().clusten_cluster_attention_plan_bytes(b, n)
+            for _ in range(2):      # the plan serves any number of calls
+                planned = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                    scale=0.2, plan=plan)
+                assert torch.equal(planned, plain)
+    # one image's lists for the whole batch
+    b, h, n = 3, 2, 200
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, torch.bfloat16, True)
+    c1, p1, m1 = cidx[:1].contiguous(), pe_idx[:1].contiguous(), mask[:1].contiguous()
+    plain = _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(p1), d(m1), d(blank_k), d(blank_v))
+    plan1 = _native.cluster_attention_plan(d(c1), d(p1), d(m1))
+    assert torch.equal(_native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                 plan=plan1), plain)
+    with pytest.raises(RuntimeError):       # a plan of other lists
+        _native.cluster_attention(d(q)[:, :, :64], d(k)[:, :, :64], d(v)[:, :, :64], None, d(table), None, None,
+                                  d(blank_k), d(blank_v), plan=plan1)
