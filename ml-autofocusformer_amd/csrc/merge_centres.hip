@@ -223,6 +223,14 @@ template <typename T>
 int launch_typed(const float* pos, const float* min_dist, const void* prob, int64_t* centre, int B, int N, int sample_num,
                  int reserve_num, int reserve_on, float alpha, int stride, hipStream_t stream) {
     const size_t lds = ((size_t)N + 256 + 16 + 4) * 4;
+    if (lds > 48 * 1024) {
+        // more LDS than a workgroup gets without asking (a CU of this device holds 160 KB)
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(merge_centres_kernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return CLUSTEN_ERR_BAD_DIMS;
+        }
+    }
     hipLaunchKernelGGL(merge_centres_kernel<T>, dim3((unsigned)B), dim3(kMergeThreads), lds, stream,
                        reinterpret_cast<const float2*>(pos), min_dist, static_cast<const T*>(prob), centre, N, sample_num,
                        reserve_num, reserve_on, alpha, stride);
@@ -231,7 +239,18 @@ int launch_typed(const float* pos, const float* min_dist, const void* prob, int6
 
 }  // namespace
 
-int merge_centres_max_tokens() { return (48 * 1024 - (256 + 16 + 4) * 4) / 4; }
+// The longest sequence whose keys the selecting workgroup holds in LDS; a thread owns at most 64 tokens (the
+// reserved-token bits of its share are one 64-bit word).
+int merge_centres_max_tokens() {
+    int dev = 0, bytes = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        bytes = 48 * 1024;
+    }
+    const int by_lds = (bytes - (256 + 16 + 4) * 4) / 4;
+    return by_lds < 64 * kMergeThreads ? by_lds : 64 * kMergeThreads;
+}
 
 int launch_merge_centres(const float* pos, const float* min_dist, const void* prob, int prob_dtype, int64_t* centre, int B,
                          int N, int sample_num, int reserve_num, int reserve_on, float alpha, int stride,

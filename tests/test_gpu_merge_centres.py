@@ -119,6 +119,18 @@ def test_centres_of_the_first_stage_of_a_384_model(device):
     assert torch.equal(got.cpu(), _expected(score, reserved, keep - reserve_num, reserve_num))
 
 
+def test_centres_of_a_sequence_past_48_kb_of_keys(device):
+    b, h, w = 2, 128, 128                      # the first stage of a 512 x 512 image: 16 384 tokens, 64 KB of keys
+    pos = _grid(b, h, w, device)
+    n = h * w
+    assert n <= _native.load().clusten_merge_centres_max_tokens()
+    prob = torch.rand(b, n, 1, generator=torch.Generator().manual_seed(10)).to(device)
+    keep, reserve_num = n // 4, 32 * 32
+    got = _native.merge_centres(pos, None, prob, 4.0, 2, keep - reserve_num, reserve_num, True)
+    score, reserved, _ = _scores(pos, prob, 4.0, 2, True)
+    assert torch.equal(got.cpu(), _expected(score, reserved, keep - reserve_num, reserve_num))
+
+
 def test_refusals(device):
     pos = _grid(1, 8, 8, device)
     with pytest.raises(RuntimeError):
