@@ -10,7 +10,8 @@
 //   shared-list path — all tokens of the tile carry the same list: the 8 products that go to one
 //     destination row are summed in registers and leave the wave as ONE fp32 atomic per (slot,
 //     channel): 8x fewer atomics than one per product, and each wave-wide atomic instruction adds
-//     to whole contiguous rows.
+//     to whole contiguous rows.  (Lists of at most 64 slots: such tiles are taken beforehand by
+//     scatter_rows_window.hip, which sums many tiles in LDS first, and are skipped here.)
 //   union path — lists that differ but are made of runs of 8 slots of which the tile's tokens share most (the
 //     neighbourhoods of a cluster-ordered sequence: a run is the 8 members of one cluster; a tile of the model's own
 //     lists holds 8-12 distinct runs): the runs are numbered by distinct value as in the forward kernels, p is laid
@@ -35,7 +36,8 @@ namespace clusten {
 template <typename T, int C, int Q, bool GUARD>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void scatter_rows_tile_kernel(
     const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out, int H,
-    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles, const int32_t* __restrict__ only_if) {
+    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles, const int32_t* __restrict__ only_if,
+    const uint8_t* __restrict__ handled) {
     constexpr int HPW = kWave / C;
     constexpr int SLOTS = 16 * Q;
     static_assert(C == 16 || C == 32 || C == 64, "a row of 16 lanes must stay inside one head");
@@ -45,6 +47,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
+    if (handled != nullptr && handled[tile] != 0) return;   // the window kernel has added this tile
     {
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
@@ -268,21 +271,21 @@ __global__ __launch_bounds__(256) void scatter_rows_elem_kernel(const T* __restr
 
 template <typename T, int C, int Q, bool GUARD>
 int scatter_tile_q(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
-                   const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
+                   const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if, const uint8_t* handled) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int grid = xcd_grid(total);
     hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(x), idx, out, s.H, s.N, s.M, xs,
-                       tiles_per_batch, total, only_if);
+                       tiles_per_batch, total, only_if, handled);
     return launch_status();
 }
 
 template <typename T, int C>
 int scatter_tile(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* out,
-                 const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
-    if (s.M == 48) return scatter_tile_q<T, C, 3, false>(p, x, xs, idx, out, s, stream, only_if);
-    return scatter_tile_q<T, C, 4, true>(p, x, xs, idx, out, s, stream, only_if);
+                 const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if, const uint8_t* handled) {
+    if (s.M == 48) return scatter_tile_q<T, C, 3, false>(p, x, xs, idx, out, s, stream, only_if, handled);
+    return scatter_tile_q<T, C, 4, true>(p, x, xs, idx, out, s, stream, only_if, handled);
 }
 
 template <typename T, typename A>
@@ -296,16 +299,22 @@ int scatter_elem(const void* p, const void* x, clusten_strides xs, const int64_t
     return launch_status();
 }
 
-// Accumulate into the zeroed fp32 buffer `acc32` (which is `out` itself for fp32 storage).
+// Whether the tile kernel takes this scatter (otherwise one thread per element does).
+template <typename T>
+bool scatter_tiles_ok(const void* p, const clusten_attn_shape& s) {
+    return s.M % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0 && (s.C == 16 || s.C == 32 || s.C == 64);
+}
+
+// Accumulate into the zeroed fp32 buffer `acc32` (which is `out` itself for fp32 storage).  `handled` (may be null)
+// marks the tiles that the window kernel has added already; it is read only when scatter_tiles_ok().
 template <typename T>
 int scatter_rows_typed(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* acc32,
-                       const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
-    const bool quads_ok = s.M % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0;
-    if (quads_ok) {
+                       const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if, const uint8_t* handled) {
+    if (scatter_tiles_ok<T>(p, s)) {
         switch (s.C) {
-            case 16: return scatter_tile<T, 16>(p, x, xs, idx, acc32, s, stream, only_if);
-            case 32: return scatter_tile<T, 32>(p, x, xs, idx, acc32, s, stream, only_if);
-            case 64: return scatter_tile<T, 64>(p, x, xs, idx, acc32, s, stream, only_if);
+            case 16: return scatter_tile<T, 16>(p, x, xs, idx, acc32, s, stream, only_if, handled);
+            case 32: return scatter_tile<T, 32>(p, x, xs, idx, acc32, s, stream, only_if, handled);
+            case 64: return scatter_tile<T, 64>(p, x, xs, idx, acc32, s, stream, only_if, handled);
             default: break;
         }
     }

@@ -368,6 +368,48 @@ def test_scatter_integer_valued_data_is_bit_exact(device):
         assert torch.equal(dq.cpu(), dq_ref) and torch.equal(dk.cpu(), dk_ref)
 
 
+def _tile_shared_lists(B, N, M, gen, kind):
+    """(B,N,M) lists in which the 8 tokens of a tile share one list (`mixed`: every other tile does)."""
+    tiles = (N + 7) // 8
+    if kind == "near":
+        return wl.windowed_cluster_lists(B, N, M, gen)
+    per_tile = torch.randint(N, (B, tiles, M), generator=gen)                  # rows anywhere in the image
+    if kind == "repeats":
+        per_tile[:, :, M // 2:] = per_tile[:, :, :M - M // 2]                   # every row named twice
+    idx = per_tile.repeat_interleave(8, dim=1)[:, :N].contiguous()
+    if kind == "mixed":
+        own = torch.randint(N, (B, N, M), generator=gen)
+        odd = (torch.arange(N) // 8) % 2 == 1
+        idx[:, odd] = own[:, odd]
+    return idx
+
+
+@pytest.mark.parametrize("kind", ["near", "far", "repeats", "mixed"])
+@pytest.mark.parametrize("c,m,n,dtype", [(32, 48, 1501, torch.float32), (32, 48, 1501, torch.bfloat16),
+                                         (16, 20, 1100, torch.float32), (64, 64, 613, torch.float16),
+                                         (32, 4, 37, torch.float32), (64, 12, 300, torch.float32)])
+def test_scatter_of_tiles_that_share_a_list(device, kind, c, m, n, dtype):
+    """The tiles whose tokens share one list are summed in an LDS window of destination rows before they reach
+    memory (rows outside the window are added directly), the other tiles by the tile kernel: sequences longer than
+    one window, rows far from their tile, rows named twice, tiles of both sorts side by side, a short last tile."""
+    g = torch.Generator().manual_seed(79)
+    B, H = 2, 3
+    idx = _tile_shared_lists(B, n, m, g, kind)
+    q = torch.randn(B, H, n, c, generator=g).to(dtype)
+    k = torch.randn(B, H, n, c, generator=g).to(dtype)
+    d_attn = torch.randn(B, H, n, m, generator=g).to(dtype)
+    dq_ref, dk_ref = oracle.qk_gather_backward(_ref(d_attn), _ref(q), _ref(k), idx)
+    dq, dk = _native.qk_backward(d_attn.to(device), q.to(device), k.to(device), idx.to(device))
+    assert oracle.rel_err(dq, dq_ref) <= TOL[dtype]
+    assert oracle.rel_err(dk, dk_ref) <= _scatter_tol(dtype)
+    # integer-valued data: every sum is exact in fp32, whatever the order of the additions
+    qi = torch.randint(-4, 5, (B, H, n, c), generator=g).to(dtype)
+    di = torch.randint(-4, 5, (B, H, n, m), generator=g).to(dtype)
+    _, dk_ref = oracle.qk_gather_backward(_ref(di), _ref(qi), _ref(qi), idx)
+    _, dk = _native.qk_backward(di.to(device), qi.to(device), qi.to(device), idx.to(device))
+    assert torch.equal(dk.float().cpu(), dk_ref.to(dtype).float())
+
+
 def test_scatter_conserves_mass_at_full_size(device):
     """Configuration 3's backward shape at full size (B64 H4 N9216 C32, fp32): the sum of d_key over
     destination rows equals the sum of all products whatever the indices are, and three batch
