@@ -110,8 +110,9 @@ int clusten_qk_forward(const void* query, clusten_strides query_strides,
  * d_query, d_key are (B,H,N,C) contiguous, need not be zeroed.  `workspace` (clusten_qk_backward_workspace_bytes,
  * 16-byte aligned) holds what the scatter needs: the pair lists of lists made of whole clusters (see
  * clusten_cluster_pairs below: built on every call; such lists take a gather without atomics whose sums repeat bit
- * for bit, chosen on the device — the host reads nothing back) and, for F16/BF16, the fp32 sums of the atomic
- * kernels that any other list takes (rounded once). */
+ * for bit, chosen on the device — the host reads nothing back), one byte per tile of 8 tokens (which tiles the
+ * kernel that sums shared lists in LDS has added) and, for F16/BF16, the fp32 sums of the atomic kernels that any
+ * other list takes (rounded once). */
 size_t clusten_qk_backward_workspace_bytes(clusten_attn_shape shape, int dtype);
 int clusten_qk_backward(const void* d_attn,
                         const void* query, clusten_strides query_strides,

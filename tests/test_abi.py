@@ -102,9 +102,10 @@ def test_workspace_contract():
     assert lib.clusten_qk_backward_workspace_bytes(s, 3) == 0          # fp64: atomics straight into d_key
     pairs = lib.clusten_cluster_pairs_bytes(2, 16, 8, 16)              # the pair lists of (B,N,M) lists over N rows
     assert pairs > 0 and pairs % 256 == 0
-    assert lib.clusten_qk_backward_workspace_bytes(s, 0) == pairs      # fp32 accumulates in place
+    tiles = 256                                                        # one byte per tile of 8 tokens, to 256 bytes
+    assert lib.clusten_qk_backward_workspace_bytes(s, 0) == pairs + tiles   # fp32 accumulates in place
     need = lib.clusten_qk_backward_workspace_bytes(s, 1)
-    assert need == pairs + 2 * 2 * 16 * 32 * 4                          # ... plus one fp32 per d_key element
+    assert need == pairs + tiles + 2 * 2 * 16 * 32 * 4                  # ... plus one fp32 per d_key element
     assert lib.clusten_av_backward_workspace_bytes(s, 2) == need
     odd = _shape(B=2, H=2, N=16, C=32, M=5)                            # no runs of 8: no pair lists
     assert lib.clusten_qk_backward_workspace_bytes(odd, 0) == 0
