@@ -5,28 +5,29 @@
 //                                                          clusten/src/clustenav_cuda_kernel.cu:93-127)
 //
 // Neighbour lists name rows near their own token, so consecutive tiles add to the same few hundred rows.  A workgroup
-// of 16 waves takes G consecutive tiles of one image and keeps an fp32 window of the destination rows around them in
-// LDS: 128 KB of cells, at 32 channels 1024 rows for 64 tiles, [first token - 256, first token + 768).  Per head:
-// every wave forms, for each of its tiles, D[slot][c] = sum_t p[t][slot] * x[t][c] on the matrix cores (operands
-// straight from memory in the instruction's layout, those of the wave's next tile requested before the present one
-// is used) and adds D into the window; a row outside the window is added to memory directly.  After a barrier the
-// non-zero cells of the window leave as one memory atomic each and are cleared for the next head.  A row is inside
-// the windows of two workgroups, so it receives two memory atomics per channel instead of one per tile that names it
-// (six at 48 neighbours).
+// of 16 waves takes 64 consecutive tiles of one image (512 tokens) and 16 of the head's channels, and keeps an fp32
+// window of the 1024 destination rows around those tokens, [first token - 256, first token + 768), in LDS (64 KB of
+// cells; two workgroups share a CU).  Per head: every wave forms, for each of its four tiles, D[slot][c] = sum_t
+// p[t][slot] * x[t][c] on the matrix cores (operands straight from memory in the instruction's layout) and adds D
+// into the window; a row outside the window is added to memory directly.  After a barrier the non-zero cells of the
+// window leave as one memory atomic each and are cleared for the next head.  A row is inside the windows of two
+// groups of tiles, so it receives two memory atomics per channel instead of one per tile that names it (six at 48
+// neighbours).
 //
 // The additions to the window are compare-and-swap loops on the cells' bits, not `ds_add_f32`: this device adds
 // floats in LDS one lane at a time (measured: 193 clocks per 64-lane instruction, whatever the addresses; an integer
 // add takes 5, a read and a write 6-10), which made the first form of this kernel 2.7 times slower than the atomics
-// to memory it replaces.  Cells are read, then swapped, eight at a time per lane; a lane goes round again only when
-// another wave, or another lane naming the same row, changed its cell in between.
+// to memory it replaces.  The four cells of a lane are read, then swapped; a lane goes round again only when another
+// wave, or another lane naming the same row, changed its cell in between.
 //
 // Which tiles have one list is found here and written to `handled` (one byte per tile); the tile kernel that follows
 // skips those tiles and takes the rest, so the two kernels together add every product exactly once.
 //
-// Measured at B128 H2 N3136 C32 M48 fp32 on lists shared by each cluster of 8 tokens (+-256-token window): 320 us
-// against the 471 us of one memory atomic per (tile, slot, channel).  Of the 320: finding the shared lists and
-// clearing the window 60, operand loads 60, matrix products and their row numbers 70, the additions 100, the
-// window's way to memory 45 - one workgroup per CU (the window fills its LDS), so these do not overlap.
+// Measured at B128 H2 N3136 C32 M48 fp32 on lists shared by each cluster of 8 tokens (+-256-token window): 255 us
+// against the 471 us of one memory atomic per (tile, slot, channel).  With all 32 channels of a head in one
+// workgroup (a 128 KB window, one workgroup per CU, the next tile's operands requested ahead) it took 311 us: the
+// phases of a workgroup - finding the shared lists, operand loads, products, additions, the window's way to memory -
+// do not overlap, and a second workgroup on the CU fills the gaps although it reads p and the lists a second time.
 #include "launch.hpp"
 #include "mfma.hpp"
 
@@ -34,27 +35,31 @@ namespace clusten {
 namespace {
 
 constexpr int kWindowWaves = 16;
-constexpr int kWindowCells = 32768;   // fp32 cells of the window, without the padding
+constexpr int kWindowRows = 1024;                              // destination rows of the window
+constexpr int kWindowTiles = 64;                               // tiles of a workgroup: half the window
+constexpr int kWindowTilesPerWave = kWindowTiles / kWindowWaves;
+constexpr int kWindowStride = 17;   // floats per row: odd, the rows of one access fall into different banks
+constexpr int kWindowLds = kWindowRows * kWindowStride * (int)sizeof(float);
 
-// Tiles of a group: their tokens span half the window, and a wave has at most four tiles (their lists stay in registers)
-constexpr int window_group_tiles(int C) { return kWindowCells / C / 16 < 64 ? kWindowCells / C / 16 : 64; }
-
-template <typename T, int C>
-__global__ __launch_bounds__(kWindowWaves* kWave) void scatter_rows_window_kernel(
+// 8 waves per SIMD: two workgroups of 16 waves on a CU
+template <typename T>
+__global__ __launch_bounds__(kWindowWaves* kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) void scatter_rows_window_kernel(
     const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out,
-    uint8_t* __restrict__ handled, int H, int N, int M, clusten_strides xs, int tiles_per_image, int groups_per_image,
-    int total_groups, const int32_t* __restrict__ only_if) {
-    constexpr int ROWS = kWindowCells / C;
-    constexpr int G = window_group_tiles(C);     // tiles of a group
-    constexpr int TPW = G / kWindowWaves;        // tiles of a wave
-    constexpr int STRIDE = C + 1;                // odd: the rows of one atomic instruction fall into different banks
+    uint8_t* __restrict__ handled, int H, int N, int M, int C, clusten_strides xs, int tiles_per_image,
+    int groups_per_image, int total_units, const int32_t* __restrict__ only_if) {
+    constexpr int ROWS = kWindowRows, G = kWindowTiles, TPW = kWindowTilesPerWave, STRIDE = kWindowStride;
     extern __shared__ float window[];            // ROWS * STRIDE
 
     if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
-    const int unit = xcd_tile(blockIdx.x, total_groups);
+    const int unit = xcd_tile(blockIdx.x, total_units);
     if (unit < 0) return;
-    const int b = unit / groups_per_image;
-    const int g = unit - b * groups_per_image;
+    // unit -> (image, group of tiles, block of 16 channels); the blocks of a group are neighbours in the grid, so they
+    // run at the same time on one XCD and the second reads p and the lists from its L2
+    const int cbn = C >> 4;
+    const int cb = unit % cbn;
+    const int bg = unit / cbn;
+    const int b = bg / groups_per_image;
+    const int g = bg - b * groups_per_image;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int r16 = lane & 15, kq = lane >> 4;
@@ -81,132 +86,74 @@ __global__ __launch_bounds__(kWindowWaves* kWave) void scatter_rows_window_kerne
             const bool shared_list = __all(same ? 1 : 0) != 0;
             rows[k] = (int)wide[0];
             if (shared_list) ok |= 1u << k;
-            if (lane == 0) handled[(int64_t)b * tiles_per_image + tile] = shared_list ? 1 : 0;
+            if (lane == 0 && cb == 0) handled[(int64_t)b * tiles_per_image + tile] = shared_list ? 1 : 0;
         }
     }
     for (int z = tid; z < ROWS * STRIDE; z += kWindowWaves * kWave) window[z] = 0.f;
     // nothing to add: the tile kernel has every tile of the group
     if (__syncthreads_or(ok != 0 ? 1 : 0) == 0) return;
 
-    // Operands of one tile and head in the layout of the matrix instruction, straight from memory:
-    //   A: p[token 4 s + kq][slot 16 blk + r16]        B: x[token 4 s + kq][channel 16 cb + r16]
-    // Those of the wave's next tile are requested before the present tile's sums are added to the window.
     const int blocks = (M + 15) >> 4;
-    struct Operands {
-        T a[2][4];
-        T xb[2][C / 16];
-    };
-    auto fetch = [&](int k, int h, Operands& o) {
-        const int tile = min(g * G + wave + kWindowWaves * k, tiles_per_image - 1);   // a tile past the end: not used
-        const int i0 = tile * kTileTokens;
-        const int nt = min(kTileTokens, N - i0);
-        const T* ph = p + (((int64_t)b * H + h) * N + i0) * M;
-        const T* xh = x + (int64_t)b * xs.b + (int64_t)h * xs.h + (int64_t)i0 * xs.n;
-#pragma unroll
-        for (int sx = 0; sx < 2; ++sx) {
-            const int tok = min(4 * sx + kq, nt - 1);
-#pragma unroll
-            for (int cb = 0; cb < C / 16; ++cb) o.xb[sx][cb] = xh[(uint32_t)(tok * (int)xs.n + 16 * cb + r16)];
-#pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
-                if (blk < blocks) o.a[sx][blk] = ph[(uint32_t)(tok * M + min(16 * blk + r16, M - 1))];
-            }
-        }
-    };
     uint32_t* cells = reinterpret_cast<uint32_t*>(window);
-    constexpr bool AHEAD = C <= 32;    // (at 64 channels two sets of operands do not fit the registers)
-    Operands cur, nxt;
-    if (AHEAD) fetch(0, 0, cur);
     for (int h = 0; h < H; ++h) {
-        float* out_h = out + ((int64_t)b * H + h) * N * C;
+        float* out_h = out + ((int64_t)b * H + h) * N * C + 16 * cb;
 #pragma unroll 1
         for (int k = 0; k < TPW; ++k) {
-            if (!AHEAD) {
-                if ((ok >> k & 1u) != 0) fetch(k, h, cur);
-            } else if (k + 1 < TPW) {
-                fetch(k + 1, h, nxt);
-            } else if (h + 1 < H) {
-                fetch(0, h + 1, nxt);
-            }
-            const Operands now = cur;
-            if (AHEAD) cur = nxt;
             if ((ok >> k & 1u) == 0) continue;
-            const int nt = min(kTileTokens, N - (g * G + wave + kWindowWaves * k) * kTileTokens);
+            const int i0 = (g * G + wave + kWindowWaves * k) * kTileTokens;
+            const int nt = min(kTileTokens, N - i0);
+            const T* ph = p + (((int64_t)b * H + h) * N + i0) * M;
+            const T* xh = x + (int64_t)b * xs.b + (int64_t)h * xs.h + (int64_t)i0 * xs.n + 16 * cb;
+            // B operands: x[token 4 s + kq][channel 16 cb + r16]
+            const float x0 = to_acc(xh[(uint32_t)(min(kq, nt - 1) * (int)xs.n + r16)]);
+            const float x1 = to_acc(xh[(uint32_t)(min(4 + kq, nt - 1) * (int)xs.n + r16)]);
+            const float xb0 = kq < nt ? x0 : 0.f, xb1 = 4 + kq < nt ? x1 : 0.f;
             int rows_k = rows[0];
 #pragma unroll
             for (int kk = 1; kk < TPW; ++kk) rows_k = k == kk ? rows[kk] : rows_k;
-            float xb[2][C / 16];
-#pragma unroll
-            for (int sx = 0; sx < 2; ++sx) {
-#pragma unroll
-                for (int cb = 0; cb < C / 16; ++cb) xb[sx][cb] = 4 * sx + kq < nt ? to_acc(now.xb[sx][cb]) : 0.f;
-            }
 #pragma unroll 1
             for (int blk = 0; blk < blocks; ++blk) {
-                T ab[2] = {now.a[0][0], now.a[1][0]};
-#pragma unroll
-                for (int bb = 1; bb < 4; ++bb) {
-                    ab[0] = blk == bb ? now.a[0][bb] : ab[0];
-                    ab[1] = blk == bb ? now.a[1][bb] : ab[1];
-                }
+                // A operands: p[token 4 s + kq][slot 16 blk + r16]
+                const int slot_a = min(16 * blk + r16, M - 1);
                 const bool slot_ok = 16 * blk + r16 < M;
-                const float a0 = (slot_ok && kq < nt) ? to_acc(ab[0]) : 0.f;
-                const float a1 = (slot_ok && 4 + kq < nt) ? to_acc(ab[1]) : 0.f;
+                const float p0 = to_acc(ph[(uint32_t)(min(kq, nt - 1) * M + slot_a)]);
+                const float p1 = to_acc(ph[(uint32_t)(min(4 + kq, nt - 1) * M + slot_a)]);
+                const float a0 = (slot_ok && kq < nt) ? p0 : 0.f;
+                const float a1 = (slot_ok && 4 + kq < nt) ? p1 : 0.f;
                 // the lane's results: slots 16 blk + 4 kq .. + 3 of channel 16 cb + r16
                 int drow[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) drow[e] = __shfl(rows_k, min(16 * blk + 4 * kq + e, M - 1));
-                // the sums are added by compare-and-swap on the cells' bits: all cells of the block are read, then
+                F32x4 d = F32x4{0.f, 0.f, 0.f, 0.f};
+                d = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, xb0, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, xb1, d, 0, 0, 0);
+                // the sums are added by compare-and-swap on the cells' bits: the lane's four cells are read, then
                 // swapped, and only the lanes that lost a race go round again
-                // ... two blocks of 16 channels at a time
-                constexpr int CB = C >= 32 ? 2 : 1;
-#pragma unroll 1
-                for (int c0 = 0; c0 < C / 16; c0 += CB) {
-                    F32x4 d[CB];
+                int cell[4];
+                uint32_t seen[4];
+                uint32_t open = 0;          // bit e: the sum still has to reach its cell
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        float b0 = xb[0][cb], b1 = xb[1][cb];
-#pragma unroll
-                        for (int cc = CB; cc < C / 16; cc += CB) {
-                            b0 = c0 == cc ? xb[0][cc + cb] : b0;
-                            b1 = c0 == cc ? xb[1][cc + cb] : b1;
-                        }
-                        d[cb] = F32x4{0.f, 0.f, 0.f, 0.f};
-                        d[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, d[cb], 0, 0, 0);
-                        d[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, d[cb], 0, 0, 0);
+                for (int e = 0; e < 4; ++e) {
+                    const int rel = drow[e] - w0;
+                    const bool valid = 16 * blk + 4 * kq + e < M;
+                    const bool inside = (uint32_t)rel < (uint32_t)ROWS;
+                    cell[e] = (inside ? rel : 0) * STRIDE + r16;
+                    seen[e] = 0;
+                    if (valid && inside) {
+                        open |= 1u << e;
+                        seen[e] = cells[cell[e]];
+                    } else if (valid) {
+                        unsafeAtomicAdd(out_h + (int64_t)drow[e] * C + r16, d[e]);
                     }
-                    int cell[4];
-                    uint32_t seen[4][CB];
-                    uint32_t open = 0;          // bit 4 cb + e: the sum still has to reach its cell
+                }
+                while (__any(open != 0 ? 1 : 0) != 0) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int rel = drow[e] - w0;
-                        const bool valid = 16 * blk + 4 * kq + e < M;
-                        const bool inside = (uint32_t)rel < (uint32_t)ROWS;
-                        cell[e] = (inside ? rel : 0) * STRIDE + 16 * c0 + r16;
-#pragma unroll
-                        for (int cb = 0; cb < CB; ++cb) {
-                            seen[e][cb] = 0;
-                            if (valid && inside) {
-                                open |= 1u << (4 * cb + e);
-                                seen[e][cb] = cells[cell[e] + 16 * cb];
-                            } else if (valid) {
-                                unsafeAtomicAdd(out_h + (int64_t)drow[e] * C + 16 * (c0 + cb) + r16, d[cb][e]);
-                            }
-                        }
-                    }
-                    while (__any(open != 0 ? 1 : 0) != 0) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-#pragma unroll
-                            for (int cb = 0; cb < CB; ++cb) {
-                                if ((open >> (4 * cb + e) & 1u) != 0) {
-                                    const uint32_t expect = seen[e][cb];
-                                    const uint32_t sum = __float_as_uint(__uint_as_float(expect) + d[cb][e]);
-                                    seen[e][cb] = atomicCAS(cells + cell[e] + 16 * cb, expect, sum);
-                                    if (seen[e][cb] == expect) open &= ~(1u << (4 * cb + e));
-                                }
-                            }
+                        if ((open >> e & 1u) != 0) {
+                            const uint32_t expect = seen[e];
+                            const uint32_t sum = __float_as_uint(__uint_as_float(expect) + d[e]);
+                            seen[e] = atomicCAS(cells + cell[e], expect, sum);
+                            if (seen[e] == expect) open &= ~(1u << e);
                         }
                     }
                 }
@@ -214,8 +161,8 @@ __global__ __launch_bounds__(kWindowWaves* kWave) void scatter_rows_window_kerne
         }
         __syncthreads();
         // the window's sums leave for memory, and the window is clear for the next head
-        for (int cell = tid; cell < ROWS * C; cell += kWindowWaves * kWave) {
-            const int r = cell / C, c = cell - r * C;
+        for (int cell = tid; cell < ROWS * 16; cell += kWindowWaves * kWave) {
+            const int r = cell >> 4, c = cell & 15;
             const float v = window[r * STRIDE + c];
             if (v != 0.f) {
                 window[r * STRIDE + c] = 0.f;
@@ -226,37 +173,23 @@ __global__ __launch_bounds__(kWindowWaves* kWave) void scatter_rows_window_kerne
     }
 }
 
-template <typename T, int C>
-int launch_c(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* acc32, uint8_t* handled,
-             const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
-    constexpr int ROWS = kWindowCells / C;
-    constexpr int G = window_group_tiles(C);
-    constexpr int LDS = ROWS * (C + 1) * (int)sizeof(float);
-    const int tiles = (s.N + kTileTokens - 1) / kTileTokens;
-    const int groups = (tiles + G - 1) / G;
-    const int64_t total = (int64_t)s.B * groups;
-    if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
-    // more LDS than a workgroup gets without asking (a CU of this device holds 160 KB)
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(scatter_rows_window_kernel<T, C>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
-        (void)hipGetLastError();
-        return CLUSTEN_ERR_LAUNCH;
-    }
-    hipLaunchKernelGGL((scatter_rows_window_kernel<T, C>), dim3(xcd_grid((int)total)), dim3(kWindowWaves * kWave), LDS,
-                       stream, static_cast<const T*>(p), static_cast<const T*>(x), idx, acc32, handled, s.H, s.N, s.M, xs,
-                       tiles, groups, (int)total, only_if);
-    return launch_status();
-}
-
 template <typename T>
 int launch_typed(const void* p, const void* x, clusten_strides xs, const int64_t* idx, float* acc32, uint8_t* handled,
                  const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if) {
-    switch (s.C) {
-        case 16: return launch_c<T, 16>(p, x, xs, idx, acc32, handled, s, stream, only_if);
-        case 32: return launch_c<T, 32>(p, x, xs, idx, acc32, handled, s, stream, only_if);
-        case 64: return launch_c<T, 64>(p, x, xs, idx, acc32, handled, s, stream, only_if);
-        default: return CLUSTEN_ERR_BAD_DIMS;
+    const int tiles = (s.N + kTileTokens - 1) / kTileTokens;
+    const int groups = (tiles + kWindowTiles - 1) / kWindowTiles;
+    const int64_t total = (int64_t)s.B * groups * (s.C / 16);
+    if (total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
+    // more LDS than a workgroup gets without asking (a CU of this device holds 160 KB)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(scatter_rows_window_kernel<T>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kWindowLds) != hipSuccess) {
+        (void)hipGetLastError();
+        return CLUSTEN_ERR_LAUNCH;
     }
+    hipLaunchKernelGGL((scatter_rows_window_kernel<T>), dim3(xcd_grid((int)total)), dim3(kWindowWaves * kWave), kWindowLds,
+                       stream, static_cast<const T*>(p), static_cast<const T*>(x), idx, acc32, handled, s.H, s.N, s.M, s.C,
+                       xs, tiles, groups, (int)total, only_if);
+    return launch_status();
 }
 
 }  // namespace
