@@ -210,7 +210,13 @@ __global__ __launch_bounds__(256) void wf_dweights_kernel(const T* __restrict__ 
 // channels in the place of the tile's tokens.  One wave per output token; the channels are taken 256 bytes of a
 // row at a time (rows and d_out rows by LDS-direct load, XOR-swizzled so that the 16-byte operand reads of the 16
 // lanes of an MFMA row fall into different bank groups), 16x16 MFMA blocks, D accumulated over the column blocks.
-// The result leaves through LDS in the (slot, ic) order of d_w as full-width stores.
+// The result leaves through LDS in the (slot, ic) order of d_w as full-width stores.  fp32 with at most four inner
+// channels takes sixteen 4x4 blocks per instruction instead, lane = slot (see below): a third of the matrix-pipe time
+// and the result already in the order of d_w.  The rows in flight are bounded by the LDS they land in (14 KB a wave),
+// so a wave takes four consecutive tokens and has the next one's list on its way while the present one's rows
+// arrive.  Stage 1 (B128, 3136 -> 784 tokens, C64, IC4, fp32): 177 -> 150 us (4x4 blocks) -> 135 us (four tokens).
+constexpr int kDwTokens = 4;   // output tokens per wave of wf_dweights_tile_kernel
+
 template <typename T, int Q>
 __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __restrict__ d_out,
                                                                  const T* __restrict__ feat,
@@ -228,20 +234,32 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
 
     __shared__ __attribute__((aligned(1024))) char stage[G_BYTES + 8 * RB];
 
-    const int token = xcd_tile(blockIdx.x, total_tokens);
-    if (token < 0) return;
-    const int b = token / Nout;
+    // a wave takes kDwTokens consecutive output tokens; the list of the next one is requested while the rows of the
+    // present one are on their way (a wave that waits for its list holds LDS that nothing is being loaded into)
+    const int unit = xcd_tile(blockIdx.x, (total_tokens + kDwTokens - 1) / kDwTokens);
+    if (unit < 0) return;
+    const int token0 = unit * kDwTokens;
     const int lane = threadIdx.x;
     const int r = lane & 15, kq = lane >> 4;      // MFMA row / k index: the lane holds quarter kq of row r
     const int g_sub = lane >> 4, g_pos = lane & 15;  // gather side: piece g_pos of staging row 4*i + g_sub
-
-    const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
-    const char* g_tok = reinterpret_cast<const char*>(d_out + (int64_t)token * IC * C);
     const uint32_t row_pitch = (uint32_t)C * sizeof(T);
     // lists of more than 16*Q slots go 16*Q slots at a time
-    for (int j0 = 0; j0 < M; j0 += ROWS) {
+    const int chunks = (M + ROWS - 1) / ROWS;
+    const int items = min(kDwTokens, total_tokens - token0) * chunks;
+    auto list_of = [&](int item) {
+        const int t = item / chunks, j0 = (item - t * chunks) * ROWS;
+        return (int)idx[(int64_t)(token0 + t) * M + j0 + min(lane, min(ROWS, M - j0) - 1)];
+    };
+    int mine_next = list_of(0);
+    for (int item = 0; item < items; ++item) {
+    const int mine = mine_next;
+    if (item + 1 < items) mine_next = list_of(item + 1);
+    const int token = token0 + item / chunks;
+    const int j0 = (item % chunks) * ROWS;
     const int mc = min(ROWS, M - j0);
-    const int mine = (int)idx[(int64_t)token * M + j0 + min(lane, mc - 1)];
+    const int b = token / Nout;
+    const char* feat_b = reinterpret_cast<const char*>(feat + (int64_t)b * N * C);
+    const char* g_tok = reinterpret_cast<const char*>(d_out + (int64_t)token * IC * C);
 
     uint32_t g_off[NI_G];
 #pragma unroll
@@ -262,19 +280,56 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
         lds_a[u] = G_BYTES + (r & 7) * RB + (((kq * NU + u) ^ (r & 7)) * 16);
     }
 
+    if constexpr (sizeof(T) == 4) {
+        if (IC <= 4) {
+            // fp32, at most four inner channels: sixteen 4x4 blocks per instruction (`v_mfma_f32_4x4x1_16b_f32`) with
+            // lane = slot.  Block l/4: A = dO[ic = l%4][c], B = G[slot l][c]; the lane ends with D[ic 0..3][slot l],
+            // the four consecutive elements of d_w it stores.  64 instructions of 8 clocks per 64 channels in the
+            // place of 48 16x16x4 instructions of 32 clocks that use four of their sixteen columns.
+            const int srow = min(lane, ROWS - 1);
+            const int ic = min(lane & 3, IC - 1);
+            F32x4 acc = F32x4{0.f, 0.f, 0.f, 0.f};
+            for (int c0 = 0; c0 < C; c0 += CB) {
+                const uint32_t col_bytes = (uint32_t)c0 * sizeof(T);
+                lds_sync();  // the previous column block's operands are in registers
+#pragma unroll
+                for (int i = 0; i < 2; ++i) CLUSTEN_LDS_DMA16(g_tok + (a_off[i] + col_bytes), stage + G_BYTES + i * 1024);
+#pragma unroll
+                for (int i = 0; i < NI_G; ++i) CLUSTEN_LDS_DMA16(feat_b + (g_off[i] + col_bytes), stage + i * 1024);
+                lds_sync_vm<0>();
+#pragma unroll 4
+                for (int u = 0; u < 16; ++u) {
+                    const Piece g = *reinterpret_cast<const Piece*>(stage + srow * RB + ((u ^ (srow & 15)) * 16));
+                    const Piece a = *reinterpret_cast<const Piece*>(stage + G_BYTES + ic * RB + ((u ^ ic) * 16));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc = mfma_4x4x1(__uint_as_float(a[e]), __uint_as_float(g[e]), acc);
+                }
+            }
+            if (lane < mc) {
+                T* dst = d_w + ((int64_t)token * M + j0 + lane) * IC;
+                if (IC == 4) {
+                    store_streaming(reinterpret_cast<Piece*>(dst), __builtin_bit_cast(Piece, acc));
+                } else {
+                    for (int v = 0; v < IC; ++v) dst[v] = acc[v];
+                }
+            }
+            lds_sync();  // the rows have been read before the next chunk's arrive
+            continue;
+        }
+    }
+
     F32x4 d[Q];
 #pragma unroll
     for (int blk = 0; blk < Q; ++blk) d[blk] = F32x4{0.f, 0.f, 0.f, 0.f};
 
     for (int c0 = 0; c0 < C; c0 += CB) {
         const uint32_t col_bytes = (uint32_t)c0 * sizeof(T);
-        __syncthreads();  // the previous column block's operands are in registers
+        lds_sync();  // the previous column block's operands are in registers
 #pragma unroll
         for (int i = 0; i < 2; ++i) CLUSTEN_LDS_DMA16(g_tok + (a_off[i] + col_bytes), stage + G_BYTES + i * 1024);
 #pragma unroll
         for (int i = 0; i < NI_G; ++i) CLUSTEN_LDS_DMA16(feat_b + (g_off[i] + col_bytes), stage + i * 1024);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-        __syncthreads();
+        lds_sync_vm<0>();
 
         typename RunIO::raw a_raw[NU];
 #pragma unroll
@@ -292,7 +347,7 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
     }
 
     // lane (r, kq) holds slots 16*blk + 4*kq .. +3 of inner channel r; d_w of the token is M*IC contiguous elements
-    __syncthreads();
+    lds_sync();
     if (r < IC) {
 #pragma unroll
         for (int blk = 0; blk < Q; ++blk) {
@@ -303,13 +358,13 @@ __global__ __launch_bounds__(kWave) void wf_dweights_tile_kernel(const T* __rest
             }
         }
     }
-    __syncthreads();
+    lds_sync();
     const int out_bytes = mc * IC * (int)sizeof(T);
     char* dst = reinterpret_cast<char*>(d_w + ((int64_t)token * M + j0) * IC);
     for (int off = lane * 16; off < out_bytes; off += kWave * 16) {
         store_streaming(reinterpret_cast<Piece*>(dst + off), *reinterpret_cast<const Piece*>(stage + off));
     }
-    __syncthreads();  // the chunk has left LDS before the next one's rows arrive
+    lds_sync();  // the chunk has left LDS before the next one's rows arrive
     }
 }
 
@@ -441,11 +496,11 @@ int wf_dweights_typed(const void* d_out, const void* feat, const int64_t* idx, v
     if constexpr (sizeof(T) <= 4) if (tile_ok) {
         const int total_tokens = s.B * s.Nout;
         if (s.M <= 48) {
-            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 3>), dim3(xcd_grid(total_tokens)), dim3(kWave), 0, stream,
+            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 3>), dim3(xcd_grid((total_tokens + kDwTokens - 1) / kDwTokens)), dim3(kWave), 0, stream,
                                static_cast<const T*>(d_out), static_cast<const T*>(feat), idx, static_cast<T*>(d_w),
                                s.N, s.Nout, s.C, s.M, s.IC, total_tokens);
         } else {
-            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 4>), dim3(xcd_grid(total_tokens)), dim3(kWave), 0, stream,
+            hipLaunchKernelGGL((wf_dweights_tile_kernel<T, 4>), dim3(xcd_grid((total_tokens + kDwTokens - 1) / kDwTokens)), dim3(kWave), 0, stream,
                                static_cast<const T*>(d_out), static_cast<const T*>(feat), idx, static_cast<T*>(d_w),
                                s.N, s.Nout, s.C, s.M, s.IC, total_tokens);
         }
