@@ -581,7 +581,26 @@ def main():
             "one_kernel_us": round(per_a[0] * 1e3, 1), "three_kernels_us": round(per_a[1] * 1e3, 1),
             "one_kernel_with_plan_us": round(per_a[2] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
-        del mcase, cidx, mattn, q16, k16, v16, pe_idx, plan
+        # the same in fp32 (inference without mixed precision)
+        table32 = table.float()
+
+        def three_kernels_fp32():
+            a = _native.qk_forward_clusters(mcase.query, mcase.key, cidx)
+            p, pb = _native.attn_softmax(a, table32, pe_idx, None, query=mcase.query, blank_key=blank_k)
+            return _native.av_forward_clusters(p, mcase.value, cidx)
+
+        _, per_f, _ = _time_kernels([lambda: _native.cluster_attention(mcase.query, mcase.key, mcase.value, cidx, table32,
+                                                                       pe_idx, None, blank_k, blank_v),
+                                     three_kernels_fp32,
+                                     lambda: _native.cluster_attention(mcase.query, mcase.key, mcase.value, None, table32,
+                                                                       None, None, blank_k, blank_v, plan=plan)],
+                                    args.steps, args.warmup)
+        fused_bytes32 = 4 * mcase.query.numel() * 4 + cidx.numel() * 4 + pe_idx.numel() * 8
+        other["cfg2_s1_local_attention_fp32_model_built_lists"] = {
+            "one_kernel_us": round(per_f[0] * 1e3, 1), "three_kernels_us": round(per_f[1] * 1e3, 1),
+            "one_kernel_with_plan_us": round(per_f[2] * 1e3, 1),
+            "one_kernel_algorithmic_bytes": fused_bytes32, "one_kernel_GBps": round(fused_bytes32 / per_f[0] / 1e6, 1)}
+        del mcase, cidx, mattn, q16, k16, v16, pe_idx, plan, table32
         # the first stage of the 384 x 384 models as the reference model builds its lists there: clusters of 24 tokens,
         # the members of the 6 nearest clusters = 144 slots (configs/aff_base_22kto1k_384.yaml:10-11), B = 16
         for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):

@@ -255,7 +255,7 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
  * regular grid have the same neighbourhoods in every image);
  * blank_key, blank_value (H,C) fp32, contiguous.  Pass the unscaled query and the model's scale, or a scaled
  * query and 1.  The probabilities are rounded to `dtype` before they weigh the value rows; sums are fp32.
- * dtype F16 or BF16 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and M = 48 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
+ * dtype F16, BF16 or F32 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and M = 48 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
  * aligned (else CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
 int clusten_cluster_attention_forward(const void* query, clusten_strides query_strides,
                                       const void* key, clusten_strides key_strides,

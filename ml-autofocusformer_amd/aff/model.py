@@ -295,8 +295,8 @@ class ClusterAttention(nn.Module):
         one_kernel = getattr(self.ops, "cluster_attention", None)
         if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
                 and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2])):
-            # inference on 16-bit data: scores, position bias, mask, blank token, softmax and the weighted sum of
-            # the values in one kernel; the query scale is applied to the scores inside it
+            # inference on 16-bit or fp32 data: scores, position bias, mask, blank token, softmax and the weighted sum
+            # of the values in one kernel; the query scale is applied to the scores inside it
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
             plan = lists[3] if len(lists) > 3 else None     # what the kernel makes of the lists, once per stage
             out = one_kernel(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, lists[0], self.bias_table(table),
@@ -581,8 +581,8 @@ class BasicLayer(nn.Module):
 
         planner = getattr(self.ops, "cluster_attention_plan", None)
         if (grid_lists is None and cluster_idx is not None and planner is not None and not torch.is_grad_enabled()
-                and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda and feat.dtype != torch.float64
-                and torch.is_autocast_enabled("cuda")):
+                and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
+                and (feat.dtype == torch.float32 or torch.is_autocast_enabled("cuda"))):
             # the one-kernel attention of every block reads what it makes of the lists from a plan built once
             grid_lists = (cluster_idx, pe_idx, mask, planner(cluster_idx, pe_idx, mask))
         carry = None

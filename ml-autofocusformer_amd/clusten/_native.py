@@ -680,8 +680,9 @@ def attn_softmax_backward(probs: torch.Tensor, blank_prob: torch.Tensor, d_probs
 
 
 def cluster_attention_supported(query: torch.Tensor, nnc: int) -> bool:
-    """True when `cluster_attention` takes this case: CUDA fp16 / bf16 queries of head dim 32, six clusters per token."""
-    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16) and query.dim() == 4
+    """True when `cluster_attention` takes this case: CUDA fp16 / bf16 / fp32 queries of head dim 32, six clusters per
+    token."""
+    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16, torch.float32) and query.dim() == 4
             and query.shape[3] == 32 and nnc == 6)
 
 
@@ -720,7 +721,7 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
                       blank_value: torch.Tensor, scale: float = 1.0, plan=None) -> torch.Tensor:
     """Local attention over the members of each token's clusters plus one blank token, in one kernel.
 
-    query, key, value (B,H,N,32) fp16 / bf16 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
+    query, key, value (B,H,N,32) fp16 / bf16 / fp32 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
     bias_table (rows,H); pe_idx (B,N,48) int64; mask (B,N,48) of 0/1 or None; blank_key, blank_value (H*32,).
     cluster_idx, pe_idx and mask may all have a leading 1 instead of B: one set of lists for every image.
     Returns softmax(scale * q.k + bias - 100 * (1 - mask) | scale * q.blank_key) applied to the gathered values and

@@ -196,7 +196,7 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
     if (!query || !key || !value || !cluster_idx || !bias_table || !pe_idx || !blank_key || !blank_value || !out) {
         return CLUSTEN_ERR_NULL_POINTER;
     }
-    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
     if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
         !strides_ok(out_strides, shape.C)) {
@@ -230,7 +230,7 @@ int clusten_cluster_attention_forward_planned(const void* query, clusten_strides
     if (!query || !key || !value || !plan || !bias_table || !blank_key || !blank_value || !out) {
         return CLUSTEN_ERR_NULL_POINTER;
     }
-    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
     if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
         !strides_ok(out_strides, shape.C)) {

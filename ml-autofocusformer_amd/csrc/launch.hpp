@@ -72,7 +72,7 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
                         float* blank_prob, clusten_attn_shape s, int dtype, hipStream_t stream);
 
 // Local attention of a cluster-ordered sequence in one kernel (QK, position bias, mask, blank token, softmax, AV,
-// blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16}, C = 32;
+// blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16, F32}, C = 32;
 //   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48) — or (1,N,.) each
 //   when lists_shared;
 //   blank_k, blank_v : fp32 (H,C).

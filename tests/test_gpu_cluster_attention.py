@@ -81,7 +81,7 @@ def _run(device, case, scale):
 
 
 @pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_against_the_oracle_composition(device, kind, dtype):
     gen = torch.Generator().manual_seed(81)
     # 396 = 49 whole clusters and one of 4 tokens (a partial tile whose pad rows list row 0); 64: few clusters
@@ -91,18 +91,19 @@ def test_against_the_oracle_composition(device, kind, dtype):
             assert err <= TOL[dtype], "%s %s n=%d mask=%s rel err %.3g" % (kind, dtype, n, with_mask, err)
 
 
-def test_strided_operands_and_unit_scale(device):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_strided_operands_and_unit_scale(device, dtype):
     """q / k / v as the views a fused qkv projection leaves (channel stride 1, token stride 3*H*C)."""
     gen = torch.Generator().manual_seed(82)
     b, h, n = 2, 2, 136
-    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True)
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", dtype, True)
     packed = torch.stack([q, k, v], dim=0).permute(1, 3, 0, 2, 4).contiguous()        # (b, n, 3, h, c)
     views = packed.to(device).permute(2, 0, 3, 1, 4)                                  # (3, b, h, n, c) views
     assert not views[0].is_contiguous()
     ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, 1.0)
     out = _native.cluster_attention(views[0], views[1], views[2], cidx.to(device), table.to(device), pe_idx.to(device),
                                     mask.to(device), blank_k.to(device), blank_v.to(device))
-    assert oracle.rel_err(out, ref) <= TOL[torch.float16]
+    assert oracle.rel_err(out, ref) <= TOL[dtype]
 
 
 def test_equals_the_three_kernel_path(device):
@@ -124,11 +125,12 @@ def test_unsupported_cases_are_refused(device):
     q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(1, 2, 64, gen, "near", torch.float16, False)
     d = lambda x: x.to(device)
     assert _native.cluster_attention_supported(d(q), 6)
-    assert not _native.cluster_attention_supported(d(q).float(), 6)
+    assert _native.cluster_attention_supported(d(q).float(), 6)
+    assert not _native.cluster_attention_supported(d(q).double(), 6)
     assert not _native.cluster_attention_supported(d(q), 8)
     assert not _native.cluster_attention_supported(q, 6)
-    with pytest.raises(RuntimeError):       # fp32 has no fused kernel
-        _native.cluster_attention(d(q).float(), d(k).float(), d(v).float(), d(cidx), d(table), d(pe_idx), None,
+    with pytest.raises(RuntimeError):       # fp64 has no fused kernel
+        _native.cluster_attention(d(q).double(), d(k).double(), d(v).double(), d(cidx), d(table), d(pe_idx), None,
                                   d(blank_k), d(blank_v))
     with pytest.raises(RuntimeError):       # CPU tensors
         _native.cluster_attention(q, k, v, cidx, table, pe_idx, None, blank_k, blank_v)
@@ -171,8 +173,9 @@ def test_cluster_numbers_out_of_range_read_row_zero(device):
     assert oracle.rel_err(out, ref) <= TOL[torch.float16]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
-def test_plan_built_once_gives_the_same_bits(device, kind):
+def test_plan_built_once_gives_the_same_bits(device, kind, dtype):
     """What the kernel works out from the index tensors, handed over as a plan (one per stage, read by every layer):
     the result is bit-equal to the call that reads the tensors, for every kind of list, with and without a mask, on
     partial tiles, and for lists shared by the batch."""
@@ -180,7 +183,7 @@ def test_plan_built_once_gives_the_same_bits(device, kind):
     d = lambda x: None if x is None else x.to(device)
     for b, h, n in ((2, 3, 396), (1, 1, 64), (3, 4, 200)):
         for with_mask in (False, True):
-            q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, torch.float16, with_mask)
+            q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, dtype, with_mask)
             plain = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k),
                                               d(blank_v), scale=0.2)
             plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
@@ -191,7 +194,7 @@ def test_plan_built_once_gives_the_same_bits(device, kind):
                 assert torch.equal(planned, plain)
     # one image's lists for the whole batch
     b, h, n = 3, 2, 200
-    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, torch.bfloat16, True)
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, torch.bfloat16 if dtype == torch.float16 else dtype, True)
     c1, p1, m1 = cidx[:1].contiguous(), pe_idx[:1].contiguous(), mask[:1].contiguous()
     plain = _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(p1), d(m1), d(blank_k), d(blank_v))
     plan1 = _native.cluster_attention_plan(d(c1), d(p1), d(m1))
