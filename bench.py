@@ -601,6 +601,18 @@ def main():
             "one_kernel_with_plan_us": round(per_f[2] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes32, "one_kernel_GBps": round(fused_bytes32 / per_f[0] / 1e6, 1)}
         del mcase, cidx, mattn, q16, k16, v16, pe_idx, plan, table32
+        # WF on the lists a merge reads (the members of the nearest clusters of every centre, centres = a sorted
+        # quarter of the tokens of a cluster-ordered sequence): consecutive output tokens name mostly the same rows
+        def _wf_merge(tag, B_, N_, C_, cluster, steps):
+            g_ = wl.generator(33)
+            lists = wl.model_built_lists(B_, N_, g_, cluster=cluster, nnc=6)
+            centres = torch.stack([torch.randperm(N_, generator=g_)[:N_ // 4].sort().values for _ in range(B_)])
+            wc = wl.wf_case(tag, 34, B=B_, N=N_, C=C_, M=lists.shape[2])
+            wc.nbhd_idx = lists.gather(1, centres[:, :, None].expand(-1, -1, lists.shape[2])).contiguous()
+            return _bench_wf(wc, steps, 5)
+
+        other["cfg2_s1_wf_merge_lists"] = _wf_merge("wf_merge", B, 3136, 64, 8, args.steps)
+        other["aff_base_384_stage1_wf_merge_lists"] = _wf_merge("wf_merge_384", 16, 9216, 128, 24, max(args.steps // 2, 5))
         # the first stage of the 384 x 384 models as the reference model builds its lists there: clusters of 24 tokens,
         # the members of the 6 nearest clusters = 144 slots (configs/aff_base_22kto1k_384.yaml:10-11), B = 16
         for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
