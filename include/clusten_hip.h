@@ -289,6 +289,40 @@ int clusten_cluster_attention_forward_planned(const void* query, clusten_strides
                                               void* out, clusten_strides out_strides, float scale,
                                               clusten_attn_shape shape, int dtype, clusten_stream stream);
 
+/* clusten_cluster_attention_forward_planned for a forward pass whose backward will follow: it also writes
+ * lse[b,h,i] = log of the denominator of token i's softmax (fp32, (B,H,N) contiguous), from which
+ * clusten_cluster_attention_backward recomputes the probabilities.  dtype F16, BF16 or F32. */
+int clusten_cluster_attention_forward_train(const void* query, clusten_strides query_strides,
+                                            const void* key, clusten_strides key_strides,
+                                            const void* value, clusten_strides value_strides,
+                                            const void* plan, const void* bias_table, int lists_shared,
+                                            const float* blank_key, const float* blank_value,
+                                            void* out, clusten_strides out_strides, float* lse, float scale,
+                                            clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* The query-side half of the backward of the kernel above, in one kernel (the backward of
+ * models/aff_transformer.py:120-155: clustenqk_cuda_kernel.cu:51-132, the tensor expressions between the operators,
+ * clustenav_cuda_kernel.cu:51-127).  With p = exp(logit - lse), delta[i] = <d_out[i], out[i]>:
+ *   d_logit[b,h,i,j] = p * (<d_out[b,h,i], value[b,h,row(i,j)]> - delta),   d_blank_logit likewise with blank_value
+ *   d_query[b,h,i]   = scale * (sum_j d_logit[b,h,i,j] * key[b,h,row(i,j)] + d_blank_logit[b,h,i] * blank_key[h])
+ * It writes d_query (strided (B,H,N,C)), probs and d_logit ((B,H,N,M) of `dtype`, contiguous), blank_prob and
+ * d_blank_logit (fp32 (B,H,N)).  The rest of the backward are sums other entry points form:
+ *   d_value = clusten_scatter_rows_by_cluster(probs, d_out),  d_key = scale * clusten_scatter_rows_by_cluster(d_logit, query),
+ *   d_bias_table = clusten_bias_table_grad(d_logit),  d_blank_key = scale * sum d_blank_logit * query,
+ *   d_blank_value = sum blank_prob * d_out.
+ * d_out, out: strided (B,H,N,C) like query (the forward's result and its gradient); dtype F16 or BF16 (else
+ * CLUSTEN_ERR_BAD_DTYPE), C = 32, M = 48.  No counterpart in the reference's extension modules. */
+int clusten_cluster_attention_backward(const void* query, clusten_strides query_strides,
+                                       const void* key, clusten_strides key_strides,
+                                       const void* value, clusten_strides value_strides,
+                                       const void* d_out, clusten_strides d_out_strides,
+                                       const void* out, clusten_strides out_strides,
+                                       const float* lse, const void* plan, const void* bias_table, int lists_shared,
+                                       const float* blank_key, const float* blank_value,
+                                       void* d_query, clusten_strides d_query_strides,
+                                       void* probs, void* d_logit, float* blank_prob, float* d_blank_logit,
+                                       float scale, clusten_attn_shape shape, int dtype, clusten_stream stream);
+
 /* ---- lists made of whole clusters: the backward scatters as gathers (optional) ------------------------------ */
 
 /* The pair lists of neighbour lists made of whole clusters, built on the device without any read-back by the host.

@@ -62,6 +62,12 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward_planned": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P,
                                                                 ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float,
                                                                 AttnShape, ctypes.c_int, _P]),
+    "clusten_cluster_attention_forward_train": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, ctypes.c_int,
+                                                               _P, _P, _P, Strides, _P, ctypes.c_float, AttnShape,
+                                                               ctypes.c_int, _P]),
+    "clusten_cluster_attention_backward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, Strides, _P, Strides,
+                                                          _P, _P, _P, ctypes.c_int, _P, _P, _P, Strides, _P, _P, _P, _P,
+                                                          ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_cluster_pairs_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "clusten_cluster_pairs": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                              ctypes.c_int, _P]),
@@ -718,7 +724,7 @@ def cluster_attention_plan(cluster_idx: torch.Tensor, pe_idx: torch.Tensor, mask
 
 def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cluster_idx: torch.Tensor,
                       bias_table: torch.Tensor, pe_idx: torch.Tensor, mask, blank_key: torch.Tensor,
-                      blank_value: torch.Tensor, scale: float = 1.0, plan=None) -> torch.Tensor:
+                      blank_value: torch.Tensor, scale: float = 1.0, plan=None, return_lse: bool = False):
     """Local attention over the members of each token's clusters plus one blank token, in one kernel.
 
     query, key, value (B,H,N,32) fp16 / bf16 / fp32 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
@@ -728,7 +734,8 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the layout the output
     projection takes).  No autograd: for inference.  The fused form of models/aff_transformer.py:120-155.
     `plan`: what `cluster_attention_plan` made of the same three index tensors; they are then not read (and may be
-    None), the result is the same.
+    None), the result is the same.  `return_lse` (needs a plan): also return the fp32 (B,H,N) logarithms of the
+    softmax denominators, what `cluster_attention_backward` recomputes the probabilities from.
     """
     lib = load()
     _require_cuda("query", query)
@@ -773,9 +780,22 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     blank_value = blank_value.detach().reshape(h, c).float().contiguous()
     out = torch.empty(b, n, h, c, dtype=dtype, device=device)
     if out.numel() == 0:
-        return out.reshape(b, n, h * c)
+        flat = out.reshape(b, n, h * c)
+        return (flat, torch.empty(b, h, n, dtype=torch.float32, device=device)) if return_lse else flat
     out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
     shape = AttnShape(b, h, n, c, m)
+    if return_lse:
+        if plan is None:
+            raise RuntimeError("return_lse needs a plan")
+        lse = torch.empty(b, h, n, dtype=torch.float32, device=device)
+        with torch.cuda.device(device):
+            _check(lib.clusten_cluster_attention_forward_train(_ptr(query), _strides(query), _ptr(key), _strides(key),
+                                                               _ptr(value), _strides(value), _ptr(plan), _ptr(bias_table),
+                                                               int(shared), _ptr(blank_key), _ptr(blank_value), _ptr(out),
+                                                               _strides(out_view), _ptr(lse), ctypes.c_float(scale), shape,
+                                                               code, _stream(device)),
+                   "clusten_cluster_attention_forward_train")
+        return out.reshape(b, n, h * c), lse
     if plan is not None:
         with torch.cuda.device(device):
             _check(lib.clusten_cluster_attention_forward_planned(_ptr(query), _strides(query), _ptr(key), _strides(key),
@@ -794,6 +814,69 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
                                                      _stream(device)),
                "clusten_cluster_attention_forward")
     return out.reshape(b, n, h * c)
+
+
+def cluster_attention_backward_supported(query: torch.Tensor, nnc: int) -> bool:
+    """True when `cluster_attention_backward` takes this case: CUDA fp16 / bf16 queries of head dim 32, six clusters
+    per token."""
+    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16) and query.dim() == 4
+            and query.shape[3] == 32 and nnc == 6)
+
+
+def cluster_attention_backward(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, d_out: torch.Tensor,
+                               out: torch.Tensor, lse: torch.Tensor, plan: torch.Tensor, bias_table: torch.Tensor,
+                               blank_key: torch.Tensor, blank_value: torch.Tensor, scale: float = 1.0):
+    """The query-side half of the backward of `cluster_attention(..., plan=plan, return_lse=True)` in one kernel.
+
+    query, key, value (B,H,N,32) fp16 / bf16 as in the forward; out (B,N,H*32) its result, d_out the gradient of it,
+    lse (B,H,N) fp32 from the forward.  Returns (d_query, probs, d_logit, blank_prob, d_blank_logit): d_query a
+    (B,H,N,32) view of (B,N,H,32) memory, probs and d_logit (B,H,N,48) of query's dtype, blank_prob and d_blank_logit
+    fp32 (B,H,N).  The other gradients are sums of these: d_value = scatter_rows_by_cluster(probs, d_out),
+    d_key = scale * scatter_rows_by_cluster(d_logit, query), d_bias_table = bias_table_grad(d_logit, ...),
+    d_blank_key = scale * sum d_blank_logit * query, d_blank_value = sum blank_prob * d_out."""
+    lib = load()
+    _require_cuda("query", query)
+    device = query.device
+    for name, t in (("key", key), ("value", value), ("d_out", d_out), ("out", out), ("lse", lse), ("plan", plan),
+                    ("bias_table", bias_table), ("blank_key", blank_key), ("blank_value", blank_value)):
+        _require_cuda(name, t, device)
+    if query.dim() != 4 or key.shape != query.shape or value.shape != query.shape:
+        raise RuntimeError("query, key and value must be (B,H,N,C) tensors of one shape")
+    b, h, n, c = query.shape
+    m = 48
+    if tuple(out.shape) != (b, n, h * c) or tuple(d_out.shape) != (b, n, h * c):
+        raise RuntimeError("out and d_out must be (B,N,H*C)")
+    if tuple(lse.shape) != (b, h, n) or lse.dtype != torch.float32:
+        raise RuntimeError("lse must be fp32 (B,H,N)")
+    lb = b if plan.numel() == lib.clusten_cluster_attention_plan_bytes(b, n) else 1
+    if plan.dtype != torch.uint8 or plan.numel() != lib.clusten_cluster_attention_plan_bytes(lb, n):
+        raise RuntimeError("plan does not belong to lists of this shape")
+    shared = b != 1 and lb == 1
+    code = _dtype_code(query, "query")
+    dtype = query.dtype
+    query, key, value = _rows(query), _rows(key.to(dtype)), _rows(value.to(dtype))
+    out_view = out.to(dtype).contiguous().view(b, n, h, c).permute(0, 2, 1, 3)
+    g_view = d_out.to(dtype).contiguous().view(b, n, h, c).permute(0, 2, 1, 3)
+    bias_table = bias_table.detach().to(dtype).contiguous()
+    blank_key = blank_key.detach().reshape(h, c).float().contiguous()
+    blank_value = blank_value.detach().reshape(h, c).float().contiguous()
+    d_query = torch.empty(b, n, h, c, dtype=dtype, device=device).permute(0, 2, 1, 3)
+    probs = torch.empty(b, h, n, m, dtype=dtype, device=device)
+    d_logit = torch.empty(b, h, n, m, dtype=dtype, device=device)
+    blank_prob = torch.empty(b, h, n, dtype=torch.float32, device=device)
+    d_blank = torch.empty(b, h, n, dtype=torch.float32, device=device)
+    if probs.numel() == 0:
+        return d_query, probs, d_logit, blank_prob, d_blank
+    with torch.cuda.device(device):
+        _check(lib.clusten_cluster_attention_backward(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(value),
+                                                      _strides(value), _ptr(g_view), _strides(g_view), _ptr(out_view),
+                                                      _strides(out_view), _ptr(lse.contiguous()), _ptr(plan),
+                                                      _ptr(bias_table), int(shared), _ptr(blank_key), _ptr(blank_value),
+                                                      _ptr(d_query), _strides(d_query), _ptr(probs), _ptr(d_logit),
+                                                      _ptr(blank_prob), _ptr(d_blank), ctypes.c_float(scale),
+                                                      AttnShape(b, h, n, c, m), code, _stream(device)),
+               "clusten_cluster_attention_backward")
+    return d_query, probs, d_logit, blank_prob, d_blank
 
 
 def dense_attention_supported(query: torch.Tensor) -> bool:
@@ -837,7 +920,8 @@ def dense_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
     blank_value = blank_value.detach().reshape(h, c).float().contiguous()
     out = torch.empty(b, n, h, c, dtype=dtype, device=device)
     if out.numel() == 0:
-        return out.reshape(b, n, h * c)
+        flat = out.reshape(b, n, h * c)
+        return (flat, torch.empty(b, h, n, dtype=torch.float32, device=device)) if return_lse else flat
     out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
     shape = AttnShape(b, h, n, c, n)
     with torch.cuda.device(device):

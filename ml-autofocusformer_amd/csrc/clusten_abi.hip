@@ -204,7 +204,7 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
     }
     return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, cluster_idx, bias_table,
                                     pe_idx, mask, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, nullptr,
-                                    shape, dtype, as_stream(stream));
+                                    nullptr, shape, dtype, as_stream(stream));
 }
 
 size_t clusten_cluster_attention_plan_bytes(int B, int N) {
@@ -239,7 +239,53 @@ int clusten_cluster_attention_forward_planned(const void* query, clusten_strides
     if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
     return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, nullptr, bias_table,
                                     nullptr, nullptr, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, plan,
-                                    shape, dtype, as_stream(stream));
+                                    nullptr, shape, dtype, as_stream(stream));
+}
+
+int clusten_cluster_attention_forward_train(const void* query, clusten_strides query_strides, const void* key,
+                                            clusten_strides key_strides, const void* value, clusten_strides value_strides,
+                                            const void* plan, const void* bias_table, int lists_shared,
+                                            const float* blank_key, const float* blank_value, void* out,
+                                            clusten_strides out_strides, float* lse, float scale, clusten_attn_shape shape,
+                                            int dtype, clusten_stream stream) {
+    if (!query || !key || !value || !plan || !bias_table || !blank_key || !blank_value || !out || !lse) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
+        !strides_ok(out_strides, shape.C)) {
+        return CLUSTEN_ERR_BAD_STRIDE;
+    }
+    if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_cluster_attention(query, query_strides, key, key_strides, value, value_strides, nullptr, bias_table,
+                                    nullptr, nullptr, blank_key, blank_value, out, out_strides, scale, lists_shared != 0, plan,
+                                    lse, shape, dtype, as_stream(stream));
+}
+
+int clusten_cluster_attention_backward(const void* query, clusten_strides query_strides, const void* key,
+                                       clusten_strides key_strides, const void* value, clusten_strides value_strides,
+                                       const void* d_out, clusten_strides d_out_strides, const void* out,
+                                       clusten_strides out_strides, const float* lse, const void* plan,
+                                       const void* bias_table, int lists_shared, const float* blank_key,
+                                       const float* blank_value, void* d_query, clusten_strides d_query_strides,
+                                       void* probs, void* d_logit, float* blank_prob, float* d_blank_logit, float scale,
+                                       clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!query || !key || !value || !d_out || !out || !lse || !plan || !bias_table || !blank_key || !blank_value ||
+        !d_query || !probs || !d_logit || !blank_prob || !d_blank_logit) {
+        return CLUSTEN_ERR_NULL_POINTER;
+    }
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (int st = check_attn_shape(shape)) return st;
+    if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
+        !strides_ok(d_out_strides, shape.C) || !strides_ok(out_strides, shape.C) || !strides_ok(d_query_strides, shape.C)) {
+        return CLUSTEN_ERR_BAD_STRIDE;
+    }
+    if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
+    return launch_cluster_attention_backward(query, query_strides, key, key_strides, value, value_strides, d_out,
+                                             d_out_strides, out, out_strides, lse, nullptr, bias_table, nullptr, nullptr,
+                                             blank_key, blank_value, d_query, d_query_strides, probs, d_logit, blank_prob,
+                                             d_blank_logit, scale, lists_shared != 0, plan, shape, dtype, as_stream(stream));
 }
 
 size_t clusten_cluster_pairs_bytes(int B, int rows, int M, int n_rows) {

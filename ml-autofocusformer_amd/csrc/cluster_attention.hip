@@ -38,7 +38,7 @@ namespace clusten {
 int launch_cluster_attention_f32(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                                 clusten_strides os, float scale, int lists_shared, const void* plan,
+                                 clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
                                  const clusten_attn_shape& s, hipStream_t stream);   // cluster_attention_f32.hip
 
 namespace {
@@ -106,7 +106,8 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     clusten_strides vs, const int32_t* __restrict__ cluster_idx, const T* __restrict__ table,
     const int64_t* __restrict__ pe_idx, const int64_t* __restrict__ mask, const float* __restrict__ blank_k,
     const float* __restrict__ blank_v, T* __restrict__ out, clusten_strides os, int H_all, int N, float scale,
-    int tiles_per_batch, int total_tiles, int lists_shared, int head_groups, const char* __restrict__ plan) {
+    int tiles_per_batch, int total_tiles, int lists_shared, int head_groups, const char* __restrict__ plan,
+    float* __restrict__ lse) {
     typedef short S4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) S4* LdsS4;
 
@@ -289,7 +290,10 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
             sum += p[r];
         }
         const float eb = __expf(bl - mx);
-        const float inv = 1.f / (oct_sum(sum) + eb);
+        const float total = oct_sum(sum) + eb;
+        const float inv = 1.f / total;
+        // for a backward pass that recomputes the probabilities: the logarithm of the softmax's denominator
+        if (lse != nullptr && i == 0 && t < nt) lse[((int64_t)b * H_all + h0 + h) * N + i0 + t] = mx + __logf(total);
 #pragma unroll
         for (int r = 0; r < kR; ++r) p[r] *= inv;
         if (i == 0) *reinterpret_cast<float*>(stage + PB_BASE + t * 4) = eb * inv;
@@ -382,14 +386,15 @@ template <typename T>
 int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out, clusten_strides os,
-                 float scale, int lists_shared, const void* plan, const clusten_attn_shape& s, hipStream_t stream) {
+                 float scale, int lists_shared, const void* plan, float* lse, const clusten_attn_shape& s,
+                 hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int groups = head_groups_for(total, s.H);  // 196 tokens x 8 heads, B = 128: 69.6 -> 63.9 us
     hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total * groups)), dim3(kWave), 0, stream,
                        static_cast<const T*>(q), qs, static_cast<const T*>(k), ks, static_cast<const T*>(v), vs,
                        cluster_idx, static_cast<const T*>(table), pe_idx, mask, blank_k, blank_v, static_cast<T*>(out),
-                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups, static_cast<const char*>(plan));
+                       os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups, static_cast<const char*>(plan), lse);
     return launch_status();
 }
 
@@ -412,8 +417,8 @@ int launch_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, int lists_shared, const void* plan, clusten_attn_shape s,
-                             int dtype, hipStream_t stream) {
+                             clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
+                             clusten_attn_shape s, int dtype, hipStream_t stream) {
     if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
     if (s.C != kC || s.M != kM) return CLUSTEN_ERR_BAD_DIMS;
     const size_t eb = dtype_size(dtype);
@@ -423,14 +428,14 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
     if (!ok) return CLUSTEN_ERR_UNALIGNED;
     if (dtype == CLUSTEN_F32) {
         return launch_cluster_attention_f32(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os,
-                                            scale, lists_shared, plan, s, stream);
+                                            scale, lists_shared, plan, lse, s, stream);
     }
     if (dtype == CLUSTEN_F16) {
         return launch_typed<f16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                   lists_shared, plan, s, stream);
+                                   lists_shared, plan, lse, s, stream);
     }
     return launch_typed<bf16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                lists_shared, plan, s, stream);
+                                lists_shared, plan, lse, s, stream);
 }
 
 }  // namespace clusten

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_f32_kernel(
     const float* __restrict__ table, const int64_t* __restrict__ pe_idx, const int64_t* __restrict__ mask,
     const float* __restrict__ blank_k, const float* __restrict__ blank_v, float* __restrict__ out, clusten_strides os,
     int H_all, int N, float scale, int tiles_per_batch, int total_tiles, int lists_shared, int head_groups,
-    const char* __restrict__ plan) {
+    const char* __restrict__ plan, float* __restrict__ lse) {
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
     // a workgroup serves the heads [h0, h0 + H) of its tile (see head_groups_for())
@@ -236,7 +236,9 @@ __global__ __launch_bounds__(kWave) void cluster_attention_f32_kernel(
             sum += p[r];
         }
         const float eb = __expf(bl - mx);
-        const float inv = 1.f / (oct_sum(sum) + eb);
+        const float total = oct_sum(sum) + eb;
+        const float inv = 1.f / total;
+        if (lse != nullptr && i == 0 && t < nt) lse[((int64_t)b * H_all + h0 + h) * N + i0 + t] = mx + __logf(total);
 #pragma unroll
         for (int r = 0; r < kR; ++r) p[r] *= inv;
         if (i == 0) *reinterpret_cast<float*>(stage + PB_BASE + t * 4) = eb * inv;
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_f32_kernel(
 int launch_cluster_attention_f32(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                                 clusten_strides os, float scale, int lists_shared, const void* plan,
+                                 clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
                                  const clusten_attn_shape& s, hipStream_t stream) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
@@ -341,7 +343,7 @@ int launch_cluster_attention_f32(const void* q, clusten_strides qs, const void* 
                        static_cast<const float*>(q), qs, static_cast<const float*>(k), ks, static_cast<const float*>(v), vs,
                        cluster_idx, static_cast<const float*>(table), pe_idx, mask, blank_k, blank_v,
                        static_cast<float*>(out), os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups,
-                       static_cast<const char*>(plan));
+                       static_cast<const char*>(plan), lse);
     return launch_status();
 }
 

@@ -75,12 +75,22 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
 // blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16, F32}, C = 32;
 //   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48) — or (1,N,.) each
 //   when lists_shared;
-//   blank_k, blank_v : fp32 (H,C).
+//   blank_k, blank_v : fp32 (H,C);  lse (may be null): fp32 (B,H,N), the logarithm of each softmax's denominator.
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                              const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
-                             clusten_strides os, float scale, int lists_shared, const void* plan, clusten_attn_shape s,
-                             int dtype, hipStream_t stream);
+                             clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
+                             clusten_attn_shape s, int dtype, hipStream_t stream);
+// The query-side half of that kernel's backward (16-bit data): d_q, the recomputed probabilities and the logit
+// gradients as (B,H,N,48) tensors of T, the blank token's probability and logit gradient as fp32 (B,H,N): see
+// cluster_attention_bwd.hip.  d_out, out: strided (B,H,N,C) like q; lse: what the forward wrote.
+int launch_cluster_attention_backward(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
+                                      clusten_strides vs, const void* d_out, clusten_strides gs, const void* out,
+                                      clusten_strides os, const float* lse, const int32_t* cluster_idx, const void* table,
+                                      const int64_t* pe_idx, const int64_t* mask, const float* blank_k,
+                                      const float* blank_v, void* d_q, clusten_strides dqs, void* probs, void* d_logit,
+                                      float* p_blank, float* ds_blank, float scale, int lists_shared, const void* plan,
+                                      clusten_attn_shape s, int dtype, hipStream_t stream);
 // The per-tile plan the kernel above reads instead of cluster_idx, pe_idx and mask when it is given one (what it
 // would work out from them before its first head): B = batch elements of the index tensors.
 size_t cluster_attention_plan_bytes(int B, int N);

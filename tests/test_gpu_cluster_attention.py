@@ -203,3 +203,61 @@ def test_plan_built_once_gives_the_same_bits(device, kind, dtype):
     with pytest.raises(RuntimeError):       # a plan of other lists
         _native.cluster_attention(d(q)[:, :, :64], d(k)[:, :, :64], d(v)[:, :, :64], None, d(table), None, None,
                                   d(blank_k), d(blank_v), plan=plan1)
+
+
+def _reference_grads(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale, d_out):
+    """Gradients of `_reference` by autograd, in fp32 from the same rounded inputs."""
+    b, h, n, c = q.shape
+    leaves = [t.float().clone().requires_grad_(True) for t in (q, k, v, table, blank_k, blank_v)]
+    qf, kf, vf, tf, bkf, bvf = leaves
+    rows = idx[:, None, :, :, None].expand(b, h, n, idx.shape[2], c)
+    kg = kf[:, :, :, None, :].expand(b, h, n, idx.shape[2], c).gather(2, rows)           # (b,h,n,m,c)
+    vg = vf[:, :, :, None, :].expand(b, h, n, idx.shape[2], c).gather(2, rows)
+    attn = (qf[:, :, :, None, :] * kg).sum(-1) * scale + tf[pe_idx].permute(0, 3, 1, 2)
+    if mask is not None:
+        attn = attn + (1 - mask.reshape(b, 1, n, -1)) * (-100.0)
+    blank = (qf * bkf.reshape(1, h, 1, c)).sum(-1, keepdim=True) * scale
+    p = torch.softmax(torch.cat([attn, blank], dim=-1), dim=-1)
+    out = (p[..., :-1, None] * vg).sum(3) + p[..., -1:] * bvf.reshape(1, h, 1, c)
+    out = out.permute(0, 2, 1, 3).reshape(b, n, h * c)
+    out.backward(d_out.float())
+    return [t.grad for t in leaves]
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_backward_against_autograd_through_the_composition(device, kind, dtype):
+    """`cluster_attention_backward` (d_query, the recomputed probabilities and the logit gradients in one kernel) with
+    the sums that complete it - the scatters over sorted pair lists, the bias table's gradient, the blank token's -
+    against autograd through the fp32 composition, with a random upstream gradient."""
+    gen = torch.Generator().manual_seed(88)
+    d = lambda x: None if x is None else x.to(device)
+    scale = C ** -0.5
+    for b, h, n in ((2, 3, 392), (1, 1, 64), (2, 4, 396)):
+        for with_mask in (False, True):
+            q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, dtype, with_mask)
+            d_out = torch.randn(b, n, h * C, generator=gen).to(dtype)
+            ref = _reference_grads(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale, d_out)
+            plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+            out, lse = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                 scale=scale, plan=plan, return_lse=True)
+            plain = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                              scale=scale, plan=plan)
+            assert torch.equal(out, plain) and lse.shape == (b, h, n) and bool(torch.isfinite(lse).all())
+            dq, probs, d_logit, p_b, ds_b = _native.cluster_attention_backward(
+                d(q), d(k), d(v), d(d_out), out, lse, plan, d(table), d(blank_k), d(blank_v), scale=scale)
+            pairs = _native.cluster_pairs(d(idx))
+            assert int(_native.pairs_not_whole(pairs)) == 0
+            g_view = d(d_out).view(b, n, h, C).permute(0, 2, 1, 3)
+            dv = _native.scatter_rows_by_cluster(probs, g_view.contiguous(), pairs)
+            dk = _native.scatter_rows_by_cluster(d_logit, d(q), pairs).float() * scale
+            d_table = _native.bias_table_grad(d_logit, d(pe_idx), table.shape[0])
+            d_bk = (ds_b.unsqueeze(-1) * d(q).float()).sum((0, 2)).reshape(-1) * scale
+            d_bv = (p_b.unsqueeze(-1) * g_view.float()).sum((0, 2)).reshape(-1)
+            tol = TOL[dtype]
+            what = "%s %s n=%d mask=%s" % (kind, dtype, n, with_mask)
+            for name, got, want in (("d_query", dq, ref[0]), ("d_key", dk, ref[1]), ("d_value", dv, ref[2]),
+                                    ("d_table", d_table, ref[3]), ("d_blank_key", d_bk, ref[4]),
+                                    ("d_blank_value", d_bv, ref[5])):
+                err = oracle.rel_err(got.float().cpu(), want)
+                assert err <= 2 * tol, "%s %s rel err %.3g" % (name, what, err)
