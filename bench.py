@@ -581,6 +581,37 @@ def main():
             "one_kernel_us": round(per_a[0] * 1e3, 1), "three_kernels_us": round(per_a[1] * 1e3, 1),
             "one_kernel_with_plan_us": round(per_a[2] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes, "one_kernel_GBps": round(fused_bytes / per_a[0] / 1e6, 1)}
+        # ... and its backward: one kernel for the query side (probabilities recomputed) + the two scatters over sorted
+        # pair lists + the bias table's gradient, against the backward functions of the three operators with the
+        # softmax kernel's backward between them (pair lists of the stage built once, outside both)
+        out16, lse = _native.cluster_attention(q16, k16, v16, None, table, None, None, blank_k, blank_v, plan=plan,
+                                               return_lse=True)
+        g16 = h16(torch.randn(out16.shape, generator=gen)).cuda()
+        pairs = _native.cluster_pairs(mcase.nbhd_idx)
+        g_view = g16.view(B, 3136, 2, 32).permute(0, 2, 1, 3)
+        probs16, pb16 = _native.attn_softmax(_native.qk_forward_clusters(q16, k16, cidx), table, pe_idx, None, query=q16,
+                                             blank_key=blank_k)
+
+        g32, v32 = g_view.float().contiguous(), mcase.value
+        def fused_backward():
+            dq, p_, ds_, pb_, dsb_ = _native.cluster_attention_backward(q16, k16, v16, g16, out16, lse, plan, table,
+                                                                      blank_k, blank_v)
+            dv = _native.scatter_rows_by_cluster(p_, g_view, pairs)
+            dk = _native.scatter_rows_by_cluster(ds_, q16, pairs)
+            return _native.bias_table_grad(ds_, pe_idx, rows), dq, dk, dv
+
+        def operator_backward():
+            # (under mixed precision the softmax kernel hands AV fp32 probabilities and the AV Function casts v up)
+            d_p, dv = _native.av_backward(g32, probs16, v32, mcase.nbhd_idx)
+            d_logit, d_blank = _native.attn_softmax_backward(probs16, pb16, d_p, torch.zeros_like(pb16), torch.float16)
+            d_table = _native.bias_table_grad(d_logit, pe_idx, rows)
+            return (d_table,) + tuple(_native.qk_backward(d_logit, q16, k16, mcase.nbhd_idx)) + (dv,)
+
+        _, per_b, _ = _time_kernels([fused_backward, operator_backward], max(args.steps // 5, 5), 3)
+        other["cfg2_s1_local_attention_fp16_backward_model_built_lists"] = {
+            "one_kernel_path_us": round(per_b[0] * 1e3, 1), "operator_path_us": round(per_b[1] * 1e3, 1),
+            "what": "d_query, d_key, d_value and the bias table's gradient of one block's local attention"}
+        del out16, lse, g16, pairs, probs16, pb16, g32, v32
         # the same in fp32 (inference without mixed precision)
         table32 = table.float()
 

@@ -39,6 +39,9 @@ def default_ops():
                            cluster_attention=_native.cluster_attention,
                            cluster_attention_plan=_native.cluster_attention_plan,
                            cluster_attention_supported=_native.cluster_attention_supported,
+                           cluster_attention_backward=_native.cluster_attention_backward,
+                           cluster_attention_backward_supported=_native.cluster_attention_backward_supported,
+                           cluster_pairs=_native.cluster_pairs, scatter_rows_by_cluster=_native.scatter_rows_by_cluster,
                            dense_attention=_native.dense_attention,
                            dense_attention_supported=_native.dense_attention_supported,
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
@@ -186,6 +189,37 @@ class _AttnSoftmax(torch.autograd.Function):
         return d_logit, d_bias, None, None, d_blank.to(blank_dtype), None
 
 
+class _ClusterAttention(torch.autograd.Function):
+    """The local attention of a block between its projections (aff_transformer.py:120-155) as one kernel forward and,
+    backward, one kernel for the query side - the probabilities are recomputed from the softmax denominators the
+    forward saved - followed by the sums that complete it: the scatters over the stage's sorted pair lists (d_key,
+    d_value), the bias table's gradient, the blank token's.  No (b,h,n,m) tensor is kept between the two passes."""
+
+    @staticmethod
+    def forward(ctx, q, key, v, bias, blank_k, blank_v, plan, pairs, pe_idx, scale, ops):
+        out, lse = ops.cluster_attention(q, key, v, None, bias, None, None, blank_k, blank_v, scale=scale, plan=plan,
+                                         return_lse=True)
+        ctx.save_for_backward(q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx)
+        ctx.meta = (scale, ops)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx = ctx.saved_tensors
+        scale, ops = ctx.meta
+        b, h, n, ch = q.shape
+        d_q, probs, d_logit, blank_prob, d_blank = ops.cluster_attention_backward(
+            q, key, v, d_out, out, lse, plan, bias, blank_k, blank_v, scale=scale)
+        g = d_out.to(q.dtype).reshape(b, n, h, ch).permute(0, 2, 1, 3)
+        d_v = ops.scatter_rows_by_cluster(probs, g, pairs)
+        d_k = ops.scatter_rows_by_cluster(d_logit, q, pairs) * scale
+        d_bias = ops.bias_table_grad(d_logit, pe_idx, bias.shape[0]).to(bias.dtype)
+        d_bk = torch.einsum("bhn,bhnc->hc", d_blank, q.float()) * scale
+        d_bv = torch.einsum("bhn,bhnc->hc", blank_prob, g.float())
+        return (d_q, d_k.to(key.dtype), d_v.to(v.dtype), d_bias, d_bk.reshape(blank_k.shape).to(blank_k.dtype),
+                d_bv.reshape(blank_v.shape).to(blank_v.dtype), None, None, None, None, None)
+
+
 def _position_bias(bias, pe_idx, ops):
     """(b, h, n, m) position bias of an attention layer: row pe_idx[b,i,j] of the (rows, h) table for every pair."""
     kernel = getattr(ops, "bias_table_grad", None)
@@ -303,6 +337,17 @@ class ClusterAttention(nn.Module):
                              lists[1], lists[2], self.blank_k, self.blank_v, scale=self.scale,
                              **({"plan": plan} if plan is not None else {}))
             return self.proj_drop(_linear(self.proj, out, self.ops))
+        train_kernel = getattr(self.ops, "cluster_attention_backward", None)
+        if (train_kernel is not None and torch.is_grad_enabled() and cluster_idx is not None and not global_attn
+                and grid_lists is not None and len(grid_lists) > 4 and not (self.training and self.attn_drop.p > 0)
+                and self.ops.cluster_attention_backward_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3),
+                                                                  cluster_idx.shape[2])):
+            # training on 16-bit data: the same kernel forward, one kernel and four sums backward
+            bias = self.bias_table(table)
+            if bias.shape[0] <= 16000:
+                out = _ClusterAttention.apply(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, bias, self.blank_k,
+                                              self.blank_v, grid_lists[3], grid_lists[4], pe_idx, self.scale, self.ops)
+                return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
         if (global_attn and dense is not None and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0)
@@ -585,6 +630,16 @@ class BasicLayer(nn.Module):
                 and (feat.dtype == torch.float32 or torch.is_autocast_enabled("cuda"))):
             # the one-kernel attention of every block reads what it makes of the lists from a plan built once
             grid_lists = (cluster_idx, pe_idx, mask, planner(cluster_idx, pe_idx, mask))
+        if ((grid_lists is None or len(grid_lists) == 3) and cluster_idx is not None and planner is not None
+                and torch.is_grad_enabled() and getattr(self.ops, "cluster_attention_backward", None) is not None
+                and not global_attn and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
+                and torch.is_autocast_enabled("cuda")):
+            # training under mixed precision: the plan of the one-kernel attention and the sorted pair lists of its
+            # backward's scatters, built once for all blocks of the stage (a grid stage hands over one image's lists)
+            pairs = self.ops.cluster_pairs(member_idx)
+            if pairs is not None:
+                lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, mask)
+                grid_lists = tuple(lists) + (planner(lists[0], lists[1], lists[2]), pairs)
         carry = None
         for blk in self.blocks:
             feat, carry = blk(feat, member_idx, mask, pe_idx, global_attn, table, cluster_idx, grid_lists, carry)

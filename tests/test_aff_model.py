@@ -769,3 +769,52 @@ def test_cached_16_bit_weights_follow_the_parameters(device):
     with torch.autocast("cuda", dtype=torch.float16):
         model(x).float().sum().backward()
     assert model.head.weight.grad is not None
+
+
+@pytest.mark.gpu
+def test_training_with_the_one_kernel_attention_matches_the_operator_path(device):
+    """A training step under fp16 autocast with the local attention as one kernel forward and `cluster_attention_backward`
+    plus its sums backward, against the same step through the three operators and the softmax kernels: same loss,
+    parameter gradients within the noise of fp16 intermediates."""
+    from aff.model import default_ops
+    fused_ops = default_ops()
+    plain = dict(vars(default_ops()))
+    plain.pop("cluster_attention_backward")
+    plain_ops = SimpleNamespace(**plain)
+    cfg = dict(embed_dim=(64, 128, 256, 512), num_heads=(2, 4, 8, 16), img_size=128)
+    a = small_model(fused_ops, **cfg).to(device).train()
+    b = small_model(plain_ops, **cfg).to(device).train()
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(2, 3, 128, 128, generator=torch.Generator().manual_seed(5)).to(device)
+    target = torch.tensor([3, 7], device=device)
+    losses = []
+    for m in (a, b):
+        with torch.autocast("cuda", dtype=torch.float16):
+            loss = torch.nn.functional.cross_entropy(m(x).float(), target)
+        loss.backward()
+        losses.append(float(loss.detach()))
+    assert abs(losses[0] - losses[1]) <= 2e-2 * max(1.0, abs(losses[1]))
+    # a gradient that is pure rounding noise (a bias in front of a batch norm) is measured against the largest gradient
+    # of the model, not against itself
+    biggest = max(float(p.grad.abs().max()) for p in b.parameters() if p.grad is not None)
+    checked = 0
+    for (name, pa), (_, pb) in zip(a.named_parameters(), b.named_parameters()):
+        assert (pa.grad is None) == (pb.grad is None), name
+        if pa.grad is None:
+            continue
+        scale = max(float(pb.grad.abs().max()), 1e-2 * biggest)
+        err = float((pa.grad - pb.grad).abs().max()) / scale
+        assert err <= 5e-2, "%s rel err %.3g" % (name, err)
+        checked += 1
+    assert checked > 50
+    # the fused path was taken: its Function is in the graph of a fresh forward
+    with torch.autocast("cuda", dtype=torch.float16):
+        y = a(x)
+    seen, stack = set(), [y.grad_fn]
+    while stack:
+        f = stack.pop()
+        if f is None or f in seen:
+            continue
+        seen.add(f)
+        stack.extend(nf for nf, _ in f.next_functions)
+    assert any("_ClusterAttention" in type(f).__name__ for f in seen)
