@@ -920,8 +920,7 @@ def dense_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
     blank_value = blank_value.detach().reshape(h, c).float().contiguous()
     out = torch.empty(b, n, h, c, dtype=dtype, device=device)
     if out.numel() == 0:
-        flat = out.reshape(b, n, h * c)
-        return (flat, torch.empty(b, h, n, dtype=torch.float32, device=device)) if return_lse else flat
+        return out.reshape(b, n, h * c)
     out_view = out.permute(0, 2, 1, 3)                                   # (B,H,N,C) view of the (B,N,H,C) memory
     shape = AttnShape(b, h, n, c, n)
     with torch.cuda.device(device):
