@@ -261,3 +261,30 @@ def test_backward_against_autograd_through_the_composition(device, kind, dtype):
                                     ("d_blank_value", d_bv, ref[5])):
                 err = oracle.rel_err(got.float().cpu(), want)
                 assert err <= 2 * tol, "%s %s rel err %.3g" % (name, what, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_softmax_denominators_of_the_training_forward(device, dtype):
+    """`return_lse=True`: the same result bit for bit, and log(sum of exp(logit)) over the 48 neighbours and the
+    blank token for every (image, head, token)."""
+    gen = torch.Generator().manual_seed(89)
+    d = lambda x: None if x is None else x.to(device)
+    b, h, n = 2, 3, 204
+    scale = C ** -0.5
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", dtype, True)
+    plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+    out, lse = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                         scale=scale, plan=plan, return_lse=True)
+    plain = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                      scale=scale, plan=plan)
+    assert torch.equal(out, plain)
+    qf, kf, tf = q.float(), k.float(), table.float()
+    attn = oracle.qk_gather_chunked(qf, kf, idx) * scale + tf[pe_idx].permute(0, 3, 1, 2)
+    attn = attn + (1 - mask.reshape(b, 1, n, -1)) * (-100.0)
+    blank = (qf * blank_k.reshape(1, h, 1, C)).sum(-1, keepdim=True) * scale
+    want = torch.logsumexp(torch.cat([attn, blank], dim=-1), dim=-1)
+    assert lse.shape == (b, h, n) and lse.dtype == torch.float32
+    assert float((lse.cpu() - want).abs().max()) <= (1e-4 if dtype == torch.float32 else 2e-3)
+    with pytest.raises(RuntimeError):       # the denominators are written by the planned kernel only
+        _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v),
+                                  return_lse=True)
