@@ -2,7 +2,8 @@
 // one kernel, with the probabilities recomputed from the saved logarithm of each softmax's denominator.
 //
 // With  x[t,j] = scale * q[t].k[row(t,j)] + bias[t,j] - 100 * (1 - mask[t,j]),  p = exp(x - lse),  p_b = exp(x_b - lse)
-// (x_b = scale * q[t].blank_k), and  delta[t] = sum_c d_out[t,c] * out[t,c] :
+// (x_b = scale * q[t].blank_k), and  delta[t] = sum_c d_out[t,c] * out[t,c]  (= sum_j p[t,j] dP[t,j] + p_b[t] dP_b[t]: a
+// tile whose distinct clusters fit one pass forms it that way, without the rounding of `out` to 16 bits) :
 //   dP[t,j]   = d_out[t] . v[row(t,j)]              dP_b[t]  = d_out[t] . blank_v
 //   dS[t,j]   = p[t,j] * (dP[t,j] - delta[t])       dS_b[t]  = p_b[t] * (dP_b[t] - delta[t])
 //   d_q[t]    = scale * (sum_j dS[t,j] * k[row(t,j)] + dS_b[t] * blank_k)
@@ -174,8 +175,10 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
 
         lds_sync_vm<0>();   // the rows of this head's first pass, its q and d_out rows, the operands above
 
-        // per token: delta = d_out . out, the blank token's logit, probability and logit gradient
-        float delta, p_b, ds_b;
+        // per token: delta = d_out . out, the blank token's logit, probability and logit gradient.  (delta also equals
+        // sum_j p_j dP_j + p_b dP_b; a tile whose clusters fit one pass takes it from there, below: the rounding of
+        // `out` to 16 bits does not enter then.)
+        float delta, p_b, ds_b, dpb_t;
         {
             float o4[4], g4[4], q4[4];
             Quad4::unpack(o_raw, o4);
@@ -186,6 +189,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
             const float bl = oct_sum(q4[0] * bk.x + q4[1] * bk.y + q4[2] * bk.z + q4[3] * bk.w) * scale;
             p_b = __expf(bl - lse_t);
             ds_b = p_b * (dpb - delta);
+            dpb_t = dpb;
         }
 
         float p_all[kR], ds_all[kR];
@@ -216,19 +220,29 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
             }
             lds_sync();
             // ---- the lane's own slots: p and dS ---------------------------------------------------------------
-            float ds_pass[kR];
+            float ds_pass[kR], pr_[kR], dp_[kR];
+            bool in_[kR];
+            float pdp = 0.f;
 #pragma unroll
             for (int r = 0; r < kR; ++r) {
                 const unsigned u = (unsigned)(us[r] - pass * kPassRuns);
-                const bool in = u < (unsigned)kPassRuns;
+                in_[r] = u < (unsigned)kPassRuns;
                 const int cell = (t * kSRow + (int)min(u, (unsigned)kPassRuns - 1) * 8 + i) * 4;
                 const float sc = *reinterpret_cast<const float*>(stage + S_BASE + cell);
-                const float dp = *reinterpret_cast<const float*>(stage + S2_BASE + cell);
-                const float pr = __expf(sc * scale + bias[r] - lse_t);
-                const float ds = pr * (dp - delta);
-                p_all[r] = in ? pr : p_all[r];
-                ds_all[r] = in ? ds : ds_all[r];
-                ds_pass[r] = in ? ds : 0.f;
+                dp_[r] = *reinterpret_cast<const float*>(stage + S2_BASE + cell);
+                pr_[r] = __expf(sc * scale + bias[r] - lse_t);
+                pdp += in_[r] ? pr_[r] * dp_[r] : 0.f;
+            }
+            if (passes == 1) {
+                delta = oct_sum(pdp) + p_b * dpb_t;
+                ds_b = p_b * (dpb_t - delta);
+            }
+#pragma unroll
+            for (int r = 0; r < kR; ++r) {
+                const float ds = pr_[r] * (dp_[r] - delta);
+                p_all[r] = in_[r] ? pr_[r] : p_all[r];
+                ds_all[r] = in_[r] ? ds : ds_all[r];
+                ds_pass[r] = in_[r] ? ds : 0.f;
             }
             if (twice) {
 #pragma unroll
