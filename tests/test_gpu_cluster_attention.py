@@ -288,3 +288,24 @@ def test_softmax_denominators_of_the_training_forward(device, dtype):
     with pytest.raises(RuntimeError):       # the denominators are written by the planned kernel only
         _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v),
                                   return_lse=True)
+
+
+def test_backward_with_lists_shared_by_the_batch(device):
+    """One image's lists (and plan) for the whole batch, as a grid stage hands them over: the backward kernel gives the
+    same bits as with the lists repeated for every image."""
+    gen = torch.Generator().manual_seed(90)
+    d = lambda x: None if x is None else x.to(device)
+    b, h, n = 3, 2, 200
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True)
+    c1, p1, m1 = cidx[:1].contiguous(), pe_idx[:1].contiguous(), mask[:1].contiguous()
+    d_out = torch.randn(b, n, h * C, generator=gen).half()
+    results = []
+    for lists in ((c1, p1, m1), (c1.expand(b, -1, -1).contiguous(), p1.expand(b, -1, -1).contiguous(),
+                                  m1.expand(b, -1, -1).contiguous())):
+        plan = _native.cluster_attention_plan(d(lists[0]), d(lists[1]), d(lists[2]))
+        out, lse = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                             plan=plan, return_lse=True)
+        results.append((out, lse) + tuple(_native.cluster_attention_backward(
+            d(q), d(k), d(v), d(d_out), out, lse, plan, d(table), d(blank_k), d(blank_v))))
+    for one, every in zip(*results):
+        assert torch.equal(one, every)
