@@ -6,12 +6,16 @@ stage-1 shape (BASELINE.json configs[2], stage 1: B128, H2, N3136, head dim 32, 
 fp32; WF 3136 -> 784 tokens, 64 channels, 4 inner channels): one QK launch, one AV launch, one WF
 launch through the C ABI, inputs resident in HBM.  `value` is the algorithmic bytes of the three ops
 (every input read once, every output written once, int64 neighbour lists) divided by the time of a
-step.  The three kernels take a third of the step each; the `roofline` object prices the one furthest
-below the 8 TB/s HBM peak among those tied for the longest (per-launch HIP-event timings taken inside
-the timed region) and carries the step's own fraction beside it; `replay_probe` times the same three
-kernels compiled without their arithmetic (same loads, LDS traffic and stores) in the same interleaved
-pass; `cpu_baseline` is the PyTorch gather oracle timed on the host cores on a batch slice of the same
-workload, `config0_cpu` the reference's own CPU-runnable configuration timed in full on both sides.
+step.  The three kernels take a third of the step each, so the `roofline` object prices the step: its
+`frac` is `value` / 8 TB/s; `kernels` lists the three kernels with the median and the minimum of at
+least 50 per-launch HIP-event timings (after at least 10 untimed launches, whatever --steps says), and
+`roofline.lowest_kernel` names the one furthest below the peak.  `parity` compares the three outputs
+of the headline tensors with the gather oracle on batch elements 0, 63 and 127 and repeats the
+comparison bit for bit on integer-valued data; `replay_probe` times the same three kernels compiled
+without their arithmetic (same loads, LDS traffic and stores; libclusten_probe.so) in the same
+interleaved pass; `cpu_baseline` is the PyTorch gather oracle timed on the host cores on a batch slice
+of the same workload, `config0_cpu` the reference's own CPU-runnable configuration timed in full on
+both sides.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
 
@@ -44,8 +48,9 @@ def _time_kernels(fns, steps, warmup):
 
     The first timed pass has one event before and one after its `steps` steps and nothing between the launches:
     its duration is the throughput figure.  The second pass records an event after every launch (a marker on
-    the stream that costs a few microseconds of gap per launch) for the per-kernel averages.
-    Returns (ms per step of the first pass, [average ms per launch of each closure], host wall ms per step)."""
+    the stream that costs a few microseconds of gap per launch) for the per-kernel figures.
+    Returns (ms per step of the first pass, [median ms per launch of each closure], host wall ms per step,
+    [minimum ms per launch of each closure])."""
     import torch
 
     for _ in range(warmup):
@@ -70,8 +75,9 @@ def _time_kernels(fns, steps, warmup):
             fn()
             marks[s][i + 1].record()
     torch.cuda.synchronize()
-    per = [sum(marks[s][i].elapsed_time(marks[s][i + 1]) for s in range(steps)) / steps for i in range(len(fns))]
-    return region_ms / steps, per, wall_ms / steps
+    samples = [sorted(marks[s][i].elapsed_time(marks[s][i + 1]) for s in range(steps)) for i in range(len(fns))]
+    med = [(x[(len(x) - 1) // 2] + x[len(x) // 2]) / 2 for x in samples]
+    return region_ms / steps, med, wall_ms / steps, [x[0] for x in samples]
 
 
 def _cpu_baseline(attn_case, wf_case, full_bytes, full_batch, slice_b=32, budget_s=12.0):
@@ -114,6 +120,45 @@ def _cpu_baseline(attn_case, wf_case, full_bytes, full_batch, slice_b=32, budget
     }
 
 
+def _parity(acase, wcase, attn_dev, dev_attn_tensors, dw, picks=(0, 63, 127)):
+    """The three outputs at the headline tensors against the gather oracle on the host, on the batch elements `picks`
+    (outside every timed region): max |x - ref| / max |ref| per operator, and the same three comparisons bit for bit on
+    integer-valued data of the same shapes and lists (sums of products of small integers are exact in fp32)."""
+    import torch
+    from clusten import _native
+    from oracle import clusten_oracle as oracle
+
+    q, k, v, idx = dev_attn_tensors
+    picks = [b for b in picks if b < q.shape[0]]
+    sel = torch.tensor(picks)
+    dsel = sel.to(q.device)
+    out = {"batch_elements": picks, "tolerance_fp32": 1e-5}
+    got_qk = _native.qk_forward(q, k, idx).index_select(0, dsel)
+    got_av = _native.av_forward(attn_dev, v, idx).index_select(0, dsel)
+    got_wf = _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx).index_select(0, dsel)
+    a_host = attn_dev.index_select(0, dsel).cpu()
+    hq, hk, hv, hidx = (t.index_select(0, sel) for t in (acase.query, acase.key, acase.value, acase.nbhd_idx))
+    hw, hf, hwidx = (t.index_select(0, sel) for t in (wcase.weights, wcase.feat, wcase.nbhd_idx))
+    out["qk_rel_err"] = float("%.3g" % oracle.rel_err(got_qk, oracle.qk_gather_chunked(hq, hk, hidx)))
+    out["av_rel_err"] = float("%.3g" % oracle.rel_err(got_av, oracle.av_gather_chunked(a_host, hv, hidx)))
+    out["wf_rel_err"] = float("%.3g" % oracle.rel_err(got_wf, oracle.wf_gather_chunked(hw, hf, hwidx)))
+    gen = torch.Generator().manual_seed(4242)
+    ints = lambda shape, lo, hi: torch.randint(lo, hi, shape, generator=gen).float()
+    iq, ik, iv = ints(hq.shape, -8, 9), ints(hk.shape, -8, 9), ints(hv.shape, -8, 9)
+    ia = ints(a_host.shape, 0, 5)
+    iw, ife = ints(hw.shape, 0, 5), ints(hf.shape, -8, 9)
+    dev = q.device
+    didx, dwidx = hidx.to(dev), hwidx.to(dev)
+    exact = {
+        "qk": torch.equal(_native.qk_forward(iq.to(dev), ik.to(dev), didx).cpu(), oracle.qk_gather_chunked(iq, ik, hidx)),
+        "av": torch.equal(_native.av_forward(ia.to(dev), iv.to(dev), didx).cpu(), oracle.av_gather_chunked(ia, iv, hidx)),
+        "wf": torch.equal(_native.wf_forward(iw.to(dev), ife.to(dev), dwidx).cpu(), oracle.wf_gather_chunked(iw, ife, hwidx)),
+    }
+    out["integer_data_bit_exact"] = exact
+    out["ok"] = bool(all(exact.values()) and max(out["qk_rel_err"], out["av_rel_err"], out["wf_rel_err"]) <= 1e-5)
+    return out
+
+
 def _config0(steps=200):
     """Configuration 0 (the reference's CPU-runnable case: QK forward, B2 H2 N1024 C32 M48 fp32) timed in full on the
     host cores (gather oracle, 3 untimed + 10 timed calls, median) and through the HIP kernel on the same tensors."""
@@ -138,7 +183,7 @@ def _config0(steps=200):
     d = case.to("cuda")
     got = _native.qk_forward(d.query, d.key, d.nbhd_idx)
     err = oracle.rel_err(got, ref)
-    _, per, _ = _time_kernels([lambda: _native.qk_forward(d.query, d.key, d.nbhd_idx)], steps, 10)
+    _, per, _, _ = _time_kernels([lambda: _native.qk_forward(d.query, d.key, d.nbhd_idx)], steps, 10)
     return {"shape": "QK forward B%d H%d N%d C%d M%d fp32" % (B, H, N, C, M), "algorithmic_bytes": nbytes,
             "cpu_ms": round(cpu_s * 1e3, 3), "cpu_GBps": round(nbytes / cpu_s / 1e9, 3),
             "cpu_cores": torch.get_num_threads(), "cpu_calls": "3 untimed + 10 timed, median",
@@ -152,7 +197,7 @@ def _stream_gather_interference(tiles=50176, gathers=24, reps=20):
     tile) and gathers that hit the L2 (24 KiB per tile inside 800 KB windows shared by 392 tiles — the QK shape), alone
     and together, without arithmetic.  The streams rotate over four buffers so that they come from memory."""
     import torch
-    from clusten import _native
+    import probe
 
     sets = 4
     ins = [torch.empty(tiles * 5120, dtype=torch.uint8, device="cuda").random_(0, 255) for _ in range(sets)]
@@ -165,9 +210,9 @@ def _stream_gather_interference(tiles=50176, gathers=24, reps=20):
         def one():
             i = turn[0] % sets
             turn[0] += 1
-            _native.stream_gather_probe(ins[i], outs[i], rows, tiles, gathers, 3136, 392, mode)
+            probe.stream_gather_probe(ins[i], outs[i], rows, tiles, gathers, 3136, 392, mode)
 
-        _, per, _ = _time_kernels([one], reps, 4)
+        _, per, _, _ = _time_kernels([one], reps, 4)
         res[name] = round(per[0] * 1e3, 1)
     res["stream_bytes"] = tiles * 8192
     res["gather_bytes"] = tiles * gathers * 1024
@@ -179,16 +224,16 @@ def _stream_gather_interference(tiles=50176, gathers=24, reps=20):
 
 def _copy_bandwidth(nbytes=1 << 30, reps=20):
     import torch
-    from clusten import _native
+    import probe
 
     src = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda").normal_()
     dst = torch.empty_like(src)
     for _ in range(3):
-        _native.copy_probe(src, dst)
+        probe.copy_probe(src, dst)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
-        _native.copy_probe(src, dst)
+        probe.copy_probe(src, dst)
     e1.record()
     torch.cuda.synchronize()
     return 2 * nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
@@ -221,7 +266,7 @@ def _bench_attn(case, steps, warmup, dtype=None):
         turn[1] += 1
         return _native.av_forward(a[4], a[2], a[3])
 
-    _, per, _ = _time_kernels([qk, av], steps, warmup)
+    _, per, _, _ = _time_kernels([qk, av], steps, warmup)
     return {"shape": "B%d H%d N%d C%d M%d %s" % (B, H, N, C, M, str(q.dtype).replace("torch.", "")),
             "qk_us": round(per[0] * 1e3, 1), "qk_GBps": round(nbytes / per[0] / 1e6, 1),
             "av_us": round(per[1] * 1e3, 1), "av_GBps": round(nbytes / per[1] / 1e6, 1), "bytes_each": nbytes,
@@ -240,7 +285,7 @@ def _bench_backward(acase, wcase, steps, warmup):
     d_feat = torch.randn_like(q)
     d_out = torch.randn(w.weights.shape[0], w.weights.shape[1], w.weights.shape[3], w.feat.shape[2],
                         dtype=w.feat.dtype, device="cuda")
-    _, per, _ = _time_kernels([lambda: _native.qk_backward(d_attn, q, k, idx),
+    _, per, _, _ = _time_kernels([lambda: _native.qk_backward(d_attn, q, k, idx),
                                lambda: _native.av_backward(d_feat, attn, v, idx),
                                lambda: _native.wf_backward(d_out, w.weights, w.feat, w.nbhd_idx)], steps, warmup)
     return {"qk_backward_us": round(per[0] * 1e3, 1), "av_backward_us": round(per[1] * 1e3, 1),
@@ -265,10 +310,34 @@ def _bench_wf(case, steps, warmup):
         turn[0] += 1
         return _native.wf_forward(*a)
 
-    _, per, _ = _time_kernels([wf], steps, warmup)
+    _, per, _, _ = _time_kernels([wf], steps, warmup)
     return {"shape": "B%d N%d->%d C%d M%d IC%d %s" % (B, N, Nout, C, M, IC, str(d.feat.dtype).replace("torch.", "")),
             "wf_us": round(per[0] * 1e3, 1), "wf_GBps": round(nbytes / per[0] / 1e6, 1), "bytes": nbytes,
             "input_sets_rotated": copies}
+
+
+def _bench_local_attention(B, H, N, dtype, steps, warmup):
+    """The one-kernel local attention (QK, bias, mask, blank token, softmax, AV) of one block at a stage's shape on
+    lists built by the model's clustering, with the plan of the stage; microseconds per call."""
+    import torch
+    import workloads as wl
+    from clusten import _native
+
+    mcase = wl.attn_case("model", 29, B=B, H=H, N=N, C=32, lists="model_built").to("cuda")
+    cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()
+    gen = torch.Generator().manual_seed(1029)
+    rows = 111 * 111
+    q, k, v = (t.to(dtype) for t in (mcase.query, mcase.key, mcase.value))
+    table = torch.randn(rows, H, generator=gen).to(dtype).cuda()
+    pe_idx = torch.randint(rows, (B, N, 48), generator=gen).cuda()
+    blank_k, blank_v = torch.randn(H * 32, generator=gen).cuda(), torch.randn(H * 32, generator=gen).cuda()
+    plan = _native.cluster_attention_plan(cidx, pe_idx, None)
+    _, per, _, per_min = _time_kernels([lambda: _native.cluster_attention(q, k, v, None, table, None, None, blank_k,
+                                                                          blank_v, plan=plan)], steps, warmup)
+    nbytes = 4 * q.numel() * q.element_size() + plan.numel()
+    return {"shape": "B%d H%d N%d C32 M48 %s, model-built lists, planned" % (B, H, N, str(dtype).replace("torch.", "")),
+            "median_us": round(per[0] * 1e3, 1), "min_us": round(per_min[0] * 1e3, 1),
+            "bytes_q_k_v_out_plan": nbytes, "GBps": round(nbytes / per[0] / 1e6, 1)}
 
 
 def _aff_tiny_throughput(batch=128, warmup=50, timed=30, tune_gemms=True):
@@ -407,8 +476,11 @@ def main():
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
+    ap.add_argument("--batch", type=int, default=None,
+                    help="batch size of the --only wf-cfg3* / ca-* profiler legs (default: the configuration's own)")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model", "replay-qk", "replay-av", "replay-wf",
-                                       "interference"),
+                                       "interference", "wf-cfg3", "wf-cfg3-f32", "ca-s1-f16", "ca-s1-f32", "ca-s2-f16",
+                                       "ca-s3-f16"),
                     default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
@@ -417,6 +489,7 @@ def main():
                  "needs no exchange); --gpus %d is not supported, use --gpus 1." % args.gpus)
 
     import torch
+    import probe
     import workloads as wl
     from clusten import _native
 
@@ -430,6 +503,17 @@ def main():
 
     if args.only == "interference":
         print(json.dumps({"only": "interference", **_stream_gather_interference()}), flush=True)
+        return
+    if args.only in ("wf-cfg3", "wf-cfg3-f32"):   # configuration 3's WF (9216 -> 2304 tokens, C = 128), bf16 or fp32
+        dt = torch.bfloat16 if args.only == "wf-cfg3" else torch.float32
+        print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
+                          **_bench_wf(wl.config3_wf(dtype=dt, B=args.batch or 64), args.steps, args.warmup)}), flush=True)
+        return
+    if args.only and args.only.startswith("ca-"):   # the one-kernel local attention at a stage's shape, with its plan
+        stage, dt = int(args.only[4]), (torch.float16 if args.only.endswith("f16") else torch.float32)
+        H, N = {1: (2, 3136), 2: (4, 784), 3: (8, 196)}[stage]
+        print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
+                          **_bench_local_attention(args.batch or 128, H, N, dt, args.steps, args.warmup)}), flush=True)
         return
     B = 128
     acase = wl.config2_attn(1, B=B)
@@ -445,10 +529,10 @@ def main():
     fns = [lambda: _native.qk_forward(q, k, idx),
            lambda: _native.av_forward(attn, v, idx),
            lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx)]
-    # the same kernels without their arithmetic (same loads, LDS traffic and stores): see include/clusten_hip.h
-    replay_fns = [lambda: _native.qk_forward(q, k, idx, replay=True),
-                  lambda: _native.av_forward(attn, v, idx, replay=True),
-                  lambda: _native.wf_forward(dw.weights, dw.feat, dw.nbhd_idx, replay=True)]
+    # the same kernels without their arithmetic (same loads, LDS traffic and stores): see include/clusten_probe.h
+    replay_fns = [lambda: probe.qk_forward_replay(q, k, idx),
+                  lambda: probe.av_forward_replay(attn, v, idx),
+                  lambda: probe.wf_forward_replay(dw.weights, dw.feat, dw.nbhd_idx)]
     torch.cuda.synchronize()
     if args.only == "bwd-model":  # the same on lists as the model builds them (whole clusters, nearest first)
         mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built")
@@ -463,39 +547,42 @@ def main():
         if args.only == "copy":  # a plain copy of known traffic, to calibrate a profiler's byte counters
             src = torch.empty(qk_bytes // 8, dtype=torch.float32, device="cuda").normal_()
             dst = torch.empty_like(src)
-            one, nbytes = (lambda: _native.copy_probe(src, dst)), 2 * src.numel() * 4
+            one, nbytes = (lambda: probe.copy_probe(src, dst)), 2 * src.numel() * 4
         elif args.only.startswith("replay-"):
             # interleaved with the other two real kernels, as in the default pass: the probe's inputs come from HBM
             i = ("qk", "av", "wf").index(args.only[7:])
             trio = list(fns)
             trio[i] = replay_fns[i]
-            _, per3, _ = _time_kernels(trio, args.steps, args.warmup)
+            _, per3, _, _ = _time_kernels(trio, args.steps, args.warmup)
             print(json.dumps({"only": args.only, "launches": args.steps + args.warmup,
                               "avg_us": round(per3[i] * 1e3, 2)}), flush=True)
             return
         else:
             i = ("qk", "av", "wf").index(args.only)
             one, nbytes = fns[i], (qk_bytes, qk_bytes, wf_bytes)[i]
-        _, per, _ = _time_kernels([one], args.steps, args.warmup)
+        _, per, _, _ = _time_kernels([one], args.steps, args.warmup)
         print(json.dumps({"only": args.only, "launches": args.steps + args.warmup, "avg_us": round(per[0] * 1e3, 2),
                           "algorithmic_bytes": nbytes, "achieved_GBps": round(nbytes / per[0] / 1e6, 1)}), flush=True)
         return
-    ms_per_step, per, wall_ms = _time_kernels(fns, args.steps, args.warmup)
+    # throughput: exactly --steps steps after --warmup untimed ones; per-kernel figures: at least 10 + 50 launches
+    ms_per_step, per, wall_ms, per_min = _time_kernels(fns, args.steps, args.warmup)
     torch.cuda.synchronize()
-    _, per_replay, _ = _time_kernels(replay_fns, args.steps, args.warmup)
+    k_steps, k_warm = max(args.steps, 50), max(args.warmup, 10)
+    if (k_steps, k_warm) != (args.steps, args.warmup):
+        _, per, _, per_min = _time_kernels(fns, k_steps, k_warm)
+        torch.cuda.synchronize()
+    _, per_replay, _, _ = _time_kernels(replay_fns, k_steps, k_warm)
     torch.cuda.synchronize()
 
     names = ("gather_dot_tile_kernel (QK)", "gather_sum_tile_kernel (AV)", "wf_forward_row_kernel (WF)")
     kbytes = (qk_bytes, qk_bytes, wf_bytes)
-    kernels = [{"kernel": n, "avg_us": round(t * 1e3, 2), "algorithmic_bytes": nb,
+    kernels = [{"kernel": n, "median_us": round(t * 1e3, 2), "min_us": round(tm * 1e3, 2), "launches_timed": k_steps,
+                "algorithmic_bytes": nb, "measured_hbm_bytes": MEASURED_TRAFFIC_BYTES[key],
                 "achieved_GBps": round(nb / t / 1e6, 1), "frac_of_hbm_peak": round(nb / t / 1e6 / HBM_PEAK_GBPS, 4)}
-               for n, t, nb in zip(names, per, kbytes)]
-    # The three kernels take a third of the step each (within 2 us of one another, less than the run-to-run spread of
-    # the event timings), so "the longest" alone would name a different kernel from run to run: kernels within 2 % of
-    # the longest count as tied, and of those the one furthest below the roofline is reported; `kernels` lists all three
-    # and `step_frac` is the whole step's fraction.
-    longest = max(per)
-    dom = min((i for i in range(3) if per[i] >= 0.98 * longest), key=lambda i: kbytes[i] / per[i])
+               for n, key, t, tm, nb in zip(names, ("qk", "av", "wf"), per, per_min, kbytes)]
+    # The three kernels take a third of the step each, so the roofline object prices the step (the north-star
+    # quantity): algorithmic bytes of the three launches over the time of a step.  `kernels` lists all three.
+    low = min(range(3), key=lambda i: kbytes[i] / per[i])
     value = total_bytes / ms_per_step / 1e6
     out = {
         "metric": "CLUSTEN QK+AV+WF forward, algorithmic GB/s (AFF-Tiny stage-1 shape)",
@@ -514,14 +601,16 @@ def main():
                                "WF 3136->784 C64; cluster-shared windowed lists (QK/AV), 48-nearest lists (WF)",
                    "global_batch": B, "algorithmic_bytes_per_step": total_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-        "roofline": {"bound": "hbm", "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": kernels[dom]["frac_of_hbm_peak"],
-                     "traffic": MEASURED_TRAFFIC_BYTES[("qk", "av", "wf")[dom]], "traffic_source": TRAFFIC_MEASURED,
-                     "kernel": names[dom], "step_frac": round(value / HBM_PEAK_GBPS, 4),
-                     "step_traffic": sum(MEASURED_TRAFFIC_BYTES.values())},
+        "roofline": {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(value / HBM_PEAK_GBPS, 4),
+                     "traffic": sum(MEASURED_TRAFFIC_BYTES.values()), "traffic_source": TRAFFIC_MEASURED,
+                     "kernel": "the step: one launch each of " + ", ".join(names),
+                     "lowest_kernel": {"kernel": names[low], "frac": kernels[low]["frac_of_hbm_peak"],
+                                       "achieved": kernels[low]["achieved_GBps"]}},
         "kernels": kernels,
+        "parity": _parity(acase, wcase, attn, (q, k, v, idx), dw),
         "replay_probe": {"what": "the same kernels compiled without their matrix instructions (same global loads, LDS "
-                                 "accesses and stores), timed in the same interleaved pass",
+                                 "accesses and stores; libclusten_probe.so), timed in the same interleaved pass",
                          "kernels": [{"kernel": n, "replay_us": round(r * 1e3, 2), "kernel_us": round(t * 1e3, 2),
                                       "kernel_over_replay": round(t / r, 3)}
                                      for n, t, r in zip(names, per, per_replay)]},
@@ -550,7 +639,7 @@ def main():
         mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built").to("cuda")
         cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()   # the same lists as cluster numbers
         mattn = torch.softmax(_native.qk_forward(mcase.query, mcase.key, mcase.nbhd_idx), dim=-1)
-        _, per_c, _ = _time_kernels([lambda: _native.qk_forward_clusters(mcase.query, mcase.key, cidx),
+        _, per_c, _, _ = _time_kernels([lambda: _native.qk_forward_clusters(mcase.query, mcase.key, cidx),
                                      lambda: _native.av_forward_clusters(mattn, mcase.value, cidx)],
                                     args.steps, args.warmup)
         other["cfg2_s1_model_built_lists_as_cluster_numbers"] = {"qk_us": round(per_c[0] * 1e3, 1),
@@ -571,7 +660,7 @@ def main():
             return _native.av_forward_clusters(p, v16, cidx)
 
         plan = _native.cluster_attention_plan(cidx, pe_idx, None)   # what a stage builds once for all its layers
-        _, per_a, _ = _time_kernels([lambda: _native.cluster_attention(q16, k16, v16, cidx, table, pe_idx, None,
+        _, per_a, _, _ = _time_kernels([lambda: _native.cluster_attention(q16, k16, v16, cidx, table, pe_idx, None,
                                                                        blank_k, blank_v), three_kernels,
                                      lambda: _native.cluster_attention(q16, k16, v16, None, table, None, None,
                                                                        blank_k, blank_v, plan=plan)],
@@ -607,7 +696,7 @@ def main():
             d_table = _native.bias_table_grad(d_logit, pe_idx, rows)
             return (d_table,) + tuple(_native.qk_backward(d_logit, q16, k16, mcase.nbhd_idx)) + (dv,)
 
-        _, per_b, _ = _time_kernels([fused_backward, operator_backward], max(args.steps // 5, 5), 3)
+        _, per_b, _, _ = _time_kernels([fused_backward, operator_backward], max(args.steps // 5, 5), 3)
         other["cfg2_s1_local_attention_fp16_backward_model_built_lists"] = {
             "one_kernel_path_us": round(per_b[0] * 1e3, 1), "operator_path_us": round(per_b[1] * 1e3, 1),
             "what": "d_query, d_key, d_value and the bias table's gradient of one block's local attention"}
@@ -620,7 +709,7 @@ def main():
             p, pb = _native.attn_softmax(a, table32, pe_idx, None, query=mcase.query, blank_key=blank_k)
             return _native.av_forward_clusters(p, mcase.value, cidx)
 
-        _, per_f, _ = _time_kernels([lambda: _native.cluster_attention(mcase.query, mcase.key, mcase.value, cidx, table32,
+        _, per_f, _, _ = _time_kernels([lambda: _native.cluster_attention(mcase.query, mcase.key, mcase.value, cidx, table32,
                                                                        pe_idx, None, blank_k, blank_v),
                                      three_kernels_fp32,
                                      lambda: _native.cluster_attention(mcase.query, mcase.key, mcase.value, None, table32,

@@ -56,8 +56,9 @@ typedef enum clusten_status {
     CLUSTEN_ERR_BAD_STRIDE = 4,     /* a stride is negative or makes rows overlap */
     CLUSTEN_ERR_WORKSPACE = 5,      /* workspace missing or smaller than *_workspace_bytes() */
     CLUSTEN_ERR_LAUNCH = 6,         /* hipGetLastError() reported a failure after a launch */
-    CLUSTEN_ERR_UNALIGNED = 7,      /* clusten_copy_probe, clusten_attn_softmax_forward: a pointer is not 16-byte aligned
-                                       (the gather ops route unaligned operands to element-wise kernels) */
+    CLUSTEN_ERR_UNALIGNED = 7,      /* an optional entry point (e.g. clusten_attn_softmax_forward) was handed a pointer
+                                       that is not 16-byte aligned (the gather ops route unaligned operands to
+                                       element-wise kernels) */
     CLUSTEN_ERR_TOO_LARGE = 8       /* clusten_qk_backward_static: the problem needs more scratch than
                                        CLUSTEN_STATIC_SCRATCH_BYTES */
 } clusten_status;
@@ -123,8 +124,7 @@ int clusten_qk_backward(const void* d_attn,
 
 /* clusten_qk_backward without a workspace argument and without any allocation, for callers that cannot call
  * hipMalloc (code under HIP graph capture, tight serving loops, harnesses that forbid it).  It has no counterpart
- * in the reference, whose backward allocates its outputs itself (clustenqk_cuda_kernel.cu:151-152).  Same
- * arguments, results and kernels as clusten_qk_backward; the fp32 buffer in which the d_key of F16/BF16 data is
+ * in the reference.  Same arguments, results and kernels as clusten_qk_backward; the fp32 buffer in which the d_key of F16/BF16 data is
  * summed is a device array of CLUSTEN_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until
  * the process ends.  clusten_qk_backward_workspace_bytes(shape, dtype) bytes of it are used: a problem that needs more
  * is refused with CLUSTEN_ERR_TOO_LARGE.  The array's address on a device is looked up on the first call made with that device
@@ -586,43 +586,6 @@ int clusten_merge_rows(const void* const* src, void* const* dst, const int* row_
  * 1 <= K <= 8 and K <= N, else CLUSTEN_ERR_BAD_DIMS. */
 int clusten_knn2d(const float* query, const float* database, int64_t* idx, float* dist,
                   int B, int Nq, int N, int K, clusten_stream stream);
-
-/* ---- measurement aid ------------------------------------------------------------------------ */
-
-/* Plain streaming copy of `bytes` bytes (multiple of 16, both pointers 16-byte aligned) with the
- * same launch shape the gather kernels use.  It has no counterpart in the reference; it exists so
- * that a profiler's HBM byte counters can be calibrated against a kernel of known traffic and so
- * that a benchmark can print the copy bandwidth the device sustains next to the roofline figure. */
-int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream);
-
-/* The two components of a gather operator's memory traffic, alone and together, with no arithmetic at all: one wave
- * per tile (`tiles` of them, dealt to the accelerator dies like the operators' tiles) that, with mode bit 0 set, reads
- * 5 KiB of `in` (tile * 5120 ...) and writes 3 KiB of `out` (tile * 3072 ...) — streams that come from and go to
- * memory — and, with mode bit 1 set, gathers `gathers` (a multiple of 12) times four 256-byte rows picked at random
- * inside its window of `rows` (window number tile / tiles_per_window, window_rows rows each) — reads that hit the L2
- * once the window has been touched.  mode 1, 2 and 3 timed on the same buffers show how far the device overlaps the
- * two (on an MI355X: not at all — the times add up).  in >= tiles * 5120 bytes, out >= tiles * 3072 bytes, rows >=
- * ceil(tiles / tiles_per_window) * window_rows * 256 bytes, all 16-byte aligned.  No counterpart in the reference. */
-int clusten_stream_gather_probe(const void* in, void* out, const void* rows, int tiles, int gathers, int window_rows,
-                                int tiles_per_window, int mode, clusten_stream stream);
-
-/* clusten_qk_forward, clusten_av_forward and clusten_wf_forward without their arithmetic: the same kernels compiled a
- * second time with every matrix instruction replaced by one integer operation on its operands, so that they issue the
- * same global loads, LDS accesses and stores in the same order and nothing else.  Arguments as for the functions they
- * shadow; dtype F32 only (else CLUSTEN_ERR_BAD_DTYPE); the outputs hold no meaningful values.  They have no
- * counterpart in the reference; they exist so that a benchmark can print, next to the time of a kernel, what its
- * memory instruction stream costs by itself on the same inputs. */
-int clusten_qk_forward_replay(const void* query, clusten_strides query_strides,
-                              const void* key, clusten_strides key_strides,
-                              const int64_t* nbhd_idx, void* attn,
-                              clusten_attn_shape shape, int dtype, clusten_stream stream);
-int clusten_av_forward_replay(const void* attn,
-                              const void* value, clusten_strides value_strides,
-                              const int64_t* nbhd_idx,
-                              void* feat, clusten_strides feat_strides,
-                              clusten_attn_shape shape, int dtype, clusten_stream stream);
-int clusten_wf_forward_replay(const void* weights, const void* feat, const int64_t* nbhd_idx,
-                              void* feat_new, clusten_wf_shape shape, int dtype, clusten_stream stream);
 
 #ifdef __cplusplus
 }

@@ -107,12 +107,6 @@ _PROTOTYPES = {
     "clusten_scanline_rank": (ctypes.c_int, [_P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                             ctypes.c_int, ctypes.c_float, ctypes.c_float, _P]),
     "clusten_knn2d": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
-    "clusten_copy_probe": (ctypes.c_int, [_P, _P, ctypes.c_size_t, _P]),
-    "clusten_stream_gather_probe": (ctypes.c_int, [_P, _P, _P, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                                   ctypes.c_int, _P]),
-    "clusten_qk_forward_replay": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
-    "clusten_av_forward_replay": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
-    "clusten_wf_forward_replay": (ctypes.c_int, [_P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
 }
 
 EXPORTS = tuple(_PROTOTYPES)
@@ -190,12 +184,33 @@ def _stream(device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def _idx(nbhd_idx: torch.Tensor, shape, device) -> torch.Tensor:
+def debug_indices() -> bool:
+    """True when the environment asks for the index-range check (CLUSTEN_DEBUG_INDICES set to anything but 0 / empty)."""
+    return os.environ.get("CLUSTEN_DEBUG_INDICES", "0") not in ("", "0")
+
+
+def check_index_range(nbhd_idx: torch.Tensor, n_rows: int, name: str = "nbhd_idx") -> None:
+    """Raise RuntimeError unless every entry of `nbhd_idx` lies in [0, n_rows).  The kernels, like the reference's
+    (clusten/src/clustenqk_cuda.cpp:21-23 checks devices and contiguity only), read rows at whatever index they are
+    given; a stray index is an out-of-bounds access on the device.  This check reads the extrema back to the host and
+    therefore synchronises: it runs only under CLUSTEN_DEBUG_INDICES=1."""
+    if nbhd_idx.numel() == 0:
+        return
+    lo, hi = int(nbhd_idx.min()), int(nbhd_idx.max())
+    if lo < 0 or hi >= n_rows:
+        raise RuntimeError("%s holds entries outside [0, %d): min %d, max %d" % (name, n_rows, lo, hi))
+
+
+def _idx(nbhd_idx: torch.Tensor, shape, device, n_rows=None) -> torch.Tensor:
+    """The list tensor as the kernels take it; `n_rows` = length of the sequence its entries point into (the second
+    entry of `shape` unless given), used by the optional range check."""
     _require_cuda("nbhd_idx", nbhd_idx, device)
     if nbhd_idx.dtype != torch.int64:
         raise RuntimeError("nbhd_idx must be int64, got %s" % nbhd_idx.dtype)
     if tuple(nbhd_idx.shape[:2]) != tuple(shape):
         raise RuntimeError("nbhd_idx has shape %s, expected (%d, %d, m)" % (tuple(nbhd_idx.shape), shape[0], shape[1]))
+    if debug_indices():
+        check_index_range(nbhd_idx, shape[1] if n_rows is None else n_rows)
     return nbhd_idx.contiguous()
 
 
@@ -216,9 +231,9 @@ def _attn_problem(a: torch.Tensor, rows: torch.Tensor, nbhd_idx: torch.Tensor, n
     return device, _dtype_code(a, names[0]), idx, AttnShape(B, H, N, C, idx.shape[2])
 
 
-def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor, replay: bool = False) -> torch.Tensor:
-    """attn (b,h,n,m) = query · key[nbhd_idx]; query/key (b,h,n,c) may be strided views.  `replay` (a measurement aid,
-    fp32): the same kernels without their arithmetic — the result holds no meaningful values."""
+def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor, _entry=None) -> torch.Tensor:
+    """attn (b,h,n,m) = query · key[nbhd_idx]; query/key (b,h,n,c) may be strided views.  (`_entry`: another library's
+    function of the same signature, for the measurement bindings of probe.py.)"""
     lib = load()
     device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
     query, key = _rows(query), _rows(key)
@@ -226,7 +241,7 @@ def qk_forward(query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor, r
     if attn.numel() == 0:
         return attn
     with torch.cuda.device(device):
-        fn = lib.clusten_qk_forward_replay if replay else lib.clusten_qk_forward
+        fn = _entry or lib.clusten_qk_forward
         _check(fn(_ptr(query), _strides(query), _ptr(key), _strides(key), _ptr(idx), _ptr(attn), shape, code,
                   _stream(device)), "clusten_qk_forward")
     return attn
@@ -343,9 +358,9 @@ def qk_backward_static(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Ten
 
 
 def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, token_major: bool = False,
-               replay: bool = False) -> torch.Tensor:
+               _entry=None) -> torch.Tensor:
     """feat (b,h,n,c) = attn · v[nbhd_idx].  With token_major=True the result is a (b,h,n,c) view of
-    (b,n,h,c) storage, so that `.permute(0,2,1,3).reshape(b,n,h*c)` needs no copy.  `replay`: see qk_forward."""
+    (b,n,h,c) storage, so that `.permute(0,2,1,3).reshape(b,n,h*c)` needs no copy.  `_entry`: see qk_forward."""
     lib = load()
     _require_cuda("attn", attn)
     device = attn.device
@@ -370,7 +385,7 @@ def av_forward(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, toke
     if shape.M == 0:
         return feat.zero_()
     with torch.cuda.device(device):
-        fn = lib.clusten_av_forward_replay if replay else lib.clusten_av_forward
+        fn = _entry or lib.clusten_av_forward
         _check(fn(_ptr(attn), _ptr(v), _strides(v), _ptr(idx), _ptr(feat), _strides(feat), shape, code, _stream(device)),
                "clusten_av_forward")
     return feat
@@ -444,14 +459,14 @@ def _wf_problem(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tenso
         raise RuntimeError("weights and feat must agree in batch size and dtype")
     B, Nout, M, IC = weights.shape
     N, C = feat.shape[1], feat.shape[2]
-    idx = _idx(nbhd_idx, (B, Nout), device)
+    idx = _idx(nbhd_idx, (B, Nout), device, n_rows=N)
     if idx.shape[2] != M:
         raise RuntimeError("weights has %d slots per token, nbhd_idx %d" % (M, idx.shape[2]))
     return device, _dtype_code(weights, "weights"), idx, WfShape(B, N, Nout, C, M, IC)
 
 
-def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor, replay: bool = False) -> torch.Tensor:
-    """feat_new (b,n_,ic,c) = weightsᵀ · feat[nbhd_idx].  `replay`: see qk_forward."""
+def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor, _entry=None) -> torch.Tensor:
+    """feat_new (b,n_,ic,c) = weightsᵀ · feat[nbhd_idx].  `_entry`: see qk_forward."""
     lib = load()
     device, code, idx, shape = _wf_problem(weights, feat, nbhd_idx)
     weights, feat = weights.contiguous(), feat.contiguous()
@@ -461,7 +476,7 @@ def wf_forward(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.Tensor
     if shape.M == 0 or shape.N == 0:
         return out.zero_()
     with torch.cuda.device(device):
-        fn = lib.clusten_wf_forward_replay if replay else lib.clusten_wf_forward
+        fn = _entry or lib.clusten_wf_forward
         _check(fn(_ptr(weights), _ptr(feat), _ptr(idx), _ptr(out), shape, code, _stream(device)), "clusten_wf_forward")
     return out
 
@@ -478,7 +493,7 @@ def wf_forward_mixed(weights: torch.Tensor, feat: torch.Tensor, nbhd_idx: torch.
         raise RuntimeError("weights must be (b,n_,m,ic), feat (b,n,c) and nbhd_idx (b,n_,m)")
     B, Nout, M, IC = weights.shape
     N, C = feat.shape[1], feat.shape[2]
-    idx = _idx(nbhd_idx, (B, Nout), device)
+    idx = _idx(nbhd_idx, (B, Nout), device, n_rows=N)
     if idx.shape[2] != M:
         raise RuntimeError("weights has %d slots per token, nbhd_idx %d" % (M, idx.shape[2]))
     shape = WfShape(B, N, Nout, C, M, IC)
@@ -1451,34 +1466,3 @@ def knn2d(query: torch.Tensor, database: torch.Tensor, k: int, return_dist: bool
             _check(lib.clusten_knn2d(_ptr(query), _ptr(database), _ptr(idx), _ptr(dist), b, nq, n, k, _stream(device)),
                    "clusten_knn2d")
     return (idx, dist) if return_dist else idx
-
-
-def copy_probe(src: torch.Tensor, dst: torch.Tensor) -> None:
-    """dst <- src with the library's streaming copy kernel (measurement aid)."""
-    lib = load()
-    _require_cuda("src", src)
-    _require_cuda("dst", dst, src.device)
-    nbytes = src.numel() * src.element_size()
-    if not (src.is_contiguous() and dst.is_contiguous()) or dst.numel() * dst.element_size() != nbytes:
-        raise RuntimeError("copy_probe needs contiguous tensors of equal byte size")
-    with torch.cuda.device(src.device):
-        _check(lib.clusten_copy_probe(_ptr(src), _ptr(dst), nbytes, _stream(src.device)), "clusten_copy_probe")
-
-
-def stream_gather_probe(stream_in: torch.Tensor, stream_out: torch.Tensor, rows: torch.Tensor, tiles: int, gathers: int,
-                        window_rows: int, tiles_per_window: int, mode: int) -> None:
-    """`clusten_stream_gather_probe` (measurement aid): per tile, mode bit 0 = read 5 KiB of `stream_in` and write 3 KiB
-    of `stream_out`, bit 1 = gather `gathers` x 1 KiB of random 256-byte rows inside the tile's window of `rows`."""
-    lib = load()
-    _require_cuda("stream_in", stream_in)
-    device = stream_in.device
-    _require_cuda("stream_out", stream_out, device)
-    _require_cuda("rows", rows, device)
-    nbytes = lambda t: t.numel() * t.element_size()
-    windows = (tiles + tiles_per_window - 1) // tiles_per_window
-    if (nbytes(stream_in) < tiles * 5120 or nbytes(stream_out) < tiles * 3072
-            or nbytes(rows) < windows * window_rows * 256):
-        raise RuntimeError("stream_gather_probe: a buffer is too small for %d tiles" % tiles)
-    with torch.cuda.device(device):
-        _check(lib.clusten_stream_gather_probe(_ptr(stream_in), _ptr(stream_out), _ptr(rows), tiles, gathers, window_rows,
-                                               tiles_per_window, mode, _stream(device)), "clusten_stream_gather_probe")

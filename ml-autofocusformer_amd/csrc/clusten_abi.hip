@@ -548,21 +548,4 @@ int clusten_knn2d(const float* query, const float* database, int64_t* idx, float
     return launch_knn2d(query, database, idx, dist, B, Nq, N, K, as_stream(stream));
 }
 
-int clusten_copy_probe(const void* src, void* dst, size_t bytes, clusten_stream stream) {
-    if (!src || !dst) return CLUSTEN_ERR_NULL_POINTER;
-    if (bytes == 0 || bytes % 16 != 0) return CLUSTEN_ERR_BAD_DIMS;
-    if (!aligned16(src) || !aligned16(dst)) return CLUSTEN_ERR_UNALIGNED;
-    return launch_copy(src, dst, bytes, as_stream(stream));
-}
-
-int clusten_stream_gather_probe(const void* in, void* out, const void* rows, int tiles, int gathers, int window_rows,
-                                int tiles_per_window, int mode, clusten_stream stream) {
-    if (!in || !out || !rows) return CLUSTEN_ERR_NULL_POINTER;
-    if (tiles <= 0 || gathers <= 0 || gathers % 12 != 0 || window_rows <= 0 || tiles_per_window <= 0 || mode < 1 || mode > 3) {
-        return CLUSTEN_ERR_BAD_DIMS;
-    }
-    if (!aligned16(in) || !aligned16(out) || !aligned16(rows)) return CLUSTEN_ERR_UNALIGNED;
-    return launch_stream_gather_probe(in, out, rows, tiles, gathers, window_rows, tiles_per_window, mode, as_stream(stream));
-}
-
 }  // extern "C"

@@ -198,7 +198,8 @@ int launch_merge_weights(const float* table_w, const int64_t* pe_idx, const int6
                          const int64_t* mask, float* out, int B, int N, int Nout, int M, hipStream_t stream);
 
 // ranking[b,:] = the order of the tokens of image b along the scan-line walk over a rows x cols anchor grid with
-//   cells of cell_w x cell_h (see scanline_rank.hip).  pos (B,N,2) fp32 as (x, y); ranking (B,N) int64; N <= 4096,
+//   cells of cell_w x cell_h (see scanline_rank.hip).  pos (B,N,2) fp32 as (x, y); ranking (B,N) int64; N <= scanline_rank_max_tokens()
+//   (the sort of an image runs in the LDS of one compute unit: 16384 tokens on an MI355X),
 //   rows * cols >= 2; workspace of scanline_rank_workspace_bytes(B, N) bytes.
 size_t scanline_rank_workspace_bytes(int B, int N);
 int scanline_rank_max_tokens();   // the longest sequence the LDS of the current device sorts (a power of two)
@@ -233,14 +234,6 @@ int launch_scanline_rank(const float* pos, int64_t* ranking, void* workspace, in
 //   idx int64; dist fp32 or null.
 int launch_knn2d(const float* query, const float* database, int64_t* idx, float* dist, int B, int Nq, int N, int K,
                  hipStream_t stream);
-
-// dst[0:bytes) = src[0:bytes), 16 bytes per lane per step.
-int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
-
-// A wave per tile: mode bit 0 = read 5 KiB of `in` and write 3 KiB of `out` per tile, bit 1 = gather `gathers` x 1 KiB
-//   of 256-byte rows at random inside the tile's window of `rows` (window = tile / tiles_per_window).  See util.hip.
-int launch_stream_gather_probe(const void* in, void* out, const void* rows, int tiles, int gathers, int window_rows,
-                               int tiles_per_window, int mode, hipStream_t stream);
 
 // Fill `count` fp32 / fp64 words with zero (a kernel, so that callers may capture it in a HIP graph).
 //   `only_if` (may be null): a device flag; the kernel does nothing when it points to zero.

@@ -1,7 +1,7 @@
 // clusten_av_forward_replay: the AV forward kernels without their arithmetic (see replay_qk.hip).
 #define CLUSTEN_REPLAY 1
 #define clusten clusten_replay   // the kernels of this file are other functions than the library's own
-#include "gather_sum_impl.hpp"
+#include "../gather_sum_impl.hpp"
 
 extern "C" int clusten_av_forward_replay(const void* attn, const void* value, clusten_strides value_strides,
                                          const int64_t* nbhd_idx, void* feat, clusten_strides feat_strides,

@@ -4,7 +4,7 @@
 // clusten_qk_forward costs by itself.  The output holds no meaningful values.
 #define CLUSTEN_REPLAY 1
 #define clusten clusten_replay   // the kernels of this file are other functions than the library's own
-#include "gather_dot_impl.hpp"
+#include "../gather_dot_impl.hpp"
 
 extern "C" int clusten_qk_forward_replay(const void* query, clusten_strides query_strides, const void* key,
                                          clusten_strides key_strides, const int64_t* nbhd_idx, void* attn,

@@ -1,7 +1,7 @@
 // clusten_wf_forward_replay: the WF forward kernels without their arithmetic (see replay_qk.hip).
 #define CLUSTEN_REPLAY 1
 #define clusten clusten_replay   // the kernels of this file are other functions than the library's own
-#include "wf_impl.hpp"
+#include "../wf_impl.hpp"
 
 extern "C" int clusten_wf_forward_replay(const void* weights, const void* feat, const int64_t* nbhd_idx, void* feat_new,
                                          clusten_wf_shape shape, int dtype, clusten_stream stream) {

@@ -1,4 +1,4 @@
-// Small streaming kernels: copy probe, zero fill, fp32 -> fp16/bf16 rounding.
+// Small streaming kernels: zero fill, fp32 -> fp16/bf16 rounding.
 #include "launch.hpp"
 
 namespace clusten {
@@ -7,14 +7,6 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kMaxGrid = 256 * 64;  // 64 workgroups of 4 waves per CU: enough to keep every CU's queues full
-
-// One 16-byte piece per thread, one short-lived workgroup per 4 KiB: on this device that streams
-// 15-20 % faster than a grid-stride loop over the same bytes.
-__global__ __launch_bounds__(kBlock) void copy_kernel(const Piece* __restrict__ src, Piece* __restrict__ dst,
-                                                     size_t pieces) {
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < pieces) dst[i] = src[i];
-}
 
 // `only_if` (may be null): a device flag; the kernel does nothing when it points to zero.
 template <typename W>
@@ -32,89 +24,12 @@ __global__ __launch_bounds__(kBlock) void round_kernel(const float* __restrict__
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < count; i += stride) dst[i] = from_acc<T>(src[i]);
 }
 
-// The memory instruction stream of a gather operator, reduced to its two components (see launch_stream_gather_probe):
-// a wave per tile reads 5 KiB of its own (STREAM), gathers `gathers` times four random 256-byte rows of its window
-// (GATHER, 12 accesses in flight) and writes 3 KiB of its own with the non-temporal hint (STREAM).
-template <bool STREAM, bool GATHER>
-__global__ __launch_bounds__(kWave) void stream_gather_kernel(const char* __restrict__ in, char* __restrict__ out,
-                                                              const char* __restrict__ rows, int total_tiles,
-                                                              int gathers, uint32_t window_rows, int tiles_per_window) {
-    constexpr int U = 12;
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
-    const uint32_t lane = threadIdx.x, sub = lane >> 4, pos = lane & 15;
-    const char* window = rows + (size_t)(tile / tiles_per_window) * window_rows * 256;
-    uint32_t h = (uint32_t)tile * 2654435761u + sub * 40503u;
-    Piece a = Piece{0, 0, 0, 0};
-    if constexpr (STREAM) {
-        Piece v[5];
-#pragma unroll
-        for (int u = 0; u < 5; ++u) v[u] = *reinterpret_cast<const Piece*>(in + (size_t)tile * 5120 + u * 1024 + lane * 16);
-#pragma unroll
-        for (int u = 0; u < 5; ++u) a ^= v[u];
-        h ^= a[0] & 1u;   // the gathers wait for the streamed data, as an operator's wait for its lists
-    }
-    if constexpr (GATHER) {
-        for (int g = 0; g < gathers; g += U) {
-            Piece v[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                h = h * 1664525u + 1013904223u;
-                v[u] = *reinterpret_cast<const Piece*>(window + (size_t)((h >> 8) % window_rows) * 256 + pos * 16);
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) a ^= v[u];
-        }
-    }
-    if constexpr (STREAM) {
-#pragma unroll
-        for (int u = 0; u < 3; ++u) {
-            store_streaming(reinterpret_cast<Piece*>(out + (size_t)tile * 3072 + u * 1024 + lane * 16), a);
-        }
-    } else {
-        if (a[0] == 0x12345678u && a[1] == 0x9abcdef0u) reinterpret_cast<Piece*>(out)[lane] = a;   // keeps the loads
-    }
-}
-
 inline int grid_for(size_t items) {
     const size_t want = (items + kBlock - 1) / kBlock;
     return (int)(want < (size_t)kMaxGrid ? (want ? want : 1) : (size_t)kMaxGrid);
 }
 
 }  // namespace
-
-int launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
-    const size_t pieces = bytes / sizeof(Piece);
-    const size_t blocks = (pieces + kBlock - 1) / kBlock;
-    if (blocks >= ((size_t)1 << 31)) return CLUSTEN_ERR_BAD_DIMS;
-    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, static_cast<const Piece*>(src),
-                       static_cast<Piece*>(dst), pieces);
-    return launch_status();
-}
-
-int launch_stream_gather_probe(const void* in, void* out, const void* rows, int tiles, int gathers, int window_rows,
-                               int tiles_per_window, int mode, hipStream_t stream) {
-    const char* i = static_cast<const char*>(in);
-    char* o = static_cast<char*>(out);
-    const char* r = static_cast<const char*>(rows);
-    const dim3 grid(xcd_grid(tiles)), block(kWave);
-    switch (mode) {
-        case 1:
-            hipLaunchKernelGGL((stream_gather_kernel<true, false>), grid, block, 0, stream, i, o, r, tiles, gathers,
-                               (uint32_t)window_rows, tiles_per_window);
-            break;
-        case 2:
-            hipLaunchKernelGGL((stream_gather_kernel<false, true>), grid, block, 0, stream, i, o, r, tiles, gathers,
-                               (uint32_t)window_rows, tiles_per_window);
-            break;
-        case 3:
-            hipLaunchKernelGGL((stream_gather_kernel<true, true>), grid, block, 0, stream, i, o, r, tiles, gathers,
-                               (uint32_t)window_rows, tiles_per_window);
-            break;
-        default: return CLUSTEN_ERR_BAD_DIMS;
-    }
-    return launch_status();
-}
 
 int launch_zero_f32(float* dst, size_t count, hipStream_t stream, const int32_t* only_if) {
     // whole 16-byte pieces when the buffer allows it

@@ -1,5 +1,5 @@
-"""The C-ABI shared library loads, exports every symbol that include/clusten_hip.h declares, and
-rejects bad arguments with the documented status codes.  No kernel is launched: every call below
+"""The C-ABI shared libraries load, export every symbol that include/clusten_hip.h (the operators) and
+include/clusten_probe.h (the measurement kernels) declare, and reject bad arguments with the documented status codes.  No kernel is launched: every call below
 returns from the argument checks, so the file runs without a GPU."""
 import ctypes
 import os
@@ -9,24 +9,37 @@ import pytest
 
 from conftest import ROOT
 from clusten import _native
+import probe
 
 HEADER = os.path.join(ROOT, "include", "clusten_hip.h")
+PROBE_HEADER = os.path.join(ROOT, "include", "clusten_probe.h")
 
 
-def _declared_functions():
-    text = open(HEADER).read()
+def _declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(clusten_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_declares_what_the_binding_binds():
     assert _declared_functions() == sorted(_native.EXPORTS)
+    assert _declared_functions(PROBE_HEADER) == sorted(probe.EXPORTS)
 
 
 def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_native.library_path())
     for name in _declared_functions():
         assert hasattr(lib, name), name
+    plib = ctypes.CDLL(probe.library_path())
+    for name in _declared_functions(PROBE_HEADER):
+        assert hasattr(plib, name), name
+
+
+def test_measurement_kernels_are_not_in_the_operator_library():
+    lib = ctypes.CDLL(_native.library_path())
+    for name in _declared_functions(PROBE_HEADER):
+        assert not hasattr(lib, name), name
+    assert probe.load().clusten_probe_abi_version() == probe.ABI_VERSION
 
 
 def test_abi_version_and_status_strings():
@@ -65,7 +78,7 @@ def test_null_pointers_are_rejected():
     assert lib.clusten_qk_backward(FAKE, FAKE, ROWS, FAKE, ROWS, FAKE, P(0), FAKE, P(0), 0, _shape(), 0, P(0)) == 1
     assert lib.clusten_av_backward(FAKE, ROWS, FAKE, FAKE, ROWS, FAKE, FAKE, P(0), P(0), 0, _shape(), 0, P(0)) == 1
     assert lib.clusten_wf_backward(FAKE, FAKE, FAKE, FAKE, FAKE, P(0), P(0), 0, _wshape(), 0, P(0)) == 1
-    assert lib.clusten_copy_probe(P(0), FAKE, 16, P(0)) == 1
+    assert probe.load().clusten_copy_probe(P(0), FAKE, 16, P(0)) == 1
 
 
 @pytest.mark.parametrize("dtype", [-1, 4, 17])
@@ -83,8 +96,8 @@ def test_bad_dims_are_rejected():
         assert lib.clusten_qk_forward(FAKE, ROWS, FAKE, ROWS, FAKE, FAKE, _shape(**bad), 0, P(0)) == 3, bad
     for bad in (dict(B=0), dict(Nout=0), dict(IC=0), dict(N=1 << 24, C=512)):
         assert lib.clusten_wf_forward(FAKE, FAKE, FAKE, FAKE, _wshape(**bad), 0, P(0)) == 3, bad
-    assert lib.clusten_copy_probe(FAKE, FAKE, 24, P(0)) == 3
-    assert lib.clusten_copy_probe(FAKE, P(0x1008), 32, P(0)) == 7
+    assert probe.load().clusten_copy_probe(FAKE, FAKE, 24, P(0)) == 3
+    assert probe.load().clusten_copy_probe(FAKE, P(0x1008), 32, P(0)) == 7
 
 
 def test_bad_strides_are_rejected():
@@ -134,3 +147,21 @@ def test_python_surface_fails_loudly_without_a_gpu_tensor():
         CLUSTENAVFunction.apply(torch.randn(1, 1, 8, 4), q, idx)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         CLUSTENWFFunction.apply(torch.randn(1, 2, 4, 4), torch.randn(1, 8, 64), torch.zeros(1, 2, 4, dtype=torch.long))
+
+
+def test_debug_index_check_raises_on_stray_entries(monkeypatch):
+    """The optional range check of the shim (the reference checks no index either: clustenqk_cuda.cpp:21-23)."""
+    import torch
+    idx = torch.tensor([[[0, 3, 7], [1, 2, 6]]])
+    _native.check_index_range(idx, 8)                       # all inside [0, 8)
+    with pytest.raises(RuntimeError, match=r"outside \[0, 7\): min 0, max 7"):
+        _native.check_index_range(idx, 7)
+    with pytest.raises(RuntimeError, match="min -1"):
+        _native.check_index_range(idx - 1, 8)
+    _native.check_index_range(idx[:, :0], 8)                # nothing to check
+    monkeypatch.delenv("CLUSTEN_DEBUG_INDICES", raising=False)
+    assert not _native.debug_indices()
+    monkeypatch.setenv("CLUSTEN_DEBUG_INDICES", "0")
+    assert not _native.debug_indices()
+    monkeypatch.setenv("CLUSTEN_DEBUG_INDICES", "1")
+    assert _native.debug_indices()

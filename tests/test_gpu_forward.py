@@ -377,7 +377,63 @@ def test_empty_inputs_give_empty_or_zero_outputs(device):
 
 
 def test_copy_probe(device):
+    import probe
     src = torch.randn(1 << 20, device=device)
     dst = torch.zeros_like(src)
-    _native.copy_probe(src, dst)
+    probe.copy_probe(src, dst)
     assert torch.equal(src, dst)
+
+
+def test_replay_probes_run_at_the_operators_shapes(device):
+    """The measurement kernels (the forward kernels without their arithmetic) live in their own library and take the
+    operators' arguments; their outputs mean nothing, so only shapes and a clean launch are checked."""
+    import probe
+    case = wl.attn_case("replay", 77, B=2, H=2, N=200, C=32).to(device)
+    attn = _native.qk_forward(case.query, case.key, case.nbhd_idx)
+    assert probe.qk_forward_replay(case.query, case.key, case.nbhd_idx).shape == attn.shape
+    assert probe.av_forward_replay(attn, case.value, case.nbhd_idx).shape == case.value.shape
+    w = wl.wf_case("replay_wf", 78, B=2, N=200, C=64).to(device)
+    assert probe.wf_forward_replay(w.weights, w.feat, w.nbhd_idx).shape == (2, 50, 4, 64)
+    torch.cuda.synchronize()
+
+
+def test_debug_index_check_on_the_device_and_no_synchronisation_without_it(device, monkeypatch):
+    """With CLUSTEN_DEBUG_INDICES=1 a stray index raises before any kernel is launched (QK / AV lists against the
+    token count, WF lists against the rows of feat); without it nothing is read back: the three forwards can be
+    recorded into a HIP graph, which a host read of device memory would break."""
+    case = wl.attn_case("dbg", 79, B=2, H=2, N=64, C=32).to(device)
+    w = wl.wf_case("dbg_wf", 80, B=2, N=64, C=64).to(device)
+    monkeypatch.setenv("CLUSTEN_DEBUG_INDICES", "1")
+    attn = _native.qk_forward(case.query, case.key, case.nbhd_idx)      # good lists pass
+    bad = case.nbhd_idx.clone()
+    bad[1, 5, 7] = 64
+    with pytest.raises(RuntimeError, match=r"outside \[0, 64\)"):
+        _native.qk_forward(case.query, case.key, bad)
+    with pytest.raises(RuntimeError, match=r"outside \[0, 64\)"):
+        _native.av_forward(attn, case.value, bad)
+    wbad = w.nbhd_idx.clone()
+    wbad[0, 0, 0] = -1
+    with pytest.raises(RuntimeError, match="min -1"):
+        _native.wf_forward(w.weights, w.feat, wbad)
+    assert int(w.nbhd_idx.max()) >= w.weights.shape[1]                  # WF lists exceed Nout and are fine: they index feat
+    _native.wf_forward(w.weights, w.feat, w.nbhd_idx)
+    monkeypatch.delenv("CLUSTEN_DEBUG_INDICES")
+
+    def step():
+        a_ = _native.qk_forward(case.query, case.key, case.nbhd_idx)
+        return a_, _native.av_forward(a_, case.value, case.nbhd_idx), _native.wf_forward(w.weights, w.feat, w.nbhd_idx)
+
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        a, f, o = step()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(a, attn)
+    assert torch.equal(f, _native.av_forward(attn, case.value, case.nbhd_idx))
+    assert torch.equal(o, _native.wf_forward(w.weights, w.feat, w.nbhd_idx))
