@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define CLUSTEN_ABI_VERSION 2
+#define CLUSTEN_ABI_VERSION 3
 
 /* Element type of every floating-point tensor of a call.  The reference dispatches
  * double / float / half (AT_DISPATCH_FLOATING_TYPES_AND_HALF, clustenqk_cuda_kernel.cu:78);
@@ -128,7 +128,8 @@ int clusten_qk_backward(const void* d_attn,
  * summed is a device array of CLUSTEN_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until
  * the process ends.  clusten_qk_backward_workspace_bytes(shape, dtype) bytes of it are used: a problem that needs more
  * is refused with CLUSTEN_ERR_TOO_LARGE.  The array's address on a device is looked up on the first call made with that device
- * current.  Calls on one GPU share the array (each clears the part it uses on its own stream first), so calls that
+ * current: make that call outside any stream capture (every later call, recorded or not, launches kernels and nothing else).
+ * Calls on one GPU share the array (each clears the part it uses on its own stream first), so calls that
  * overlap in time on one GPU race: keep them on one stream or order them with events. */
 #define CLUSTEN_STATIC_SCRATCH_BYTES (32u << 20)
 int clusten_qk_backward_static(const void* d_attn,
@@ -248,15 +249,17 @@ int clusten_attn_softmax_forward(const void* attn, const void* bias_table, const
  *   blank[b,h,i]   = scale * <query[b,h,i], blank_key[h]>
  *   p, p_blank     = softmax over the M neighbours and the blank token
  *   out[b,h,i]     = sum_j p[b,h,i,j] * value[b,h,row(i,j)] + p_blank[b,h,i] * blank_value[h]
- *   row(i,j)       = 8 * cluster_idx[b,i,j/8] + j%8, row 0 where that is not in [0,N)
+ *   row(i,j)       = S * cluster_idx[b,i,j/S] + j%S, row 0 where that is not in [0,N);  S = M / 6, the cluster size
  * query, key, value, out: strided (B,H,N,C) of `dtype`; bias_table (rows,H) of `dtype`, contiguous;
- * cluster_idx (B,N,M/8) int32; pe_idx (B,N,M) int64 in [0,rows) — unchecked; mask (B,N,M) int64 of 0/1 or NULL;
+ * cluster_idx (B,N,6) int32; pe_idx (B,N,M) int64 in [0,rows) — unchecked; mask (B,N,M) int64 of 0/1 or NULL;
  * with lists_shared != 0 these three are (1,N,.) tensors that serve every batch element (the tokens of a
  * regular grid have the same neighbourhoods in every image);
  * blank_key, blank_value (H,C) fp32, contiguous.  Pass the unscaled query and the model's scale, or a scaled
  * query and 1.  The probabilities are rounded to `dtype` before they weigh the value rows; sums are fp32.
- * dtype F16, BF16 or F32 (else CLUSTEN_ERR_BAD_DTYPE), C = 32 and M = 48 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte
- * aligned (else CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
+ * dtype F16, BF16 or F32 (else CLUSTEN_ERR_BAD_DTYPE); C = 32; M = 48 (six clusters of 8: the 224 x 224 models) or,
+ * for F16 / BF16, M = 144 (six clusters of 24: the 384 x 384 models, configs/aff_base_22kto1k_384.yaml:10-11), else
+ * CLUSTEN_ERR_BAD_DIMS; rows 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's
+ * extension modules. */
 int clusten_cluster_attention_forward(const void* query, clusten_strides query_strides,
                                       const void* key, clusten_strides key_strides,
                                       const void* value, clusten_strides value_strides,
@@ -270,17 +273,17 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
  * clusters of every tile of 8 tokens, the bias-table row and mask bit of every slot, the runs a token repeats —
  * handed over as a plan: the lists of a stage serve all its layers (models/aff_transformer.py:454-487 builds them once
  * per stage, :505-507 runs the blocks on them), so the plan is built once per stage and read by every layer.
- *   clusten_cluster_attention_plan_bytes(B, N): size of the plan for index tensors of B batch elements (B = 1 when
- *   the lists are shared by every image);
- *   clusten_cluster_attention_plan: fills it from cluster_idx (B,N,6) int32, pe_idx (B,N,48) int64 and mask (B,N,48)
+ *   clusten_cluster_attention_plan_bytes(B, N, M): size of the plan for index tensors of B batch elements (B = 1 when
+ *   the lists are shared by every image) and M = 48 or 144 neighbours per token (0 for any other M);
+ *   clusten_cluster_attention_plan: fills it from cluster_idx (B,N,6) int32, pe_idx (B,N,M) int64 and mask (B,N,M)
  *   int64 or NULL; plan 16-byte aligned (else CLUSTEN_ERR_UNALIGNED), plan_bytes at least the size above (else
  *   CLUSTEN_ERR_WORKSPACE);
  *   clusten_cluster_attention_forward_planned: clusten_cluster_attention_forward with `plan` in the place of the three
  *   index tensors; same results bit for bit.
  * No counterpart in the reference's extension modules. */
-size_t clusten_cluster_attention_plan_bytes(int B, int N);
+size_t clusten_cluster_attention_plan_bytes(int B, int N, int M);
 int clusten_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
-                                   size_t plan_bytes, int B, int N, clusten_stream stream);
+                                   size_t plan_bytes, int B, int N, int M, clusten_stream stream);
 int clusten_cluster_attention_forward_planned(const void* query, clusten_strides query_strides,
                                               const void* key, clusten_strides key_strides,
                                               const void* value, clusten_strides value_strides,
@@ -355,6 +358,21 @@ int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair
  * CLUSTEN_ERR_UNALIGNED).  No counterpart in the reference's extension modules. */
 int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_strides x_strides, const void* pair_lists,
                                     void* y, clusten_attn_shape shape, int dtype, clusten_stream stream);
+
+/* The scatter of the two attention backward passes alone, for any lists:
+ *   y[b,h,nbhd_idx[b,i,j],:] += p[b,h,i,j] * x[b,h,i,:]          (y need not be zeroed)
+ * the d_key of clusten_qk_backward (p = d_attn, x = query; clustenqk_cuda_kernel.cu:91-132) and the d_value of
+ * clusten_av_backward (p = attn, x = d_feat; clustenav_cuda_kernel.cu:93-127), with the kernels of those two entry
+ * points: the gather over pair lists when the lists are made of whole clusters, atomics otherwise, chosen on the device.
+ * pair_lists: the block clusten_cluster_pairs filled for (B, N, M, N), or NULL.  A caller that keeps the block of a
+ * list tensor (one per stage of a model: it serves every layer and head) saves the rebuild on every call; when the
+ * block's flag says the lists are not made of whole clusters the atomic kernels run, so y is always the full sum.
+ * p (B,H,N,M) and y (B,H,N,C) contiguous, x strided (B,H,N,C); workspace of clusten_scatter_rows_workspace_bytes
+ * (= clusten_qk_backward_workspace_bytes) bytes, 16-byte aligned, whether or not pair_lists is given. */
+size_t clusten_scatter_rows_workspace_bytes(clusten_attn_shape shape, int dtype);
+int clusten_scatter_rows(const void* p, const void* x, clusten_strides x_strides, const int64_t* nbhd_idx,
+                         const void* pair_lists, void* y, void* workspace, size_t workspace_bytes,
+                         clusten_attn_shape shape, int dtype, clusten_stream stream);
 
 /* clusten_wf_backward for lists made of whole clusters, the feature gradient as a gather (no atomics, no workspace,
  * every row of d_feat written once from an fp32 sum in a fixed order):
@@ -556,8 +574,9 @@ int clusten_gather_rows(const void* x, const int64_t* order, void* out, int64_t 
  * `topk(sorted=False)` leaves the order of the sampled tokens open; here it is fixed: the tokens whose score is above
  * the sample_num-th highest by ascending index, then as many of those equal to it as are needed, by ascending index.
  * pos (B,N,2) fp32, 8-byte aligned; min_dist (B,N) fp32 or NULL; learned_prob (B,N) of prob_dtype or NULL; centre
- * (B, sample_num + (reserve_on ? reserve_num : 0)) int64.  An image must hold at least reserve_num tokens on the coarse
- * grid (the reference's reshape demands exactly that many); further ones are left out.  0 < sample_num, sample_num
+ * (B, sample_num + (reserve_on ? reserve_num : 0)) int64.  An image should hold reserve_num tokens on the coarse
+ * grid (the reference's reshape demands exactly that many and raises otherwise): further ones are left out, and the
+ * slots of missing ones hold -1, which clusten_merge_rows reads as row 0.  0 < sample_num, sample_num
  * [+ reserve_num] <= N <= clusten_merge_centres_max_tokens(), else CLUSTEN_ERR_BAD_DIMS.  No counterpart in the
  * reference's extension modules. */
 int clusten_merge_centres_max_tokens(void);
@@ -570,8 +589,8 @@ int clusten_merge_centres(const float* pos, const float* min_dist, const void* l
  *   dst[t][b,i,:] = src[t][b, centre[b,i], :]      t < count, 1 <= count <= 4
  * src[t] (B,N,.) and dst[t] (B,n_out,.) contiguous with rows of row_bytes[t] bytes, a multiple of 8 (else
  * CLUSTEN_ERR_BAD_DIMS), 8-byte aligned (else CLUSTEN_ERR_UNALIGNED); src, dst and row_bytes are host arrays of
- * `count` entries; centre (B,n_out) int64 with values in [0,N) — unchecked.  No counterpart in the reference's
- * extension modules. */
+ * `count` entries; centre (B,n_out) int64 with values in [0,N); a value outside that range reads row 0.  No
+ * counterpart in the reference's extension modules. */
 int clusten_merge_rows(const void* const* src, void* const* dst, const int* row_bytes, int count,
                        const int64_t* centre, int64_t B, int N, int n_out, clusten_stream stream);
 

@@ -41,7 +41,7 @@ def default_ops():
                            cluster_attention_supported=_native.cluster_attention_supported,
                            cluster_attention_backward=_native.cluster_attention_backward,
                            cluster_attention_backward_supported=_native.cluster_attention_backward_supported,
-                           cluster_pairs=_native.cluster_pairs, scatter_rows_by_cluster=_native.scatter_rows_by_cluster,
+                           cluster_pairs=_native.cluster_pairs, scatter_rows=_native.scatter_rows,
                            dense_attention=_native.dense_attention,
                            dense_attention_supported=_native.dense_attention_supported,
                            layer_norm=_native.layer_norm, layer_norm_supported=_native.layer_norm_supported,
@@ -193,31 +193,34 @@ class _ClusterAttention(torch.autograd.Function):
     """The local attention of a block between its projections (aff_transformer.py:120-155) as one kernel forward and,
     backward, one kernel for the query side - the probabilities are recomputed from the softmax denominators the
     forward saved - followed by the sums that complete it: the scatters over the stage's sorted pair lists (d_key,
-    d_value), the bias table's gradient, the blank token's.  No (b,h,n,m) tensor is kept between the two passes."""
+    d_value), the bias table's gradient, the blank token's.  No (b,h,n,m) tensor is kept between the two passes.
+    The scatters go through the operators' own scatter, which reads the flag of the pair lists on the device: lists
+    that turn out not to be made of whole clusters (never the model's own) take its atomic kernels, so d_key and d_value
+    are complete sums whatever `member_idx` holds."""
 
     @staticmethod
-    def forward(ctx, q, key, v, bias, blank_k, blank_v, plan, pairs, pe_idx, scale, ops):
+    def forward(ctx, q, key, v, bias, blank_k, blank_v, plan, pairs, pe_idx, member_idx, scale, ops):
         out, lse = ops.cluster_attention(q, key, v, None, bias, None, None, blank_k, blank_v, scale=scale, plan=plan,
                                          return_lse=True)
-        ctx.save_for_backward(q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx)
+        ctx.save_for_backward(q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx, member_idx)
         ctx.meta = (scale, ops)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
-        q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx = ctx.saved_tensors
+        q, key, v, out, lse, bias, blank_k, blank_v, plan, pairs, pe_idx, member_idx = ctx.saved_tensors
         scale, ops = ctx.meta
         b, h, n, ch = q.shape
         d_q, probs, d_logit, blank_prob, d_blank = ops.cluster_attention_backward(
             q, key, v, d_out, out, lse, plan, bias, blank_k, blank_v, scale=scale)
         g = d_out.to(q.dtype).reshape(b, n, h, ch).permute(0, 2, 1, 3)
-        d_v = ops.scatter_rows_by_cluster(probs, g, pairs)
-        d_k = ops.scatter_rows_by_cluster(d_logit, q, pairs) * scale
+        d_v = ops.scatter_rows(probs, g, member_idx, pairs)
+        d_k = ops.scatter_rows(d_logit, q, member_idx, pairs) * scale
         d_bias = ops.bias_table_grad(d_logit, pe_idx, bias.shape[0]).to(bias.dtype)
         d_bk = torch.einsum("bhn,bhnc->hc", d_blank, q.float()) * scale
         d_bv = torch.einsum("bhn,bhnc->hc", blank_prob, g.float())
         return (d_q, d_k.to(key.dtype), d_v.to(v.dtype), d_bias, d_bk.reshape(blank_k.shape).to(blank_k.dtype),
-                d_bv.reshape(blank_v.shape).to(blank_v.dtype), None, None, None, None, None)
+                d_bv.reshape(blank_v.shape).to(blank_v.dtype), None, None, None, None, None, None)
 
 
 def _position_bias(bias, pe_idx, ops):
@@ -309,6 +312,7 @@ class ClusterAttention(nn.Module):
         self.proj = nn.Linear(dim, dim)
         self.proj_drop = nn.Dropout(proj_drop)
         self.ops = ops
+        self.cluster_size = 8     # tokens per cluster of the lists this layer is given (its stage sets it)
 
     def bias_table(self, table):
         """(rows, heads) position bias for every row of the relative-position table (aff_transformer.py:125-129)."""
@@ -320,15 +324,16 @@ class ClusterAttention(nn.Module):
         b, n, c = feat.shape
         h = self.num_heads
         ch = c // h
-        # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,8*nnc) row lists
-        compact = (cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
-                   and getattr(self.ops, "qk_clusters", None) is not None)
+        # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,m*nnc) row lists
+        numbered = cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
+        compact = numbered and self.cluster_size == 8 and getattr(self.ops, "qk_clusters", None) is not None
         q, kv = _linear_pair(self.q, self.kv, feat, self.ops)
         kv = kv.view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                                                 # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
         one_kernel = getattr(self.ops, "cluster_attention", None)
-        if (compact and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
-                and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2])):
+        if (numbered and one_kernel is not None and not (self.training and self.attn_drop.p > 0)
+                and self.ops.cluster_attention_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3), cluster_idx.shape[2],
+                                                         self.cluster_size)):
             # inference on 16-bit or fp32 data: scores, position bias, mask, blank token, softmax and the weighted sum
             # of the values in one kernel; the query scale is applied to the scores inside it
             lists = grid_lists if grid_lists is not None else (cluster_idx, pe_idx, cluster_mask)
@@ -339,14 +344,15 @@ class ClusterAttention(nn.Module):
             return self.proj_drop(_linear(self.proj, out, self.ops))
         train_kernel = getattr(self.ops, "cluster_attention_backward", None)
         if (train_kernel is not None and torch.is_grad_enabled() and cluster_idx is not None and not global_attn
-                and grid_lists is not None and len(grid_lists) > 4 and not (self.training and self.attn_drop.p > 0)
+                and self.cluster_size == 8 and grid_lists is not None and len(grid_lists) > 4 and not (self.training and self.attn_drop.p > 0)
                 and self.ops.cluster_attention_backward_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3),
                                                                   cluster_idx.shape[2])):
             # training on 16-bit data: the same kernel forward, one kernel and four sums backward
             bias = self.bias_table(table)
             if bias.shape[0] <= 16000:
                 out = _ClusterAttention.apply(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, bias, self.blank_k,
-                                              self.blank_v, grid_lists[3], grid_lists[4], pe_idx, self.scale, self.ops)
+                                              self.blank_v, grid_lists[3], grid_lists[4], pe_idx, member_idx,
+                                              self.scale, self.ops)
                 return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
         if (global_attn and dense is not None and not torch.is_grad_enabled()
@@ -520,6 +526,8 @@ class BasicLayer(nn.Module):
         self.blocks = nn.ModuleList([
             ClusterTransformerBlock(dim, num_heads, mlp_ratio, drop, attn_drop, rates[i], layer_scale, ops=ops)
             for i in range(depth)])
+        for blk in self.blocks:
+            blk.attn.cluster_size = cluster_size
         if downsample:
             self.downsample = ClusterMerging(dim, out_dim, alpha, ds_rate, reserve_on, ops=ops)
             self.prob_net = nn.Linear(dim, 1)
@@ -549,7 +557,7 @@ class BasicLayer(nn.Module):
                 and self.ops.neighbour_lists_supported(pos, nearest)):
             # the four index tensors in one kernel
             member_idx, mask, pe_idx, cluster_idx = one_pass(pos, nearest, m, radius, table_width, mask is not None)
-            return pos, ranking, member_idx, mask, pe_idx, (cluster_idx if m == 8 else None)
+            return pos, ranking, member_idx, mask, pe_idx, (cluster_idx if m in (8, 24) else None)
         if ranking is not None:
             # cluster order: cluster g owns tokens g*m .. g*m+m-1, pad slots of the last one hold index 0 and mask 0
             rows = nearest.unsqueeze(3) * m + torch.arange(m, device=pos.device)
@@ -565,9 +573,9 @@ class BasicLayer(nn.Module):
         nb_pos = pos.gather(1, member_idx.reshape(b, -1, 1).expand(-1, -1, d)).reshape(b, n, nnc * m, d)
         rel = nb_pos - (pos.unsqueeze(2) - radius)
         pe_idx = (rel[..., 1] * table_width + rel[..., 0]).long()
-        # with clusters of 8 in cluster order, member_idx[b,i,8r+t] = 8*nearest[b,i,r]+t (0 past the last token):
-        # the cluster numbers alone describe the lists
-        cluster_idx = nearest.to(torch.int32).contiguous() if (ranking is not None and m == 8) else None
+        # with clusters of m in cluster order, member_idx[b,i,m*r+t] = m*nearest[b,i,r]+t (0 past the last token):
+        # the cluster numbers alone describe the lists (the kernels take clusters of 8 and, in part, of 24)
+        cluster_idx = nearest.to(torch.int32).contiguous() if (ranking is not None and m in (8, 24)) else None
         return pos, ranking, member_idx, mask, pe_idx, cluster_idx
 
     def grid_order(self, pos1, h, w, radius):
@@ -607,7 +615,8 @@ class BasicLayer(nn.Module):
                 if cluster_idx is not None:
                     grid_lists = (cluster_idx, pe_idx, mask)           # one image's lists, for the one-kernel attention
                     planner = getattr(self.ops, "cluster_attention_plan", None)
-                    if planner is not None and not torch.is_grad_enabled() and cluster_idx.shape[2] == 6 and pe_idx.is_cuda:
+                    if (planner is not None and not torch.is_grad_enabled() and cluster_idx.shape[2] == 6 and pe_idx.is_cuda
+                            and (self.cluster_size == 8 or torch.is_autocast_enabled("cuda"))):
                         if (key, "plan") not in self._grid_cache:      # what that kernel makes of them, kept with them
                             self._grid_cache[(key, "plan")] = planner(cluster_idx, pe_idx, mask)
                         grid_lists = grid_lists + (self._grid_cache[(key, "plan")],)
@@ -627,12 +636,12 @@ class BasicLayer(nn.Module):
         planner = getattr(self.ops, "cluster_attention_plan", None)
         if (grid_lists is None and cluster_idx is not None and planner is not None and not torch.is_grad_enabled()
                 and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
-                and (feat.dtype == torch.float32 or torch.is_autocast_enabled("cuda"))):
+                and ((feat.dtype == torch.float32 and self.cluster_size == 8) or torch.is_autocast_enabled("cuda"))):
             # the one-kernel attention of every block reads what it makes of the lists from a plan built once
             grid_lists = (cluster_idx, pe_idx, mask, planner(cluster_idx, pe_idx, mask))
         if ((grid_lists is None or len(grid_lists) == 3) and cluster_idx is not None and planner is not None
                 and torch.is_grad_enabled() and getattr(self.ops, "cluster_attention_backward", None) is not None
-                and not global_attn and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
+                and not global_attn and self.cluster_size == 8 and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
                 and torch.is_autocast_enabled("cuda")):
             # training under mixed precision: the plan of the one-kernel attention and the sorted pair lists of its
             # backward's scatters, built once for all blocks of the stage (a grid stage hands over one image's lists)

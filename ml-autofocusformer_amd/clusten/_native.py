@@ -14,7 +14,7 @@ import torch
 
 _LIB_PATH = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "lib", "libclusten_hip.so"))
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
 
@@ -57,8 +57,9 @@ _PROTOTYPES = {
     "clusten_cluster_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P,
                                                         ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float, AttnShape,
                                                         ctypes.c_int, _P]),
-    "clusten_cluster_attention_plan_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
-    "clusten_cluster_attention_plan": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, _P]),
+    "clusten_cluster_attention_plan_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "clusten_cluster_attention_plan": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                                     ctypes.c_int, _P]),
     "clusten_cluster_attention_forward_planned": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P,
                                                                 ctypes.c_int, _P, _P, _P, Strides, ctypes.c_float,
                                                                 AttnShape, ctypes.c_int, _P]),
@@ -73,6 +74,9 @@ _PROTOTYPES = {
                                              ctypes.c_int, _P]),
     "clusten_wf_backward_by_cluster": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, WfShape, ctypes.c_int, _P]),
     "clusten_scatter_rows_by_cluster": (ctypes.c_int, [_P, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
+    "clusten_scatter_rows_workspace_bytes": (ctypes.c_size_t, [AttnShape, ctypes.c_int]),
+    "clusten_scatter_rows": (ctypes.c_int, [_P, _P, Strides, _P, _P, _P, _P, ctypes.c_size_t, AttnShape, ctypes.c_int,
+                                            _P]),
     "clusten_dense_attention_forward": (ctypes.c_int, [_P, Strides, _P, Strides, _P, Strides, _P, _P, _P, _P, _P, Strides,
                                                       ctypes.c_float, AttnShape, ctypes.c_int, _P]),
     "clusten_linear_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -307,8 +311,40 @@ def _workspace(nbytes: int, device):
     return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
 
 
-def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor):
-    """(d_query, d_key), both contiguous (b,h,n,c)."""
+def scatter_rows(p: torch.Tensor, x: torch.Tensor, nbhd_idx: torch.Tensor, pair_lists=None) -> torch.Tensor:
+    """y (b,h,n,c) with y[b,h,nbhd_idx[b,i,j]] += p[b,h,i,j] * x[b,h,i]: the d_key (p = d_attn, x = query) and d_value
+    (p = attn, x = d_feat) of the attention backward passes, for any lists.  Lists made of whole clusters take the
+    gather over pair lists, anything else the atomic kernels; the device chooses.  `pair_lists`: the block
+    `cluster_pairs(nbhd_idx)` made of these lists, kept by the caller across calls (it is otherwise rebuilt here)."""
+    lib = load()
+    device, code, idx, shape = _attn_problem(x, x, nbhd_idx, ("x", "x"))
+    _require_cuda("p", p, device)
+    if tuple(p.shape) != (shape.B, shape.H, shape.N, shape.M) or p.dtype != x.dtype:
+        raise RuntimeError("p must be (b,h,n,m) with the dtype of x")
+    p, x = p.contiguous(), _rows(x)
+    y = torch.empty((shape.B, shape.H, shape.N, shape.C), dtype=x.dtype, device=device)
+    if y.numel() == 0 or shape.M == 0:
+        return y.zero_()
+    if pair_lists is not None:
+        _require_cuda("pair_lists", pair_lists, device)
+        if pair_lists.numel() != lib.clusten_cluster_pairs_bytes(shape.B, shape.N, shape.M, shape.N):
+            raise RuntimeError("scatter_rows: pair_lists does not belong to lists of this shape (cluster_pairs)")
+    ws_bytes = lib.clusten_scatter_rows_workspace_bytes(shape, code)
+    ws = _workspace(ws_bytes, device)
+    with torch.cuda.device(device):
+        _check(lib.clusten_scatter_rows(_ptr(p), _ptr(x), _strides(x), _ptr(idx), _ptr(pair_lists), _ptr(y), _ptr(ws),
+                                        ws_bytes, shape, code, _stream(device)), "clusten_scatter_rows")
+    return y
+
+
+def qk_backward(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, nbhd_idx: torch.Tensor, pairs=None):
+    """(d_query, d_key), both contiguous (b,h,n,c).  `pairs`: the block `cluster_pairs(nbhd_idx)` of a caller that keeps
+    it across the layers of a stage; the call then runs as its two halves (same kernels, same results) and skips the
+    rebuild of the pair lists."""
+    if pairs is not None:
+        if tuple(d_attn.shape) != tuple(query.shape[:3]) + (nbhd_idx.shape[2],) or d_attn.dtype != query.dtype:
+            raise RuntimeError("d_attn must be (b,h,n,m) with the dtype of query")
+        return av_forward(d_attn, key, nbhd_idx), scatter_rows(d_attn, query, nbhd_idx, pairs)
     lib = load()
     device, code, idx, shape = _attn_problem(query, key, nbhd_idx, ("query", "key"))
     _require_cuda("d_attn", d_attn, device)
@@ -427,8 +463,12 @@ def av_forward_mixed(attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor
     return feat
 
 
-def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor):
-    """(d_attn (b,h,n,m), d_v (b,h,n,c)), both contiguous."""
+def av_backward(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, nbhd_idx: torch.Tensor, pairs=None):
+    """(d_attn (b,h,n,m), d_v (b,h,n,c)), both contiguous.  `pairs`: see qk_backward."""
+    if pairs is not None:
+        if tuple(attn.shape) != tuple(v.shape[:3]) + (nbhd_idx.shape[2],) or attn.dtype != v.dtype:
+            raise RuntimeError("attn must be (b,h,n,m) with the dtype of v")
+        return qk_forward(d_feat, v, nbhd_idx), scatter_rows(attn, d_feat, nbhd_idx, pairs)
     lib = load()
     device, code, idx, shape = _attn_problem(d_feat, v, nbhd_idx, ("d_feat", "v"))
     _require_cuda("attn", attn, device)
@@ -700,18 +740,18 @@ def attn_softmax_backward(probs: torch.Tensor, blank_prob: torch.Tensor, d_probs
     return d_logit, d_blank_logit
 
 
-def cluster_attention_supported(query: torch.Tensor, nnc: int) -> bool:
-    """True when `cluster_attention` takes this case: CUDA fp16 / bf16 / fp32 queries of head dim 32, six clusters per
-    token."""
-    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16, torch.float32) and query.dim() == 4
-            and query.shape[3] == 32 and nnc == 6)
+def cluster_attention_supported(query: torch.Tensor, nnc: int, cluster_size: int = 8) -> bool:
+    """True when `cluster_attention` takes this case: CUDA queries of head dim 32, six clusters per token; clusters of 8
+    tokens (fp16 / bf16 / fp32) or of 24 tokens (fp16 / bf16)."""
+    types = {8: (torch.float16, torch.bfloat16, torch.float32), 24: (torch.float16, torch.bfloat16)}.get(cluster_size, ())
+    return query.is_cuda and query.dtype in types and query.dim() == 4 and query.shape[3] == 32 and nnc == 6
 
 
 def cluster_attention_plan(cluster_idx: torch.Tensor, pe_idx: torch.Tensor, mask) -> torch.Tensor:
     """What `cluster_attention` works out from its three index tensors before its first head, for every tile of 8
     tokens: a uint8 tensor to hand to every call that uses these lists (`plan=`), e.g. all layers of a stage.
-    cluster_idx (B,N,6) int32, pe_idx (B,N,48) int64, mask (B,N,48) of 0/1 or None — B = 1 for lists shared by every
-    image."""
+    cluster_idx (B,N,6) int32, pe_idx (B,N,M) int64, mask (B,N,M) of 0/1 or None — B = 1 for lists shared by every
+    image; M = 48 (clusters of 8 tokens) or 144 (clusters of 24)."""
     lib = load()
     _require_cuda("cluster_idx", cluster_idx)
     device = cluster_idx.device
@@ -720,19 +760,20 @@ def cluster_attention_plan(cluster_idx: torch.Tensor, pe_idx: torch.Tensor, mask
         raise RuntimeError("cluster_idx must be (B,N,6)")
     lb, n = cluster_idx.shape[:2]
     cidx = _cluster_idx(cluster_idx, (lb, n), device)
-    if pe_idx.shape != (lb, n, 48) or pe_idx.dtype != torch.int64:
-        raise RuntimeError("pe_idx must be int64 of shape (B,N,48) like cluster_idx")
+    m = pe_idx.shape[2] if pe_idx.dim() == 3 else 0
+    if pe_idx.shape != (lb, n, m) or m not in (48, 144) or pe_idx.dtype != torch.int64:
+        raise RuntimeError("pe_idx must be int64 of shape (B,N,48) or (B,N,144), B and N like cluster_idx")
     pe_idx = pe_idx.contiguous()
     if mask is not None:
         _require_cuda("mask", mask, device)
-        if mask.shape != (lb, n, 48):
-            raise RuntimeError("mask must have shape (B,N,48) like cluster_idx")
+        if mask.shape != (lb, n, m):
+            raise RuntimeError("mask must have the shape of pe_idx")
         mask = mask.to(torch.int64).contiguous()
-    nbytes = lib.clusten_cluster_attention_plan_bytes(lb, n)
+    nbytes = lib.clusten_cluster_attention_plan_bytes(lb, n, m)
     plan = torch.empty(nbytes, dtype=torch.uint8, device=device)
     if nbytes:
         with torch.cuda.device(device):
-            _check(lib.clusten_cluster_attention_plan(_ptr(cidx), _ptr(pe_idx), _ptr(mask), _ptr(plan), nbytes, lb, n,
+            _check(lib.clusten_cluster_attention_plan(_ptr(cidx), _ptr(pe_idx), _ptr(mask), _ptr(plan), nbytes, lb, n, m,
                                                       _stream(device)), "clusten_cluster_attention_plan")
     return plan
 
@@ -743,7 +784,8 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     """Local attention over the members of each token's clusters plus one blank token, in one kernel.
 
     query, key, value (B,H,N,32) fp16 / bf16 / fp32 (any strides, channel stride 1); cluster_idx (B,N,6) int32;
-    bias_table (rows,H); pe_idx (B,N,48) int64; mask (B,N,48) of 0/1 or None; blank_key, blank_value (H*32,).
+    bias_table (rows,H); pe_idx (B,N,M) int64; mask (B,N,M) of 0/1 or None; blank_key, blank_value (H*32,).
+    M = 48: clusters of 8 tokens (row(i,j) = 8 * cluster + j % 8); M = 144, fp16 / bf16 only: clusters of 24.
     cluster_idx, pe_idx and mask may all have a leading 1 instead of B: one set of lists for every image.
     Returns softmax(scale * q.k + bias - 100 * (1 - mask) | scale * q.blank_key) applied to the gathered values and
     the blank value, as a (B,N,H*32) tensor of query's dtype (heads side by side, the layout the output
@@ -764,17 +806,21 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
     b, h, n, c = query.shape
     if plan is not None:
         _require_cuda("plan", plan, device)
-        lb = b if plan.numel() == lib.clusten_cluster_attention_plan_bytes(b, n) else 1
-        if plan.dtype != torch.uint8 or plan.numel() != lib.clusten_cluster_attention_plan_bytes(lb, n):
+        # the plan's size tells the batch elements of its lists (b, or 1 for shared lists) and their length
+        fits = [(lb_, m_) for m_ in (48, 144) for lb_ in (b, 1)
+                if plan.numel() == lib.clusten_cluster_attention_plan_bytes(lb_, n, m_)]
+        if plan.dtype != torch.uint8 or not fits:
             raise RuntimeError("plan does not belong to lists of this shape")
+        lb, m = fits[0]
         shared = b != 1 and lb == 1
-        m = 48
         cidx = pe_idx = mask = None
     else:
         shared = b != 1 and cluster_idx.dim() == 3 and cluster_idx.shape[0] == 1
         lb = 1 if shared else b
         cidx = _cluster_idx(cluster_idx, (lb, n), device)
-        m = 8 * cidx.shape[2]
+        m = pe_idx.shape[2] if pe_idx.dim() == 3 else 0
+        if cidx.shape[2] != 6 or m not in (48, 144):
+            raise RuntimeError("cluster_idx must be (B,N,6) and pe_idx (B,N,48) or (B,N,144)")
         if pe_idx.shape != (lb, n, m) or pe_idx.dtype != torch.int64:
             raise RuntimeError("pe_idx must be int64 of shape (B,N,M), or (1,N,M) like cluster_idx")
         pe_idx = pe_idx.contiguous()
@@ -863,8 +909,8 @@ def cluster_attention_backward(query: torch.Tensor, key: torch.Tensor, value: to
         raise RuntimeError("out and d_out must be (B,N,H*C)")
     if tuple(lse.shape) != (b, h, n) or lse.dtype != torch.float32:
         raise RuntimeError("lse must be fp32 (B,H,N)")
-    lb = b if plan.numel() == lib.clusten_cluster_attention_plan_bytes(b, n) else 1
-    if plan.dtype != torch.uint8 or plan.numel() != lib.clusten_cluster_attention_plan_bytes(lb, n):
+    lb = b if plan.numel() == lib.clusten_cluster_attention_plan_bytes(b, n, 48) else 1
+    if plan.dtype != torch.uint8 or plan.numel() != lib.clusten_cluster_attention_plan_bytes(lb, n, 48):
         raise RuntimeError("plan does not belong to lists of this shape")
     shared = b != 1 and lb == 1
     code = _dtype_code(query, "query")
@@ -1377,6 +1423,11 @@ def merge_centres(pos: torch.Tensor, min_dist, learned_prob, alpha: float, strid
         _check(lib.clusten_merge_centres(_ptr(pos), _ptr(min_dist), _ptr(learned_prob), code, _ptr(centre), b, n,
                                          sample_num, reserve_num, int(bool(reserve_on)), ctypes.c_float(alpha),
                                          stride, _stream(device)), "clusten_merge_centres")
+    if reserve_on and debug_indices() and centre.numel() and int(centre.min()) < 0:
+        # the kernel marks the slots of reserved tokens an image does not have with -1; the reference's
+        # `reserve_mask.nonzero().reshape(b, reserve_num)` raises there (aff_transformer.py:323)
+        raise RuntimeError("merge_centres: an image holds fewer than reserve_num = %d tokens on the coarse grid"
+                           % reserve_num)
     return centre
 
 

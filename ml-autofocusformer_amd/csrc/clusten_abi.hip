@@ -207,18 +207,18 @@ int clusten_cluster_attention_forward(const void* query, clusten_strides query_s
                                     nullptr, shape, dtype, as_stream(stream));
 }
 
-size_t clusten_cluster_attention_plan_bytes(int B, int N) {
+size_t clusten_cluster_attention_plan_bytes(int B, int N, int M) {
     if (B <= 0 || N <= 0) return 0;
-    return cluster_attention_plan_bytes(B, N);
+    return cluster_attention_plan_bytes(B, N, M);
 }
 
 int clusten_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
-                                   size_t plan_bytes, int B, int N, clusten_stream stream) {
+                                   size_t plan_bytes, int B, int N, int M, clusten_stream stream) {
     if (!cluster_idx || !pe_idx || !plan) return CLUSTEN_ERR_NULL_POINTER;
-    if (B <= 0 || N <= 0) return CLUSTEN_ERR_BAD_DIMS;
-    if (plan_bytes < cluster_attention_plan_bytes(B, N)) return CLUSTEN_ERR_WORKSPACE;
+    if (B <= 0 || N <= 0 || cluster_attention_plan_bytes(1, 8, M) == 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (plan_bytes < cluster_attention_plan_bytes(B, N, M)) return CLUSTEN_ERR_WORKSPACE;
     if (!aligned16(plan)) return CLUSTEN_ERR_UNALIGNED;
-    return launch_cluster_attention_plan(cluster_idx, pe_idx, mask, plan, B, N, as_stream(stream));
+    return launch_cluster_attention_plan(cluster_idx, pe_idx, mask, plan, B, N, M, as_stream(stream));
 }
 
 int clusten_cluster_attention_forward_planned(const void* query, clusten_strides query_strides, const void* key,
@@ -341,6 +341,26 @@ int clusten_scatter_rows_by_cluster(const void* p, const void* x, clusten_stride
                                      reinterpret_cast<const int32_t*>(ws + l.ends),
                                      reinterpret_cast<const int32_t*>(ws + l.pairs),
                                      reinterpret_cast<const int32_t*>(ws + l.flag), y, shape, dtype, as_stream(stream));
+}
+
+size_t clusten_scatter_rows_workspace_bytes(clusten_attn_shape shape, int dtype) {
+    if (!dtype_ok(dtype) || check_attn_shape(shape) != CLUSTEN_OK) return 0;
+    return scatter_rows_workspace_bytes(shape, dtype);
+}
+
+int clusten_scatter_rows(const void* p, const void* x, clusten_strides x_strides, const int64_t* nbhd_idx,
+                         const void* pair_lists, void* y, void* workspace, size_t workspace_bytes,
+                         clusten_attn_shape shape, int dtype, clusten_stream stream) {
+    if (!p || !x || !nbhd_idx || !y) return CLUSTEN_ERR_NULL_POINTER;
+    if (int st = check_attn_call(shape, dtype)) return st;
+    if (!strides_ok(x_strides, shape.C)) return CLUSTEN_ERR_BAD_STRIDE;
+    const size_t need = scatter_rows_workspace_bytes(shape, dtype);
+    if (need && (!workspace || workspace_bytes < need)) return CLUSTEN_ERR_WORKSPACE;
+    if (pair_lists) {
+        if (!cluster_pairs_supported(shape.B, shape.N, shape.M, shape.N)) return CLUSTEN_ERR_BAD_DIMS;
+        if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
+    }
+    return launch_scatter_rows(p, x, x_strides, nbhd_idx, y, workspace, shape, dtype, as_stream(stream), pair_lists);
 }
 
 int clusten_dense_attention_forward(const void* query, clusten_strides query_strides, const void* key,

@@ -4,13 +4,15 @@
 //   blank[b,h,i]   = scale * sum_c q[b,h,i,c] * blank_k[h,c]
 //   p[b,h,i,:], p_blank[b,h,i] = softmax over the M neighbours and the blank token
 //   out[b,h,i,c]   = sum_j p[b,h,i,j] * v[b,h,row(i,j),c] + p_blank[b,h,i] * blank_v[h,c]
-//   row(i,j)       = 8 * cluster_idx[b,i,j/8] + j%8   (row 0 where that is not in [0,N))
+//   row(i,j)       = CS * cluster_idx[b,i,j/CS] + j%CS   (row 0 where that is not in [0,N)); CS = cluster size
 //
 // This is CLUSTENQKFunction, the tensor expressions between the two operators and CLUSTENAVFunction of the
 // reference model (models/aff_transformer.py:120-155; kernels clusten/src/clustenqk_cuda_kernel.cu:18-49 and
 // clusten/src/clustenav_cuda_kernel.cu:18-49) with the (B,H,N,M) logits and probabilities never leaving the
-// chip.  16-bit data (fp16 / bf16), head dim 32, M = 48 (six clusters of 8 per token): the shape of every
-// attention layer of the shipped models under mixed precision.
+// chip.  16-bit data (fp16 / bf16), head dim 32, six clusters per token: M = 48 for clusters of 8 (every attention
+// layer of the shipped 224 x 224 models under mixed precision), M = 144 for clusters of 24 (the 384 x 384 models,
+// configs/aff_base_22kto1k_384.yaml:10-11), which the kernel treats as three runs of 8 rows each: a tile of 8 tokens
+// then names some 8 distinct clusters = 24 runs and a head takes two or three passes.
 //
 // One wave owns 8 consecutive tokens (one cluster) and walks the heads.  The tile's 48 cluster numbers are
 // numbered by distinct value (`U` of them; 7-12 in the shipped models: neighbouring tokens choose among the same
@@ -68,19 +70,21 @@ constexpr int O_BASE = V_BASE + kPassRows * kRB;           // output chunk of a 
 constexpr int Q_BASE = O_BASE + kTileTokens * kRB;         // q rows of two heads (slot h % 2)
 constexpr int Q_SLOT = kTileTokens * kRB;
 constexpr int UL_BASE = Q_BASE + 2 * Q_SLOT;               // cluster number of each distinct cluster
-constexpr int PB_BASE = UL_BASE + kTileTokens * kR * 4;    // blank-token probability per token
+constexpr int PB_BASE = UL_BASE + kTileTokens * kNnc * 4;  // blank-token probability per token
 constexpr int LDS_BYTES = PB_BASE + kTileTokens * 4;
 static_assert(P_BYTES % 16 == 0 && P_BYTES <= kPassRows * kRB, "the probabilities fit the K area");
 static_assert(kTileTokens * kSRow * 4 <= kPassRows * kRB, "the scores fit the K area");
 static_assert(kPassRows % 32 == 0 && Q_BASE % 16 == 0, "whole 32-row steps");
 
 // One wave per tile: the plan of every tile of the index tensors (B_lists batch elements).
+template <int CS>
 __global__ __launch_bounds__(kWave) void cluster_attention_plan_kernel(const int32_t* __restrict__ cluster_idx,
                                                                        const int64_t* __restrict__ pe_idx,
                                                                        const int64_t* __restrict__ mask,
                                                                        char* __restrict__ plan, int N, int tiles_per_batch,
                                                                        int total_tiles) {
-    __shared__ int ulist[kTileTokens * kR];
+    typedef Geo<CS> G;
+    __shared__ int ulist[kTileTokens * kNnc];
     const int tile = blockIdx.x;
     if (tile >= total_tiles) return;
     const int b = tile / tiles_per_batch;
@@ -88,19 +92,28 @@ __global__ __launch_bounds__(kWave) void cluster_attention_plan_kernel(const int
     const int nt = min(kTileTokens, N - i0);
     const int lane = threadIdx.x;
     const int64_t tok = (int64_t)b * N + i0 + min(lane >> 3, nt - 1);
-    int pe[kR], us[kR], repeats, U;
-    tile_setup(cluster_idx, pe_idx, mask, b, N, i0, nt, tok, pe, us, repeats, U, ulist);
+    int pe[G::kR], us[kNnc], repeats, U;
+    tile_setup<CS>(cluster_idx, pe_idx, mask, b, N, i0, nt, tok, pe, us, repeats, U, ulist);
     lds_sync();
-    char* mine = plan + (int64_t)tile * kPlanBytes;
+    char* mine = plan + (int64_t)tile * G::kPlanBytes;
     if (lane == 0) *reinterpret_cast<int*>(mine) = U;
-    if (lane < kTileTokens * kR) *reinterpret_cast<int*>(mine + 16 + lane * 4) = lane < U ? ulist[lane] : 0;
-    const uint32_t w2 = (uint32_t)us[0] | ((uint32_t)us[1] << 8) | ((uint32_t)us[2] << 16) | ((uint32_t)us[3] << 24);
-    const uint32_t w3 = (uint32_t)us[4] | ((uint32_t)us[5] << 8) | ((uint32_t)repeats << 16);
-    *reinterpret_cast<Piece*>(mine + kPlanLane + lane * 32) = Piece{(uint32_t)pe[0], (uint32_t)pe[1], (uint32_t)pe[2], (uint32_t)pe[3]};
-    *reinterpret_cast<Piece*>(mine + kPlanLane + lane * 32 + 16) = Piece{(uint32_t)pe[4], (uint32_t)pe[5], w2, w3};
+    if (lane < kTileTokens * kNnc) *reinterpret_cast<int*>(mine + 16 + lane * 4) = lane < U ? ulist[lane] : 0;
+    // the lane's record: pe[kR], then the six distinct-cluster numbers and the repeat bits, one byte each
+    uint32_t words[G::kPlanLaneBytes / 4];
+#pragma unroll
+    for (int w = 0; w < G::kPlanLaneBytes / 4; ++w) words[w] = 0u;
+#pragma unroll
+    for (int r = 0; r < G::kR; ++r) words[r] = (uint32_t)pe[r];
+    words[G::kR] = (uint32_t)us[0] | ((uint32_t)us[1] << 8) | ((uint32_t)us[2] << 16) | ((uint32_t)us[3] << 24);
+    words[G::kR + 1] = (uint32_t)us[4] | ((uint32_t)us[5] << 8) | ((uint32_t)repeats << 16);
+#pragma unroll
+    for (int q = 0; q < G::kPlanLaneBytes / 16; ++q) {
+        *reinterpret_cast<Piece*>(mine + kPlanLane + lane * G::kPlanLaneBytes + q * 16) =
+            Piece{words[4 * q], words[4 * q + 1], words[4 * q + 2], words[4 * q + 3]};
+    }
 }
 
-template <typename T>
+template <typename T, int CS>
 __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     const T* __restrict__ q, clusten_strides qs, const T* __restrict__ k, clusten_strides ks, const T* __restrict__ v,
     clusten_strides vs, const int32_t* __restrict__ cluster_idx, const T* __restrict__ table,
@@ -110,6 +123,9 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     float* __restrict__ lse) {
     typedef short S4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) S4* LdsS4;
+    typedef Geo<CS> G;
+    constexpr int kRuns = G::kR;     // runs of 8 slots per token
+    constexpr int kSub = G::kSub;    // runs per cluster
 
     __shared__ __attribute__((aligned(1024))) char stage[LDS_BYTES];
 
@@ -147,43 +163,57 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     fetch_q(0);
     if (H > 1) fetch_q(1);
 
-    int pe[kR];      // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
-    int us[kR];      // distinct-cluster number of this lane's token's runs
-    int repeats = 0; // bit r: run r repeats an earlier run of the token; its probability is added to that run's
-    int U = 0;
+    int pe[kRuns];   // per-slot inputs the heads share: row of the bias table; the sign bit marks a masked slot
+    int usc[kNnc];   // distinct-cluster number of each of this lane's token's clusters
+    int repeats = 0; // bit k: cluster k repeats an earlier one of the token; its probabilities are added to that one's
+    int U = 0;       // distinct clusters of the tile
     int* ulist = reinterpret_cast<int*>(stage + UL_BASE);
     if (plan != nullptr) {
         // the tile's plan, built once for all layers that use these lists
-        const char* mine = plan + (list_b * tiles_per_batch + (tile - b * tiles_per_batch)) * (int64_t)kPlanBytes;
-        const Piece lo = *reinterpret_cast<const Piece*>(mine + kPlanLane + lane * 32);
-        const Piece hi = *reinterpret_cast<const Piece*>(mine + kPlanLane + lane * 32 + 16);
+        const char* mine = plan + (list_b * tiles_per_batch + (tile - b * tiles_per_batch)) * (int64_t)G::kPlanBytes;
+        uint32_t words[G::kPlanLaneBytes / 4];
+#pragma unroll
+        for (int q = 0; q < G::kPlanLaneBytes / 16; ++q) {
+            const Piece w4 = *reinterpret_cast<const Piece*>(mine + kPlanLane + lane * G::kPlanLaneBytes + q * 16);
+            words[4 * q] = w4[0]; words[4 * q + 1] = w4[1]; words[4 * q + 2] = w4[2]; words[4 * q + 3] = w4[3];
+        }
         U = *reinterpret_cast<const int*>(mine);
-        if (lane < kTileTokens * kR) ulist[lane] = *reinterpret_cast<const int*>(mine + 16 + lane * 4);
-        pe[0] = (int)lo[0]; pe[1] = (int)lo[1]; pe[2] = (int)lo[2]; pe[3] = (int)lo[3];
-        pe[4] = (int)hi[0]; pe[5] = (int)hi[1];
-        us[0] = hi[2] & 0xff; us[1] = (hi[2] >> 8) & 0xff; us[2] = (hi[2] >> 16) & 0xff; us[3] = hi[2] >> 24;
-        us[4] = hi[3] & 0xff; us[5] = (hi[3] >> 8) & 0xff;
-        repeats = (hi[3] >> 16) & 0xff;
+        if (lane < kTileTokens * kNnc) ulist[lane] = *reinterpret_cast<const int*>(mine + 16 + lane * 4);
+#pragma unroll
+        for (int r = 0; r < kRuns; ++r) pe[r] = (int)words[r];
+        const uint32_t w2 = words[kRuns], w3 = words[kRuns + 1];
+        usc[0] = w2 & 0xff; usc[1] = (w2 >> 8) & 0xff; usc[2] = (w2 >> 16) & 0xff; usc[3] = w2 >> 24;
+        usc[4] = w3 & 0xff; usc[5] = (w3 >> 8) & 0xff;
+        repeats = (w3 >> 16) & 0xff;
     } else {
-        tile_setup(cluster_idx, pe_idx, mask, list_b, N, i0, nt, tok, pe, us, repeats, U, ulist);
+        tile_setup<CS>(cluster_idx, pe_idx, mask, list_b, N, i0, nt, tok, pe, usc, repeats, U, ulist);
     }
     const bool twice = __any(repeats) != 0;
     lds_sync();
+    // in units of runs of 8 rows: distinct cluster u holds the units kSub * u .. kSub * u + kSub - 1
+    int ub[kNnc];
+#pragma unroll
+    for (int c = 0; c < kNnc; ++c) ub[c] = usc[c] * kSub;
+    auto unit_of = [&](auto ri) -> int {   // the unit of the token's run r (a compile-time number)
+        constexpr int r = decltype(ri)::value;
+        return ub[r / kSub] + r % kSub;
+    };
+    const int units = U * kSub;
 
-    const int total_rows = 8 * U;
-    const int passes = (U + kPassRuns - 1) / kPassRuns;
+    const int total_rows = 8 * units;
+    const int passes = (units + kPassRuns - 1) / kPassRuns;
     const uint32_t k_pitch = (uint32_t)ks.n * 2, v_pitch = (uint32_t)vs.n * 2;
     const char* k_b = reinterpret_cast<const char*>(k + (int64_t)b * ks.b + (int64_t)h0 * ks.h);
     const char* v_b = reinterpret_cast<const char*>(v + (int64_t)b * vs.b + (int64_t)h0 * vs.h);
 
-    // rows of the distinct clusters 8*pass .. 8*pass+7, as this lane gathers them: access a moves row 16*a + g_sub of
-    // the pass; clusters past the last one repeat it so that every row of a 32-row step holds data
+    // rows of the units 12*pass .. 12*pass+11, as this lane gathers them: access a moves row 16*a + g_sub of the
+    // pass; units past the last one repeat it so that every row of a 32-row step holds data
     auto pass_rows = [&](int pass, uint32_t (&rr)[kAccesses]) {
 #pragma unroll
         for (int a = 0; a < kAccesses; ++a) {
             const int urow = a * 16 + g_sub;
-            const int c = ulist[min(pass * kPassRuns + (urow >> 3), U - 1)];
-            const int row = c * 8 + (urow & 7);
+            const int unit = min(pass * kPassRuns + (urow >> 3), units - 1);
+            const int row = ulist[unit / kSub] * CS + (unit % kSub) * 8 + (urow & 7);
             rr[a] = (unsigned)row < (unsigned)N ? (uint32_t)row : 0u;
         }
     };
@@ -215,9 +245,9 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         }
 
         // small per-head operands: their latency passes under the score computation
-        float bias[kR];
+        float bias[kRuns];
 #pragma unroll
-        for (int r = 0; r < kR; ++r) {
+        for (int r = 0; r < kRuns; ++r) {
             const uint32_t cell = lane_offset(((uint32_t)(pe[r] & 0x7fffffff) * (uint32_t)H_all + (uint32_t)(h0 + h)) * 2);
             bias[r] = to_acc(*reinterpret_cast<const T*>(reinterpret_cast<const char*>(table) + cell)) +
                       (pe[r] < 0 ? -100.f : 0.f);
@@ -226,9 +256,9 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         const float bv[2] = {blank_v[(h0 + h) * kC + r16], blank_v[(h0 + h) * kC + 16 + r16]};
 
         // ---- scores -------------------------------------------------------------------------------------
-        float logit[kR];
+        float logit[kRuns];
 #pragma unroll
-        for (int r = 0; r < kR; ++r) logit[r] = 0.f;
+        for (int r = 0; r < kRuns; ++r) logit[r] = 0.f;
         for (int pass = 0; pass < passes; ++pass) {
             const int rows_here = min(kPassRows, total_rows - pass * kPassRows);
             if (pass > 0) lds_sync_vm<0>();  // the K rows of this pass are in LDS
@@ -252,13 +282,13 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
                 }
             }
             lds_sync();
-#pragma unroll
-            for (int r = 0; r < kR; ++r) {
-                const unsigned u = (unsigned)(us[r] - pass * kPassRuns);
+            static_for<0, kRuns>([&](auto ri) {
+                constexpr int r = decltype(ri)::value;
+                const unsigned u = (unsigned)(unit_of(ri) - pass * kPassRuns);
                 const float sc = *reinterpret_cast<const float*>(
                     stage + S_BASE + (t * kSRow + (int)min(u, (unsigned)kPassRuns - 1) * 8 + i) * 4);
                 logit[r] = u < (unsigned)kPassRuns ? sc : logit[r];
-            }
+            });
             if (pass + 1 < passes) {
                 lds_sync();  // the scores are picked: the area takes the next K rows
                 uint32_t rr[kAccesses];
@@ -267,11 +297,11 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
             }
         }
 
-        // ---- softmax over the 48 neighbours and the blank token ----------------------------------------------
-        float x[kR];
+        // ---- softmax over the neighbours and the blank token ---------------------------------------------------
+        float x[kRuns];
         float mx = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < kR; ++r) {
+        for (int r = 0; r < kRuns; ++r) {
             x[r] = logit[r] * scale + bias[r];
             mx = fmaxf(mx, x[r]);
         }
@@ -282,10 +312,10 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         }
         const float bl = oct_sum(part) * scale;
         mx = fmaxf(oct_max(mx), bl);
-        float p[kR];
+        float p[kRuns];
         float sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < kR; ++r) {
+        for (int r = 0; r < kRuns; ++r) {
             p[r] = __expf(x[r] - mx);
             sum += p[r];
         }
@@ -295,16 +325,17 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         // for a backward pass that recomputes the probabilities: the logarithm of the softmax's denominator
         if (lse != nullptr && i == 0 && t < nt) lse[((int64_t)b * H_all + h0 + h) * N + i0 + t] = mx + __logf(total);
 #pragma unroll
-        for (int r = 0; r < kR; ++r) p[r] *= inv;
+        for (int r = 0; r < kRuns; ++r) p[r] *= inv;
         if (i == 0) *reinterpret_cast<float*>(stage + PB_BASE + t * 4) = eb * inv;
         if (twice) {
 #pragma unroll
-            for (int r = kR - 1; r >= 1; --r) {
+            for (int c = kNnc - 1; c >= 1; --c) {
 #pragma unroll
-                for (int r2 = 0; r2 < r; ++r2) {
-                    // the first run with the same cluster collects the probabilities of its repeats
-                    bool firstmatch = us[r] == us[r2] && ((repeats >> r) & 1) && !((repeats >> r2) & 1);
-                    p[r2] += firstmatch ? p[r] : 0.f;
+                for (int c2 = 0; c2 < c; ++c2) {
+                    // the first listing of a cluster collects the probabilities of its repeats
+                    const bool firstmatch = usc[c] == usc[c2] && ((repeats >> c) & 1) && !((repeats >> c2) & 1);
+#pragma unroll
+                    for (int q = 0; q < kSub; ++q) p[c2 * kSub + q] += firstmatch ? p[c * kSub + q] : 0.f;
                 }
             }
         }
@@ -322,12 +353,12 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
             }
             lds_sync();
             T* prow = reinterpret_cast<T*>(stage + P_BASE) + t * kPRow + i;
-#pragma unroll
-            for (int r = 0; r < kR; ++r) {
-                // runs of other passes, and repeats (already added to their first run), go to the spare cells
-                const unsigned u = ((repeats >> r) & 1) ? ~0u : (unsigned)(us[r] - pass * kPassRuns);
+            static_for<0, kRuns>([&](auto ri) {
+                constexpr int r = decltype(ri)::value;
+                // runs of other passes, and repeats (already added to their first listing), go to the spare cells
+                const unsigned u = ((repeats >> (r / kSub)) & 1) ? ~0u : (unsigned)(unit_of(ri) - pass * kPassRuns);
                 prow[min(u, (unsigned)kPassRuns) * 8] = from_acc<T>(p[r]);
-            }
+            });
             if (pass > 0) {
                 lds_sync_vm<0>();  // the V rows of this pass are in LDS, the probabilities are written
             } else {
@@ -382,7 +413,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
     }
 }
 
-template <typename T>
+template <typename T, int CS>
 int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                  clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out, clusten_strides os,
@@ -391,7 +422,7 @@ int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strid
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     const int groups = head_groups_for(total, s.H);  // 196 tokens x 8 heads, B = 128: 69.6 -> 63.9 us
-    hipLaunchKernelGGL((cluster_attention_kernel<T>), dim3(xcd_grid(total * groups)), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((cluster_attention_kernel<T, CS>), dim3(xcd_grid(total * groups)), dim3(kWave), 0, stream,
                        static_cast<const T*>(q), qs, static_cast<const T*>(k), ks, static_cast<const T*>(v), vs,
                        cluster_idx, static_cast<const T*>(table), pe_idx, mask, blank_k, blank_v, static_cast<T*>(out),
                        os, s.H, s.N, scale, tiles_per_batch, total, lists_shared, groups, static_cast<const char*>(plan), lse);
@@ -400,17 +431,27 @@ int launch_typed(const void* q, clusten_strides qs, const void* k, clusten_strid
 
 }  // namespace
 
-size_t cluster_attention_plan_bytes(int B, int N) {
-    return (size_t)B * ((N + kTileTokens - 1) / kTileTokens) * kPlanBytes;
+size_t cluster_attention_plan_bytes(int B, int N, int M) {
+    const size_t per_tile = M == Geo<24>::kM ? Geo<24>::kPlanBytes : (M == Geo<8>::kM ? Geo<8>::kPlanBytes : 0);
+    return (size_t)B * ((N + kTileTokens - 1) / kTileTokens) * per_tile;
 }
 
 int launch_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
-                                  int B, int N, hipStream_t stream) {
+                                  int B, int N, int M, hipStream_t stream) {
     const int tiles_per_batch = (N + kTileTokens - 1) / kTileTokens;
     const int64_t total = (int64_t)B * tiles_per_batch;
     if (total <= 0 || total >= ((int64_t)1 << 30)) return CLUSTEN_ERR_BAD_DIMS;
-    hipLaunchKernelGGL(cluster_attention_plan_kernel, dim3((unsigned)total), dim3(kWave), 0, stream, cluster_idx, pe_idx, mask,
-                       static_cast<char*>(plan), N, tiles_per_batch, (int)total);
+    const int cluster_size = M / kNnc;
+    if (M % kNnc != 0) return CLUSTEN_ERR_BAD_DIMS;
+    if (cluster_size == 8) {
+        hipLaunchKernelGGL(cluster_attention_plan_kernel<8>, dim3((unsigned)total), dim3(kWave), 0, stream, cluster_idx,
+                           pe_idx, mask, static_cast<char*>(plan), N, tiles_per_batch, (int)total);
+    } else if (cluster_size == 24) {
+        hipLaunchKernelGGL(cluster_attention_plan_kernel<24>, dim3((unsigned)total), dim3(kWave), 0, stream, cluster_idx,
+                           pe_idx, mask, static_cast<char*>(plan), N, tiles_per_batch, (int)total);
+    } else {
+        return CLUSTEN_ERR_BAD_DIMS;
+    }
     return launch_status();
 }
 
@@ -420,7 +461,10 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
                              clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
                              clusten_attn_shape s, int dtype, hipStream_t stream) {
     if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
-    if (s.C != kC || s.M != kM) return CLUSTEN_ERR_BAD_DIMS;
+    // six clusters per token: 48 neighbours = clusters of 8, 144 = clusters of 24
+    if (s.C != kC || (s.M != Geo<8>::kM && s.M != Geo<24>::kM)) return CLUSTEN_ERR_BAD_DIMS;
+    const int cluster_size = s.M / kNnc;
+    if (cluster_size == 24 && dtype == CLUSTEN_F32) return CLUSTEN_ERR_BAD_DIMS;   // clusters of 24: 16-bit data only
     const size_t eb = dtype_size(dtype);
     const bool ok = rows_aligned16(q, qs, eb) && rows_aligned16(k, ks, eb) && rows_aligned16(v, vs, eb) &&
                     rows_aligned16(out, os, eb) && aligned16(blank_k) && slice_fits_int32(ks, s.H, s.N, s.C) &&
@@ -430,12 +474,20 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
         return launch_cluster_attention_f32(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os,
                                             scale, lists_shared, plan, lse, s, stream);
     }
-    if (dtype == CLUSTEN_F16) {
-        return launch_typed<f16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                   lists_shared, plan, lse, s, stream);
+    if (cluster_size == 24) {
+        if (dtype == CLUSTEN_F16) {
+            return launch_typed<f16_t, 24>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os,
+                                           scale, lists_shared, plan, lse, s, stream);
+        }
+        return launch_typed<bf16_t, 24>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os,
+                                        scale, lists_shared, plan, lse, s, stream);
     }
-    return launch_typed<bf16_t>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
-                                lists_shared, plan, lse, s, stream);
+    if (dtype == CLUSTEN_F16) {
+        return launch_typed<f16_t, 8>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
+                                      lists_shared, plan, lse, s, stream);
+    }
+    return launch_typed<bf16_t, 8>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,
+                                   lists_shared, plan, lse, s, stream);
 }
 
 }  // namespace clusten

@@ -42,9 +42,12 @@ int launch_gather_sum_clusters(const void* p, const void* rows, clusten_strides 
 //   p : contiguous (B,H,N,M);  x : strided (B,H,N,C);  out : contiguous (B,H,N,C), zeroed here.
 //   Lists made of whole clusters (found out on the device) go through pair lists in `workspace` and a gather without
 //   atomics; for any other list the sum is built with fp32 atomics (for F16/BF16 in `workspace`, rounded once).
+//   `pair_lists` (may be null): the block launch_cluster_pairs filled for these lists (layout cluster_pairs_layout(B,
+//   N, M, N)); the pair lists are then not rebuilt in the workspace.
 size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype);
 int launch_scatter_rows(const void* p, const void* x, clusten_strides x_strides, const int64_t* idx, void* out,
-                        void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream);
+                        void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream,
+                        const void* pair_lists = nullptr);
 
 // out[b,i,ic,c] = sum_j w[b,i,j,ic] * feat[b,idx[b,i,j],c]      (WF forward)
 int launch_wf_forward(const void* w, const void* feat, const int64_t* idx, void* out, clusten_wf_shape s, int dtype,
@@ -73,8 +76,8 @@ int launch_attn_softmax(const void* attn, const void* table, const int64_t* pe_i
 
 // Local attention of a cluster-ordered sequence in one kernel (QK, position bias, mask, blank token, softmax, AV,
 // blank value): see cluster_attention.hip.  q, k, v, out : strided (B,H,N,C) of T in {F16, BF16, F32}, C = 32;
-//   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,48) — or (1,N,.) each
-//   when lists_shared;
+//   cluster_idx (B,N,6) int32; table (rows,H) of T; pe_idx, mask (may be null) : int64 (B,N,M) — or (1,N,.) each
+//   when lists_shared; M = 48 (clusters of 8) or, for 16-bit data, 144 (clusters of 24);
 //   blank_k, blank_v : fp32 (H,C);  lse (may be null): fp32 (B,H,N), the logarithm of each softmax's denominator.
 int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
                              clusten_strides vs, const int32_t* cluster_idx, const void* table, const int64_t* pe_idx,
@@ -92,10 +95,10 @@ int launch_cluster_attention_backward(const void* q, clusten_strides qs, const v
                                       float* p_blank, float* ds_blank, float scale, int lists_shared, const void* plan,
                                       clusten_attn_shape s, int dtype, hipStream_t stream);
 // The per-tile plan the kernel above reads instead of cluster_idx, pe_idx and mask when it is given one (what it
-// would work out from them before its first head): B = batch elements of the index tensors.
-size_t cluster_attention_plan_bytes(int B, int N);
+// would work out from them before its first head): B = batch elements of the index tensors, M = 48 or 144.
+size_t cluster_attention_plan_bytes(int B, int N, int M);
 int launch_cluster_attention_plan(const int32_t* cluster_idx, const int64_t* pe_idx, const int64_t* mask, void* plan,
-                                  int B, int N, hipStream_t stream);
+                                  int B, int N, int M, hipStream_t stream);
 
 // The pair lists of lists made of whole clusters (cluster_pairs.hip), built on the device: for `rows` list rows per
 //   image of M slots that point into a sequence of D rows (K = ceil(D/8) clusters), pairs[starts[b*K+g] .. ends[b*K+g])

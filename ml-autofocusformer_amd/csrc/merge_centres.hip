@@ -179,6 +179,12 @@ __global__ __launch_bounds__(kMergeThreads) void merge_centres_kernel(const floa
     int at_equal = scan_threads(n_equal, scratch, &total);
     int at_res = scan_threads(n_res, scratch, &total);
     int64_t* out = centre + (int64_t)b * out_n;
+    // an image with fewer reserved tokens than reserve_num (the reference's reshape raises there,
+    // models/aff_transformer.py:323): the slots nobody fills hold -1, which the caller can test for and which
+    // merge_rows_kernel reads as row 0
+    if (reserve_on) {
+        for (int s = total + (int)threadIdx.x; s < reserve_num; s += (int)blockDim.x) out[sample_num + s] = -1;
+    }
     for (int i = lo; i < hi; ++i) {
         const uint32_t k = keys[i];
         if (k > kth) {
@@ -211,7 +217,8 @@ __global__ __launch_bounds__(256) void merge_rows_kernel(MergeRows r, const int6
     const int64_t row = e / W;
     const int w = (int)(e - row * W);
     const int64_t b = row / n_out;
-    const int64_t from = b * N + centre[row];
+    const int64_t c = centre[row];
+    const int64_t from = b * N + ((uint64_t)c < (uint64_t)N ? c : 0);   // an index outside [0,N) reads row 0
     int t = 0;
 #pragma unroll
     for (int u = 1; u < 4; ++u) t += (u < r.count && w >= r.first[u]);

@@ -40,6 +40,23 @@ __device__ __forceinline__ F32x4 mfma_4x4x1(float a, float b, F32x4 d) {
     }
 }
 
+// Sixteen independent 4x4 blocks, D += A (4x4) * B (4x4) over four k steps of 16-bit operands, fp32 sums:
+// `v_mfma_f32_4x4x4_16b_f16` / `_bf16`.  Lane t of a block holds row t of A (k = 0..3, two registers), column t of B
+// (k = 0..3) and column t of D (rows 0..3).  Products of fp16 / bf16 values are exact in fp32.
+template <typename T>
+__device__ __forceinline__ F32x4 mfma_4x4x4_16b(const U32x2& a, const U32x2& b, F32x4 d) {
+    static_assert(sizeof(T) == 2, "16-bit operands");
+    typedef _Float16 H4 __attribute__((ext_vector_type(4)));
+    typedef short S4 __attribute__((ext_vector_type(4)));
+    if constexpr (CLUSTEN_REPLAY != 0) {
+        return replay_touch(a[0] ^ a[1], b[0] ^ b[1], d);
+    } else if constexpr (std::is_same<T, f16_t>::value) {
+        return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(H4, a), __builtin_bit_cast(H4, b), d, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(S4, a), __builtin_bit_cast(S4, b), d, 0, 0, 0);
+    }
+}
+
 // s_waitcnt immediate (gfx9 encoding) that waits until at most `vm` vector-memory operations are
 // outstanding and leaves the LDS/scalar and export counters alone.
 constexpr int waitcnt_vm(int vm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (15 << 8); }

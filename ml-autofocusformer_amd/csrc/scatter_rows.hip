@@ -52,7 +52,7 @@ ScatterPlan scatter_plan(const clusten_attn_shape& s, int dtype) {
 size_t scatter_rows_workspace_bytes(clusten_attn_shape s, int dtype) { return scatter_plan(s, dtype).bytes; }
 
 int launch_scatter_rows(const void* p, const void* x, clusten_strides xs, const int64_t* idx, void* out,
-                        void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream) {
+                        void* workspace, clusten_attn_shape s, int dtype, hipStream_t stream, const void* pair_lists) {
     const size_t count = (size_t)s.B * s.H * s.N * s.C;
     const ScatterPlan plan = scatter_plan(s, dtype);
     if (plan.bytes != 0 && !aligned16(workspace)) return CLUSTEN_ERR_UNALIGNED;
@@ -61,14 +61,19 @@ int launch_scatter_rows(const void* p, const void* x, clusten_strides xs, const 
     // lists made of whole clusters: a gather over sorted pair lists, chosen on the device through `flag`
     const int32_t* flag = nullptr;
     if (plan.by_cluster && scatter_by_cluster_supported(p, x, xs, out, s, dtype)) {
-        int32_t* not_whole = reinterpret_cast<int32_t*>(ws + plan.pairs.flag);
-        int32_t* keys = reinterpret_cast<int32_t*>(ws + plan.pairs.keys);
-        int32_t* wg_bad = reinterpret_cast<int32_t*>(ws + plan.pairs.wg_bad);
-        int32_t* pairs = reinterpret_cast<int32_t*>(ws + plan.pairs.pairs);
-        int32_t* starts = reinterpret_cast<int32_t*>(ws + plan.pairs.starts);
-        int32_t* ends = reinterpret_cast<int32_t*>(ws + plan.pairs.ends);
-        st = launch_cluster_pairs(idx, keys, wg_bad, not_whole, pairs, starts, ends, s.B, s.N, s.M, s.N, stream);
-        if (st != CLUSTEN_OK) return st;
+        // the caller's pair lists of these lists (built once for every layer and head that uses them), or the
+        // workspace's, built now
+        char* block = pair_lists != nullptr ? const_cast<char*>(static_cast<const char*>(pair_lists)) : ws;
+        int32_t* not_whole = reinterpret_cast<int32_t*>(block + plan.pairs.flag);
+        int32_t* pairs = reinterpret_cast<int32_t*>(block + plan.pairs.pairs);
+        int32_t* starts = reinterpret_cast<int32_t*>(block + plan.pairs.starts);
+        int32_t* ends = reinterpret_cast<int32_t*>(block + plan.pairs.ends);
+        if (pair_lists == nullptr) {
+            int32_t* keys = reinterpret_cast<int32_t*>(block + plan.pairs.keys);
+            int32_t* wg_bad = reinterpret_cast<int32_t*>(block + plan.pairs.wg_bad);
+            st = launch_cluster_pairs(idx, keys, wg_bad, not_whole, pairs, starts, ends, s.B, s.N, s.M, s.N, stream);
+            if (st != CLUSTEN_OK) return st;
+        }
         st = launch_scatter_by_cluster(p, x, xs, starts, ends, pairs, not_whole, out, s, dtype, stream);
         if (st != CLUSTEN_OK) return st;
         flag = not_whole;

@@ -12,6 +12,9 @@
 // fp32 channels) and every gather instruction moves whole rows, 1 KiB per wave access, straight
 // into registers.  Each row is read once for all IC inner channels (the reference re-gathers it
 // IC times).
+// fp16 / bf16 weights over rows of the same type go four slots per instruction through `v_mfma_f32_4x4x4_16b_f16` /
+// `_bf16` with the operands as they are stored (a quarter of the matrix instructions, no widening); everything else
+// as below.
 // The products run on the matrix cores as `v_mfma_f32_4x4x1_16b_f32`: 16 independent 4x4 blocks,
 // one slot (k = 1) per instruction.  Block l/4 takes, as its B row, element e of the 16-byte groups
 // that lanes 4*(l/4)..+3 hold (four channels of one token), and as its A column the token's four
@@ -59,6 +62,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     constexpr int NI_W = (W_BYTES + 1023) / 1024;
     static_assert(LPT == 16 || LPT == 32 || LPT == 64, "a row of 16 lanes must belong to one token");
     static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
+    static_assert(GS == 4, "the 16-bit path multiplies the four slots of a pipeline group at once");
 
     __shared__ __attribute__((aligned(1024))) char wbuf[NI_W * 1024];
 
@@ -140,13 +144,39 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
                 },
                 [&](auto ji) {
                     constexpr int j = decltype(ji)::value;
-                    const float aop = (!GUARD || j < mc) ? to_acc(wv[j]) : 0.f;
-                    float x[VEC];
-                    VecIO<TF, VEC>::unpack(fv[j], x);
+                    if constexpr (sizeof(T) == 2 && std::is_same<T, TF>::value) {
+                        // 16-bit weights and rows: four slots per matrix instruction (k = 4), operands as stored.
+                        // A = the lane's inner channel of the weights of slots j-3..j; B = one channel of the four
+                        // gathered rows: the low (high) halves of word d of the four rows are channel 2d (2d+1).
+                        if constexpr (j % 4 == 3) {
+                            uint32_t wbits[4];
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        const float bop = (!GUARD || j < mc) ? x[e] : 0.f;
-                        acc[e] = mfma_4x4x1(aop, bop, acc[e]);
+                            for (int q = 0; q < 4; ++q) {
+                                wbits[q] = (!GUARD || j - 3 + q < mc) ? storage_bits(wv[j - 3 + q]) : 0u;
+                            }
+                            const U32x2 aop = U32x2{wbits[0] | (wbits[1] << 16), wbits[2] | (wbits[3] << 16)};
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) {
+                                uint32_t x[4];
+#pragma unroll
+                                for (int q = 0; q < 4; ++q) x[q] = (!GUARD || j - 3 + q < mc) ? fv[j - 3 + q][d] : 0u;
+                                const U32x2 lo = U32x2{__builtin_amdgcn_perm(x[1], x[0], 0x05040100u),
+                                                       __builtin_amdgcn_perm(x[3], x[2], 0x05040100u)};
+                                const U32x2 hi = U32x2{__builtin_amdgcn_perm(x[1], x[0], 0x07060302u),
+                                                       __builtin_amdgcn_perm(x[3], x[2], 0x07060302u)};
+                                acc[2 * d] = mfma_4x4x4_16b<T>(aop, lo, acc[2 * d]);
+                                acc[2 * d + 1] = mfma_4x4x4_16b<T>(aop, hi, acc[2 * d + 1]);
+                            }
+                        }
+                    } else {
+                        const float aop = (!GUARD || j < mc) ? to_acc(wv[j]) : 0.f;
+                        float x[VEC];
+                        VecIO<TF, VEC>::unpack(fv[j], x);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            const float bop = (!GUARD || j < mc) ? x[e] : 0.f;
+                            acc[e] = mfma_4x4x1(aop, bop, acc[e]);
+                        }
                     }
                 });
         }

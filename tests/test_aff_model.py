@@ -199,7 +199,16 @@ def test_clusters_of_24_with_144_neighbours_as_in_the_384_models(device, amp):
     same model on the oracle."""
     from aff.model import default_ops
     kw = dict(img_size=192, num_classes=12, embed_dim=(64, 128, 256, 512), cluster_size=24, nbhd_size=(144, 144, 144, 144))
-    hip = small_model(default_ops(), **kw).to(device)
+    ops = default_ops()
+    fused_calls = []
+    one_kernel = ops.cluster_attention
+
+    def counted(q, *a, **k):
+        fused_calls.append(tuple(q.shape))
+        return one_kernel(q, *a, **k)
+
+    ops.cluster_attention = counted
+    hip = small_model(ops, **kw).to(device)
     ref = small_model(oracle_ops(), **kw).to(device)
     ref.load_state_dict(hip.state_dict())
     x = torch.randn(2, 3, 192, 192, generator=torch.Generator().manual_seed(17)).to(device)
@@ -208,7 +217,10 @@ def test_clusters_of_24_with_144_neighbours_as_in_the_384_models(device, amp):
     assert torch.isfinite(y_hip).all()
     assert oracle.rel_err(y_hip.float(), y_ref.float()) < (2e-2 if amp else 1e-4)
     if amp:
+        # under mixed precision the local attention of the first two stages (1 + 2 blocks) ran as one kernel each
+        assert [s[2] for s in fused_calls] == [2304, 576, 576] and all(s[3] == 32 for s in fused_calls)
         return
+    assert not fused_calls      # fp32 data: clusters of 24 go through the three operators
     hip.train(), ref.train()
     target = torch.randn(2, 12, generator=torch.Generator().manual_seed(18)).to(device)
     for model in (hip, ref):
@@ -772,20 +784,22 @@ def test_cached_16_bit_weights_follow_the_parameters(device):
 
 
 @pytest.mark.gpu
-def test_training_with_the_one_kernel_attention_matches_the_operator_path(device):
+@pytest.mark.parametrize("img_size", [128, 120])
+def test_training_with_the_one_kernel_attention_matches_the_operator_path(device, img_size):
     """A training step under fp16 autocast with the local attention as one kernel forward and `cluster_attention_backward`
     plus its sums backward, against the same step through the three operators and the softmax kernels: same loss,
-    parameter gradients within the noise of fp16 intermediates."""
+    parameter gradients within the noise of fp16 intermediates.  At 120 x 120 pixels the stages hold 900, 225 and 56
+    tokens: short last clusters, pad slots and masks in every local stage."""
     from aff.model import default_ops
     fused_ops = default_ops()
     plain = dict(vars(default_ops()))
     plain.pop("cluster_attention_backward")
     plain_ops = SimpleNamespace(**plain)
-    cfg = dict(embed_dim=(64, 128, 256, 512), num_heads=(2, 4, 8, 16), img_size=128)
+    cfg = dict(embed_dim=(64, 128, 256, 512), num_heads=(2, 4, 8, 16), img_size=img_size)
     a = small_model(fused_ops, **cfg).to(device).train()
     b = small_model(plain_ops, **cfg).to(device).train()
     b.load_state_dict(a.state_dict())
-    x = torch.randn(2, 3, 128, 128, generator=torch.Generator().manual_seed(5)).to(device)
+    x = torch.randn(2, 3, img_size, img_size, generator=torch.Generator().manual_seed(5)).to(device)
     target = torch.tensor([3, 7], device=device)
     losses = []
     for m in (a, b):

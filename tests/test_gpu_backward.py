@@ -203,6 +203,45 @@ def test_cluster_by_cluster_scatter_properties(device):
     assert _native.cluster_pairs(idx[:, :, :44].contiguous()) is None
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_scatter_alone_with_the_callers_pair_lists(device, dtype):
+    """`clusten_scatter_rows`: the scatter of the attention backward passes by itself, with pair lists the caller keeps.
+    On lists made of whole clusters it is the gather over those lists (bit-equal to the entry point that only does
+    that, and to the drop-in backward); on any other list the block's flag sends it to the atomic kernels, so the
+    output is the full sum either way - nothing is left unwritten.  `qk_backward` / `av_backward` with `pairs=` are
+    the same kernels as without."""
+    g = torch.Generator().manual_seed(84)
+    B, H, N, C = 2, 2, 203, 32                       # a short last cluster: 3 rows and 5 pad slots
+    tol = TOL_SCATTER_F32 if dtype == torch.float32 else TOL[dtype]
+    x = torch.randn(B, H, N, C, generator=g).to(dtype)
+    k = torch.randn(B, H, N, C, generator=g).to(dtype)
+    for kind in ("runs:padded", "model_built", "random", "windowed"):
+        idx = wl.attn_case("s", 85, B=B, H=H, N=N, C=C, lists=kind).nbhd_idx
+        M = idx.shape[-1]
+        p = torch.randn(B, H, N, M, generator=g).to(dtype)
+        xd, kd, pd, idxd = x.to(device), k.to(device), p.to(device), idx.to(device)
+        pairs = _native.cluster_pairs(idxd)
+        whole = int(_native.pairs_not_whole(pairs)) == 0
+        assert whole == (kind in ("runs:padded", "model_built")), kind
+        want_dq, want_dk = oracle.qk_gather_backward(p.float(), x.float(), k.float(), idx)
+        got = _native.scatter_rows(pd, xd, idxd, pairs)
+        assert got.dtype == dtype and oracle.rel_err(got, want_dk) <= tol, kind
+        assert oracle.rel_err(_native.scatter_rows(pd, xd, idxd), want_dk) <= tol, kind      # pair lists built inside
+        dq, dk = _native.qk_backward(pd, xd, kd, idxd, pairs=pairs)
+        dq0, dk0 = _native.qk_backward(pd, xd, kd, idxd)
+        assert torch.equal(dq, dq0) and oracle.rel_err(dq, want_dq) <= tol
+        da, dv = _native.av_backward(xd, pd, kd, idxd, pairs=pairs)
+        da0, dv0 = _native.av_backward(xd, pd, kd, idxd)
+        assert torch.equal(da, da0)
+        if whole:   # fixed summation order: the same bits through every door
+            assert torch.equal(got, _native.scatter_rows_by_cluster(pd, xd, pairs))
+            assert torch.equal(got, dk0) and torch.equal(dk, dk0) and torch.equal(dv, dv0)
+        else:
+            assert oracle.rel_err(dk, want_dk) <= tol and oracle.rel_err(dv, dv0.float().cpu()) <= 2 * tol
+    with pytest.raises(RuntimeError, match="does not belong"):
+        _native.scatter_rows(pd, xd, idxd, pairs[:-256])
+
+
 def test_backward_never_reads_the_device_from_the_host(device):
     """The drop-in backward of the three operators recorded into a HIP graph (a capture fails on any synchronisation or
     read-back) and replayed with eager work between the replays: every replay equals the eager result bit for bit on

@@ -17,10 +17,10 @@ pytestmark = pytest.mark.gpu
 C, NNC, M = 32, 6, 48
 
 
-def _cluster_numbers(b, n, gen, kind):
-    """(B,N,6) int32 cluster numbers out of ceil(N/8) clusters (the last may be short: its pad slots list row 0)."""
-    k = (n + 7) // 8
-    own = torch.arange(n) // 8
+def _cluster_numbers(b, n, gen, kind, cs=8):
+    """(B,N,6) int32 cluster numbers out of ceil(N/cs) clusters (the last may be short: its pad slots list row 0)."""
+    k = (n + cs - 1) // cs
+    own = torch.arange(n) // cs
     if kind == "shared":        # the 8 tokens of a cluster list the same clusters
         per = torch.stack([torch.randperm(k, generator=gen)[:NNC] for _ in range(b * k)]).reshape(b, k, NNC)
         return per[:, own].to(torch.int32).contiguous()
@@ -32,8 +32,8 @@ def _cluster_numbers(b, n, gen, kind):
     return pick.to(torch.int32).contiguous()
 
 
-def _expand(cidx, n):
-    rows = cidx.long().unsqueeze(3) * 8 + torch.arange(8)
+def _expand(cidx, n, cs=8):
+    rows = cidx.long().unsqueeze(3) * cs + torch.arange(cs)
     rows = torch.where((rows < n) & (rows >= 0), rows, torch.zeros_like(rows))
     return rows.reshape(cidx.shape[0], cidx.shape[1], -1).contiguous()
 
@@ -52,19 +52,20 @@ def _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale):
     return out.permute(0, 2, 1, 3).reshape(b, n, h * c)
 
 
-def _case(b, h, n, gen, kind, dtype, with_mask, rows=97):
+def _case(b, h, n, gen, kind, dtype, with_mask, rows=97, cs=8):
+    m = NNC * cs
     q = torch.randn(b, h, n, C, generator=gen).to(dtype)
     k = torch.randn(b, h, n, C, generator=gen).to(dtype)
     v = torch.randn(b, h, n, C, generator=gen).to(dtype)
-    cidx = _cluster_numbers(b, n, gen, kind)
+    cidx = _cluster_numbers(b, n, gen, kind, cs)
     table = torch.randn(rows, h, generator=gen).to(dtype)
-    pe_idx = torch.randint(rows, (b, n, M), generator=gen)
-    idx = _expand(cidx, n)
+    pe_idx = torch.randint(rows, (b, n, m), generator=gen)
+    idx = _expand(cidx, n, cs)
     mask = None
     if with_mask:
         # pad slots of a short last cluster are masked, as the model's cluster mask does, plus a few others
-        mask = ((cidx.long().unsqueeze(3) * 8 + torch.arange(8)) < n).reshape(b, n, M).long()
-        mask = mask * (torch.rand(b, n, M, generator=gen) > 0.05).long()
+        mask = ((cidx.long().unsqueeze(3) * cs + torch.arange(cs)) < n).reshape(b, n, m).long()
+        mask = mask * (torch.rand(b, n, m, generator=gen) > 0.05).long()
     blank_k = torch.randn(h * C, generator=gen)
     blank_v = torch.randn(h * C, generator=gen)
     return q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v
@@ -89,6 +90,65 @@ def test_against_the_oracle_composition(device, kind, dtype):
         for with_mask in (False, True):
             err = _run(device, _case(b, h, n, gen, kind, dtype, with_mask), scale=C ** -0.5)
             assert err <= TOL[dtype], "%s %s n=%d mask=%s rel err %.3g" % (kind, dtype, n, with_mask, err)
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_clusters_of_24_against_the_oracle_composition(device, kind, dtype):
+    """Clusters of 24 tokens, the members of the 6 nearest = 144 neighbours (the 384 x 384 models,
+    configs/aff_base_22kto1k_384.yaml:10-11): three runs of 8 rows per cluster, two or three passes per head on lists
+    like the model's, up to twelve on lists with nothing in common.  With and without a mask, a short last cluster
+    (400 = 16 clusters and one of 16 tokens; 148: a last cluster of 4), partial tiles, through the tensors and through
+    a plan (bit-equal), per-image lists and one image's lists for the batch."""
+    gen = torch.Generator().manual_seed(91)
+    d = lambda x: None if x is None else x.to(device)
+    for b, h, n in ((2, 3, 400), (1, 2, 148), (2, 4, 192)):
+        for with_mask in (False, True):
+            case = _case(b, h, n, gen, kind, dtype, with_mask, cs=24)
+            q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = case
+            assert idx.shape == (b, n, 144)
+            ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, C ** -0.5)
+            out = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k),
+                                            d(blank_v), scale=C ** -0.5)
+            err = oracle.rel_err(out, ref)
+            assert err <= TOL[dtype], "%s %s n=%d mask=%s rel err %.3g" % (kind, dtype, n, with_mask, err)
+            plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+            assert plan.numel() == _native.load().clusten_cluster_attention_plan_bytes(b, n, 144)
+            planned = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                scale=C ** -0.5, plan=plan)
+            assert torch.equal(planned, out)
+    # one image's lists for the whole batch
+    b, h, n = 3, 2, 240
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, dtype, True, cs=24)
+    c1, p1, m1 = cidx[:1].contiguous(), pe_idx[:1].contiguous(), mask[:1].contiguous()
+    full = _native.cluster_attention(d(q), d(k), d(v), d(c1.expand(b, -1, -1).contiguous()), d(table),
+                                     d(p1.expand(b, -1, -1).contiguous()), d(m1.expand(b, -1, -1).contiguous()),
+                                     d(blank_k), d(blank_v), scale=0.25)
+    shared = _native.cluster_attention(d(q), d(k), d(v), d(c1), d(table), d(p1), d(m1), d(blank_k), d(blank_v), scale=0.25)
+    assert torch.equal(shared, full)
+    plan1 = _native.cluster_attention_plan(d(c1), d(p1), d(m1))
+    assert torch.equal(_native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                 scale=0.25, plan=plan1), full)
+    # fp32 data has no kernel for clusters of 24
+    assert not _native.cluster_attention_supported(d(q).float(), 6, 24) and _native.cluster_attention_supported(d(q), 6, 24)
+    with pytest.raises(RuntimeError):
+        _native.cluster_attention(d(q).float(), d(k).float(), d(v).float(), d(c1), d(table), d(p1), d(m1), d(blank_k),
+                                  d(blank_v))
+
+
+def test_clusters_of_24_equal_the_operators_on_the_expanded_lists(device):
+    """The same attention through QK on the 144-slot lists, the softmax kernel and AV (the path the 384 x 384 models took
+    before): equal within the 16-bit tolerance."""
+    gen = torch.Generator().manual_seed(92)
+    b, h, n = 2, 4, 480
+    q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, "near", torch.float16, True, cs=24)
+    d = lambda x: x.to(device)
+    attn = _native.qk_forward(d(q), d(k), d(idx))
+    probs, blank = _native.attn_softmax(attn, d(table), d(pe_idx), d(mask), query=d(q), blank_key=d(blank_k))
+    three = _native.av_forward(probs.to(torch.float16), d(v), d(idx)).float() + blank * d(blank_v).reshape(1, h, 1, C)
+    three = three.permute(0, 2, 1, 3).reshape(b, n, h * C)
+    one = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v))
+    assert oracle.rel_err(one.float().cpu(), three.cpu()) <= TOL[torch.float16]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
@@ -187,7 +247,7 @@ def test_plan_built_once_gives_the_same_bits(device, kind, dtype):
             plain = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k),
                                               d(blank_v), scale=0.2)
             plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
-            assert plan.dtype == torch.uint8 and plan.numel() == _native.load().clusten_cluster_attention_plan_bytes(b, n)
+            assert plan.dtype == torch.uint8 and plan.numel() == _native.load().clusten_cluster_attention_plan_bytes(b, n, 48)
             for _ in range(2):      # the plan serves any number of calls
                 planned = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
                                                     scale=0.2, plan=plan)

@@ -285,6 +285,23 @@ def test_wf_other_shapes(device, c, ic, m):
     _check_wf(wl.wf_case("wf", 62, B=2, N=196, C=c, IC=ic, M=m, Nout=64), device, torch.float32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("c,ic,m", [(128, 4, 48), (128, 3, 48), (256, 2, 48), (128, 1, 48), (128, 4, 16), (128, 4, 144),
+                                    (128, 4, 20), (128, 2, 100), (512, 4, 52), (64, 4, 48)])
+def test_wf_16_bit_rows_on_the_16_bit_matrix_path(device, dtype, c, ic, m):
+    """fp16 / bf16 weights over rows of the same type: four slots per matrix instruction.  Lists of 48 slots (no range
+    checks) and other lengths (64 slots at a time, the tail of the last four-slot group zeroed), 1 to 4 inner channels,
+    rows of 128 bytes (element kernel) to 1 KiB; sums of small integers must come out exactly rounded."""
+    _check_wf(wl.wf_case("wf16", 64, B=2, N=196, C=c, IC=ic, M=m, Nout=50, dtype=dtype), device, dtype)
+    g = torch.Generator().manual_seed(65)
+    w = torch.randint(-4, 5, (2, 50, m, ic), generator=g).float()
+    f = torch.randint(-8, 9, (2, 196, c), generator=g).float()
+    idx = torch.randint(196, (2, 50, m), generator=g)
+    out = _native.wf_forward(w.to(dtype).to(device), f.to(dtype).to(device), idx.to(device))
+    # the fp32 sums of these integers are exact, so the result is their one rounding to the storage type
+    assert torch.equal(out.cpu(), oracle.wf_gather(w, f, idx).to(dtype))
+
+
 def test_wf_integer_valued_data_is_bit_exact(device):
     g = torch.Generator().manual_seed(63)
     B, N, Nout, C, M, IC = 2, 196, 49, 128, 48, 4

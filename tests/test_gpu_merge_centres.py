@@ -143,6 +143,29 @@ def test_refusals(device):
         _native.merge_centres(pos.cpu(), None, None, 4.0, 2, 4, 4, True)
 
 
+def test_an_image_with_fewer_reserved_tokens_than_asked_for(device, monkeypatch):
+    """The reference's reshape raises when an image does not hold reserve_num tokens on the coarse grid
+    (aff_transformer.py:323).  The kernel fills the slots of the missing ones with -1 (nothing stays unwritten), the row
+    gather reads row 0 for them, and under CLUSTEN_DEBUG_INDICES=1 the wrapper raises like the reference; a surplus of
+    reserved tokens is cut to the first reserve_num."""
+    pos = _grid(2, 8, 8, device)                       # 4 tokens of each image lie on the grid of spacing 4
+    pos[1, 0] = torch.tensor([1.0, 1.0])               # ... but image 1 loses one: 3
+    got = _native.merge_centres(pos, None, None, 4.0, 2, 8, 4, True)
+    res = got[:, 8:].cpu()
+    grid4 = ((pos.cpu() % 4).sum(-1) == 0)
+    assert torch.equal(res[0], grid4[0].nonzero()[:, 0]) and res[0].tolist() == [0, 4, 32, 36]
+    assert torch.equal(res[1, :3], grid4[1].nonzero()[:, 0]) and int(res[1, 3]) == -1
+    assert int(got[:, :8].min()) >= 0
+    rows = _native.merge_rows(got, pos)[0]
+    assert torch.equal(rows[1, 8 + 3], pos[1, 0]) and torch.equal(rows[1, 8 + 2], pos[1, 36])
+    few = _native.merge_centres(pos, None, None, 4.0, 2, 8, 2, True)           # more reserved tokens than slots
+    assert torch.equal(few[:, 8:].cpu(), torch.stack([grid4[b].nonzero()[:2, 0] for b in range(2)]))
+    monkeypatch.setenv("CLUSTEN_DEBUG_INDICES", "1")
+    with pytest.raises(RuntimeError, match="fewer than reserve_num"):
+        _native.merge_centres(pos, None, None, 4.0, 2, 8, 4, True)
+    _native.merge_centres(pos, None, None, 4.0, 2, 8, 3, True)
+
+
 @pytest.mark.parametrize("with_mask", [False, True])
 def test_rows_at_the_centres(device, with_mask):
     gen = torch.Generator().manual_seed(11)

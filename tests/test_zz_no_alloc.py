@@ -62,6 +62,44 @@ def test_two_calls_in_a_row_the_second_smaller(device, dtype):
                 assert oracle.rel_err(got_q, ref_q) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_a_warmed_call_allocates_nothing_and_replays_from_a_graph(device, dtype):
+    """After one call on the device (which looks the scratch array's address up) a call changes neither the device's
+    free memory nor the framework's allocation count, and it can be recorded into a HIP graph: replays, with eager
+    calls between them, equal the eager result (integer-valued data, so the order of the atomics cannot show)."""
+    d_attn, q, k, idx = (t.to(device) for t in _inputs(310, 2, 2, 200, 32, 48, dtype, "windowed", True))
+    got_q, got_k = torch.empty_like(q), torch.empty_like(q)
+    _native.qk_backward_static(d_attn, q, k, idx, got_q, got_k)       # the first call on this device
+    torch.cuda.synchronize()
+    want_q, want_k = got_q.clone(), got_k.clone()
+    free0 = torch.cuda.mem_get_info()[0]
+    count0 = torch.cuda.memory_stats()["allocation.all.allocated"]
+    segs0 = torch.cuda.memory_stats()["segment.all.allocated"]
+    _native.qk_backward_static(d_attn, q, k, idx, got_q, got_k)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == count0
+    assert torch.cuda.memory_stats()["segment.all.allocated"] == segs0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _native.qk_backward_static(d_attn, q, k, idx, got_q, got_k)   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _native.qk_backward_static(d_attn, q, k, idx, got_q, got_k)
+    for _ in range(3):
+        got_q.fill_(float("nan"))
+        got_k.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_q, want_q) and torch.equal(got_k, want_k)
+        small = [t.to(device) for t in _inputs(311, 1, 2, 64, 32, 48, dtype, "random", True)]   # eager work between
+        sq, sk = torch.empty_like(small[1]), torch.empty_like(small[1])
+        _native.qk_backward_static(*small, sq, sk)
+        assert torch.equal(sk, _native.qk_backward(*small)[1])
+
+
 def test_a_problem_beyond_the_scratch_is_refused(device):
     lib = _native.load()
     # 16-bit data: at least 4 bytes of scratch per d_key element
