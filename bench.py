@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # runs of `bench.py --only {qk,av,wf}`, each counter scaled by what it reads for the copy probe of known
 # size; see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md, which names the source revision the
 # counters were read at.  A constant of that run, not a measurement of this one: TRAFFIC_MEASURED says when.
-MEASURED_TRAFFIC_BYTES = {"qk": 359.56e6 + 154.14e6, "av": 410.98e6 + 102.76e6, "wf": 219.18e6 + 102.76e6}
+MEASURED_TRAFFIC_BYTES = {"qk": 359.59e6 + 154.14e6, "av": 410.97e6 + 102.76e6, "wf": 219.49e6 + 102.76e6}
 TRAFFIC_MEASURED = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md"
 
 
@@ -316,26 +316,29 @@ def _bench_wf(case, steps, warmup):
             "input_sets_rotated": copies}
 
 
-def _bench_local_attention(B, H, N, dtype, steps, warmup):
+def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8):
     """The one-kernel local attention (QK, bias, mask, blank token, softmax, AV) of one block at a stage's shape on
     lists built by the model's clustering, with the plan of the stage; microseconds per call."""
     import torch
     import workloads as wl
     from clusten import _native
 
-    mcase = wl.attn_case("model", 29, B=B, H=H, N=N, C=32, lists="model_built").to("cuda")
-    cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()
+    mcase = wl.attn_case("model", 29, B=B, H=H, N=N, C=32, M=6 * cluster, lists="random")
+    mcase.nbhd_idx = wl.model_built_lists(B, N, wl.generator(29), cluster=cluster, nnc=6)
+    mcase = mcase.to("cuda")
+    cidx = (mcase.nbhd_idx[:, :, ::cluster] // cluster).to(torch.int32).contiguous()
     gen = torch.Generator().manual_seed(1029)
     rows = 111 * 111
     q, k, v = (t.to(dtype) for t in (mcase.query, mcase.key, mcase.value))
     table = torch.randn(rows, H, generator=gen).to(dtype).cuda()
-    pe_idx = torch.randint(rows, (B, N, 48), generator=gen).cuda()
+    pe_idx = torch.randint(rows, (B, N, 6 * cluster), generator=gen).cuda()
     blank_k, blank_v = torch.randn(H * 32, generator=gen).cuda(), torch.randn(H * 32, generator=gen).cuda()
     plan = _native.cluster_attention_plan(cidx, pe_idx, None)
     _, per, _, per_min = _time_kernels([lambda: _native.cluster_attention(q, k, v, None, table, None, None, blank_k,
                                                                           blank_v, plan=plan)], steps, warmup)
     nbytes = 4 * q.numel() * q.element_size() + plan.numel()
-    return {"shape": "B%d H%d N%d C32 M48 %s, model-built lists, planned" % (B, H, N, str(dtype).replace("torch.", "")),
+    return {"shape": "B%d H%d N%d C32 M%d %s, model-built lists, planned" % (B, H, N, 6 * cluster,
+                                                                            str(dtype).replace("torch.", "")),
             "median_us": round(per[0] * 1e3, 1), "min_us": round(per_min[0] * 1e3, 1),
             "bytes_q_k_v_out_plan": nbytes, "GBps": round(nbytes / per[0] / 1e6, 1)}
 
@@ -473,6 +476,8 @@ def main():
                     help="headline only: leave out the other configurations and the GEMM tuning of the images/s leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs (the baseline and configuration 0)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the AFF-Tiny images/s leg")
+    ap.add_argument("--no-parity", action="store_true",
+                    help="skip the parity leg (its small launches would enter a profiler's per-kernel averages)")
     ap.add_argument("--e2e-only", action="store_true", help="run just the AFF-Tiny images/s leg")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
@@ -480,7 +485,7 @@ def main():
                     help="batch size of the --only wf-cfg3* / ca-* profiler legs (default: the configuration's own)")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model", "replay-qk", "replay-av", "replay-wf",
                                        "interference", "wf-cfg3", "wf-cfg3-f32", "ca-s1-f16", "ca-s1-f32", "ca-s2-f16",
-                                       "ca-s3-f16"),
+                                       "ca-s3-f16", "ca-384-f16"),
                     default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
@@ -508,6 +513,11 @@ def main():
         dt = torch.bfloat16 if args.only == "wf-cfg3" else torch.float32
         print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
                           **_bench_wf(wl.config3_wf(dtype=dt, B=args.batch or 64), args.steps, args.warmup)}), flush=True)
+        return
+    if args.only == "ca-384-f16":   # ... at the first stage of a 384 x 384 model: clusters of 24, 144 neighbours
+        print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
+                          **_bench_local_attention(args.batch or 16, 4, 9216, torch.float16, args.steps, args.warmup,
+                                                   cluster=24)}), flush=True)
         return
     if args.only and args.only.startswith("ca-"):   # the one-kernel local attention at a stage's shape, with its plan
         stage, dt = int(args.only[4]), (torch.float16 if args.only.endswith("f16") else torch.float32)
@@ -608,7 +618,7 @@ def main():
                      "lowest_kernel": {"kernel": names[low], "frac": kernels[low]["frac_of_hbm_peak"],
                                        "achieved": kernels[low]["achieved_GBps"]}},
         "kernels": kernels,
-        "parity": _parity(acase, wcase, attn, (q, k, v, idx), dw),
+        "parity": None if args.no_parity else _parity(acase, wcase, attn, (q, k, v, idx), dw),
         "replay_probe": {"what": "the same kernels compiled without their matrix instructions (same global loads, LDS "
                                  "accesses and stores; libclusten_probe.so), timed in the same interleaved pass",
                          "kernels": [{"kernel": n, "replay_us": round(r * 1e3, 2), "kernel_us": round(t * 1e3, 2),
@@ -740,6 +750,36 @@ def main():
             c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
             c384.nbhd_idx = wl.model_built_lists(16, 9216, gen384, cluster=24, nnc=6)
             other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
+            if dt == torch.bfloat16:
+                # local attention of one block of that stage under mixed precision: one kernel (clusters of 24 as
+                # three runs of 8) against what the model ran before it existed - QK on the 144-slot lists, the
+                # softmax kernel (fp32 probabilities), the cast of v that clusten/clusten.py:52-53 makes, AV in fp32
+                d384 = c384.to("cuda")
+                g2 = torch.Generator().manual_seed(1031)
+                rows384 = 191 * 191                          # offsets between two tokens of a 96 x 96 grid
+                table384 = torch.randn(rows384, 4, generator=g2).to(dt).cuda()
+                pe384 = torch.randint(rows384, (16, 9216, 144), generator=g2).cuda()
+                bk384, bv384 = torch.randn(128, generator=g2).cuda(), torch.randn(128, generator=g2).cuda()
+                cidx24 = (d384.nbhd_idx[:, :, ::24] // 24).to(torch.int32).contiguous()
+                plan384 = _native.cluster_attention_plan(cidx24, pe384, None)
+
+                def three_kernels_384():
+                    a = _native.qk_forward(d384.query, d384.key, d384.nbhd_idx)
+                    p, pb = _native.attn_softmax(a, table384, pe384, None, query=d384.query, blank_key=bk384)
+                    return _native.av_forward(p, d384.value.float(), d384.nbhd_idx)
+
+                _, per_x, _, _ = _time_kernels(
+                    [lambda: _native.cluster_attention(d384.query, d384.key, d384.value, cidx24, table384, pe384, None,
+                                                       bk384, bv384),
+                     three_kernels_384,
+                     lambda: _native.cluster_attention(d384.query, d384.key, d384.value, None, table384, None, None,
+                                                       bk384, bv384, plan=plan384)], max(args.steps // 2, 5), 5)
+                fb = 4 * d384.query.numel() * 2 + cidx24.numel() * 4 + pe384.numel() * 8
+                other["aff_base_384_stage1_local_attention_bf16_model_lists"] = {
+                    "one_kernel_us": round(per_x[0] * 1e3, 1), "three_kernels_us": round(per_x[1] * 1e3, 1),
+                    "one_kernel_with_plan_us": round(per_x[2] * 1e3, 1), "one_kernel_algorithmic_bytes": fb,
+                    "one_kernel_GBps": round(fb / per_x[0] / 1e6, 1)}
+                del d384, table384, pe384, cidx24, plan384
             if dt == torch.float32:
                 # merge lists of the same stage: the 144-slot lists of every fourth token, 9216 -> 2304 tokens, C = 128
                 w384 = wl.wf_case("aff_base_384_wf", 32, B=16, N=9216, C=128, M=144)

@@ -723,6 +723,37 @@ def test_recorded_forward_replays_equal_the_eager_forward(device):
 
 
 @pytest.mark.gpu
+def test_aff_tiny_224_at_the_benchmarked_batch_equals_the_small_batch(device):
+    """The images/s figure is taken at batch 128, where the grid stage hands over one image's lists for the whole batch,
+    the Linear layers of stage 1 go through the library's kernel and the forward is replayed from a HIP graph.  The
+    logits of images 0 and 1 inside that batch equal those of a batch of just the two (itself checked against the
+    oracle model above) within the mixed-precision tolerance, eager and replayed; the replay equals eager bit for bit."""
+    from aff.model import CapturedForward
+    torch.manual_seed(0)
+    net = aff_tiny().to(device).eval()
+    x = torch.randn(128, 3, 224, 224, generator=torch.Generator().manual_seed(6)).to(device)
+
+    def eager(inp):
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+            return net(inp)
+
+    small = eager(x[:2]).float()
+    big = eager(x)
+    assert big.shape == (128, 1000) and torch.isfinite(big).all()
+    assert oracle.rel_err(big[:2].float(), small) < 2e-2
+    recorded = CapturedForward(net, x)
+    for _ in range(2):
+        replayed = recorded(x).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, big)
+    assert oracle.rel_err(replayed[:2].float(), small) < 2e-2
+    # every image of the batch is its own problem: a permutation of the batch permutes the logits
+    perm = torch.randperm(128, generator=torch.Generator().manual_seed(7)).to(device)
+    assert oracle.rel_err(eager(x[perm]).float(), big[perm].float()) < 2e-2
+    del recorded
+
+
+@pytest.mark.gpu
 def test_aff_tiny_224_forward_and_gradients(device):
     model = aff_tiny().to(device)
     x = torch.randn(2, 3, 224, 224, device=device)
