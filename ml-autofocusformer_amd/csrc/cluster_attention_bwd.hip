@@ -2,8 +2,9 @@
 // one kernel, with the probabilities recomputed from the saved logarithm of each softmax's denominator.
 //
 // With  x[t,j] = scale * q[t].k[row(t,j)] + bias[t,j] - 100 * (1 - mask[t,j]),  p = exp(x - lse),  p_b = exp(x_b - lse)
-// (x_b = scale * q[t].blank_k), and  delta[t] = sum_c d_out[t,c] * out[t,c]  (= sum_j p[t,j] dP[t,j] + p_b[t] dP_b[t]: a
-// tile whose distinct clusters fit one pass forms it that way, without the rounding of `out` to 16 bits) :
+// (x_b = scale * q[t].blank_k), and  delta[t] = sum_c d_out[t,c] * out[t,c]  (= sum_j p[t,j] dP[t,j] + p_b[t] dP_b[t]: the
+// kernel forms it that way, without the rounding of `out` to 16 bits - inside its one pass, or in a sweep of its own
+// ahead of the passes for a tile that needs several) :
 //   dP[t,j]   = d_out[t] . v[row(t,j)]              dP_b[t]  = d_out[t] . blank_v
 //   dS[t,j]   = p[t,j] * (dP[t,j] - delta[t])       dS_b[t]  = p_b[t] * (dP_b[t] - delta[t])
 //   d_q[t]    = scale * (sum_j dS[t,j] * k[row(t,j)] + dS_b[t] * blank_k)
@@ -176,8 +177,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
         lds_sync_vm<0>();   // the rows of this head's first pass, its q and d_out rows, the operands above
 
         // per token: delta = d_out . out, the blank token's logit, probability and logit gradient.  (delta also equals
-        // sum_j p_j dP_j + p_b dP_b; a tile whose clusters fit one pass takes it from there, below: the rounding of
-        // `out` to 16 bits does not enter then.)
+        // sum_j p_j dP_j + p_b dP_b and is replaced by that sum below: the rounding of `out` to 16 bits does not enter.)
         float delta, p_b, ds_b, dpb_t;
         {
             float o4[4], g4[4], q4[4];
@@ -190,6 +190,52 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
             p_b = __expf(bl - lse_t);
             ds_b = p_b * (dpb - delta);
             dpb_t = dpb;
+        }
+
+        if (passes > 1) {
+            // A tile whose clusters take several passes: a first sweep over the passes forms only S and dP and adds up
+            // p * dP, so that delta is the same fp32 sum a one-pass tile uses and does not depend on the 16-bit rounding
+            // of `out` either (such tiles are rare on lists like the model's: more than 12 distinct clusters among the
+            // 48 a tile names; they pay their rows twice).
+            float pdp = 0.f;
+            for (int pass = 0; pass < passes; ++pass) {
+                const int rows_here = min(kPassRows, total_rows - pass * kPassRows);
+                if (pass > 0) lds_sync_vm<0>();  // the K and V rows of this pass are in LDS
+                const Piece qraw = *reinterpret_cast<const Piece*>(q_lds + (r16 & 7) * kRB + kq * 16);
+                const Piece graw = *reinterpret_cast<const Piece*>(g_lds + (r16 & 7) * kRB + kq * 16);
+#pragma unroll
+                for (int blk = 0; blk < kBlocks; ++blk) {
+                    if (blk * 16 < rows_here) {
+                        const Piece kraw = *reinterpret_cast<const Piece*>(stage + K_BASE + (blk * 16 + r16) * kRB + kq * 16);
+                        const Piece vraw = *reinterpret_cast<const Piece*>(stage + V_BASE + (blk * 16 + r16) * kRB + kq * 16);
+                        const F32x4 s = tile_mfma<T>(kraw, qraw, F32x4{0.f, 0.f, 0.f, 0.f});
+                        const F32x4 d = tile_mfma<T>(vraw, graw, F32x4{0.f, 0.f, 0.f, 0.f});
+                        if (r16 < kTileTokens) {
+                            *reinterpret_cast<F32x4*>(stage + S_BASE + (r16 * kSRow + 16 * blk + 4 * kq) * 4) = s;
+                            *reinterpret_cast<F32x4*>(stage + S2_BASE + (r16 * kSRow + 16 * blk + 4 * kq) * 4) = d;
+                        }
+                    }
+                }
+                lds_sync();
+#pragma unroll
+                for (int r = 0; r < kR; ++r) {
+                    const unsigned u = (unsigned)(us[r] - pass * kPassRuns);
+                    const int cell = (t * kSRow + (int)min(u, (unsigned)kPassRuns - 1) * 8 + i) * 4;
+                    const float sc = *reinterpret_cast<const float*>(stage + S_BASE + cell);
+                    const float dp = *reinterpret_cast<const float*>(stage + S2_BASE + cell);
+                    pdp += u < (unsigned)kPassRuns ? __expf(sc * scale + bias[r] - lse_t) * dp : 0.f;
+                }
+                lds_sync();  // rows and scores have been read: the next pass's rows, or the first pass's again
+                const int nxt = pass + 1 < passes ? pass + 1 : 0;
+                uint32_t rr[kAccesses];
+                pass_rows(nxt, rr);
+                const int next_rows = min(kPassRows, total_rows - nxt * kPassRows);
+                gather(k_bh, k_pitch, rr, next_rows, K_BASE);
+                gather(v_bh, v_pitch, rr, next_rows, V_BASE);
+            }
+            delta = oct_sum(pdp) + p_b * dpb_t;
+            ds_b = p_b * (dpb_t - delta);
+            lds_sync_vm<0>();   // the rows of the first pass are back
         }
 
         float p_all[kR], ds_all[kR];
