@@ -583,6 +583,22 @@ def main():
         torch.cuda.synchronize()
     _, per_replay, _, _ = _time_kernels(replay_fns, k_steps, k_warm)
     torch.cuda.synchronize()
+    # The same step over three sets of tensors taken in turn (lists included), so that no launch finds anything of the
+    # step before it in the 256 MB memory-side cache.  Within a step QK and AV share their lists, as in an attention layer.
+    sets = [(q, k, v, idx, attn, dw.weights, dw.feat, dw.nbhd_idx)]
+    for _ in range(2):
+        sets.append(tuple(t.clone() for t in sets[0]))
+    turn = [0]
+
+    def _next_set():
+        turn[0] += 1
+
+    rot_fns = [lambda: _native.qk_forward(sets[turn[0] % 3][0], sets[turn[0] % 3][1], sets[turn[0] % 3][3]),
+               lambda: _native.av_forward(sets[turn[0] % 3][4], sets[turn[0] % 3][2], sets[turn[0] % 3][3]),
+               lambda: (_native.wf_forward(sets[turn[0] % 3][5], sets[turn[0] % 3][6], sets[turn[0] % 3][7]), _next_set())]
+    rot_ms, rot_per, _, _ = _time_kernels(rot_fns, k_steps, k_warm)
+    torch.cuda.synchronize()
+    del sets[1:]
 
     names = ("gather_dot_tile_kernel (QK)", "gather_sum_tile_kernel (AV)", "wf_forward_row_kernel (WF)")
     kbytes = (qk_bytes, qk_bytes, wf_bytes)
@@ -618,6 +634,10 @@ def main():
                      "lowest_kernel": {"kernel": names[low], "frac": kernels[low]["frac_of_hbm_peak"],
                                        "achieved": kernels[low]["achieved_GBps"]}},
         "kernels": kernels,
+        "rotating_inputs": {"what": "the same step over three sets of tensors taken in turn (lists too): nothing of the "
+                                    "step before is in the memory-side cache; QK and AV of a step share their lists",
+                            "sets": 3, "ms_per_step": round(rot_ms, 4), "GBps": round(total_bytes / rot_ms / 1e6, 1),
+                            "median_us": [round(t * 1e3, 2) for t in rot_per]},
         "parity": None if args.no_parity else _parity(acase, wcase, attn, (q, k, v, idx), dw),
         "replay_probe": {"what": "the same kernels compiled without their matrix instructions (same global loads, LDS "
                                  "accesses and stores; libclusten_probe.so), timed in the same interleaved pass",

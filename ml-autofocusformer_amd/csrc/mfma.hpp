@@ -90,6 +90,16 @@ __device__ __forceinline__ uint32_t lane_offset(uint32_t off) {
 #define CLUSTEN_LDS_DMA16(gptr, lptr)                                                       \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr), \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+// The same for data that is read once, with the non-temporal hint when NT is set (a compile-time 0 / 1).
+#define CLUSTEN_LDS_DMA16_STREAM(gptr, lptr, NT)                                            \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr), \
+                                     (__attribute__((address_space(3))) void*)(lptr), 16, 0, (NT) ? 2 : 0)
+template <bool NT, typename V>
+__device__ __forceinline__ V load_stream(const V* p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+
 
 // D(16x16) += A * B over the channels two lanes hold in one register group of 8 or 16 bytes each: `a` belongs to
 // row lane % 16 of A, `b` to column lane % 16 of B, and lane / 16 selects which quarter of the channel range
