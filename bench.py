@@ -750,6 +750,33 @@ def main():
             "one_kernel_us": round(per_f[0] * 1e3, 1), "three_kernels_us": round(per_f[1] * 1e3, 1),
             "one_kernel_with_plan_us": round(per_f[2] * 1e3, 1),
             "one_kernel_algorithmic_bytes": fused_bytes32, "one_kernel_GBps": round(fused_bytes32 / per_f[0] / 1e6, 1)}
+        # ... and its backward in fp32, against the backward functions of the three operators around the softmax's
+        out32, lse32 = _native.cluster_attention(mcase.query, mcase.key, mcase.value, None, table32, None, None, blank_k,
+                                                 blank_v, plan=plan, return_lse=True)
+        gout32 = torch.randn(out32.shape, generator=gen).cuda()
+        gview32 = gout32.view(B, 3136, 2, 32).permute(0, 2, 1, 3)
+        pairs = _native.cluster_pairs(mcase.nbhd_idx)
+        probs32, pb32 = _native.attn_softmax(_native.qk_forward_clusters(mcase.query, mcase.key, cidx), table32, pe_idx,
+                                             None, query=mcase.query, blank_key=blank_k)
+
+        def fused_backward_fp32():
+            dq, p_, ds_, pb_, dsb_ = _native.cluster_attention_backward(mcase.query, mcase.key, mcase.value, gout32, out32,
+                                                                      lse32, plan, table32, blank_k, blank_v)
+            dv = _native.scatter_rows_by_cluster(p_, gview32, pairs)
+            dk = _native.scatter_rows_by_cluster(ds_, mcase.query, pairs)
+            return _native.bias_table_grad(ds_, pe_idx, rows), dq, dk, dv
+
+        def operator_backward_fp32():
+            d_p, dv = _native.av_backward(gview32, probs32, mcase.value, mcase.nbhd_idx, pairs=pairs)
+            d_logit, d_blank = _native.attn_softmax_backward(probs32, pb32, d_p, torch.zeros_like(pb32), torch.float32)
+            d_table = _native.bias_table_grad(d_logit, pe_idx, rows)
+            return (d_table,) + tuple(_native.qk_backward(d_logit, mcase.query, mcase.key, mcase.nbhd_idx, pairs=pairs)) + (dv,)
+
+        _, per_g, _, _ = _time_kernels([fused_backward_fp32, operator_backward_fp32], max(args.steps // 5, 5), 3)
+        other["cfg2_s1_local_attention_fp32_backward_model_built_lists"] = {
+            "one_kernel_path_us": round(per_g[0] * 1e3, 1), "operator_path_us": round(per_g[1] * 1e3, 1),
+            "what": "d_query, d_key, d_value and the bias table's gradient of one block's local attention, fp32"}
+        del out32, lse32, gout32, gview32, pairs, probs32, pb32
         del mcase, cidx, mattn, q16, k16, v16, pe_idx, plan, table32
         # WF on the lists a merge reads (the members of the nearest clusters of every centre, centres = a sorted
         # quarter of the tokens of a cluster-ordered sequence): consecutive output tokens name mostly the same rows

@@ -313,8 +313,9 @@ int clusten_cluster_attention_forward_train(const void* query, clusten_strides q
  *   d_value = clusten_scatter_rows_by_cluster(probs, d_out),  d_key = scale * clusten_scatter_rows_by_cluster(d_logit, query),
  *   d_bias_table = clusten_bias_table_grad(d_logit),  d_blank_key = scale * sum d_blank_logit * query,
  *   d_blank_value = sum blank_prob * d_out.
- * d_out, out: strided (B,H,N,C) like query (the forward's result and its gradient); dtype F16 or BF16 (else
- * CLUSTEN_ERR_BAD_DTYPE), C = 32, M = 48.  No counterpart in the reference's extension modules. */
+ * d_out, out: strided (B,H,N,C) like query (the forward's result and its gradient); dtype F16, BF16 or F32 (for F32
+ * the bias table is fp32 too, as in the forward), C = 32, M = 48.  No counterpart in the reference's extension
+ * modules. */
 int clusten_cluster_attention_backward(const void* query, clusten_strides query_strides,
                                        const void* key, clusten_strides key_strides,
                                        const void* value, clusten_strides value_strides,

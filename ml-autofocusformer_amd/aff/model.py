@@ -347,7 +347,7 @@ class ClusterAttention(nn.Module):
                 and self.cluster_size == 8 and grid_lists is not None and len(grid_lists) > 4 and not (self.training and self.attn_drop.p > 0)
                 and self.ops.cluster_attention_backward_supported(q.view(b, n, h, ch).permute(0, 2, 1, 3),
                                                                   cluster_idx.shape[2])):
-            # training on 16-bit data: the same kernel forward, one kernel and four sums backward
+            # training: the same kernel forward, one kernel and four sums backward
             bias = self.bias_table(table)
             if bias.shape[0] <= 16000:
                 out = _ClusterAttention.apply(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, bias, self.blank_k,
@@ -642,8 +642,8 @@ class BasicLayer(nn.Module):
         if ((grid_lists is None or len(grid_lists) == 3) and cluster_idx is not None and planner is not None
                 and torch.is_grad_enabled() and getattr(self.ops, "cluster_attention_backward", None) is not None
                 and not global_attn and self.cluster_size == 8 and cluster_idx.shape[2] == 6 and cluster_idx.is_cuda
-                and torch.is_autocast_enabled("cuda")):
-            # training under mixed precision: the plan of the one-kernel attention and the sorted pair lists of its
+                and (torch.is_autocast_enabled("cuda") or feat.dtype == torch.float32)):
+            # training (fp32, or mixed precision): the plan of the one-kernel attention and the sorted pair lists of its
             # backward's scatters, built once for all blocks of the stage (a grid stage hands over one image's lists)
             pairs = self.ops.cluster_pairs(member_idx)
             if pairs is not None:

@@ -878,9 +878,9 @@ def cluster_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tenso
 
 
 def cluster_attention_backward_supported(query: torch.Tensor, nnc: int) -> bool:
-    """True when `cluster_attention_backward` takes this case: CUDA fp16 / bf16 queries of head dim 32, six clusters
-    per token."""
-    return (query.is_cuda and query.dtype in (torch.float16, torch.bfloat16) and query.dim() == 4
+    """True when `cluster_attention_backward` takes this case: CUDA fp32 / fp16 / bf16 queries of head dim 32, six
+    clusters per token."""
+    return (query.is_cuda and query.dtype in (torch.float32, torch.float16, torch.bfloat16) and query.dim() == 4
             and query.shape[3] == 32 and nnc == 6)
 
 
@@ -889,7 +889,7 @@ def cluster_attention_backward(query: torch.Tensor, key: torch.Tensor, value: to
                                blank_key: torch.Tensor, blank_value: torch.Tensor, scale: float = 1.0):
     """The query-side half of the backward of `cluster_attention(..., plan=plan, return_lse=True)` in one kernel.
 
-    query, key, value (B,H,N,32) fp16 / bf16 as in the forward; out (B,N,H*32) its result, d_out the gradient of it,
+    query, key, value (B,H,N,32) fp32 / fp16 / bf16 as in the forward; out (B,N,H*32) its result, d_out the gradient of it,
     lse (B,H,N) fp32 from the forward.  Returns (d_query, probs, d_logit, blank_prob, d_blank_logit): d_query a
     (B,H,N,32) view of (B,N,H,32) memory, probs and d_logit (B,H,N,48) of query's dtype, blank_prob and d_blank_logit
     fp32 (B,H,N).  The other gradients are sums of these: d_value = scatter_rows_by_cluster(probs, d_out),

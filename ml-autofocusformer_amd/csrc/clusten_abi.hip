@@ -275,7 +275,7 @@ int clusten_cluster_attention_backward(const void* query, clusten_strides query_
         !d_query || !probs || !d_logit || !blank_prob || !d_blank_logit) {
         return CLUSTEN_ERR_NULL_POINTER;
     }
-    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
     if (int st = check_attn_shape(shape)) return st;
     if (!strides_ok(query_strides, shape.C) || !strides_ok(key_strides, shape.C) || !strides_ok(value_strides, shape.C) ||
         !strides_ok(d_out_strides, shape.C) || !strides_ok(out_strides, shape.C) || !strides_ok(d_query_strides, shape.C)) {

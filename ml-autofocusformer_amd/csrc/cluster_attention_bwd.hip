@@ -21,10 +21,20 @@
 // pass.  Per pass: S = K q^T and dP = V d_out^T are six 16x16x32 matrix instructions each; every lane picks the scores
 // and dP of its own slots, forms p and dS; dS re-indexed by distinct cluster (as the forward does with p) times the K
 // rows is the query gradient, with the K operand read by `ds_read_b64_tr_b16` from the same row-major rows.
-// 16-bit data (fp16 / bf16), head dim 32, M = 48.
+// 16-bit data (fp16 / bf16), head dim 32, M = 48; fp32 data goes to cluster_attention_bwd_f32.hip.
 #include "cluster_attention_plan.hpp"
 
 namespace clusten {
+
+int launch_cluster_attention_backward_f32(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
+                                          clusten_strides vs, const void* d_out, clusten_strides gs, const void* out,
+                                          clusten_strides os, const float* lse, const int32_t* cluster_idx,
+                                          const void* table, const int64_t* pe_idx, const int64_t* mask,
+                                          const float* blank_k, const float* blank_v, void* d_q, clusten_strides dqs,
+                                          void* probs, void* d_logit, float* p_blank, float* ds_blank, float scale,
+                                          int lists_shared, const void* plan, const clusten_attn_shape& s,
+                                          hipStream_t stream);   // cluster_attention_bwd_f32.hip
+
 namespace {
 
 using namespace ca;
@@ -424,14 +434,20 @@ int launch_cluster_attention_backward(const void* q, clusten_strides qs, const v
                                       const float* blank_v, void* d_q, clusten_strides dqs, void* probs, void* d_logit,
                                       float* p_blank, float* ds_blank, float scale, int lists_shared, const void* plan,
                                       clusten_attn_shape s, int dtype, hipStream_t stream) {
-    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16) return CLUSTEN_ERR_BAD_DTYPE;
+    if (dtype != CLUSTEN_F16 && dtype != CLUSTEN_BF16 && dtype != CLUSTEN_F32) return CLUSTEN_ERR_BAD_DTYPE;
     if (s.C != kC || s.M != kM) return CLUSTEN_ERR_BAD_DIMS;
-    const bool ok = rows_aligned16(q, qs, 2) && rows_aligned16(k, ks, 2) && rows_aligned16(v, vs, 2) &&
-                    rows_aligned16(d_out, gs, 2) && rows_aligned16(out, os, 2) && rows_aligned16(d_q, dqs, 2) &&
+    const int es = dtype == CLUSTEN_F32 ? 4 : 2;
+    const bool ok = rows_aligned16(q, qs, es) && rows_aligned16(k, ks, es) && rows_aligned16(v, vs, es) &&
+                    rows_aligned16(d_out, gs, es) && rows_aligned16(out, os, es) && rows_aligned16(d_q, dqs, es) &&
                     aligned16(probs) && aligned16(d_logit) && aligned16(blank_k) && aligned16(blank_v) &&
                     slice_fits_int32(ks, s.H, s.N, s.C) && slice_fits_int32(vs, s.H, s.N, s.C) &&
                     slice_fits_int32(qs, s.H, s.N, s.C) && slice_fits_int32(gs, s.H, s.N, s.C);
     if (!ok) return CLUSTEN_ERR_UNALIGNED;
+    if (dtype == CLUSTEN_F32) {
+        return launch_cluster_attention_backward_f32(q, qs, k, ks, v, vs, d_out, gs, out, os, lse, cluster_idx, table, pe_idx,
+                                                     mask, blank_k, blank_v, d_q, dqs, probs, d_logit, p_blank, ds_blank,
+                                                     scale, lists_shared, plan, s, stream);
+    }
     if (dtype == CLUSTEN_F16) {
         return launch_typed<f16_t>(q, qs, k, ks, v, vs, d_out, gs, out, os, lse, cluster_idx, table, pe_idx, mask, blank_k,
                                    blank_v, d_q, dqs, probs, d_logit, p_blank, ds_blank, scale, lists_shared, plan, s, stream);

@@ -250,7 +250,9 @@ def test_parameter_gradients_with_the_cluster_by_cluster_backward(device, monkey
     monkeypatch.setattr(_native, "qk_backward", watched("qk", _native.qk_backward, lambda a: None))
     monkeypatch.setattr(_native, "av_backward", watched("av", _native.av_backward, lambda a: None))
     monkeypatch.setattr(_native, "wf_backward", watched("wf", _native.wf_backward, lambda a: a[2].shape[1]))
-    hip = small_model(default_ops(), img_size=128, num_classes=16, embed_dim=embed_dim).to(device).train()
+    ops = dict(vars(default_ops()))
+    ops.pop("cluster_attention_backward")      # the three operators, not the one-kernel attention (head dim 32 would take it)
+    hip = small_model(SimpleNamespace(**ops), img_size=128, num_classes=16, embed_dim=embed_dim).to(device).train()
     ref = small_model(oracle_ops(), img_size=128, num_classes=16, embed_dim=embed_dim).to(device).train()
     ref.load_state_dict(hip.state_dict())
     x = torch.randn(4, 3, 128, 128, generator=torch.Generator().manual_seed(8)).to(device)
@@ -816,12 +818,16 @@ def test_cached_16_bit_weights_follow_the_parameters(device):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("img_size", [128, 120])
-def test_training_with_the_one_kernel_attention_matches_the_operator_path(device, img_size):
-    """A training step under fp16 autocast with the local attention as one kernel forward and `cluster_attention_backward`
-    plus its sums backward, against the same step through the three operators and the softmax kernels: same loss,
-    parameter gradients within the noise of fp16 intermediates.  At 120 x 120 pixels the stages hold 900, 225 and 56
-    tokens: short last clusters, pad slots and masks in every local stage."""
+@pytest.mark.parametrize("amp", [True, False])
+def test_training_with_the_one_kernel_attention_matches_the_operator_path(device, img_size, amp):
+    """A training step (under fp16 autocast, or in fp32) with the local attention as one kernel forward and
+    `cluster_attention_backward` plus its sums backward, against the same step through the three operators and the
+    softmax kernels: same loss, parameter gradients within the noise of fp16 intermediates (fp32: within 1e-3 of the
+    largest entry).  At 120 x 120 pixels the stages hold 900, 225 and 56 tokens: short last clusters, pad slots and
+    masks in every local stage."""
+    import contextlib
     from aff.model import default_ops
+    mode = (lambda: torch.autocast("cuda", dtype=torch.float16)) if amp else contextlib.nullcontext
     fused_ops = default_ops()
     plain = dict(vars(default_ops()))
     plain.pop("cluster_attention_backward")
@@ -834,11 +840,11 @@ def test_training_with_the_one_kernel_attention_matches_the_operator_path(device
     target = torch.tensor([3, 7], device=device)
     losses = []
     for m in (a, b):
-        with torch.autocast("cuda", dtype=torch.float16):
+        with mode():
             loss = torch.nn.functional.cross_entropy(m(x).float(), target)
         loss.backward()
         losses.append(float(loss.detach()))
-    assert abs(losses[0] - losses[1]) <= 2e-2 * max(1.0, abs(losses[1]))
+    assert abs(losses[0] - losses[1]) <= (2e-2 if amp else 1e-5) * max(1.0, abs(losses[1]))
     # a gradient that is pure rounding noise (a bias in front of a batch norm) is measured against the largest gradient
     # of the model, not against itself
     biggest = max(float(p.grad.abs().max()) for p in b.parameters() if p.grad is not None)
@@ -849,11 +855,11 @@ def test_training_with_the_one_kernel_attention_matches_the_operator_path(device
             continue
         scale = max(float(pb.grad.abs().max()), 1e-2 * biggest)
         err = float((pa.grad - pb.grad).abs().max()) / scale
-        assert err <= 5e-2, "%s rel err %.3g" % (name, err)
+        assert err <= (5e-2 if amp else 1e-3), "%s rel err %.3g" % (name, err)
         checked += 1
     assert checked > 50
     # the fused path was taken: its Function is in the graph of a fresh forward
-    with torch.autocast("cuda", dtype=torch.float16):
+    with mode():
         y = a(x)
     seen, stack = set(), [y.grad_fn]
     while stack:

@@ -285,7 +285,7 @@ def _reference_grads(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale,
 
 
 @pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_backward_against_autograd_through_the_composition(device, kind, dtype):
     """`cluster_attention_backward` (d_query, the recomputed probabilities and the logit gradients in one kernel) with
     the sums that complete it - the scatters over sorted pair lists, the bias table's gradient, the blank token's -
