@@ -7,13 +7,10 @@
 // value, all of them on the same few hundred kilobytes.  Here a workgroup takes one head and a contiguous slice of the
 // head's values (images one after the other) and sums into a copy of that head's column of the table in LDS (LDS
 // atomics; at most 16 000 rows); what it has collected goes to memory with one global atomic per touched row.
-// The grid is about a thousand workgroups of 512 threads: the global atomics of the flush all land on the same few
-// kilobytes, so a workgroup should flush once for a long slice, and a column of 12 000 rows is 48 KB of LDS, so few
-// workgroups fit a compute unit and each has to bring many waves.  A thread reads four consecutive values at a time
-// (two 16-byte loads of indices, one load of gradients) and keeps four such groups in flight.  What bounds the kernel
-// is the rate of the fp32 LDS atomics, about one every three cycles per compute unit whatever the rows are (38.5 M
-// values: 205 us in fp32 and fp16, over 3000 or 12 321 rows, uniform or clustered; the same loop with integer atomics
-// takes 73 us on fp16 values).
+// The grid is one round of workgroups of 512 threads (768 to 1024 of them): the global atomics of the flush all land
+// on the same few kilobytes, so a workgroup should flush once for a long slice, and a column of 12 000 rows is 48 KB
+// of LDS, so few workgroups fit a compute unit and each has to bring many waves.  A thread reads four consecutive values at a time
+// (two 16-byte loads of indices, one load of gradients) and keeps four such groups in flight.
 // d_table is fp32 and zeroed by the caller.  It has no counterpart in the reference's extension modules.
 #include "launch.hpp"
 
@@ -34,6 +31,7 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
     typedef typename RawBytes<VEC == 4 ? 16 : 8>::type IdxRaw;   // two indices (VEC = 4: a group is two of them) or one
     constexpr int IR = VEC == 4 ? 2 : 1;
     extern __shared__ float col[];   // rows floats
+    uint32_t* cells = reinterpret_cast<uint32_t*>(col);
     const int h = blockIdx.y;
     for (int r = threadIdx.x; r < rows; r += kGradThreads) col[r] = 0.f;
     __syncthreads();
@@ -66,14 +64,33 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
         }
 #pragma unroll
         for (int k = 0; k < kGradGroups; ++k) {
+            // The values are added by compare-and-swap on the cells' bits (an fp32 LDS atomic add takes some 190 cycles
+            // per wave instruction here, a compare-and-swap a few): the group's cells are read, then swapped, and only
+            // the lanes that lost a race go round again.
+            float x[VEC];
+            uint32_t cell[VEC], seen[VEC];
+            uint32_t open = 0;          // bit v: the value still has to reach its cell
             if (in[k]) {
-                float x[VEC];
                 GIO::unpack(g[k], x);
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
                     // the index as two 32-bit words: a row is below 2^31
                     const uint32_t lo32 = raw_word(r[k][v / 2], 2 * (v % 2)), hi32 = raw_word(r[k][v / 2], 2 * (v % 2) + 1);
-                    if (hi32 == 0u && lo32 < (uint32_t)rows) atomicAdd(&col[lo32], x[v]);
+                    const bool ok = hi32 == 0u && lo32 < (uint32_t)rows;
+                    cell[v] = ok ? lo32 : 0u;
+                    seen[v] = ok ? cells[cell[v]] : 0u;
+                    open |= ok ? 1u << v : 0u;
+                }
+            }
+            while (open != 0) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    if ((open >> v & 1u) != 0) {
+                        const uint32_t expect = seen[v];
+                        const uint32_t sum = __float_as_uint(__uint_as_float(expect) + x[v]);
+                        seen[v] = atomicCAS(cells + cell[v], expect, sum);
+                        if (seen[v] == expect) open &= ~(1u << v);
+                    }
                 }
             }
         }
@@ -90,14 +107,17 @@ void launch_typed(const void* d_logit, const int64_t* pe_idx, float* d_table, in
                   hipStream_t stream) {
     const bool wide = per_image % 4 == 0 && aligned16(d_logit) && aligned16(pe_idx);
     const int vec = wide ? 4 : 1;
-    // about 1024 workgroups in all, and no slice shorter than 16 000 values
+    // one round of workgroups: as many as fit the 256 compute units at once (4 of 512 threads each, fewer when the
+    // column takes more than a quarter of a unit's 160 KB of LDS), and no slice shorter than 16 000 values
+    const size_t lds_bytes = (size_t)rows * sizeof(float);
+    const int per_unit = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / max(lds_bytes, (size_t)1)));
     const int64_t total = per_image / vec * B;
     const int64_t want = (total * vec + 16383) / 16384;
-    const int64_t cap = max(1, 1024 / H);
+    const int64_t cap = max(1, 256 * per_unit / H);
     const int slices = (int)max((int64_t)1, min(want, cap));
     const int64_t per_slice = (total + slices - 1) / slices;
     const dim3 grid((unsigned)slices, (unsigned)H);
-    const size_t lds = (size_t)rows * sizeof(float);
+    const size_t lds = lds_bytes;
     if (wide) {
         hipLaunchKernelGGL((bias_table_grad_kernel<T, 4>), grid, dim3(kGradThreads), lds, stream,
                            static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, per_image, per_slice, B);
