@@ -574,7 +574,12 @@ def main():
         print(json.dumps({"only": args.only, "launches": args.steps + args.warmup, "avg_us": round(per[0] * 1e3, 2),
                           "algorithmic_bytes": nbytes, "achieved_GBps": round(nbytes / per[0] / 1e6, 1)}), flush=True)
         return
-    # throughput: exactly --steps steps after --warmup untimed ones; per-kernel figures: at least 10 + 50 launches
+    # throughput: exactly --steps steps after --warmup untimed ones; per-kernel figures: at least 10 + 50 launches.
+    # A process that has just started runs its first few tens of milliseconds of kernels some 5 % slower (the device's
+    # clocks are still rising), so the same measurement is taken twice: `cold_start` is the one right after start-up,
+    # `value` the one that follows it, with the device in the state a training or serving loop keeps it in.
+    cold_ms, _, _, _ = _time_kernels(fns, args.steps, args.warmup)
+    torch.cuda.synchronize()
     ms_per_step, per, wall_ms, per_min = _time_kernels(fns, args.steps, args.warmup)
     torch.cuda.synchronize()
     k_steps, k_warm = max(args.steps, 50), max(args.warmup, 10)
@@ -634,6 +639,8 @@ def main():
                      "lowest_kernel": {"kernel": names[low], "frac": kernels[low]["frac_of_hbm_peak"],
                                        "achieved": kernels[low]["achieved_GBps"]}},
         "kernels": kernels,
+        "cold_start": {"what": "the same --warmup + --steps measurement taken first, right after the process started",
+                       "ms_per_step": round(cold_ms, 4), "GBps": round(total_bytes / cold_ms / 1e6, 1)},
         "rotating_inputs": {"what": "the same step over three sets of tensors taken in turn (lists too): nothing of the "
                                     "step before is in the memory-side cache; QK and AV of a step share their lists",
                             "sets": 3, "ms_per_step": round(rot_ms, 4), "GBps": round(total_bytes / rot_ms / 1e6, 1),
