@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # runs of `bench.py --only {qk,av,wf}`, each counter scaled by what it reads for the copy probe of known
 # size; see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md, which names the source revision the
 # counters were read at.  A constant of that run, not a measurement of this one: TRAFFIC_MEASURED says when.
-MEASURED_TRAFFIC_BYTES = {"qk": 359.59e6 + 154.14e6, "av": 410.97e6 + 102.76e6, "wf": 219.49e6 + 102.76e6}
+MEASURED_TRAFFIC_BYTES = {"qk": 359.59e6 + 154.14e6, "av": 411.70e6 + 102.76e6, "wf": 218.48e6 + 102.76e6}
 TRAFFIC_MEASURED = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/pmc_hbm_traffic_qk_av_wf_tiny_stage1.md"
 
 
