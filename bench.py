@@ -804,6 +804,17 @@ def main():
             c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
             c384.nbhd_idx = wl.model_built_lists(16, 9216, gen384, cluster=24, nnc=6)
             other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
+            if dt == torch.float32:
+                # the same lists as (B,N,6) int32 numbers of clusters of 24 rows instead of (B,N,144) int64 rows
+                dn = c384.to("cuda")
+                cn = (dn.nbhd_idx[:, :, ::24] // 24).to(torch.int32).contiguous()
+                pn = torch.softmax(_native.qk_forward(dn.query, dn.key, dn.nbhd_idx), dim=-1)
+                _, per_n, _, _ = _time_kernels([lambda: _native.qk_forward_clusters(dn.query, dn.key, cn, cluster_size=24),
+                                                lambda: _native.av_forward_clusters(pn, dn.value, cn, cluster_size=24)],
+                                               max(args.steps // 2, 5), 5)
+                other["aff_base_384_stage1_model_lists_fp32_as_cluster_numbers"] = {
+                    "qk_us": round(per_n[0] * 1e3, 1), "av_us": round(per_n[1] * 1e3, 1)}
+                del dn, cn, pn
             if dt == torch.bfloat16:
                 # local attention of one block of that stage under mixed precision: one kernel (clusters of 24 as
                 # three runs of 8) against what the model ran before it existed - QK on the 144-slot lists, the

@@ -207,10 +207,17 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
  * themselves, as int32 — 1/16 of the bytes — and compute exactly what clusten_qk_forward /
  * clusten_av_forward compute on the expanded lists:
  *     nbhd_idx[b,i,8*r+t] = 8*cluster_idx[b,i,r]+t   if that is < N,   else 0.
- * shape.M = 8 * nnc (a multiple of 8, at most 64).  Tile kernels only: dtype F32/F16/BF16, head dim
- * 16/32/64 (else CLUSTEN_ERR_BAD_DIMS), rows 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).  Forward only:
+ * shape.M = 8 * nnc (a multiple of 8, at most 64).  Longer lists are lists of larger clusters: for 64 < M <= 256 the
+ * cluster size is L = clusten_cluster_size_for(M) (24 if M is a multiple of 24 of at most 8 clusters, else 32, else
+ * 16 by the same rule: M = 144 is the 6 clusters of 24 tokens of the 384 x 384 configurations,
+ * configs/aff_base_22kto1k_384.yaml:10-11), cluster_idx is (B,N,M/L) and
+ *     nbhd_idx[b,i,L*r+t] = L*cluster_idx[b,i,r]+t   if that is < N,   else 0
+ * (a cluster number whose first row is outside [0,N) stands for L slots of row 0).
+ * Tile kernels only: dtype F32/F16/BF16, head dim 16/32/64 (for M > 64: rows of at least 64 bytes), else
+ * CLUSTEN_ERR_BAD_DIMS; rows 16-byte aligned (else CLUSTEN_ERR_UNALIGNED).  Forward only:
  * for training expand the lists and use the functions above.  No counterpart in the reference's extension
  * modules. */
+int clusten_cluster_size_for(int M);   /* 8 for M <= 64 (M % 8 == 0), L as above for 64 < M <= 256, 0 otherwise */
 int clusten_qk_forward_clusters(const void* query, clusten_strides query_strides,
                                 const void* key, clusten_strides key_strides,
                                 const int32_t* cluster_idx, void* attn,

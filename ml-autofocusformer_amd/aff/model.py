@@ -326,7 +326,8 @@ class ClusterAttention(nn.Module):
         ch = c // h
         # inference: the neighbourhoods as (b,n,nnc) cluster numbers instead of the expanded (b,n,m*nnc) row lists
         numbered = cluster_idx is not None and not global_attn and not torch.is_grad_enabled()
-        compact = numbered and self.cluster_size == 8 and getattr(self.ops, "qk_clusters", None) is not None
+        compact = numbered and getattr(self.ops, "qk_clusters", None) is not None
+        sized = {} if self.cluster_size == 8 else {"cluster_size": self.cluster_size}
         q, kv = _linear_pair(self.q, self.kv, feat, self.ops)
         kv = kv.view(b, n, h, 2, ch).permute(3, 0, 2, 1, 4)                                                 # (2,b,h,n,ch) view
         key, v = kv[0], kv[1]
@@ -365,8 +366,8 @@ class ClusterAttention(nn.Module):
         q = (q * self.scale).reshape(b, n, h, ch).permute(0, 2, 1, 3)                    # (b,h,n,ch) view
         if global_attn:
             attn = q @ key.transpose(-1, -2)                                             # (b,h,n,n)
-        elif compact and self.ops.clusters_supported(q, cluster_idx.shape[2]):
-            attn = self.ops.qk_clusters(q, key, cluster_idx)                             # (b,h,n,m)
+        elif compact and self.ops.clusters_supported(q, cluster_idx.shape[2], **sized):
+            attn = self.ops.qk_clusters(q, key, cluster_idx, **sized)                    # (b,h,n,m)
         else:
             compact = False
             attn = self.ops.qk(q, key, member_idx)                                       # (b,h,n,m)
@@ -397,7 +398,7 @@ class ClusterAttention(nn.Module):
         if global_attn:
             out = attn @ v
         elif compact:
-            out = self.ops.av_clusters(attn, v, cluster_idx)
+            out = self.ops.av_clusters(attn, v, cluster_idx, **sized)
         else:
             out = self.ops.av(attn, v, member_idx)                                       # (b,h,n,ch)
         out = out + blank * self.blank_v.reshape(1, h, 1, ch)

@@ -50,6 +50,7 @@ _PROTOTYPES = {
     "clusten_wf_forward_mixed": (ctypes.c_int, [_P, _P, ctypes.c_int, _P, _P, WfShape, _P]),
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
+    "clusten_cluster_size_for": (ctypes.c_int, [ctypes.c_int]),
     "clusten_qk_forward_clusters": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_av_forward_clusters": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
@@ -592,10 +593,15 @@ def wf_backward_by_cluster(d_feat_new: torch.Tensor, weights: torch.Tensor, feat
     return d_weights, d_feat
 
 
-def clusters_supported(a: torch.Tensor, nnc: int) -> bool:
-    """True when the cluster-number entry points take this case (head dim 16/32/64, at most 8 clusters per token)."""
-    return (a.is_cuda and a.dtype in (torch.float32, torch.float16, torch.bfloat16) and a.shape[3] in (16, 32, 64)
-            and 1 <= nnc <= 8)
+def clusters_supported(a: torch.Tensor, nnc: int, cluster_size: int = 8) -> bool:
+    """True when the cluster-number entry points take this case: head dim 16/32/64, at most 8 clusters per token, of 8
+    rows or of the size `cluster_size_for` gives their slot count (24 for 144 slots; rows of at least 64 bytes there)."""
+    if not (a.is_cuda and a.dtype in (torch.float32, torch.float16, torch.bfloat16) and a.shape[3] in (16, 32, 64)
+            and 1 <= nnc <= 8):
+        return False
+    if cluster_size == 8:
+        return True
+    return cluster_size_for(cluster_size * nnc) == cluster_size and a.shape[3] * a.element_size() >= 64
 
 
 def _cluster_idx(cluster_idx: torch.Tensor, shape, device) -> torch.Tensor:
@@ -605,8 +611,23 @@ def _cluster_idx(cluster_idx: torch.Tensor, shape, device) -> torch.Tensor:
     return cluster_idx.contiguous()
 
 
-def qk_forward_clusters(query: torch.Tensor, key: torch.Tensor, cluster_idx: torch.Tensor) -> torch.Tensor:
-    """qk_forward on nbhd_idx[b,i,8r+t] = 8*cluster_idx[b,i,r]+t (0 where that is >= N), without building it."""
+def cluster_size_for(m: int) -> int:
+    """The cluster size the cluster-number forms read a list of m slots in (0: no such form)."""
+    return int(load().clusten_cluster_size_for(int(m)))
+
+
+def _clusters_slots(cidx: torch.Tensor, cluster_size: int) -> int:
+    m = cluster_size * cidx.shape[2]
+    if cluster_size_for(m) != cluster_size:
+        raise RuntimeError("lists of %d clusters of %d rows are not taken by the cluster-number forms" %
+                           (cidx.shape[2], cluster_size))
+    return m
+
+
+def qk_forward_clusters(query: torch.Tensor, key: torch.Tensor, cluster_idx: torch.Tensor,
+                        cluster_size: int = 8) -> torch.Tensor:
+    """qk_forward on nbhd_idx[b,i,L*r+t] = L*cluster_idx[b,i,r]+t (0 where that is >= N), without building it;
+    L = `cluster_size` (8, or the cluster size `cluster_size_for(L * clusters per token)` names: 24 for 144 slots)."""
     lib = load()
     _require_cuda("query", query)
     device = query.device
@@ -615,7 +636,7 @@ def qk_forward_clusters(query: torch.Tensor, key: torch.Tensor, cluster_idx: tor
         raise RuntimeError("query and key must be (B,H,N,C) tensors of one dtype")
     B, H, N, C = query.shape
     cidx = _cluster_idx(cluster_idx, (B, N), device)
-    shape = AttnShape(B, H, N, C, 8 * cidx.shape[2])
+    shape = AttnShape(B, H, N, C, _clusters_slots(cidx, cluster_size))
     query, key = _rows(query), _rows(key)
     attn = torch.empty((B, H, N, shape.M), dtype=query.dtype, device=device)
     if attn.numel() == 0:
@@ -627,7 +648,8 @@ def qk_forward_clusters(query: torch.Tensor, key: torch.Tensor, cluster_idx: tor
     return attn
 
 
-def av_forward_clusters(attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.Tensor) -> torch.Tensor:
+def av_forward_clusters(attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.Tensor,
+                        cluster_size: int = 8) -> torch.Tensor:
     """av_forward on the lists qk_forward_clusters describes; v is cast to attn's dtype like the AV Function does."""
     lib = load()
     _require_cuda("attn", attn)
@@ -635,9 +657,10 @@ def av_forward_clusters(attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.
     _require_cuda("v", v, device)
     B, H, N, C = v.shape
     cidx = _cluster_idx(cluster_idx, (B, N), device)
-    if tuple(attn.shape) != (B, H, N, 8 * cidx.shape[2]):
-        raise RuntimeError("attn must be (B,H,N,8 * clusters per token)")
-    shape = AttnShape(B, H, N, C, 8 * cidx.shape[2])
+    m = _clusters_slots(cidx, cluster_size)
+    if tuple(attn.shape) != (B, H, N, m):
+        raise RuntimeError("attn must be (B,H,N,cluster size * clusters per token)")
+    shape = AttnShape(B, H, N, C, m)
     attn, v = attn.contiguous(), _rows(v.to(attn.dtype))
     feat = torch.empty((B, H, N, C), dtype=attn.dtype, device=device)
     if feat.numel() == 0:

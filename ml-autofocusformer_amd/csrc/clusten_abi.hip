@@ -152,6 +152,8 @@ int clusten_wf_backward(const void* d_feat_new, const void* weights, const void*
     return launch_wf_dfeat(d_feat_new, weights, nbhd_idx, d_feat, workspace, shape, dtype, as_stream(stream));
 }
 
+int clusten_cluster_size_for(int M) { return cluster_size_for(M); }
+
 int clusten_qk_forward_clusters(const void* query, clusten_strides query_strides, const void* key,
                                 clusten_strides key_strides, const int32_t* cluster_idx, void* attn,
                                 clusten_attn_shape shape, int dtype, clusten_stream stream) {

@@ -17,6 +17,11 @@ int gather_dot_clusters_f16(const void*, clusten_strides, const void*, clusten_s
 int gather_dot_clusters_bf16(const void*, clusten_strides, const void*, clusten_strides, const int32_t*, void*,
                              const clusten_attn_shape&, hipStream_t);
 
+int cluster_size_for(int M) {
+    if (M > 0 && M <= 64 && M % 8 == 0) return 8;
+    return runs_length_for(M);
+}
+
 int launch_gather_dot_clusters(const void* a, clusten_strides as, const void* rows, clusten_strides rs,
                                const int32_t* cluster_idx, void* out, clusten_attn_shape s, int dtype,
                                hipStream_t stream) {

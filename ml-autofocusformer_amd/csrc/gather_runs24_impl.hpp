@@ -45,9 +45,11 @@ struct Runs24Staging {
 // The runs of the nt <= 24 tokens of a tile (R <= 8 runs of 24 each): distinct runs numbered in order of first
 // appearance, their rows listed (ulist: 24 per distinct run), inv[token * U_MAX + number] = run of the token.
 // Returns the number of distinct runs, or -1 when the tile is not for this path.
+// `cid_tile` != nullptr: the lists as cluster numbers (R per token, int32; run r of a token = rows 24 c .. 24 c + 23, row
+// 0 where that is outside [0, N)); nothing is read from `idx_tile` then.
 template <int U_MAX>
-__device__ __forceinline__ int number_runs24(const int64_t* __restrict__ idx_tile, int nt, int M, int R, int N, int* ulist,
-                                             unsigned char* inv) {
+__device__ __forceinline__ int number_runs24(const int64_t* __restrict__ idx_tile, const int32_t* __restrict__ cid_tile,
+                                             int nt, int M, int R, int N, int* ulist, unsigned char* inv) {
     typedef long long I64x2 __attribute__((ext_vector_type(2)));
     constexpr int L = kRun24;
     const int lane = threadIdx.x;
@@ -60,6 +62,11 @@ __device__ __forceinline__ int number_runs24(const int64_t* __restrict__ idx_til
         const int nruns = ntg * R;
         live[g] = lane < nruns;
         const int rho = min(lane, max(nruns, 1) - 1);
+        if (cid_tile != nullptr) {
+            const int64_t first = (int64_t)cid_tile[(kTileTokens * min(g, (nt - 1) / kTileTokens) + rho / R) * R + rho % R] * L;
+            key[g] = (first >= 0 && first < N) ? (int)first : -1;   // a run outside the sequence: 24 times row 0
+            continue;
+        }
         const int64_t* run = idx_tile + (int64_t)(kTileTokens * min(g, (nt - 1) / kTileTokens) + rho / R) * M + (rho % R) * L;
         I64x2 two[12];
 #pragma unroll
@@ -124,7 +131,7 @@ __device__ __forceinline__ int number_runs24(const int64_t* __restrict__ idx_til
         }
         if (first[g] && live[g]) {   // consecutive rows from key[g] on; past the end of the sequence: row 0
 #pragma unroll
-            for (int t = 0; t < L; ++t) ulist[uslot[g] * L + t] = key[g] + t < N ? key[g] + t : 0;
+            for (int t = 0; t < L; ++t) ulist[uslot[g] * L + t] = (key[g] >= 0 && key[g] + t < N) ? key[g] + t : 0;
         }
     }
     return U;
@@ -134,7 +141,8 @@ __device__ __forceinline__ int number_runs24(const int64_t* __restrict__ idx_til
 
 template <typename T, int C>
 __global__ __launch_bounds__(kWave) void gather_sum_runs24_kernel(const T* __restrict__ p, const T* __restrict__ rows,
-                                                                  const int64_t* __restrict__ idx, T* __restrict__ out, int H,
+                                                                  const int64_t* __restrict__ idx,
+                                                                  const int32_t* __restrict__ cid, T* __restrict__ out, int H,
                                                                   int N, int M, clusten_strides rs, clusten_strides os,
                                                                   int tiles_per_batch, int total_tiles) {
     typedef Runs24Staging<T, C> S;
@@ -158,10 +166,11 @@ __global__ __launch_bounds__(kWave) void gather_sum_runs24_kernel(const T* __res
     float* weights = reinterpret_cast<float*>(stage + S::S_BASE);   // p of the pass by union row: [token][SROW]
     float* chunk = reinterpret_cast<float*>(stage + S::A_BASE);     // the tile's output rows, fp32: 24 x C
 
-    const int U = number_runs24<S::U_MAX>(idx + ((int64_t)b * N + i0) * M, nt, M, R, N, ulist, inv);
+    const int U = number_runs24<S::U_MAX>(idx + ((int64_t)b * N + i0) * M,
+                                          cid != nullptr ? cid + ((int64_t)b * N + i0) * R : nullptr, nt, M, R, N, ulist, inv);
     if (U < 0) {
         for (int g = 0; g * kTileTokens < nt; ++g) {
-            gather_sum_runs_tokens<T, C>(stage, p, rows, idx, out, H, N, M, L, rs, os, b, i0 + g * kTileTokens,
+            gather_sum_runs_tokens<T, C>(stage, p, rows, idx, cid, out, H, N, M, L, rs, os, b, i0 + g * kTileTokens,
                                          min(kTileTokens, nt - g * kTileTokens));
         }
         return;
@@ -289,23 +298,24 @@ __global__ __launch_bounds__(kWave) void gather_sum_runs24_kernel(const T* __res
 
 template <typename T, int C>
 int launch_gather_sum_runs24_c(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
-                               clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
+                               clusten_strides os, const clusten_attn_shape& s, hipStream_t stream, const int32_t* cid) {
     const int tiles_per_batch = (s.N + kTile24 - 1) / kTile24;
     const int total = s.B * tiles_per_batch;
     hipLaunchKernelGGL((gather_sum_runs24_kernel<T, C>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
-                       static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N, s.M, rs, os,
-                       tiles_per_batch, total);
+                       static_cast<const T*>(p), static_cast<const T*>(rows), idx, cid, static_cast<T*>(out), s.H, s.N, s.M, rs,
+                       os, tiles_per_batch, total);
     return launch_status();
 }
 
 template <typename T>
 int launch_gather_sum_runs24(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
-                             clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
+                             clusten_strides os, const clusten_attn_shape& s, hipStream_t stream,
+                             const int32_t* cid = nullptr) {
     if constexpr (sizeof(T) == 4) {
-        if (s.C == 16) return launch_gather_sum_runs24_c<T, 16>(p, rows, rs, idx, out, os, s, stream);
+        if (s.C == 16) return launch_gather_sum_runs24_c<T, 16>(p, rows, rs, idx, out, os, s, stream, cid);
     }
-    if (s.C == 32) return launch_gather_sum_runs24_c<T, 32>(p, rows, rs, idx, out, os, s, stream);
-    return launch_gather_sum_runs24_c<T, 64>(p, rows, rs, idx, out, os, s, stream);
+    if (s.C == 32) return launch_gather_sum_runs24_c<T, 32>(p, rows, rs, idx, out, os, s, stream, cid);
+    return launch_gather_sum_runs24_c<T, 64>(p, rows, rs, idx, out, os, s, stream, cid);
 }
 
 }  // namespace clusten

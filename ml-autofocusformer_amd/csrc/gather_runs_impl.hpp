@@ -59,13 +59,39 @@ struct RunsStaging {
 // The runs of tokens [t0, t0 + ntok) of a tile: distinct runs numbered, their rows listed in LDS.  Returns the number
 // of distinct runs, or -1 when there are more than U_MAX.  `uslots[rho]` = number of run rho (token-major), `ulist` =
 // L rows per distinct run.
+// `cid_tokens` != nullptr: the lists are given as cluster numbers instead (R per token, int32): run r of a token is rows
+// L c .. L c + L - 1 of the sequence, row 0 where that is outside [0, N) — every run is regular by construction and
+// nothing is read from `idx_tokens`.
 template <int U_MAX>
-__device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_tokens, int ntok, int M, int L, int R, int N,
-                                           int* ulist, int* uslots) {
+__device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_tokens, const int32_t* __restrict__ cid_tokens,
+                                           int ntok, int M, int L, int R, int N, int* ulist, int* uslots) {
     typedef long long I64x2 __attribute__((ext_vector_type(2)));
     const int lane = threadIdx.x;
     const int nruns = ntok * R;
     const int rho = min(lane, nruns - 1);
+    if (cid_tokens != nullptr) {
+        const int64_t first = (int64_t)cid_tokens[rho] * L;
+        const int key = (first >= 0 && first < N) ? (int)first : -1;   // runs outside the sequence: L times row 0
+        uint64_t remaining = nruns >= 64 ? ~0ull : ((1ull << nruns) - 1);
+        int uslot = 0, U = 0;
+        bool lead = false;
+        while (remaining != 0 && U < U_MAX) {
+            const int s = __builtin_ctzll(remaining);
+            const int ks = __builtin_amdgcn_readlane(key, s);
+            const bool hit = key == ks;
+            const uint64_t match = __ballot(hit) & remaining;
+            if (hit) uslot = U;
+            lead = lead || lane == s;
+            remaining &= ~match;
+            ++U;
+        }
+        if (remaining != 0) return -1;
+        if (lead && lane < nruns) {
+            for (int t = 0; t < L; ++t) ulist[uslot * L + t] = (key >= 0 && key + t < N) ? key + t : 0;
+        }
+        if (lane < nruns) uslots[lane] = uslot;
+        return U;
+    }
     const int64_t* run = idx_tokens + (int64_t)(rho / R) * M + (rho % R) * L;
     const int v0 = (int)run[0];
     // L consecutive rows, or the short last cluster of the sequence followed by the row 0 its pad slots hold?
@@ -134,9 +160,9 @@ __device__ __forceinline__ int number_runs(const int64_t* __restrict__ idx_token
 // Tokens [i0, i0 + nt) (nt <= 8) of batch element b, all heads; `stage`: RunsStaging<T, C>::BYTES bytes of LDS.
 template <typename T, int C>
 __device__ __forceinline__ void gather_dot_runs_tokens(char* stage, const T* __restrict__ a, const T* __restrict__ rows,
-                                                       const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
-                                                       int M, int L, clusten_strides as, clusten_strides rs, int b, int i0,
-                                                       int nt) {
+                                                       const int64_t* __restrict__ idx, const int32_t* __restrict__ cid,
+                                                       T* __restrict__ out, int H, int N, int M, int L, clusten_strides as,
+                                                       clusten_strides rs, int b, int i0, int nt) {
     typedef RunsStaging<T, C> S;
     typedef VecIO<T, S::VEC> PieceIO;
     typedef VecIO<T, 4> OutIO;
@@ -155,7 +181,9 @@ __device__ __forceinline__ void gather_dot_runs_tokens(char* stage, const T* __r
     int ntok = nt;
     for (int t0 = 0; t0 < nt;) {
         lds_sync();
-        const int U = number_runs<S::U_MAX>(idx + ((int64_t)b * N + i0 + t0) * M, ntok, M, L, R, N, ulist, uslots);
+        const int U = number_runs<S::U_MAX>(idx + ((int64_t)b * N + i0 + t0) * M,
+                                            cid != nullptr ? cid + ((int64_t)b * N + i0 + t0) * R : nullptr, ntok, M, L, R, N,
+                                            ulist, uslots);
         if (U < 0) {   // more distinct runs than the tables hold: one token at a time (at most R <= 8 runs)
             ntok = 1;
             continue;
@@ -292,14 +320,15 @@ __device__ __forceinline__ void gather_dot_runs_tokens(char* stage, const T* __r
 
 template <typename T, int C>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ? 3 : 1))) void gather_dot_runs_kernel(
-    const T* __restrict__ a, const T* __restrict__ rows, const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
-    int M, int L, clusten_strides as, clusten_strides rs, int tiles_per_batch, int total_tiles) {
+    const T* __restrict__ a, const T* __restrict__ rows, const int64_t* __restrict__ idx, const int32_t* __restrict__ cid,
+    T* __restrict__ out, int H, int N, int M, int L, clusten_strides as, clusten_strides rs, int tiles_per_batch,
+    int total_tiles) {
     __shared__ __attribute__((aligned(1024))) char stage[RunsStaging<T, C>::BYTES];
     const int tile = xcd_tile(blockIdx.x, total_tiles);
     if (tile < 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
-    gather_dot_runs_tokens<T, C>(stage, a, rows, idx, out, H, N, M, L, as, rs, b, i0, min(kTileTokens, N - i0));
+    gather_dot_runs_tokens<T, C>(stage, a, rows, idx, cid, out, H, N, M, L, as, rs, b, i0, min(kTileTokens, N - i0));
 }
 
 // ---- gather_sum ----------------------------------------------------------------------------------------------------
@@ -307,9 +336,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(C <= 32 ?
 // Tokens [i0, i0 + nt) (nt <= 8) of batch element b, all heads; `stage`: RunsStaging<T, C>::BYTES bytes of LDS.
 template <typename T, int C>
 __device__ __forceinline__ void gather_sum_runs_tokens(char* stage, const T* __restrict__ p, const T* __restrict__ rows,
-                                                       const int64_t* __restrict__ idx, T* __restrict__ out, int H, int N,
-                                                       int M, int L, clusten_strides rs, clusten_strides os, int b, int i0,
-                                                       int nt) {
+                                                       const int64_t* __restrict__ idx, const int32_t* __restrict__ cid,
+                                                       T* __restrict__ out, int H, int N, int M, int L, clusten_strides rs,
+                                                       clusten_strides os, int b, int i0, int nt) {
     typedef RunsStaging<T, C> S;
     typedef VecIO<T, 4> OutIO;
     constexpr int CB = C / 16;   // channel blocks of 16
@@ -328,7 +357,9 @@ __device__ __forceinline__ void gather_sum_runs_tokens(char* stage, const T* __r
     int ntok = nt;
     for (int t0 = 0; t0 < nt;) {
         lds_sync();
-        const int U = number_runs<S::U_MAX>(idx + ((int64_t)b * N + i0 + t0) * M, ntok, M, L, R, N, ulist, uslots);
+        const int U = number_runs<S::U_MAX>(idx + ((int64_t)b * N + i0 + t0) * M,
+                                            cid != nullptr ? cid + ((int64_t)b * N + i0 + t0) * R : nullptr, ntok, M, L, R, N,
+                                            ulist, uslots);
         if (U < 0) {   // more distinct runs than the tables hold: one token at a time (at most R <= 8 runs)
             ntok = 1;
             continue;
@@ -429,7 +460,8 @@ __device__ __forceinline__ void gather_sum_runs_tokens(char* stage, const T* __r
 
 template <typename T, int C>
 __global__ __launch_bounds__(kWave) void gather_sum_runs_kernel(const T* __restrict__ p, const T* __restrict__ rows,
-                                                                const int64_t* __restrict__ idx, T* __restrict__ out,
+                                                                const int64_t* __restrict__ idx,
+                                                                const int32_t* __restrict__ cid, T* __restrict__ out,
                                                                 int H, int N, int M, int L, clusten_strides rs,
                                                                 clusten_strides os, int tiles_per_batch, int total_tiles) {
     __shared__ __attribute__((aligned(1024))) char stage[RunsStaging<T, C>::BYTES];
@@ -437,7 +469,7 @@ __global__ __launch_bounds__(kWave) void gather_sum_runs_kernel(const T* __restr
     if (tile < 0) return;
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
-    gather_sum_runs_tokens<T, C>(stage, p, rows, idx, out, H, N, M, L, rs, os, b, i0, min(kTileTokens, N - i0));
+    gather_sum_runs_tokens<T, C>(stage, p, rows, idx, cid, out, H, N, M, L, rs, os, b, i0, min(kTileTokens, N - i0));
 }
 
 // ---- launch ----------------------------------------------------------------------------------------------------------
@@ -459,44 +491,46 @@ constexpr bool runs_head_dim_ok(int C) {
 
 template <typename T, int C>
 int launch_gather_dot_runs_c(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
-                             void* out, const clusten_attn_shape& s, int L, hipStream_t stream) {
+                             void* out, const clusten_attn_shape& s, int L, hipStream_t stream, const int32_t* cid) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     hipLaunchKernelGGL((gather_dot_runs_kernel<T, C>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
-                       static_cast<const T*>(a), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N, s.M, L, as,
-                       rs, tiles_per_batch, total);
+                       static_cast<const T*>(a), static_cast<const T*>(rows), idx, cid, static_cast<T*>(out), s.H, s.N, s.M, L,
+                       as, rs, tiles_per_batch, total);
     return launch_status();
 }
 
+// `cid` != nullptr: the lists as cluster numbers, (B, N, M / L) int32 (see number_runs); `idx` is not read then.
 template <typename T>
 int launch_gather_dot_runs(const void* a, clusten_strides as, const void* rows, clusten_strides rs, const int64_t* idx,
-                           void* out, const clusten_attn_shape& s, int L, hipStream_t stream) {
+                           void* out, const clusten_attn_shape& s, int L, hipStream_t stream, const int32_t* cid = nullptr) {
     if constexpr (sizeof(T) == 4) {
-        if (s.C == 16) return launch_gather_dot_runs_c<T, 16>(a, as, rows, rs, idx, out, s, L, stream);
+        if (s.C == 16) return launch_gather_dot_runs_c<T, 16>(a, as, rows, rs, idx, out, s, L, stream, cid);
     }
-    if (s.C == 32) return launch_gather_dot_runs_c<T, 32>(a, as, rows, rs, idx, out, s, L, stream);
-    return launch_gather_dot_runs_c<T, 64>(a, as, rows, rs, idx, out, s, L, stream);
+    if (s.C == 32) return launch_gather_dot_runs_c<T, 32>(a, as, rows, rs, idx, out, s, L, stream, cid);
+    return launch_gather_dot_runs_c<T, 64>(a, as, rows, rs, idx, out, s, L, stream, cid);
 }
 
 template <typename T, int C>
 int launch_gather_sum_runs_c(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
-                             clusten_strides os, const clusten_attn_shape& s, int L, hipStream_t stream) {
+                             clusten_strides os, const clusten_attn_shape& s, int L, hipStream_t stream, const int32_t* cid) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
     hipLaunchKernelGGL((gather_sum_runs_kernel<T, C>), dim3(xcd_grid(total)), dim3(kWave), 0, stream,
-                       static_cast<const T*>(p), static_cast<const T*>(rows), idx, static_cast<T*>(out), s.H, s.N, s.M, L, rs,
-                       os, tiles_per_batch, total);
+                       static_cast<const T*>(p), static_cast<const T*>(rows), idx, cid, static_cast<T*>(out), s.H, s.N, s.M, L,
+                       rs, os, tiles_per_batch, total);
     return launch_status();
 }
 
 template <typename T>
 int launch_gather_sum_runs(const void* p, const void* rows, clusten_strides rs, const int64_t* idx, void* out,
-                           clusten_strides os, const clusten_attn_shape& s, int L, hipStream_t stream) {
+                           clusten_strides os, const clusten_attn_shape& s, int L, hipStream_t stream,
+                           const int32_t* cid = nullptr) {
     if constexpr (sizeof(T) == 4) {
-        if (s.C == 16) return launch_gather_sum_runs_c<T, 16>(p, rows, rs, idx, out, os, s, L, stream);
+        if (s.C == 16) return launch_gather_sum_runs_c<T, 16>(p, rows, rs, idx, out, os, s, L, stream, cid);
     }
-    if (s.C == 32) return launch_gather_sum_runs_c<T, 32>(p, rows, rs, idx, out, os, s, L, stream);
-    return launch_gather_sum_runs_c<T, 64>(p, rows, rs, idx, out, os, s, L, stream);
+    if (s.C == 32) return launch_gather_sum_runs_c<T, 32>(p, rows, rs, idx, out, os, s, L, stream, cid);
+    return launch_gather_sum_runs_c<T, 64>(p, rows, rs, idx, out, os, s, L, stream, cid);
 }
 
 }  // namespace clusten

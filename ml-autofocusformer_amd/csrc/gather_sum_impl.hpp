@@ -666,14 +666,19 @@ int launch_elem(const void* p, const void* rows, clusten_strides rs, const int64
     return launch_status();
 }
 
-// Lists given as cluster numbers (see CLUSTERS above): `cluster_idx` is (B, N, M/8) int32.  Only the tile kernels
-// take this format: head dim 16/32/64, M a multiple of 8 up to 64, 16-byte aligned rows.
+// Lists given as cluster numbers (see CLUSTERS above): `cluster_idx` is (B, N, M/8) int32 for M <= 64 (clusters of 8)
+// and (B, N, M/L) for longer lists, L = runs_length_for(M) the cluster size (24 for the 144 slots of the 384 x 384
+// models).  Only the tile kernels take this format: head dim 16/32/64, 16-byte aligned rows.
 template <typename T>
 int gather_sum_clusters_typed(const void* p, const void* rows, clusten_strides rs, const int32_t* cluster_idx, void* out,
                               clusten_strides os, const clusten_attn_shape& s, hipStream_t stream) {
     const bool quads_ok = ((int64_t)s.M * sizeof(T)) % 16 == 0 && aligned16(p) && rows_aligned16(rows, rs, sizeof(T)) &&
                           rows_aligned16(out, os, sizeof(T)) && slice_fits_int32(rs, s.H, s.N, s.C);
     if (!quads_ok) return CLUSTEN_ERR_UNALIGNED;
+    if (const int L = runs_length_for(s.M); L != 0 && runs_head_dim_ok<T>(s.C)) {
+        if (L == kRun24) return launch_gather_sum_runs24<T>(p, rows, rs, nullptr, out, os, s, stream, cluster_idx);
+        return launch_gather_sum_runs<T>(p, rows, rs, nullptr, out, os, s, L, stream, cluster_idx);
+    }
     if (s.M % 8 != 0 || s.M > 64) return CLUSTEN_ERR_BAD_DIMS;
     const int64_t* idx = reinterpret_cast<const int64_t*>(cluster_idx);
     switch (s.C) {

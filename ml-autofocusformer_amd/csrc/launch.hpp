@@ -33,6 +33,9 @@ int launch_gather_sum(const void* p, const void* rows, clusten_strides rows_stri
 int launch_gather_sum_mixed(const void* p, const void* rows, clusten_strides rows_strides, const int64_t* idx, void* out,
                             clusten_strides out_strides, clusten_attn_shape s, int rows_dtype, hipStream_t stream);
 
+// Cluster size the cluster-number forms read a list of M slots in: 8 up to 64 slots, then the run length of the kernels
+// for long runs (24, 32 or 16; gather_runs_impl.hpp), 0 when M is neither.
+int cluster_size_for(int M);
 // The same with the lists given as cluster numbers (see launch_gather_dot_clusters).
 int launch_gather_sum_clusters(const void* p, const void* rows, clusten_strides rows_strides, const int32_t* cluster_idx,
                                void* out, clusten_strides out_strides, clusten_attn_shape s, int dtype,

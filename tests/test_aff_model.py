@@ -208,6 +208,14 @@ def test_clusters_of_24_with_144_neighbours_as_in_the_384_models(device, amp):
         return one_kernel(q, *a, **k)
 
     ops.cluster_attention = counted
+    numbered_calls = []
+    qk_numbers = ops.qk_clusters
+
+    def counted_numbers(q, k, cidx, **k2):
+        numbered_calls.append((q.shape[2], cidx.shape[2], k2.get("cluster_size", 8)))
+        return qk_numbers(q, k, cidx, **k2)
+
+    ops.qk_clusters = counted_numbers
     hip = small_model(ops, **kw).to(device)
     ref = small_model(oracle_ops(), **kw).to(device)
     ref.load_state_dict(hip.state_dict())
@@ -220,7 +228,8 @@ def test_clusters_of_24_with_144_neighbours_as_in_the_384_models(device, amp):
         # under mixed precision the local attention of the first two stages (1 + 2 blocks) ran as one kernel each
         assert [s[2] for s in fused_calls] == [2304, 576, 576] and all(s[3] == 32 for s in fused_calls)
         return
-    assert not fused_calls      # fp32 data: clusters of 24 go through the three operators
+    # fp32 data: clusters of 24 go through the three operators, in inference on (b,n,6) cluster numbers
+    assert not fused_calls and numbered_calls == [(2304, 6, 24), (576, 6, 24), (576, 6, 24)]
     hip.train(), ref.train()
     target = torch.randn(2, 12, generator=torch.Generator().manual_seed(18)).to(device)
     for model in (hip, ref):

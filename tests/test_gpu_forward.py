@@ -376,6 +376,57 @@ def test_lists_given_as_cluster_numbers(device, kind, dtype):
         _native.qk_forward_clusters(q.to(device), k.to(device), cidx.long().to(device))
 
 
+def _cluster_numbers_of(b, n, nnc, cs, gen, kind):
+    """(B,N,nnc) int32 numbers of clusters of `cs` rows; tokens of one cluster pick theirs from the same dozen."""
+    k = (n + cs - 1) // cs
+    own = torch.arange(n) // cs
+    if kind == "shared":
+        per_cluster = torch.stack([torch.randperm(k, generator=gen)[:nnc] for _ in range(b * k)]).reshape(b, k, nnc)
+        return per_cluster[:, own].to(torch.int32).contiguous()
+    width = k if kind == "scattered" else min(9, k)
+    lo = torch.zeros(n, dtype=torch.int64) if kind == "scattered" else (own - width // 2).clamp(0, k - width)
+    pick = torch.rand(b, n, width, generator=gen).argsort(dim=2)[:, :, :nnc] + lo.view(1, n, 1)
+    return pick.to(torch.int32).contiguous()
+
+
+@pytest.mark.parametrize("kind", ["near", "shared", "scattered", "outside"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_long_lists_given_as_numbers_of_larger_clusters(device, kind, dtype):
+    """The cluster-number forms on lists of more than 64 slots: clusters of 24 rows (6 of them: the 144 slots of the
+    384 x 384 models), of 32 and of 16, against the oracle and against the row-list entry points on the expanded lists
+    (bit for bit: same kernels, same order of sums).  A short last cluster, tiles of 20 tokens, and cluster numbers
+    whose rows lie outside the sequence (they stand for row 0)."""
+    gen = torch.Generator().manual_seed(72)
+    for n, c, nnc, cs in ((596, 32, 6, 24), (240, 64, 6, 24), (300, 32, 4, 32), (212, 32, 5, 16), (148, 32, 4, 24)):
+        b, h = 2, 3
+        q = (torch.randn(b, h, n, c, generator=gen) * c ** -0.5).to(dtype)
+        k = torch.randn(b, h, n, c, generator=gen).to(dtype)
+        v = torch.randn(b, h, n, c, generator=gen).to(dtype)
+        assert _native.cluster_size_for(cs * nnc) == cs
+        cidx = _cluster_numbers_of(b, n, nnc, cs, gen, "near" if kind == "outside" else kind)
+        if kind == "outside":
+            far = torch.rand(b, n, nnc, generator=gen) < 0.1
+            cidx = torch.where(far, torch.full_like(cidx, (n + cs - 1) // cs + 3), cidx)
+            cidx[:, ::17, 0] = -2
+        rows = cidx.long().unsqueeze(3) * cs + torch.arange(cs)
+        idx = torch.where((rows >= 0) & (rows < n), rows, torch.zeros_like(rows)).reshape(b, n, cs * nnc).contiguous()
+        qr, kr, vr = _ref_inputs(q, k, v)
+        attn_ref = oracle.qk_gather_chunked(qr, kr, idx)
+        attn = _native.qk_forward_clusters(q.to(device), k.to(device), cidx.to(device), cluster_size=cs)
+        what = "%s %s n=%d c=%d %dx%d" % (kind, dtype, n, c, nnc, cs)
+        assert attn.dtype == dtype and oracle.rel_err(attn, attn_ref) <= TOL[dtype], what
+        p = torch.softmax(attn_ref, dim=-1).to(dtype)
+        feat_ref = oracle.av_gather_chunked(_ref_inputs(p)[0], vr, idx)
+        feat = _native.av_forward_clusters(p.to(device), v.to(device), cidx.to(device), cluster_size=cs)
+        assert feat.dtype == dtype and oracle.rel_err(feat, feat_ref) <= TOL[dtype], what
+        assert oracle.rel_err(attn, _native.qk_forward(q.to(device), k.to(device), idx.to(device)).cpu()) <= TOL[dtype], what
+        assert oracle.rel_err(feat, _native.av_forward(p.to(device), v.to(device), idx.to(device)).cpu()) <= TOL[dtype], what
+    assert _native.clusters_supported(q.to(device), 6, 24) and not _native.clusters_supported(q.to(device), 9, 24)
+    assert not _native.clusters_supported(q.to(device), 6, 20)
+    with pytest.raises(RuntimeError):   # 6 clusters of 20 rows: no such form
+        _native.qk_forward_clusters(q.to(device), k.to(device), cidx.to(device)[:, :, :6].contiguous(), cluster_size=20)
+
+
 def test_empty_inputs_give_empty_or_zero_outputs(device):
     # no batch elements, no tokens, or empty lists: nothing is launched
     for b, n, m in ((0, 16, 8), (2, 0, 8), (2, 16, 0)):
