@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define CLUSTEN_ABI_VERSION 3
+#define CLUSTEN_ABI_VERSION 4
 
 /* Element type of every floating-point tensor of a call.  The reference dispatches
  * double / float / half (AT_DISPATCH_FLOATING_TYPES_AND_HALF, clustenqk_cuda_kernel.cu:78);

@@ -14,7 +14,7 @@ import torch
 
 _LIB_PATH = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "lib", "libclusten_hip.so"))
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
 
