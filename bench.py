@@ -285,11 +285,20 @@ def _bench_backward(acase, wcase, steps, warmup):
     d_feat = torch.randn_like(q)
     d_out = torch.randn(w.weights.shape[0], w.weights.shape[1], w.weights.shape[3], w.feat.shape[2],
                         dtype=w.feat.dtype, device="cuda")
-    _, per, _, _ = _time_kernels([lambda: _native.qk_backward(d_attn, q, k, idx),
-                               lambda: _native.av_backward(d_feat, attn, v, idx),
-                               lambda: _native.wf_backward(d_out, w.weights, w.feat, w.nbhd_idx)], steps, warmup)
-    return {"qk_backward_us": round(per[0] * 1e3, 1), "av_backward_us": round(per[1] * 1e3, 1),
-            "wf_backward_us": round(per[2] * 1e3, 1)}
+    pairs = _native.cluster_pairs(idx)     # what a harness builds once per stage and hands to every layer's backward
+    fns = [lambda: _native.qk_backward(d_attn, q, k, idx),
+           lambda: _native.av_backward(d_feat, attn, v, idx),
+           lambda: _native.wf_backward(d_out, w.weights, w.feat, w.nbhd_idx)]
+    if pairs is not None:
+        fns += [lambda: _native.qk_backward(d_attn, q, k, idx, pairs=pairs),
+                lambda: _native.av_backward(d_feat, attn, v, idx, pairs=pairs)]
+    _, per, _, _ = _time_kernels(fns, steps, warmup)
+    out = {"qk_backward_us": round(per[0] * 1e3, 1), "av_backward_us": round(per[1] * 1e3, 1),
+           "wf_backward_us": round(per[2] * 1e3, 1)}
+    if pairs is not None:
+        out["qk_backward_with_the_callers_pair_lists_us"] = round(per[3] * 1e3, 1)
+        out["av_backward_with_the_callers_pair_lists_us"] = round(per[4] * 1e3, 1)
+    return out
 
 
 def _bench_wf(case, steps, warmup):

@@ -33,21 +33,16 @@
 
 namespace clusten {
 
+// One tile of 8 tokens (all heads) of the atomic scatter.
 template <typename T, int C, int Q, bool GUARD>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void scatter_rows_tile_kernel(
-    const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out, int H,
-    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles, const int32_t* __restrict__ only_if,
-    const uint8_t* __restrict__ handled) {
+__device__ __forceinline__ void scatter_rows_tile(const T* __restrict__ p, const T* __restrict__ x,
+                                                  const int64_t* __restrict__ idx, float* __restrict__ out, int H, int N,
+                                                  int M, clusten_strides xs, int tiles_per_batch, int tile) {
     constexpr int HPW = kWave / C;
     constexpr int SLOTS = 16 * Q;
     static_assert(C == 16 || C == 32 || C == 64, "a row of 16 lanes must stay inside one head");
     static_assert(!GUARD || Q == 4, "guarded lists are taken 64 slots at a time");
     typedef typename Quad<T>::raw QuadRaw;
-
-    if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
-    const int tile = xcd_tile(blockIdx.x, total_tiles);
-    if (tile < 0) return;
-    if (handled != nullptr && handled[tile] != 0) return;   // the window kernel has added this tile
     {
     const int b = tile / tiles_per_batch;
     const int i0 = (tile - b * tiles_per_batch) * kTileTokens;
@@ -245,6 +240,34 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void
     }
 }
 
+constexpr int kScatterGroupTiles = 8;   // tiles of a workgroup when most tiles are expected to be skipped
+
+// A workgroup takes `group` consecutive tiles: 1 when this kernel has every tile, kScatterGroupTiles when the window
+// kernel ran first and left one byte per tile in `handled` (non-zero: added there).  With lists shared by the tokens of
+// a tile nothing is left for this kernel, and a launch of one workgroup per tile costs 12 us at 50 000 tiles just for
+// its waves to start and read their byte; a group's eight bytes are read with one load and the grid is an eighth.
+template <typename T, int C, int Q, bool GUARD>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4))) void scatter_rows_tile_kernel(
+    const T* __restrict__ p, const T* __restrict__ x, const int64_t* __restrict__ idx, float* __restrict__ out, int H,
+    int N, int M, clusten_strides xs, int tiles_per_batch, int total_tiles, int group, int total_groups,
+    const int32_t* __restrict__ only_if, const uint8_t* __restrict__ handled) {
+    if (only_if != nullptr && *only_if == 0) return;   // the cluster-by-cluster kernel has these lists
+    const int g = xcd_tile(blockIdx.x, total_groups);
+    if (g < 0) return;
+    const int tile0 = g * group;
+    const int lane = threadIdx.x;
+    const int mine = tile0 + lane;
+    bool open = lane < group && mine < total_tiles;
+    if (open && handled != nullptr) open = handled[mine] == 0;   // the window kernel has added the others
+    uint64_t todo = __ballot(open);
+    while (todo != 0) {
+        const int k = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        __syncthreads();   // the LDS tables of the tile before have been read
+        scatter_rows_tile<T, C, Q, GUARD>(p, x, idx, out, H, N, M, xs, tiles_per_batch, tile0 + k);
+    }
+}
+
 // One thread per (b,h,i,c); loops over the list with one atomic per product.  Any dtype whose
 // accumulation type A has a hardware atomic add (float, double).
 template <typename T, typename A>
@@ -274,10 +297,11 @@ int scatter_tile_q(const void* p, const void* x, clusten_strides xs, const int64
                    const clusten_attn_shape& s, hipStream_t stream, const int32_t* only_if, const uint8_t* handled) {
     const int tiles_per_batch = (s.N + kTileTokens - 1) / kTileTokens;
     const int total = s.B * tiles_per_batch;
-    const int grid = xcd_grid(total);
-    hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(grid), dim3(kWave), 0, stream,
+    const int group = handled != nullptr ? kScatterGroupTiles : 1;
+    const int groups = (total + group - 1) / group;
+    hipLaunchKernelGGL((scatter_rows_tile_kernel<T, C, Q, GUARD>), dim3(xcd_grid(groups)), dim3(kWave), 0, stream,
                        static_cast<const T*>(p), static_cast<const T*>(x), idx, out, s.H, s.N, s.M, xs,
-                       tiles_per_batch, total, only_if, handled);
+                       tiles_per_batch, total, group, groups, only_if, handled);
     return launch_status();
 }
 
