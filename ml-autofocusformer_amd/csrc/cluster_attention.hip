@@ -408,7 +408,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
         if (lane < 32 && g_sub < nt) {
             const Piece o = *reinterpret_cast<const Piece*>(stage + O_BASE + lane * 16);
             char* dst = reinterpret_cast<char*>(out + (int64_t)b * os.b + (int64_t)(h0 + h) * os.h + (int64_t)(i0 + g_sub) * os.n);
-            store_streaming(reinterpret_cast<Piece*>(dst + g_pos * 16), o);
+            *reinterpret_cast<Piece*>(dst + g_pos * 16) = o;   // plain: the output projection reads it next
         }
     }
 }

@@ -220,7 +220,8 @@ __global__ __launch_bounds__(kWave) void dense_attention_kernel(
         const int row = 16 * a + g_sub;
         if (row < N) {
             const Piece o = *reinterpret_cast<const Piece*>(stage + O_BASE + a * 1024 + lane * 16);
-            store_streaming(reinterpret_cast<Piece*>(out_bh + (int64_t)row * os.n * 2 + g_pos * 16), o);
+            // plain store: the output projection reads it next
+            *reinterpret_cast<Piece*>(out_bh + (int64_t)row * os.n * 2 + g_pos * 16) = o;
         }
     }
 }

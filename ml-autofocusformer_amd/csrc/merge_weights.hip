@@ -25,10 +25,7 @@ __global__ __launch_bounds__(256) void merge_weights_kernel(const float* __restr
     if (prob) s = prob[(e / pairs_per_batch) * N + nbhd_idx[e]];
     if (mask) s *= (float)mask[e];
     w.x *= s, w.y *= s, w.z *= s, w.w *= s;
-    __builtin_nontemporal_store(w.x, out + e * 4);
-    __builtin_nontemporal_store(w.y, out + e * 4 + 1);
-    __builtin_nontemporal_store(w.z, out + e * 4 + 2);
-    __builtin_nontemporal_store(w.w, out + e * 4 + 3);
+    *reinterpret_cast<float4*>(out + e * 4) = w;   // plain: the merge kernel reads it next
 }
 
 }  // namespace
