@@ -42,6 +42,14 @@ int launch_cluster_attention_f32(const void* q, clusten_strides qs, const void* 
                                  const int64_t* mask, const float* blank_k, const float* blank_v, void* out,
                                  clusten_strides os, float scale, int lists_shared, const void* plan, float* lse,
                                  const clusten_attn_shape& s, hipStream_t stream);   // cluster_attention_f32.hip
+// cluster_attention_resident.hip: short sequences, the K and V rows of an (image, head) resident in LDS
+bool cluster_attention_resident_takes(const clusten_attn_shape& s, int dtype);
+int launch_cluster_attention_resident(const void* q, clusten_strides qs, const void* k, clusten_strides ks, const void* v,
+                                      clusten_strides vs, const int32_t* cluster_idx, const void* table,
+                                      const int64_t* pe_idx, const int64_t* mask, const float* blank_k,
+                                      const float* blank_v, void* out, clusten_strides os, float scale, int lists_shared,
+                                      const void* plan, float* lse, const clusten_attn_shape& s, int dtype,
+                                      hipStream_t stream);
 
 namespace {
 
@@ -481,6 +489,10 @@ int launch_cluster_attention(const void* q, clusten_strides qs, const void* k, c
         }
         return launch_typed<bf16_t, 24>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os,
                                         scale, lists_shared, plan, lse, s, stream);
+    }
+    if (cluster_attention_resident_takes(s, dtype)) {
+        return launch_cluster_attention_resident(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out,
+                                                 os, scale, lists_shared, plan, lse, s, dtype, stream);
     }
     if (dtype == CLUSTEN_F16) {
         return launch_typed<f16_t, 8>(q, qs, k, ks, v, vs, cluster_idx, table, pe_idx, mask, blank_k, blank_v, out, os, scale,

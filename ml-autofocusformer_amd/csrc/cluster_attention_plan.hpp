@@ -65,7 +65,7 @@ __device__ __forceinline__ void tile_setup(const int32_t* __restrict__ cluster_i
                                            int64_t tok, int (&pe)[Geo<CS>::kR], int (&us)[kNnc], int& repeats, int& U,
                                            int* ulist) {
     constexpr int kRuns = Geo<CS>::kR, kSlots = Geo<CS>::kM;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;   // (the callers are one wave per tile; some have several waves a workgroup)
     const int t = lane >> 3, i = lane & 7;
     // cluster numbers: lane rho < 48 owns entry rho = token * 6 + cluster of the tile
     const int rho = min(lane, kTileTokens * kNnc - 1);

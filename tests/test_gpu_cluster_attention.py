@@ -265,6 +265,41 @@ def test_plan_built_once_gives_the_same_bits(device, kind, dtype):
                                   d(blank_k), d(blank_v), plan=plan1)
 
 
+@pytest.mark.parametrize("kind", ["near", "scattered", "repeated"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_short_sequences_with_the_rows_of_a_head_resident_in_lds(device, kind, dtype):
+    """512 or more (image, head) pairs of at most 256 tokens go to the kernel that keeps the K and V rows of a head in
+    LDS (the 196-token stage of the 224 x 224 models): against the oracle composition, and bit for bit against the same
+    images computed a quarter of the batch at a time, which the kernel with one workgroup per tile takes - with and
+    without plan, masks, a short last cluster (196 = 24 clusters and 4 tokens), the training forward's denominators."""
+    gen = torch.Generator().manual_seed(95)
+    d = lambda x: None if x is None else x.to(device)
+    scale = C ** -0.5
+    for b, h, n, with_mask in ((64, 8, 196, True), (128, 4, 104, False), (32, 16, 250, True)):
+        q, k, v, cidx, idx, table, pe_idx, mask, blank_k, blank_v = _case(b, h, n, gen, kind, dtype, with_mask)
+        ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale)
+        out = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v),
+                                        scale=scale)
+        what = "%s %s b=%d h=%d n=%d" % (kind, dtype, b, h, n)
+        assert oracle.rel_err(out, ref) <= TOL[dtype], what
+        plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+        planned, lse = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                                 scale=scale, plan=plan, return_lse=True)
+        assert torch.equal(planned, out), what
+        quarter = b // 4
+        parts, lses = [], []
+        for lo in range(0, b, quarter):
+            sl = slice(lo, lo + quarter)
+            assert quarter * h < 512
+            pl = _native.cluster_attention_plan(d(cidx[sl]), d(pe_idx[sl]), d(None if mask is None else mask[sl]))
+            o, l = _native.cluster_attention(d(q[sl]), d(k[sl]), d(v[sl]), None, d(table), None, None, d(blank_k),
+                                             d(blank_v), scale=scale, plan=pl, return_lse=True)
+            parts.append(o)
+            lses.append(l)
+        assert torch.equal(torch.cat(parts), out), what
+        assert torch.equal(torch.cat(lses), lse), what
+
+
 def _reference_grads(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, scale, d_out):
     """Gradients of `_reference` by autograd, in fp32 from the same rounded inputs."""
     b, h, n, c = q.shape
