@@ -325,7 +325,7 @@ def _bench_wf(case, steps, warmup):
             "input_sets_rotated": copies}
 
 
-def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8):
+def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8, views=False):
     """The one-kernel local attention (QK, bias, mask, blank token, softmax, AV) of one block at a stage's shape on
     lists built by the model's clustering, with the plan of the stage; microseconds per call."""
     import torch
@@ -339,6 +339,12 @@ def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8):
     gen = torch.Generator().manual_seed(1029)
     rows = 111 * 111
     q, k, v = (t.to(dtype) for t in (mcase.query, mcase.key, mcase.value))
+    if views:
+        # the operands as a model's projections leave them: q a (B,N,H,C) tensor, k and v the two halves of a
+        # (B,N,H,2,C) tensor (models/aff_transformer.py:112-118), all three handed over as permuted views
+        kv = torch.stack([k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)], dim=3).contiguous()      # (B,N,H,2,C)
+        q = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        k, v = kv[:, :, :, 0].permute(0, 2, 1, 3), kv[:, :, :, 1].permute(0, 2, 1, 3)
     table = torch.randn(rows, H, generator=gen).to(dtype).cuda()
     pe_idx = torch.randint(rows, (B, N, 6 * cluster), generator=gen).cuda()
     blank_k, blank_v = torch.randn(H * 32, generator=gen).cuda(), torch.randn(H * 32, generator=gen).cuda()
@@ -346,8 +352,8 @@ def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8):
     _, per, _, per_min = _time_kernels([lambda: _native.cluster_attention(q, k, v, None, table, None, None, blank_k,
                                                                           blank_v, plan=plan)], steps, warmup)
     nbytes = 4 * q.numel() * q.element_size() + plan.numel()
-    return {"shape": "B%d H%d N%d C32 M%d %s, model-built lists, planned" % (B, H, N, 6 * cluster,
-                                                                            str(dtype).replace("torch.", "")),
+    return {"shape": "B%d H%d N%d C32 M%d %s, model-built lists, planned%s" % (
+                B, H, N, 6 * cluster, str(dtype).replace("torch.", ""), ", q / k / v as views of the projections" if views else ""),
             "median_us": round(per[0] * 1e3, 1), "min_us": round(per_min[0] * 1e3, 1),
             "bytes_q_k_v_out_plan": nbytes, "GBps": round(nbytes / per[0] / 1e6, 1)}
 
@@ -494,7 +500,7 @@ def main():
                     help="batch size of the --only wf-cfg3* / ca-* profiler legs (default: the configuration's own)")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model", "replay-qk", "replay-av", "replay-wf",
                                        "interference", "wf-cfg3", "wf-cfg3-f32", "ca-s1-f16", "ca-s1-f32", "ca-s2-f16",
-                                       "ca-s3-f16", "ca-384-f16"),
+                                       "ca-s3-f16", "ca-384-f16", "ca-s1-f16-views", "ca-s2-f16-views", "ca-s3-f16-views"),
                     default=None,
                     help="launch just this kernel warmup+steps times (for profilers); prints a short JSON line")
     args = ap.parse_args()
@@ -529,10 +535,11 @@ def main():
                                                    cluster=24)}), flush=True)
         return
     if args.only and args.only.startswith("ca-"):   # the one-kernel local attention at a stage's shape, with its plan
-        stage, dt = int(args.only[4]), (torch.float16 if args.only.endswith("f16") else torch.float32)
+        stage, dt = int(args.only[4]), (torch.float16 if "f16" in args.only else torch.float32)
         H, N = {1: (2, 3136), 2: (4, 784), 3: (8, 196)}[stage]
         print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
-                          **_bench_local_attention(args.batch or 128, H, N, dt, args.steps, args.warmup)}), flush=True)
+                          **_bench_local_attention(args.batch or 128, H, N, dt, args.steps, args.warmup,
+                                                   views=args.only.endswith("-views"))}), flush=True)
         return
     B = 128
     acase = wl.config2_attn(1, B=B)

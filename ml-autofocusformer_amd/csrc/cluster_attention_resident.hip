@@ -45,7 +45,9 @@ constexpr int UL_OFF = O_OFF + kTileTokens * kRB;          // cluster number of 
 constexpr int PB_OFF = UL_OFF + kTileTokens * kNnc * 4;    // blank-token probability per token
 constexpr int W_BYTES = (PB_OFF + kTileTokens * 4 + 1023) / 1024 * 1024;
 static_assert(P_BYTES <= S_BYTES && P_BYTES > 1024 && P_BYTES <= 2048, "the probabilities fit the score area");
-inline int resident_rows_bytes(int N) { return (N + 15) / 16 * 16 * kRB; }
+// rows of the sequence padded to whole 16-row accesses (the pad rows hold copies of row 0, as the pad slots of a short
+// last cluster name row 0), then one more access of copies of row 0: the rows of a cluster number outside the sequence
+inline int resident_rows_bytes(int N) { return ((N + 15) / 16 * 16 + 16) * kRB; }
 inline int resident_lds_bytes(int N) { return 2 * resident_rows_bytes(N) + kResWaves * W_BYTES; }
 
 template <typename T>
@@ -60,8 +62,11 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
 
     extern __shared__ __attribute__((aligned(1024))) char stage[];
     const int KF_BASE = 0;
-    const int VF_BASE = (N + 15) / 16 * 16 * kRB;
+    const int n_pad = (N + 15) / 16 * 16;
+    const int VF_BASE = (n_pad + 16) * kRB;
     const int W_BASE = 2 * VF_BASE;
+    const int clusters = (N + 7) / 8;           // clusters of the sequence; number `clusters` and beyond: rows of row 0
+    const int zero_cluster_bytes = n_pad * kRB;
 
     // unit -> (image, head): the heads of an image are neighbours in the grid (they read the same plan and lists)
     const int unit = xcd_tile(blockIdx.x, total_units);
@@ -82,8 +87,9 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
     {
         const char* k_bh = reinterpret_cast<const char*>(k + (int64_t)b * ks.b + (int64_t)h * ks.h);
         const char* v_bh = reinterpret_cast<const char*>(v + (int64_t)b * vs.b + (int64_t)h * vs.h);
-        for (int a = wave; a * 16 < N; a += kResWaves) {
-            const uint32_t row = (uint32_t)min(a * 16 + g_sub, N - 1);
+        for (int a = wave; a * 16 < n_pad + 16; a += kResWaves) {
+            const int r = a * 16 + g_sub;
+            const uint32_t row = (uint32_t)(r < N ? r : 0);
             CLUSTEN_LDS_DMA16(k_bh + lane_offset(row * (uint32_t)ks.n * 2 + (uint32_t)g_pos * 16), stage + KF_BASE + a * 1024);
             CLUSTEN_LDS_DMA16(v_bh + lane_offset(row * (uint32_t)vs.n * 2 + (uint32_t)g_pos * 16), stage + VF_BASE + a * 1024);
         }
@@ -98,17 +104,34 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
             CLUSTEN_LDS_DMA16(q_bh + lane_offset(row * (uint32_t)qs.n * 2 + (uint32_t)g_pos * 16), mine + Q_OFF + slot * Q_SLOT);
         }
     };
-    if (wave < tiles_per_batch) fetch_q(wave, 0);
+    // byte offset of a cluster's 8 rows in the LDS copies (the copies of row 0 for a number outside the sequence)
+    auto cluster_bytes = [&](int c) -> int {
+        return (unsigned)c < (unsigned)clusters ? c * (8 * kRB) : zero_cluster_bytes;
+    };
+    // a tile's plan as it is loaded: two 16-byte pieces per lane, the number of distinct clusters, one cluster number
+    struct PlanRegs {
+        Piece lo, hi;
+        int U, cluster;
+    };
+    auto load_plan = [&](int tile) -> PlanRegs {
+        const char* pl = plan + (list_b * tiles_per_batch + tile) * (int64_t)kPlanBytes;
+        PlanRegs r;
+        r.lo = *reinterpret_cast<const Piece*>(pl + kPlanLane + lane * 32);
+        r.hi = *reinterpret_cast<const Piece*>(pl + kPlanLane + lane * 32 + 16);
+        r.U = *reinterpret_cast<const int*>(pl);
+        r.cluster = *reinterpret_cast<const int*>(pl + 16 + min(lane, kTileTokens * kNnc - 1) * 4);
+        return r;
+    };
+    // the wave's first tile: q rows and plan requested along with the K and V rows
+    PlanRegs ahead = PlanRegs{Piece{0u, 0u, 0u, 0u}, Piece{0u, 0u, 0u, 0u}, 0, 0};
+    if (wave < tiles_per_batch) {
+        fetch_q(wave, 0);
+        if (plan != nullptr) ahead = load_plan(wave);
+    }
     // per-head constants
     const float4 bk = *reinterpret_cast<const float4*>(blank_k + h * kC + 4 * i);
     const float bv[2] = {blank_v[h * kC + r16], blank_v[h * kC + 16 + r16]};
     __syncthreads();   // (waits for every load above: the rows are in LDS for all waves)
-
-    // a row of the sequence in the LDS copies: member m of cluster c, row 0 when that is outside the sequence
-    auto row_bytes = [&](int c, int m) -> int {
-        const int row = c * 8 + m;
-        return ((unsigned)row < (unsigned)N ? row : 0) * kRB;
-    };
 
     int turn = 0;
     for (int tile = wave; tile < tiles_per_batch; tile += kResWaves, ++turn) {
@@ -116,28 +139,31 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
         const int nt = min(kTileTokens, N - i0);
         const int64_t tok = list_b * N + i0 + min(t, nt - 1);
         const char* q_lds = mine + Q_OFF + (turn & 1) * Q_SLOT;
+        const bool more = tile + kResWaves < tiles_per_batch;
 
         int pe[kR];      // per-slot inputs: row of the bias table; the sign bit marks a masked slot
         int usc[kNnc];   // distinct-cluster number of each of this lane's token's clusters
         int repeats = 0; // bit c: cluster c repeats an earlier one of the token
         int U = 0;       // distinct clusters of the tile
-        lds_sync();      // the tile before has read its cluster numbers
+        lds_sync();      // the tile before has read its cluster offsets
         if (plan != nullptr) {
-            const char* pl = plan + (list_b * tiles_per_batch + tile) * (int64_t)kPlanBytes;
-            const Piece lo = *reinterpret_cast<const Piece*>(pl + kPlanLane + lane * 32);
-            const Piece hi = *reinterpret_cast<const Piece*>(pl + kPlanLane + lane * 32 + 16);
-            U = *reinterpret_cast<const int*>(pl);
-            if (lane < kTileTokens * kNnc) ulist[lane] = *reinterpret_cast<const int*>(pl + 16 + lane * 4);
-            pe[0] = (int)lo[0]; pe[1] = (int)lo[1]; pe[2] = (int)lo[2]; pe[3] = (int)lo[3];
-            pe[4] = (int)hi[0]; pe[5] = (int)hi[1];
-            usc[0] = hi[2] & 0xff; usc[1] = (hi[2] >> 8) & 0xff; usc[2] = (hi[2] >> 16) & 0xff; usc[3] = hi[2] >> 24;
-            usc[4] = hi[3] & 0xff; usc[5] = (hi[3] >> 8) & 0xff;
-            repeats = (hi[3] >> 16) & 0xff;
+            const PlanRegs now = ahead;
+            U = now.U;
+            // `ulist` holds where each distinct cluster's rows lie in the LDS copies
+            if (lane < kTileTokens * kNnc) ulist[lane] = cluster_bytes(now.cluster);
+            pe[0] = (int)now.lo[0]; pe[1] = (int)now.lo[1]; pe[2] = (int)now.lo[2]; pe[3] = (int)now.lo[3];
+            pe[4] = (int)now.hi[0]; pe[5] = (int)now.hi[1];
+            usc[0] = now.hi[2] & 0xff; usc[1] = (now.hi[2] >> 8) & 0xff; usc[2] = (now.hi[2] >> 16) & 0xff;
+            usc[3] = now.hi[2] >> 24;
+            usc[4] = now.hi[3] & 0xff; usc[5] = (now.hi[3] >> 8) & 0xff;
+            repeats = (now.hi[3] >> 16) & 0xff;
         } else {
             tile_setup<8>(cluster_idx, pe_idx, mask, list_b, N, i0, nt, tok, pe, usc, repeats, U, ulist);
+            lds_sync();
+            if (lane < kTileTokens * kNnc) ulist[lane] = cluster_bytes(ulist[lane]);   // cluster numbers -> offsets
         }
         const bool twice = __any(repeats) != 0;
-        // the bias of the lane's slots, and the next tile's q rows, requested before the wait for this tile's
+        // the bias of the lane's slots, then the next tile's plan and q rows: requested before the wait for this tile's
         float bias[kR];
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
@@ -145,9 +171,11 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
             bias[r] = to_acc(*reinterpret_cast<const T*>(reinterpret_cast<const char*>(table) + cell)) +
                       (pe[r] < 0 ? -100.f : 0.f);
         }
-        if (tile + kResWaves < tiles_per_batch) {
+        if (more) {
+            if (plan != nullptr) ahead = load_plan(tile + kResWaves);
             fetch_q(tile + kResWaves, (turn + 1) & 1);
-            lds_sync_vm<1>();   // everything but the rows just requested: this tile's q rows, the cluster numbers
+            // this tile's q rows were requested a tile ago: before the loads above, which may stay in flight
+            lds_sync_vm<5>();
         } else {
             lds_sync_vm<0>();
         }
@@ -167,13 +195,13 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
             int kaddr[kBlocks];
 #pragma unroll
             for (int blk = 0; blk < kBlocks; ++blk) {
-                kaddr[blk] = ulist[min(pass * kPassRuns + 2 * blk + (r16 >> 3), U - 1)];
+                kaddr[blk] = ulist[min(pass * kPassRuns + 2 * blk + (r16 >> 3), U - 1)] + (r16 & 7) * kRB + kq * 16;
             }
             if (pass > 0) lds_sync();   // the scores of the pass before have been picked
 #pragma unroll
             for (int blk = 0; blk < kBlocks; ++blk) {
                 if (blk * 16 < rows_here) {
-                    const Piece kraw = *reinterpret_cast<const Piece*>(stage + KF_BASE + row_bytes(kaddr[blk], r16 & 7) + kq * 16);
+                    const Piece kraw = *reinterpret_cast<const Piece*>(stage + KF_BASE + kaddr[blk]);
                     const F32x4 d = tile_mfma<T>(kraw, qraw, F32x4{0.f, 0.f, 0.f, 0.f});
                     // lane (r16, kq): pass rows 16*blk + 4*kq .. +3 of token r16
                     if (r16 < kTileTokens) {
@@ -239,7 +267,9 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
             // the lane's rows of each 32-row step: members r16 / 4 and r16 / 4 + 4 of distinct cluster 4 s + kq
             int vaddr[kSteps];
 #pragma unroll
-            for (int s = 0; s < kSteps; ++s) vaddr[s] = ulist[min(pass * kPassRuns + 4 * s + kq, U - 1)];
+            for (int s = 0; s < kSteps; ++s) {
+                vaddr[s] = ulist[min(pass * kPassRuns + 4 * s + kq, U - 1)] + (r16 >> 2) * kRB + (r16 & 3) * 8;
+            }
             lds_sync();  // the scores have been picked (the probabilities of the pass before have been read)
             // probabilities of this pass, re-indexed by distinct cluster: zero, then each lane puts in its own
             *reinterpret_cast<Piece*>(mine + S_OFF + lane * 16) = Piece{0u, 0u, 0u, 0u};
@@ -259,8 +289,8 @@ __global__ __launch_bounds__(kResWaves* kWave) void cluster_attention_resident_k
             for (int s = 0; s < kSteps; ++s) {
                 if (s * 32 < rows_here) {
                     const Piece a = *reinterpret_cast<const Piece*>(mine + S_OFF + ((r16 & 7) * kPRow + 32 * s + 8 * kq) * 2);
-                    const char* lo_row = stage + VF_BASE + row_bytes(vaddr[s], r16 >> 2) + (r16 & 3) * 8;
-                    const char* hi_row = stage + VF_BASE + row_bytes(vaddr[s], (r16 >> 2) + 4) + (r16 & 3) * 8;
+                    const char* lo_row = stage + VF_BASE + vaddr[s];
+                    const char* hi_row = lo_row + 4 * kRB;
 #pragma unroll
                     for (int cb = 0; cb < 2; ++cb) {
                         // rows 0-3 and 4-7 of the lane's cluster, transposed to channel 16*cb + r16
