@@ -354,6 +354,16 @@ int clusten_cluster_attention_backward(const void* query, clusten_strides query_
 size_t clusten_cluster_pairs_bytes(int B, int rows, int M, int n_rows);
 int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair_lists_bytes, int B, int rows, int M,
                           int n_rows, clusten_stream stream);
+/* The same block from the lists given as cluster numbers (the format of clusten_qk_forward_clusters, clusters of 8
+ * rows): cluster_idx (B,rows,nnc) int32, block of clusten_cluster_pairs_bytes(B, rows, 8 * nnc, n_rows) bytes.  With it the
+ * backward of the cluster-number forms needs no row lists at all:
+ *   d_query = clusten_av_forward_clusters(d_attn, key, cluster_idx),  d_key   = clusten_scatter_rows_by_cluster(d_attn, query, block)
+ *   d_attn  = clusten_qk_forward_clusters(d_feat, value, cluster_idx), d_value = clusten_scatter_rows_by_cluster(attn, d_feat, block)
+ * A number outside [0, ceil(n_rows / 8)) sets the block's flag (the forward forms read row 0 for such a number; the
+ * by-cluster scatter then leaves its output untouched: check the flag, or keep the numbers in range, as the lists of
+ * models/aff_transformer.py:476 are).  No counterpart in the reference's extension modules. */
+int clusten_cluster_pairs_from_numbers(const int32_t* cluster_idx, void* pair_lists, size_t pair_lists_bytes, int B,
+                                       int rows, int nnc, int n_rows, clusten_stream stream);
 
 /* The scatter of the two attention backward passes as a gather, for lists made of whole clusters:
  *   y[b,h, 8g+t, :] = sum over the pairs (i,r) with c(b,i,r) = g of  p[b,h,i,8r+t] * x[b,h,i,:]

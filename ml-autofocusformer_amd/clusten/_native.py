@@ -51,6 +51,8 @@ _PROTOTYPES = {
     "clusten_wf_backward_workspace_bytes": (ctypes.c_size_t, [WfShape, ctypes.c_int]),
     "clusten_wf_backward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, WfShape, ctypes.c_int, _P]),
     "clusten_cluster_size_for": (ctypes.c_int, [ctypes.c_int]),
+    "clusten_cluster_pairs_from_numbers": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                          ctypes.c_int, _P]),
     "clusten_qk_forward_clusters": (ctypes.c_int, [_P, Strides, _P, Strides, _P, _P, AttnShape, ctypes.c_int, _P]),
     "clusten_av_forward_clusters": (ctypes.c_int, [_P, _P, Strides, _P, _P, Strides, AttnShape, ctypes.c_int, _P]),
     "clusten_attn_softmax_forward": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, Strides, _P, _P, _P, AttnShape, ctypes.c_int,
@@ -274,6 +276,49 @@ def cluster_pairs(nbhd_idx: torch.Tensor, n_rows=None):
         _check(lib.clusten_cluster_pairs(_ptr(idx), _ptr(block), nbytes, B, rows, M, D, _stream(device)),
                "clusten_cluster_pairs")
     return block
+
+
+def cluster_pairs_from_numbers(cluster_idx: torch.Tensor, n_rows=None):
+    """The block `cluster_pairs` builds for the expanded lists, from the (b,rows,nnc) int32 numbers of clusters of 8 rows
+    themselves (`clusten_cluster_pairs_from_numbers`).  A number outside [0, ceil(n_rows / 8)) sets the block's flag.
+    None when the shape is not supported."""
+    lib = load()
+    _require_cuda("cluster_idx", cluster_idx)
+    if cluster_idx.dim() != 3 or cluster_idx.dtype != torch.int32:
+        raise RuntimeError("cluster_idx must be an int32 (b,rows,clusters per token) tensor")
+    B, rows, nnc = cluster_idx.shape
+    D = rows if n_rows is None else int(n_rows)
+    nbytes = lib.clusten_cluster_pairs_bytes(B, rows, 8 * nnc, D) if B and rows and nnc else 0
+    if nbytes == 0:
+        return None
+    cidx = cluster_idx.contiguous()
+    device = cidx.device
+    block = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        _check(lib.clusten_cluster_pairs_from_numbers(_ptr(cidx), _ptr(block), nbytes, B, rows, nnc, D, _stream(device)),
+               "clusten_cluster_pairs_from_numbers")
+    return block
+
+
+def qk_backward_clusters(d_attn: torch.Tensor, query: torch.Tensor, key: torch.Tensor, cluster_idx: torch.Tensor,
+                         pairs=None):
+    """(d_query, d_key) of `qk_forward_clusters` (clusters of 8 rows, numbers inside the sequence): a gather on the
+    numbers and the by-cluster scatter over `pairs` = `cluster_pairs_from_numbers(cluster_idx)` (built here when not
+    given; a caller keeps it for all layers of a stage)."""
+    if pairs is None:
+        pairs = cluster_pairs_from_numbers(cluster_idx)
+    if pairs is None:
+        raise RuntimeError("qk_backward_clusters: lists of this shape have no pair lists")
+    return av_forward_clusters(d_attn, key, cluster_idx), scatter_rows_by_cluster(d_attn, query, pairs)
+
+
+def av_backward_clusters(d_feat: torch.Tensor, attn: torch.Tensor, v: torch.Tensor, cluster_idx: torch.Tensor, pairs=None):
+    """(d_attn, d_v) of `av_forward_clusters`: see `qk_backward_clusters`."""
+    if pairs is None:
+        pairs = cluster_pairs_from_numbers(cluster_idx)
+    if pairs is None:
+        raise RuntimeError("av_backward_clusters: lists of this shape have no pair lists")
+    return qk_forward_clusters(d_feat, v, cluster_idx), scatter_rows_by_cluster(attn, d_feat, pairs)
 
 
 def pairs_not_whole(pair_lists: torch.Tensor) -> torch.Tensor:

@@ -309,6 +309,22 @@ int clusten_cluster_pairs(const int64_t* nbhd_idx, void* pair_lists, size_t pair
                                 reinterpret_cast<int32_t*>(ws + l.ends), B, rows, M, n_rows, as_stream(stream));
 }
 
+int clusten_cluster_pairs_from_numbers(const int32_t* cluster_idx, void* pair_lists, size_t pair_lists_bytes, int B, int rows,
+                                       int nnc, int n_rows, clusten_stream stream) {
+    if (!cluster_idx || !pair_lists) return CLUSTEN_ERR_NULL_POINTER;
+    if (nnc <= 0 || nnc > kPairMaxSlots / 8) return CLUSTEN_ERR_BAD_DIMS;
+    const int M = 8 * nnc;
+    if (!cluster_pairs_supported(B, rows, M, n_rows)) return CLUSTEN_ERR_BAD_DIMS;
+    const ClusterPairsLayout l = cluster_pairs_layout(B, rows, M, n_rows);
+    if (pair_lists_bytes < l.bytes) return CLUSTEN_ERR_WORKSPACE;
+    if (!aligned16(pair_lists)) return CLUSTEN_ERR_UNALIGNED;
+    char* ws = static_cast<char*>(pair_lists);
+    return launch_cluster_pairs(nullptr, reinterpret_cast<int32_t*>(ws + l.keys), reinterpret_cast<int32_t*>(ws + l.wg_bad),
+                                reinterpret_cast<int32_t*>(ws + l.flag), reinterpret_cast<int32_t*>(ws + l.pairs),
+                                reinterpret_cast<int32_t*>(ws + l.starts), reinterpret_cast<int32_t*>(ws + l.ends), B, rows, M,
+                                n_rows, as_stream(stream), cluster_idx);
+}
+
 int clusten_wf_backward_by_cluster(const void* d_feat_new, const void* weights, const void* feat, const int64_t* nbhd_idx,
                                    const void* pair_lists, void* d_weights, void* d_feat, clusten_wf_shape shape, int dtype,
                                    clusten_stream stream) {

@@ -69,6 +69,27 @@ __global__ __launch_bounds__(kKeysBlock) void cluster_keys_kernel(const int64_t*
     if (threadIdx.x == 0) wg_bad[blockIdx.x] = found ? 1 : 0;
 }
 
+// The same table of keys from cluster numbers (the lists given as (B,rows,R) int32, R numbers of clusters of 8 rows per
+// token): the numbers are the keys; a number outside [0, K) raises the flag.
+__global__ __launch_bounds__(kKeysBlock) void cluster_number_keys_kernel(const int32_t* __restrict__ numbers,
+                                                                         int32_t* __restrict__ keys,
+                                                                         int32_t* __restrict__ wg_bad, int K, int64_t runs) {
+    const int64_t first = (int64_t)blockIdx.x * (kKeysBlock * kKeysPerThread) + threadIdx.x;
+    bool any_bad = false;
+#pragma unroll
+    for (int u = 0; u < kKeysPerThread; ++u) {
+        const int64_t e = first + u * kKeysBlock;
+        if (e < runs) {
+            const int c = numbers[e];
+            const bool ok = (unsigned)c < (unsigned)K;
+            keys[e] = ok ? c : 0;
+            any_bad = any_bad || !ok;
+        }
+    }
+    const int found = __syncthreads_or(any_bad);
+    if (threadIdx.x == 0) wg_bad[blockIdx.x] = found ? 1 : 0;
+}
+
 // Exclusive scan of one value per thread over the workgroup; `scratch` holds one int per wave.  Returns the sum of
 // the values of the threads before this one; *total receives the sum over the workgroup.
 __device__ __forceinline__ int block_exclusive_scan(int v, int* scratch, int* total) {
@@ -256,13 +277,19 @@ ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D) {
 }
 
 int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int32_t* not_whole, int32_t* pairs,
-                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream) {
+                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream,
+                         const int32_t* numbers) {
     const int R = M / 8, K = (D + 7) / 8;
     const int64_t E = (int64_t)rows * R;
     const int64_t runs = (int64_t)B * E;
     const int cap = (int)((D % 8) ? 2 * E : E);
-    const int n_wg = (int)keys_workgroups(runs);
-    hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)n_wg), dim3(kKeysBlock), 0, stream, idx, keys, wg_bad, D, runs);
+    const int n_wg = (int)keys_workgroups(runs);   // (sized for the lists: four threads per run; the numbers use fewer)
+    if (numbers != nullptr) {
+        hipLaunchKernelGGL(cluster_number_keys_kernel, dim3((unsigned)n_wg), dim3(kKeysBlock), 0, stream, numbers, keys,
+                           wg_bad, K, runs);
+    } else {
+        hipLaunchKernelGGL(cluster_keys_kernel, dim3((unsigned)n_wg), dim3(kKeysBlock), 0, stream, idx, keys, wg_bad, D, runs);
+    }
     int waves = (kSortLdsBytes / 4 - 16) / K - 1;    // (waves + 1) * K + waves ints of LDS
     waves = waves > 16 ? 16 : waves;
     const int64_t steps = (E + 63) / 64;

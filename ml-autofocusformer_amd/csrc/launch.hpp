@@ -113,8 +113,11 @@ struct ClusterPairsLayout {
 };
 bool cluster_pairs_supported(int B, int rows, int M, int D);
 ClusterPairsLayout cluster_pairs_layout(int B, int rows, int M, int D);
+// `numbers` != nullptr: the lists as (B,rows,M/8) int32 cluster numbers instead of `idx` (not read then); a number
+//   outside [0, ceil(D/8)) raises *not_whole.
 int launch_cluster_pairs(const int64_t* idx, int32_t* keys, int32_t* wg_bad, int32_t* not_whole, int32_t* pairs,
-                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream);
+                         int32_t* starts, int32_t* ends, int B, int rows, int M, int D, hipStream_t stream,
+                         const int32_t* numbers = nullptr);
 // The entries (i, j) of a list tensor (B, rows, M) by the row of the D-row sequence they name, built on the device
 //   (cluster_pairs.hip): entries[starts[b*D+n] .. ends[b*D+n]) holds e = i*M + j for every idx[b,i,j] = n, ascending.
 //   `only_if` (may be null): device flag; nothing is done when it points to zero.  Sizes as row_entries_layout() gives

@@ -204,6 +204,41 @@ def test_cluster_by_cluster_scatter_properties(device):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_backward_of_the_cluster_number_forms(device, dtype):
+    """`qk_backward_clusters` / `av_backward_clusters`: the lists as (b,n,nnc) int32 cluster numbers in the backward too
+    (pair lists straight from the numbers, `clusten_cluster_pairs_from_numbers`).  Against the oracle's backward on the
+    expanded lists and bit for bit against the row-list backward (same kernels, same pair lists); a short last cluster;
+    a number outside the sequence raises the block's flag."""
+    g = torch.Generator().manual_seed(86)
+    tol = TOL_SCATTER_F32 if dtype == torch.float32 else TOL[dtype]
+    for B, H, N, C, nnc in ((2, 2, 203, 32, 6), (1, 3, 96, 64, 4), (2, 1, 400, 16, 8)):
+        if C == 16 and dtype != torch.float32:
+            continue
+        idx = wl.model_built_lists(B, N, g, cluster=8, nnc=nnc)
+        cidx = (idx[:, :, ::8] // 8).to(torch.int32).contiguous()
+        q = torch.randn(B, H, N, C, generator=g).to(dtype)
+        k = torch.randn(B, H, N, C, generator=g).to(dtype)
+        p = torch.randn(B, H, N, 8 * nnc, generator=g).to(dtype)
+        qd, kd, pd, idxd, cd = q.to(device), k.to(device), p.to(device), idx.to(device), cidx.to(device)
+        pairs = _native.cluster_pairs_from_numbers(cd)
+        assert int(_native.pairs_not_whole(pairs)) == 0
+        want_dq, want_dk = oracle.qk_gather_backward(p.float(), q.float(), k.float(), idx)
+        dq, dk = _native.qk_backward_clusters(pd, qd, kd, cd)
+        what = "%s N=%d C=%d nnc=%d" % (dtype, N, C, nnc)
+        assert oracle.rel_err(dq, want_dq) <= tol and oracle.rel_err(dk, want_dk) <= tol, what
+        dq0, dk0 = _native.qk_backward(pd, qd, kd, idxd)
+        assert torch.equal(dk, dk0) and oracle.rel_err(dq, dq0.float().cpu()) <= tol, what
+        da, dv = _native.av_backward_clusters(qd, pd, kd, cd, pairs=pairs)
+        da0, dv0 = _native.av_backward(qd, pd, kd, idxd)
+        assert torch.equal(dv, dv0) and oracle.rel_err(da, da0.float().cpu()) <= tol, what
+    stray = cd.clone()
+    stray[0, 5, 1] = (N + 7) // 8
+    assert int(_native.pairs_not_whole(_native.cluster_pairs_from_numbers(stray))) == 1
+    stray[0, 5, 1] = -1
+    assert int(_native.pairs_not_whole(_native.cluster_pairs_from_numbers(stray))) == 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_scatter_alone_with_the_callers_pair_lists(device, dtype):
     """`clusten_scatter_rows`: the scatter of the attention backward passes by itself, with pair lists the caller keeps.
     On lists made of whole clusters it is the gather over those lists (bit-equal to the entry point that only does
