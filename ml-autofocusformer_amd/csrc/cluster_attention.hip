@@ -233,11 +233,22 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
             }
         }
     };
+    // K and V rows of the same pass together, access by access: when k and v are the two halves of one projection output
+    // (a model hands them over so) a K row and its V row share a 128-byte line, and the V access finds in the L1 what
+    // the K access just asked for
+    auto gather_both = [&](const char* k_bh, const char* v_bh, const uint32_t (&rr)[kAccesses], int rows_here) {
+#pragma unroll
+        for (int a = 0; a < kAccesses; ++a) {
+            if ((a & ~1) * 16 < rows_here) {
+                CLUSTEN_LDS_DMA16(k_bh + lane_offset(rr[a] * k_pitch + (uint32_t)g_pos * 16), stage + K_BASE + a * 1024);
+                CLUSTEN_LDS_DMA16(v_bh + lane_offset(rr[a] * v_pitch + (uint32_t)g_pos * 16), stage + V_BASE + a * 1024);
+            }
+        }
+    };
     uint32_t rr0[kAccesses];  // pass 0: used by every head
     pass_rows(0, rr0);
     const int rows0 = min(kPassRows, total_rows);
-    gather(k_b, k_pitch, rr0, rows0, K_BASE);
-    gather(v_b, v_pitch, rr0, rows0, V_BASE);
+    gather_both(k_b, v_b, rr0, rows0);
 
     for (int h = 0; h < H; ++h) {
         const char* k_bh = k_b + (int64_t)h * ks.h * 2;
@@ -393,8 +404,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_kernel(
                 pass_rows(pass + 1, rr);
                 gather(v_bh, v_pitch, rr, min(kPassRows, total_rows - (pass + 1) * kPassRows), V_BASE);
             } else if (h + 1 < H) {
-                gather(k_b + (int64_t)(h + 1) * ks.h * 2, k_pitch, rr0, rows0, K_BASE);
-                gather(v_b + (int64_t)(h + 1) * vs.h * 2, v_pitch, rr0, rows0, V_BASE);
+                gather_both(k_b + (int64_t)(h + 1) * ks.h * 2, v_b + (int64_t)(h + 1) * vs.h * 2, rr0, rows0);
                 if (h + 2 < H) fetch_q(h + 2);
             }
         }

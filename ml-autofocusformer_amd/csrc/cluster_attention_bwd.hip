@@ -149,19 +149,21 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
             rr[a] = (unsigned)row < (unsigned)N ? (uint32_t)row : 0u;
         }
     };
-    auto gather = [&](const char* rows_bh, uint32_t pitch, const uint32_t (&rr)[kAccesses], int rows_here, int lds_base) {
+    // K and V rows together, access by access: when k and v are the two halves of one projection output a K row and its V
+    // row share a 128-byte line, and the V access finds in the L1 what the K access just asked for
+    auto gather_both = [&](const char* k_bh, const char* v_bh, const uint32_t (&rr)[kAccesses], int rows_here) {
 #pragma unroll
         for (int a = 0; a < kAccesses; ++a) {
             if ((a & ~1) * 16 < rows_here) {
-                CLUSTEN_LDS_DMA16(rows_bh + lane_offset(rr[a] * pitch + (uint32_t)g_pos * 16), stage + lds_base + a * 1024);
+                CLUSTEN_LDS_DMA16(k_bh + lane_offset(rr[a] * k_pitch + (uint32_t)g_pos * 16), stage + K_BASE + a * 1024);
+                CLUSTEN_LDS_DMA16(v_bh + lane_offset(rr[a] * v_pitch + (uint32_t)g_pos * 16), stage + V_BASE + a * 1024);
             }
         }
     };
     uint32_t rr0[kAccesses];
     pass_rows(0, rr0);
     const int rows0 = min(kPassRows, total_rows);
-    gather(k_b, k_pitch, rr0, rows0, K_BASE);
-    gather(v_b, v_pitch, rr0, rows0, V_BASE);
+    gather_both(k_b, v_b, rr0, rows0);
 
     for (int h = 0; h < H; ++h) {
         const int hh = h0 + h;
@@ -240,8 +242,7 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
                 uint32_t rr[kAccesses];
                 pass_rows(nxt, rr);
                 const int next_rows = min(kPassRows, total_rows - nxt * kPassRows);
-                gather(k_bh, k_pitch, rr, next_rows, K_BASE);
-                gather(v_bh, v_pitch, rr, next_rows, V_BASE);
+                gather_both(k_bh, v_bh, rr, next_rows);
             }
             delta = oct_sum(pdp) + p_b * dpb_t;
             ds_b = p_b * (dpb_t - delta);
@@ -346,11 +347,9 @@ __global__ __launch_bounds__(kWave) void cluster_attention_bwd_kernel(
                 uint32_t rr[kAccesses];
                 pass_rows(pass + 1, rr);
                 const int next_rows = min(kPassRows, total_rows - (pass + 1) * kPassRows);
-                gather(k_bh, k_pitch, rr, next_rows, K_BASE);
-                gather(v_bh, v_pitch, rr, next_rows, V_BASE);
+                gather_both(k_bh, v_bh, rr, next_rows);
             } else if (h + 1 < H) {
-                gather(k_b + (int64_t)(h + 1) * ks.h * 2, k_pitch, rr0, rows0, K_BASE);
-                gather(v_b + (int64_t)(h + 1) * vs.h * 2, v_pitch, rr0, rows0, V_BASE);
+                gather_both(k_b + (int64_t)(h + 1) * ks.h * 2, v_b + (int64_t)(h + 1) * vs.h * 2, rr0, rows0);
                 if (h + 2 < H) fetch_rows(h + 2);
             }
         }
