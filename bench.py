@@ -325,7 +325,7 @@ def _bench_wf(case, steps, warmup):
             "input_sets_rotated": copies}
 
 
-def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8, views=False):
+def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8, views=False, random_bias_rows=False):
     """The one-kernel local attention (QK, bias, mask, blank token, softmax, AV) of one block at a stage's shape on
     lists built by the model's clustering, with the plan of the stage; microseconds per call."""
     import torch
@@ -333,11 +333,13 @@ def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8, views=False
     from clusten import _native
 
     mcase = wl.attn_case("model", 29, B=B, H=H, N=N, C=32, M=6 * cluster, lists="random")
-    mcase.nbhd_idx = wl.model_built_lists(B, N, wl.generator(29), cluster=cluster, nnc=6)
+    mcase.nbhd_idx, pe_idx, rows = wl.model_built_geometry(B, N, wl.generator(29), cluster=cluster, nnc=6)
     mcase = mcase.to("cuda")
     cidx = (mcase.nbhd_idx[:, :, ::cluster] // cluster).to(torch.int32).contiguous()
     gen = torch.Generator().manual_seed(1029)
-    rows = 111 * 111
+    if random_bias_rows:
+        pe_idx = torch.randint(rows, pe_idx.shape, generator=gen)
+    pe_idx = pe_idx.cuda()
     q, k, v = (t.to(dtype) for t in (mcase.query, mcase.key, mcase.value))
     if views:
         # the operands as a model's projections leave them: q a (B,N,H,C) tensor, k and v the two halves of a
@@ -346,14 +348,14 @@ def _bench_local_attention(B, H, N, dtype, steps, warmup, cluster=8, views=False
         q = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
         k, v = kv[:, :, :, 0].permute(0, 2, 1, 3), kv[:, :, :, 1].permute(0, 2, 1, 3)
     table = torch.randn(rows, H, generator=gen).to(dtype).cuda()
-    pe_idx = torch.randint(rows, (B, N, 6 * cluster), generator=gen).cuda()
     blank_k, blank_v = torch.randn(H * 32, generator=gen).cuda(), torch.randn(H * 32, generator=gen).cuda()
     plan = _native.cluster_attention_plan(cidx, pe_idx, None)
     _, per, _, per_min = _time_kernels([lambda: _native.cluster_attention(q, k, v, None, table, None, None, blank_k,
                                                                           blank_v, plan=plan)], steps, warmup)
     nbytes = 4 * q.numel() * q.element_size() + plan.numel()
-    return {"shape": "B%d H%d N%d C32 M%d %s, model-built lists, planned%s" % (
-                B, H, N, 6 * cluster, str(dtype).replace("torch.", ""), ", q / k / v as views of the projections" if views else ""),
+    return {"shape": "B%d H%d N%d C32 M%d %s, model-built lists and position indices, planned%s%s" % (
+                B, H, N, 6 * cluster, str(dtype).replace("torch.", ""), ", q / k / v as views of the projections" if views else "",
+                ", position indices drawn uniformly from the table instead" if random_bias_rows else ""),
             "median_us": round(per[0] * 1e3, 1), "min_us": round(per_min[0] * 1e3, 1),
             "bytes_q_k_v_out_plan": nbytes, "GBps": round(nbytes / per[0] / 1e6, 1)}
 
@@ -498,6 +500,9 @@ def main():
                     help="images/s leg: keep the GEMM libraries' default solutions (no TunableOp pass; for profilers)")
     ap.add_argument("--batch", type=int, default=None,
                     help="batch size of the --only wf-cfg3* / ca-* profiler legs (default: the configuration's own)")
+    ap.add_argument("--random-bias-rows", action="store_true",
+                    help="ca-* legs: position indices drawn uniformly from the table (every slot another cache line) "
+                         "instead of the offsets between the tokens' positions")
     ap.add_argument("--only", choices=("qk", "av", "wf", "copy", "bwd", "bwd-model", "replay-qk", "replay-av", "replay-wf",
                                        "interference", "wf-cfg3", "wf-cfg3-f32", "ca-s1-f16", "ca-s1-f32", "ca-s2-f16",
                                        "ca-s3-f16", "ca-384-f16", "ca-s1-f16-views", "ca-s2-f16-views", "ca-s3-f16-views"),
@@ -532,14 +537,15 @@ def main():
     if args.only == "ca-384-f16":   # ... at the first stage of a 384 x 384 model: clusters of 24, 144 neighbours
         print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
                           **_bench_local_attention(args.batch or 16, 4, 9216, torch.float16, args.steps, args.warmup,
-                                                   cluster=24)}), flush=True)
+                                                   cluster=24, random_bias_rows=args.random_bias_rows)}), flush=True)
         return
     if args.only and args.only.startswith("ca-"):   # the one-kernel local attention at a stage's shape, with its plan
         stage, dt = int(args.only[4]), (torch.float16 if "f16" in args.only else torch.float32)
         H, N = {1: (2, 3136), 2: (4, 784), 3: (8, 196)}[stage]
         print(json.dumps({"only": args.only, "launches": 2 * (args.steps + args.warmup),
                           **_bench_local_attention(args.batch or 128, H, N, dt, args.steps, args.warmup,
-                                                   views=args.only.endswith("-views"))}), flush=True)
+                                                   views=args.only.endswith("-views"),
+                                                   random_bias_rows=args.random_bias_rows)}), flush=True)
         return
     B = 128
     acase = wl.config2_attn(1, B=B)
@@ -689,7 +695,11 @@ def main():
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built"), args.steps, args.warmup)
         other["cfg2_s1_model_like_lists"] = _bench_attn(
             wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model"), args.steps, args.warmup)
-        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="model_built").to("cuda")
+        mcase = wl.attn_case("model", 29, B=B, H=2, N=3136, C=32, lists="random")
+        # the lists with the position indices that go with them: offsets between the tokens' positions, as the model
+        # computes them (uniformly drawn indices would make every slot's bias another cache line)
+        mcase.nbhd_idx, pe_idx, rows = wl.model_built_geometry(B, 3136, wl.generator(29))
+        mcase, pe_idx = mcase.to("cuda"), pe_idx.cuda()
         cidx = (mcase.nbhd_idx[:, :, ::8] // 8).to(torch.int32).contiguous()   # the same lists as cluster numbers
         mattn = torch.softmax(_native.qk_forward(mcase.query, mcase.key, mcase.nbhd_idx), dim=-1)
         _, per_c, _, _ = _time_kernels([lambda: _native.qk_forward_clusters(mcase.query, mcase.key, cidx),
@@ -702,9 +712,7 @@ def main():
         h16 = lambda t: t.to(torch.float16)
         q16, k16, v16 = h16(mcase.query), h16(mcase.key), h16(mcase.value)
         gen = torch.Generator().manual_seed(1029)
-        rows = 111 * 111                                  # offsets between two tokens of a 56 x 56 grid
         table = h16(torch.randn(rows, 2, generator=gen)).cuda()
-        pe_idx = torch.randint(rows, (B, 3136, 48), generator=gen).cuda()
         blank_k, blank_v = torch.randn(64, generator=gen).cuda(), torch.randn(64, generator=gen).cuda()
 
         def three_kernels():
@@ -818,7 +826,7 @@ def main():
         for dt, tag in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             gen384 = wl.generator(31)
             c384 = wl.attn_case("aff_base_384", 31, B=16, H=4, N=9216, C=32, M=144, dtype=dt, lists="random")
-            c384.nbhd_idx = wl.model_built_lists(16, 9216, gen384, cluster=24, nnc=6)
+            c384.nbhd_idx, pe384, rows384 = wl.model_built_geometry(16, 9216, gen384, cluster=24, nnc=6)
             other["aff_base_384_stage1_model_lists_%s" % tag] = _bench_attn(c384, max(args.steps // 2, 5), 5)
             if dt == torch.float32:
                 # the same lists as (B,N,6) int32 numbers of clusters of 24 rows instead of (B,N,144) int64 rows
@@ -837,9 +845,8 @@ def main():
                 # softmax kernel (fp32 probabilities), the cast of v that clusten/clusten.py:52-53 makes, AV in fp32
                 d384 = c384.to("cuda")
                 g2 = torch.Generator().manual_seed(1031)
-                rows384 = 191 * 191                          # offsets between two tokens of a 96 x 96 grid
                 table384 = torch.randn(rows384, 4, generator=g2).to(dt).cuda()
-                pe384 = torch.randint(rows384, (16, 9216, 144), generator=g2).cuda()
+                pe384 = pe384.cuda()
                 bk384, bv384 = torch.randn(128, generator=g2).cuda(), torch.randn(128, generator=g2).cuda()
                 cidx24 = (d384.nbhd_idx[:, :, ::24] // 24).to(torch.int32).contiguous()
                 plan384 = _native.cluster_attention_plan(cidx24, pe384, None)

@@ -532,7 +532,7 @@ int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, c
  *   d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]
  * summed per workgroup in LDS before it reaches memory.  d_logit (B,H,N,M) of `dtype` (F32, F16 or BF16), pe_idx
  * (B,N,M) int64 (entries outside [0,rows) are skipped), d_table (rows,H) fp32, zeroed by the caller; all
- * contiguous.  rows <= 16000 (else CLUSTEN_ERR_BAD_DIMS).  The order of the additions varies from run to run, as a
+ * contiguous.  rows <= 40000 (else CLUSTEN_ERR_BAD_DIMS).  The order of the additions varies from run to run, as a
  * scatter-add's does.  No counterpart in the reference's extension modules. */
 int clusten_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M,
                             int rows, int dtype, clusten_stream stream);

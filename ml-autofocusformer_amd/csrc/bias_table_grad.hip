@@ -5,24 +5,68 @@
 // the backward of `pe_table.gather(index=pe_idx...)` added to the attention logits (models/aff_transformer.py:131-133).
 // The framework runs it as a scatter-add of B*H*N*M values into a table of some 12 000 rows: one global atomic per
 // value, all of them on the same few hundred kilobytes.  Here a workgroup takes one head and a contiguous slice of the
-// head's values (images one after the other) and sums into a copy of that head's column of the table in LDS (LDS
-// atomics; at most 16 000 rows); what it has collected goes to memory with one global atomic per touched row.
-// The grid is one round of workgroups of 512 threads (768 to 1024 of them): the global atomics of the flush all land
-// on the same few kilobytes, so a workgroup should flush once for a long slice, and a column of 12 000 rows is 48 KB
-// of LDS, so few workgroups fit a compute unit and each has to bring many waves.  A thread reads four consecutive values at a time
+// head's values (images one after the other) and sums into a copy of that head's column of the table in LDS; what it
+// has collected goes to memory with one global atomic per touched row.
+// The position indices of a model are offsets between neighbouring tokens: a few hundred cells around the table's
+// centre take all the additions (on such indices a loop of compare-and-swap additions of floats spends its time on
+// lost races, 420 us against 90 us on indices spread over the table).  So a cell is a 64-bit integer: a value enters
+// as a multiple of 2^-40 of the power of two above the slice's largest magnitude, the additions are LDS integer
+// atomics, which the hardware serialises without a retry, and the sum of a slice is exact whatever the order.  fp16
+// values need no look at the slice (all are multiples of 2^-24 below 2^16: every sum is exact); for fp32 and bf16 the
+// workgroup first sweeps its slice for the largest magnitude.  Tables of more than 20 000 rows (a column of 64-bit
+// cells would not fit the 160 KB of LDS) keep fp32 cells and the compare-and-swap additions, up to 40 000 rows.
+// The grid is one round of workgroups of 512 threads: the global atomics of the flush all land on the same few
+// kilobytes, so a workgroup should flush once for a long slice.  A thread reads four consecutive values at a time
 // (two 16-byte loads of indices, one load of gradients) and keeps four such groups in flight.
 // d_table is fp32 and zeroed by the caller.  It has no counterpart in the reference's extension modules.
+#include <type_traits>
+
 #include "launch.hpp"
 
 namespace clusten {
 namespace {
 
 constexpr int kGradThreads = 512;
-constexpr int kGradRowsMax = 16000;   // 64 000 bytes of LDS
-constexpr int kGradGroups = 4;        // groups of 4 values in flight per thread
+constexpr int kGradRowsMax = 40000;        // 160 000 bytes of LDS as fp32 cells: one workgroup per compute unit at that size
+constexpr int kGradRowsFixed = 20000;      // ... as 64-bit cells
+constexpr int kGradGroups = 4;             // groups of 4 values in flight per thread
+constexpr int kFixedBits = 40;             // a value of the slice's top binade has 41 bits; 2^21 of them fit a cell
+constexpr int64_t kFixedSliceMax = 1 << 21;   // values of a slice with 64-bit cells
+constexpr int kHalfTop = 142;              // fp32 exponent field of the binade [2^15, 2^16): no fp16 value lies above it
+
+// x in units of 2^(e_top - 127 - kFixedBits), truncated towards zero; |x| < 2^(e_top - 126) gives |result| < 2^41.
+__device__ __forceinline__ long long to_fixed(float x, int e_top) {
+    const uint32_t bits = __float_as_uint(x);
+    const int e = (int)(bits >> 23) & 0xff;
+    const uint32_t mant = (bits & 0x7fffffu) | (e != 0 ? 0x800000u : 0u);
+    // x = mant * 2^(max(e,1) - 150); the unit is 2^(e_top - 127 - 40)
+    const int sh = max(e, 1) - e_top + (kFixedBits - 23);
+    const unsigned long long mag = sh >= 0 ? (unsigned long long)mant << min(sh, kFixedBits - 23)
+                                           : (unsigned long long)(mant >> min(-sh, 31));
+    return (bits >> 31) != 0 ? -(long long)mag : (long long)mag;
+}
+
+// The position (image, group in the image) of a thread's next group of VEC values inside the head's slice, stepped
+// without a division.
+struct SliceWalk {
+    int64_t f, b, e;
+    __device__ __forceinline__ void start(int64_t lo, int64_t groups_per_image) {
+        f = lo + threadIdx.x;
+        b = f / groups_per_image;
+        e = f - b * groups_per_image;
+    }
+    __device__ __forceinline__ void step(int64_t groups_per_image, int B) {
+        e += kGradThreads;
+        while (e >= groups_per_image) {   // (at most once unless an image holds fewer groups than there are threads)
+            e -= groups_per_image;
+            b = min(b + 1, (int64_t)B - 1);
+        }
+    }
+};
 
 // VEC = 4: per_image % 4 == 0 and both tensors 16-byte aligned (a group never straddles two images); VEC = 1 otherwise.
-template <typename T, int VEC>
+// FIXED: 64-bit cells (rows * 8 bytes of dynamic LDS), else fp32 cells (rows * 4 bytes).
+template <typename T, int VEC, bool FIXED>
 __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* __restrict__ d_logit,
                                                                        const int64_t* __restrict__ pe_idx,
                                                                        float* __restrict__ d_table, int H, int rows,
@@ -30,45 +74,78 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
     typedef VecIO<T, VEC> GIO;
     typedef typename RawBytes<VEC == 4 ? 16 : 8>::type IdxRaw;   // two indices (VEC = 4: a group is two of them) or one
     constexpr int IR = VEC == 4 ? 2 : 1;
-    extern __shared__ float col[];   // rows floats
+    // rows floats, or rows 64-bit sums and behind them the bits of the slice's largest finite magnitude; no other LDS
+    // variable, so that the array starts at offset 0 (64-bit LDS atomics fault on an address that is not 8-byte aligned)
+    extern __shared__ __attribute__((aligned(16))) float col[];
     uint32_t* cells = reinterpret_cast<uint32_t*>(col);
+    unsigned long long* sums = reinterpret_cast<unsigned long long*>(col);
+    uint32_t* slice_top = reinterpret_cast<uint32_t*>(sums + rows);
     const int h = blockIdx.y;
-    for (int r = threadIdx.x; r < rows; r += kGradThreads) col[r] = 0.f;
+    if constexpr (FIXED) {
+        for (int r = threadIdx.x; r < rows; r += kGradThreads) sums[r] = 0ull;
+    } else {
+        for (int r = threadIdx.x; r < rows; r += kGradThreads) col[r] = 0.f;
+    }
+    if (FIXED && threadIdx.x == 0) *slice_top = 0u;
     __syncthreads();
-    // slice blockIdx.x of the head's B * per_image / VEC groups of values: the thread keeps (image, group in the image)
-    // of its next group and steps it, so that no division enters the loop
+    // slice blockIdx.x of the head's B * per_image / VEC groups of values
     const int64_t groups_per_image = per_image / VEC;
     const int64_t total = groups_per_image * B;
     const int64_t lo = (int64_t)blockIdx.x * per_slice, hi = min(total, lo + per_slice);
-    int64_t f = lo + threadIdx.x;
-    int64_t b = f / groups_per_image, e = f - b * groups_per_image;
-    for (; f < hi; f += kGradGroups * kGradThreads) {
+    int e_top = kHalfTop;
+    if constexpr (FIXED && !std::is_same<T, f16_t>::value) {
+        // first sweep: the largest finite magnitude of the slice names the binade the cells' unit hangs on
+        uint32_t top = 0u;
+        SliceWalk w;
+        w.start(lo, groups_per_image);
+        for (; w.f < hi; w.f += kGradGroups * kGradThreads) {
+            typename GIO::raw g[kGradGroups];
+            bool in[kGradGroups];
+#pragma unroll
+            for (int k = 0; k < kGradGroups; ++k) {
+                in[k] = w.f + k * kGradThreads < hi;
+                if (in[k]) g[k] = *reinterpret_cast<const typename GIO::raw*>(d_logit + ((w.b * H + h) * groups_per_image + w.e) * VEC);
+                w.step(groups_per_image, B);
+            }
+#pragma unroll
+            for (int k = 0; k < kGradGroups; ++k) {
+                if (in[k]) {
+                    float x[VEC];
+                    GIO::unpack(g[k], x);
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        const uint32_t m = __float_as_uint(x[v]) & 0x7fffffffu;
+                        top = m < 0x7f800000u ? max(top, m) : top;
+                    }
+                }
+            }
+        }
+        atomicMax(slice_top, top);
+        __syncthreads();
+        e_top = max(1, (int)(*slice_top >> 23));
+    }
+    SliceWalk w;
+    w.start(lo, groups_per_image);
+    for (; w.f < hi; w.f += kGradGroups * kGradThreads) {
         IdxRaw r[kGradGroups][IR];
         typename GIO::raw g[kGradGroups];
         bool in[kGradGroups];
 #pragma unroll
         for (int k = 0; k < kGradGroups; ++k) {   // independent loads before the first addition
-            in[k] = f + k * kGradThreads < hi;
+            in[k] = w.f + k * kGradThreads < hi;
             if (in[k]) {
 #pragma unroll
-                for (int w = 0; w < IR; ++w) {
-                    r[k][w] = *reinterpret_cast<const IdxRaw*>(pe_idx + (b * groups_per_image + e) * VEC + 2 * w);
+                for (int q = 0; q < IR; ++q) {
+                    r[k][q] = *reinterpret_cast<const IdxRaw*>(pe_idx + (w.b * groups_per_image + w.e) * VEC + 2 * q);
                 }
-                g[k] = *reinterpret_cast<const typename GIO::raw*>(d_logit + ((b * H + h) * groups_per_image + e) * VEC);
+                g[k] = *reinterpret_cast<const typename GIO::raw*>(d_logit + ((w.b * H + h) * groups_per_image + w.e) * VEC);
             }
-            e += kGradThreads;
-            while (e >= groups_per_image) {   // (at most once unless an image holds fewer groups than there are threads)
-                e -= groups_per_image;
-                b = min(b + 1, (int64_t)B - 1);
-            }
+            w.step(groups_per_image, B);
         }
 #pragma unroll
         for (int k = 0; k < kGradGroups; ++k) {
-            // The values are added by compare-and-swap on the cells' bits (an fp32 LDS atomic add takes some 190 cycles
-            // per wave instruction here, a compare-and-swap a few): the group's cells are read, then swapped, and only
-            // the lanes that lost a race go round again.
             float x[VEC];
-            uint32_t cell[VEC], seen[VEC];
+            uint32_t cell[VEC];
             uint32_t open = 0;          // bit v: the value still has to reach its cell
             if (in[k]) {
                 GIO::unpack(g[k], x);
@@ -78,53 +155,96 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
                     const uint32_t lo32 = raw_word(r[k][v / 2], 2 * (v % 2)), hi32 = raw_word(r[k][v / 2], 2 * (v % 2) + 1);
                     const bool ok = hi32 == 0u && lo32 < (uint32_t)rows;
                     cell[v] = ok ? lo32 : 0u;
-                    seen[v] = ok ? cells[cell[v]] : 0u;
                     open |= ok ? 1u << v : 0u;
                 }
             }
-            while (open != 0) {
+            if constexpr (FIXED) {
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
                     if ((open >> v & 1u) != 0) {
-                        const uint32_t expect = seen[v];
-                        const uint32_t sum = __float_as_uint(__uint_as_float(expect) + x[v]);
-                        seen[v] = atomicCAS(cells + cell[v], expect, sum);
-                        if (seen[v] == expect) open &= ~(1u << v);
+                        if ((__float_as_uint(x[v]) & 0x7f800000u) == 0x7f800000u) {
+                            // an infinity or a NaN has no integer: it goes to the table as it is
+                            unsafeAtomicAdd(d_table + (int64_t)cell[v] * H + h, x[v]);
+                        } else {
+                            atomicAdd(sums + cell[v], (unsigned long long)to_fixed(x[v], e_top));
+                        }
+                    }
+                }
+            } else {
+                // fp32 cells: the values are added by compare-and-swap on the cells' bits (an fp32 LDS atomic add
+                // takes some 190 cycles per wave instruction here, a compare-and-swap a few): the group's cells are
+                // read, then swapped, and only the lanes that lost a race go round again.
+                uint32_t seen[VEC];
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) seen[v] = (open >> v & 1u) != 0 ? cells[cell[v]] : 0u;
+                while (open != 0) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) {
+                        if ((open >> v & 1u) != 0) {
+                            const uint32_t expect = seen[v];
+                            const uint32_t sum = __float_as_uint(__uint_as_float(expect) + x[v]);
+                            seen[v] = atomicCAS(cells + cell[v], expect, sum);
+                            if (seen[v] == expect) open &= ~(1u << v);
+                        }
                     }
                 }
             }
         }
     }
     __syncthreads();
-    for (int r = threadIdx.x; r < rows; r += kGradThreads) {
-        const float v = col[r];
-        if (v != 0.f) unsafeAtomicAdd(d_table + (int64_t)r * H + h, v);
+    if constexpr (FIXED) {
+        for (int r = threadIdx.x; r < rows; r += kGradThreads) {
+            const long long v = (long long)sums[r];
+            if (v != 0) unsafeAtomicAdd(d_table + (int64_t)r * H + h, (float)ldexp((double)v, e_top - 127 - kFixedBits));
+        }
+    } else {
+        for (int r = threadIdx.x; r < rows; r += kGradThreads) {
+            const float v = col[r];
+            if (v != 0.f) unsafeAtomicAdd(d_table + (int64_t)r * H + h, v);
+        }
     }
 }
 
-template <typename T>
-void launch_typed(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int rows, int64_t per_image,
-                  hipStream_t stream) {
+template <typename T, bool FIXED>
+int launch_cells(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int rows, int64_t per_image,
+                 hipStream_t stream) {
     const bool wide = per_image % 4 == 0 && aligned16(d_logit) && aligned16(pe_idx);
     const int vec = wide ? 4 : 1;
     // one round of workgroups: as many as fit the 256 compute units at once (4 of 512 threads each, fewer when the
-    // column takes more than a quarter of a unit's 160 KB of LDS), and no slice shorter than 16 000 values
-    const size_t lds_bytes = (size_t)rows * sizeof(float);
-    const int per_unit = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / max(lds_bytes, (size_t)1)));
+    // column takes more than a quarter of a unit's 160 KB of LDS), and no slice shorter than 16 000 values; with
+    // 64-bit cells no slice longer than 2^21 values (41 bits a value, 62 bits a sum) either
+    const size_t lds = FIXED ? (size_t)rows * sizeof(long long) + 16 : (size_t)rows * sizeof(float);
+    const int per_unit = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / max(lds, (size_t)1)));
     const int64_t total = per_image / vec * B;
     const int64_t want = (total * vec + 16383) / 16384;
     const int64_t cap = max(1, 256 * per_unit / H);
-    const int slices = (int)max((int64_t)1, min(want, cap));
+    int64_t slices = max((int64_t)1, min(want, cap));
+    if (FIXED) slices = max(slices, (total * vec + kFixedSliceMax - 1) / kFixedSliceMax);
     const int64_t per_slice = (total + slices - 1) / slices;
     const dim3 grid((unsigned)slices, (unsigned)H);
-    const size_t lds = lds_bytes;
+    const void* fn = wide ? reinterpret_cast<const void*>(bias_table_grad_kernel<T, 4, FIXED>)
+                          : reinterpret_cast<const void*>(bias_table_grad_kernel<T, 1, FIXED>);
+    if (lds > 48 * 1024) {   // more LDS than a workgroup gets without asking
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160016) != hipSuccess) {
+            (void)hipGetLastError();
+            return CLUSTEN_ERR_LAUNCH;
+        }
+    }
     if (wide) {
-        hipLaunchKernelGGL((bias_table_grad_kernel<T, 4>), grid, dim3(kGradThreads), lds, stream,
+        hipLaunchKernelGGL((bias_table_grad_kernel<T, 4, FIXED>), grid, dim3(kGradThreads), lds, stream,
                            static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, per_image, per_slice, B);
     } else {
-        hipLaunchKernelGGL((bias_table_grad_kernel<T, 1>), grid, dim3(kGradThreads), lds, stream,
+        hipLaunchKernelGGL((bias_table_grad_kernel<T, 1, FIXED>), grid, dim3(kGradThreads), lds, stream,
                            static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, per_image, per_slice, B);
     }
+    return CLUSTEN_OK;
+}
+
+template <typename T>
+int launch_typed(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int rows, int64_t per_image,
+                 hipStream_t stream) {
+    if (rows <= kGradRowsFixed) return launch_cells<T, true>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream);
+    return launch_cells<T, false>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream);
 }
 
 }  // namespace
@@ -133,13 +253,14 @@ int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_
                            int dtype, hipStream_t stream) {
     if (rows > kGradRowsMax) return CLUSTEN_ERR_BAD_DIMS;
     const int64_t per_image = (int64_t)N * M;
+    int rc;
     switch (dtype) {
-        case CLUSTEN_F32: launch_typed<float>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
-        case CLUSTEN_F16: launch_typed<f16_t>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
-        case CLUSTEN_BF16: launch_typed<bf16_t>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
+        case CLUSTEN_F32: rc = launch_typed<float>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
+        case CLUSTEN_F16: rc = launch_typed<f16_t>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
+        case CLUSTEN_BF16: rc = launch_typed<bf16_t>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream); break;
         default: return CLUSTEN_ERR_BAD_DTYPE;
     }
-    return launch_status();
+    return rc != CLUSTEN_OK ? rc : launch_status();
 }
 
 }  // namespace clusten

@@ -99,26 +99,39 @@ def model_like_lists(B: int, N: int, gen: torch.Generator, cluster: int = CLUSTE
     return out
 
 
-def model_built_lists(B: int, N: int, gen: torch.Generator, cluster: int = CLUSTER, nnc: int = 6,
-                      keep: float = 0.77) -> torch.Tensor:
-    """(B,N,nnc*cluster) int64 lists built the way the reference model builds them for a stage of adaptively kept
-    tokens (models/aff_transformer.py:454-487): per image N tokens at distinct integer positions of a square canvas (a
-    random `keep` of its pixels), ordered and cut into clusters by the balanced clustering
-    (`aff.points.space_filling_cluster`), each token listing the members of the `nnc` clusters whose centres are
-    nearest, nearest first; the pad slots of a short last cluster hold row 0.  Unlike `model_like_lists` (strips of a
-    regular grid) neighbouring clusters here are neighbours in the plane, as in the model."""
+def model_built_geometry(B: int, N: int, gen: torch.Generator, cluster: int = CLUSTER, nnc: int = 6,
+                         keep: float = 0.77):
+    """((B,N,nnc*cluster) int64 lists, (B,N,nnc*cluster) int64 position indices, rows of the position table) built
+    the way the reference model builds them for a stage of adaptively kept tokens (models/aff_transformer.py:454-487):
+    per image N tokens at distinct integer positions of a square canvas (a random `keep` of its pixels), ordered and
+    cut into clusters by the balanced clustering (`aff.points.space_filling_cluster`), each token listing the members
+    of the `nnc` clusters whose centres are nearest, nearest first; the pad slots of a short last cluster hold row 0.
+    The position index of (token, slot) is the offset between the two positions as a row of a (2 side - 1)^2 table
+    (:483-485): neighbours are near, so a tile's indices fall into a few dozen adjacent rows of the table.
+    Unlike `model_like_lists` (strips of a regular grid) neighbouring clusters here are neighbours in the plane, as
+    in the model."""
     from aff.points import knn, space_filling_cluster
     side = int(math.ceil(math.sqrt(N / keep)))
+    radius, width = side - 1, 2 * side - 1
     ys, xs = torch.meshgrid(torch.arange(side), torch.arange(side), indexing="ij")
     canvas = torch.stack([xs.reshape(-1), ys.reshape(-1)], dim=1).float()
     out = torch.empty(B, N, nnc * cluster, dtype=torch.int64)
+    pe = torch.empty(B, N, nnc * cluster, dtype=torch.int64)
     for b in range(B):
         pos = canvas[torch.randperm(side * side, generator=gen)[:N].sort().values][None]
         pos, centres, _, _, _ = space_filling_cluster(pos, cluster, side, side)
         near = knn(pos, centres, nnc)[0]                                              # (N,nnc)
         rows = near.unsqueeze(2) * cluster + torch.arange(cluster)
         out[b] = torch.where(rows < N, rows, torch.zeros_like(rows)).reshape(N, nnc * cluster)
-    return out
+        rel = pos[0][out[b]] - (pos[0][:, None, :] - radius)                          # (N,M,2), every entry in [0, width)
+        pe[b] = (rel[..., 1] * width + rel[..., 0]).long()
+    return out, pe, width * width
+
+
+def model_built_lists(B: int, N: int, gen: torch.Generator, cluster: int = CLUSTER, nnc: int = 6,
+                      keep: float = 0.77) -> torch.Tensor:
+    """The lists of `model_built_geometry` alone."""
+    return model_built_geometry(B, N, gen, cluster, nnc, keep)[0]
 
 
 @dataclass

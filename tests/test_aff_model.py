@@ -567,7 +567,8 @@ def test_bias_table_grad_kernel_equals_the_scatter_add(device, dtype):
     """Gradient of the position-bias table: per-workgroup sums in LDS against index_add in fp64."""
     from clusten import _native
     gen = torch.Generator().manual_seed(43)
-    for b, h, n, m, rows in ((3, 2, 200, 48, 12321), (2, 8, 49, 49, 12321), (1, 1, 5, 8, 7), (4, 16, 64, 48, 16000)):
+    for b, h, n, m, rows in ((3, 2, 200, 48, 12321), (2, 8, 49, 49, 12321), (1, 1, 5, 8, 7), (4, 16, 64, 48, 16000),
+                             (2, 4, 96, 144, 36481), (1, 2, 33, 7, 40000)):
         g = torch.randn(b, h, n, m, generator=gen).to(dtype)
         # positions near the table's centre, as relative offsets of neighbours are, plus a few anywhere
         idx = (rows // 2 + torch.randint(-min(60, rows // 2), min(61, rows - rows // 2), (b, n, m), generator=gen))
@@ -578,10 +579,54 @@ def test_bias_table_grad_kernel_equals_the_scatter_add(device, dtype):
         got = _native.bias_table_grad(g.to(device), idx.to(device), rows)
         assert got.dtype == torch.float32 and got.shape == (rows, h)
         assert oracle.rel_err(got.cpu().double(), want) <= 1e-5
-    assert not _native.bias_table_grad_supported(g.to(device), 16001)
+    assert not _native.bias_table_grad_supported(g.to(device), 40001)
     assert not _native.bias_table_grad_supported(g, 100)
     with pytest.raises(RuntimeError):
         _native.bias_table_grad(g.to(device), idx.to(device)[:, :, :3], rows)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_bias_table_grad_on_offsets_between_neighbours_and_on_values_of_any_size(device, dtype):
+    """The indices of a model are offsets between near tokens: a few hundred cells take every addition.  Tables of up
+    to 20 000 rows are summed in 64-bit integer cells whose unit hangs on the largest magnitude of a workgroup's slice:
+    values of very different sizes, zeros, subnormals, infinities and NaNs must come out as fp64 sums rounded once."""
+    from clusten import _native
+    gen = torch.Generator().manual_seed(47)
+    b, h, n, m, rows = 6, 2, 784, 48, 12321
+    dx, dy = torch.randint(-4, 5, (b, n, m), generator=gen), torch.randint(-4, 5, (b, n, m), generator=gen)
+    idx = (dy + 55) * 111 + dx + 55                                   # 81 distinct cells
+    big = {torch.float32: 1e30, torch.float16: 1e4, torch.bfloat16: 1e30}[dtype]   # (fp16: randn * 1e4 stays finite)
+    tiny = {torch.float32: 1e-36, torch.float16: 6e-8, torch.bfloat16: 1e-36}[dtype]
+    for scale_of_image in ((1.0,) * b, (big, 1.0, tiny, 1e-3, 0.0, 1e3)):
+        g = torch.randn(b, h, n, m, generator=gen) * torch.tensor(scale_of_image).view(b, 1, 1, 1)
+        g = g.to(dtype)
+        want = torch.zeros(rows, h, dtype=torch.float64)
+        want.index_add_(0, idx.reshape(-1), g.double().permute(0, 2, 3, 1).reshape(-1, h))
+        got = _native.bias_table_grad(g.to(device), idx.to(device), rows).cpu().double()
+        # fp64 sums of at most 6 * 784 * 48 values per cell, rounded to fp32 by at most a few hundred workgroups
+        assert torch.isfinite(got).all()
+        assert oracle.rel_err(got, want) <= 2e-6
+        touched = want != 0
+        assert (got[~touched] == 0).all()
+    # values a slice can hold exactly: integers in fp16 sum without any rounding, whatever the order
+    gi = torch.randint(-8, 9, (b, h, n, m), generator=gen).to(dtype)
+    want = torch.zeros(rows, h, dtype=torch.float64)
+    want.index_add_(0, idx.reshape(-1), gi.double().permute(0, 2, 3, 1).reshape(-1, h))
+    got = _native.bias_table_grad(gi.to(device), idx.to(device), rows).cpu().double()
+    assert torch.equal(got, want)
+    # an infinity and a NaN reach their cells as they are and leave the others alone
+    gs = torch.randn(b, h, n, m, generator=gen).to(dtype)
+    gs[1, 0, 5, 7], gs[2, 1, 9, 3] = float("inf"), float("nan")
+    got = _native.bias_table_grad(gs.to(device), idx.to(device), rows).cpu()
+    assert torch.isinf(got[idx[1, 5, 7], 0]) and torch.isnan(got[idx[2, 9, 3], 1])
+    clean = gs.clone()
+    clean[1, 0, 5, 7], clean[2, 1, 9, 3] = 0.0, 0.0
+    want = torch.zeros(rows, h, dtype=torch.float64)
+    want.index_add_(0, idx.reshape(-1), clean.double().permute(0, 2, 3, 1).reshape(-1, h))
+    keep = torch.ones(rows, h, dtype=torch.bool)
+    keep[idx[1, 5, 7], 0], keep[idx[2, 9, 3], 1] = False, False
+    assert oracle.rel_err(got.double()[keep], want[keep]) <= 2e-6
 
 
 @pytest.mark.gpu

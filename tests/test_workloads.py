@@ -94,6 +94,32 @@ def test_model_built_lists_are_whole_clusters_of_neighbouring_tokens():
     assert short.numel() > 0 and (short[:, 4:] == 0).all() and (short[:, :4] == torch.arange(96, 100)).all()
 
 
+def test_model_built_geometry_gives_the_lists_and_position_indices_of_the_models_own_layer():
+    """The benchmark's attention legs take their lists and position indices from `model_built_geometry`: both equal
+    what a layer of this build's model (`BasicLayer.neighbourhoods`, models/aff_transformer.py:454-487) computes for
+    the same tokens, and the indices of a tile fall into a small part of the table."""
+    import math
+    from aff.model import BasicLayer
+    for cluster, n in ((8, 784), (8, 100), (24, 600)):
+        lists, pe, rows = wl.model_built_geometry(2, n, wl.generator(6), cluster=cluster, nnc=6)
+        side = int(math.ceil(math.sqrt(n / 0.77)))
+        assert rows == (2 * side - 1) ** 2 and lists.shape == pe.shape == (2, n, 6 * cluster)
+        assert int(pe.min()) >= 0 and int(pe.max()) < rows
+        assert torch.equal(lists, wl.model_built_lists(2, n, wl.generator(6), cluster=cluster, nnc=6))
+        # the same canvas positions through the model's layer
+        gen = wl.generator(6)
+        ys, xs = torch.meshgrid(torch.arange(side), torch.arange(side), indexing="ij")
+        canvas = torch.stack([xs.reshape(-1), ys.reshape(-1)], dim=1).float()
+        pos = torch.stack([canvas[torch.randperm(side * side, generator=gen)[:n].sort().values] for _ in range(2)])
+        layer = BasicLayer(8, 8, cluster, 6 * cluster, depth=0, num_heads=1, mlp_ratio=1.0, downsample=False)
+        _, _, member_idx, _, pe_idx, _ = layer.neighbourhoods(pos, side, side, side - 1, 2 * side - 1)
+        assert torch.equal(member_idx, lists) and torch.equal(pe_idx, pe)
+        # offsets between near tokens: a tile of `cluster` tokens names a small share of the table's rows
+        per_tile = pe[0, :n // cluster * cluster].reshape(-1, cluster * 6 * cluster)
+        distinct = torch.tensor([len(set((r // (2 * side - 1)).tolist())) for r in per_tile]).float().mean()
+        assert float(distinct) < 0.6 * (2 * side - 1)
+
+
 def test_algorithmic_bytes_match_the_published_table():
     # AFF-Tiny stage 1, fp32: QK = AV = 513.8 MB, WF IC4 = 321.1 MB, IC1 = 186.3 MB
     assert round(wl.attn_bytes(128, 2, 3136, 32, 48, 4) / 1e6, 1) == 513.8
