@@ -532,11 +532,10 @@ int clusten_attn_softmax_backward(const float* probs, const float* blank_prob, c
  *   d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]
  * summed per workgroup in LDS before it reaches memory.  d_logit (B,H,N,M) of `dtype` (F32, F16 or BF16), pe_idx
  * (B,N,M) int64 (entries outside [0,rows) are skipped), d_table (rows,H) fp32, zeroed by the caller; all
- * contiguous.  rows <= 40000 (else CLUSTEN_ERR_BAD_DIMS).  Up to 20000 rows a workgroup sums its share of the values
- * exactly (64-bit integer cells scaled to the share's largest magnitude; an infinity or a NaN is added to the table
- * as it is) and only the workgroups' partial sums meet in fp32 atomics, whose order varies from run to run; above
- * that the cells are fp32 and the order of all additions varies, as a scatter-add's does.  No counterpart in the
- * reference's extension modules. */
+ * contiguous.  A workgroup sums its share of the values for the table's 20000 middle rows (all rows of a smaller
+ * table) exactly, in 64-bit integer cells scaled to the share's largest magnitude, and only the workgroups' partial
+ * sums meet in fp32 atomics, whose order varies from run to run; values for other rows, infinities and NaNs are added
+ * to the table one atomic each, as a scatter-add does.  No counterpart in the reference's extension modules. */
 int clusten_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M,
                             int rows, int dtype, clusten_stream stream);
 

@@ -227,7 +227,7 @@ def _position_bias(bias, pe_idx, ops):
     """(b, h, n, m) position bias of an attention layer: row pe_idx[b,i,j] of the (rows, h) table for every pair."""
     kernel = getattr(ops, "bias_table_grad", None)
     if (kernel is not None and torch.is_grad_enabled() and bias.requires_grad and bias.is_cuda
-            and bias.dtype in (torch.float32, torch.float16, torch.bfloat16) and bias.shape[0] <= 40000):
+            and bias.dtype in (torch.float32, torch.float16, torch.bfloat16)):
         return _PositionBias.apply(bias, pe_idx, kernel)
     return _table_rows(bias, pe_idx).permute(0, 3, 1, 2)
 
@@ -350,11 +350,10 @@ class ClusterAttention(nn.Module):
                                                                   cluster_idx.shape[2])):
             # training: the same kernel forward, one kernel and four sums backward
             bias = self.bias_table(table)
-            if bias.shape[0] <= 40000:
-                out = _ClusterAttention.apply(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, bias, self.blank_k,
-                                              self.blank_v, grid_lists[3], grid_lists[4], pe_idx, member_idx,
-                                              self.scale, self.ops)
-                return self.proj_drop(_linear(self.proj, out, self.ops))
+            out = _ClusterAttention.apply(q.view(b, n, h, ch).permute(0, 2, 1, 3), key, v, bias, self.blank_k,
+                                          self.blank_v, grid_lists[3], grid_lists[4], pe_idx, member_idx,
+                                          self.scale, self.ops)
+            return self.proj_drop(_linear(self.proj, out, self.ops))
         dense = getattr(self.ops, "dense_attention", None)
         if (global_attn and dense is not None and not torch.is_grad_enabled()
                 and not (self.training and self.attn_drop.p > 0)
@@ -382,7 +381,7 @@ class ClusterAttention(nn.Module):
             blank = (q * self.blank_k.reshape(1, h, 1, ch)).sum(-1, keepdim=True)        # (b,h,n,1)
             if (fused is not None and getattr(self.ops, "attn_softmax_backward", None) is not None
                     and getattr(self.ops, "bias_table_grad", None) is not None and torch.is_grad_enabled()
-                    and not global_attn and attn.is_cuda and bias.shape[0] <= 40000
+                    and not global_attn and attn.is_cuda
                     and not (self.training and self.attn_drop.p > 0)
                     and self.ops.attn_softmax_supported(attn, attn.shape[-1])):
                 # training: the same glue as one kernel forward and one backward

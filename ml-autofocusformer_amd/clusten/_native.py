@@ -1327,8 +1327,8 @@ def add_row_score(x: torch.Tensor, branch, weight: torch.Tensor, bias):
 
 
 def bias_table_grad_supported(d_logit: torch.Tensor, rows: int) -> bool:
-    """True when `bias_table_grad` takes this case: a CUDA fp32 / fp16 / bf16 (B,H,N,M) gradient, at most 40000 rows."""
-    return d_logit.is_cuda and d_logit.dtype in _DTYPE_CODES and d_logit.dim() == 4 and 0 < rows <= 40000
+    """True when `bias_table_grad` takes this case: a CUDA fp32 / fp16 / bf16 (B,H,N,M) gradient and a table of any number of rows."""
+    return d_logit.is_cuda and d_logit.dtype in _DTYPE_CODES and d_logit.dim() == 4 and 0 < rows < 2 ** 31
 
 
 def bias_table_grad(d_logit: torch.Tensor, pe_idx: torch.Tensor, rows: int) -> torch.Tensor:
@@ -1339,7 +1339,7 @@ def bias_table_grad(d_logit: torch.Tensor, pe_idx: torch.Tensor, rows: int) -> t
     device = d_logit.device
     _require_cuda("pe_idx", pe_idx, device)
     if not bias_table_grad_supported(d_logit, rows):
-        raise RuntimeError("bias_table_grad takes a fp32 / fp16 / bf16 (B,H,N,M) gradient and a table of at most 40000 rows")
+        raise RuntimeError("bias_table_grad takes a CUDA fp32 / fp16 / bf16 (B,H,N,M) gradient and a table of 1 to 2^31 - 1 rows")
     B, H, N, M = d_logit.shape
     if pe_idx.shape != (B, N, M) or pe_idx.dtype != torch.int64:
         raise RuntimeError("pe_idx must be int64 of shape (B,N,M)")

@@ -13,8 +13,10 @@
 // as a multiple of 2^-40 of the power of two above the slice's largest magnitude, the additions are LDS integer
 // atomics, which the hardware serialises without a retry, and the sum of a slice is exact whatever the order.  fp16
 // values need no look at the slice (all are multiples of 2^-24 below 2^16: every sum is exact); for fp32 and bf16 the
-// workgroup first sweeps its slice for the largest magnitude.  Tables of more than 20 000 rows (a column of 64-bit
-// cells would not fit the 160 KB of LDS) keep fp32 cells and the compare-and-swap additions, up to 40 000 rows.
+// workgroup first sweeps its slice for the largest magnitude.
+// The LDS copy holds 20 000 cells (160 KB): the whole column of a table of up to 20 000 rows, else the 20 000 rows
+// around the table's centre (the offset zero of a (2r+1)^2 table is its middle row); values for rows outside that
+// window go to the table with a global atomic each.
 // The grid is one round of workgroups of 512 threads: the global atomics of the flush all land on the same few
 // kilobytes, so a workgroup should flush once for a long slice.  A thread reads four consecutive values at a time
 // (two 16-byte loads of indices, one load of gradients) and keeps four such groups in flight.
@@ -27,11 +29,10 @@ namespace clusten {
 namespace {
 
 constexpr int kGradThreads = 512;
-constexpr int kGradRowsMax = 40000;        // 160 000 bytes of LDS as fp32 cells: one workgroup per compute unit at that size
-constexpr int kGradRowsFixed = 20000;      // ... as 64-bit cells
+constexpr int kGradWindow = 20000;         // 64-bit cells of the LDS copy: 160 000 bytes
 constexpr int kGradGroups = 4;             // groups of 4 values in flight per thread
 constexpr int kFixedBits = 40;             // a value of the slice's top binade has 41 bits; 2^21 of them fit a cell
-constexpr int64_t kFixedSliceMax = 1 << 21;   // values of a slice with 64-bit cells
+constexpr int64_t kFixedSliceMax = 1 << 21;   // values of a slice
 constexpr int kHalfTop = 142;              // fp32 exponent field of the binade [2^15, 2^16): no fp16 value lies above it
 
 // x in units of 2^(e_top - 127 - kFixedBits), truncated towards zero; |x| < 2^(e_top - 126) gives |result| < 2^41.
@@ -65,35 +66,30 @@ struct SliceWalk {
 };
 
 // VEC = 4: per_image % 4 == 0 and both tensors 16-byte aligned (a group never straddles two images); VEC = 1 otherwise.
-// FIXED: 64-bit cells (rows * 8 bytes of dynamic LDS), else fp32 cells (rows * 4 bytes).
-template <typename T, int VEC, bool FIXED>
+// The LDS copy covers the rows [win_lo, win_lo + win_cells) of the table (win_cells * 8 + 16 bytes of dynamic LDS).
+template <typename T, int VEC>
 __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* __restrict__ d_logit,
                                                                        const int64_t* __restrict__ pe_idx,
                                                                        float* __restrict__ d_table, int H, int rows,
-                                                                       int64_t per_image, int64_t per_slice, int B) {
+                                                                       int win_lo, int win_cells, int64_t per_image,
+                                                                       int64_t per_slice, int B) {
     typedef VecIO<T, VEC> GIO;
     typedef typename RawBytes<VEC == 4 ? 16 : 8>::type IdxRaw;   // two indices (VEC = 4: a group is two of them) or one
     constexpr int IR = VEC == 4 ? 2 : 1;
-    // rows floats, or rows 64-bit sums and behind them the bits of the slice's largest finite magnitude; no other LDS
-    // variable, so that the array starts at offset 0 (64-bit LDS atomics fault on an address that is not 8-byte aligned)
-    extern __shared__ __attribute__((aligned(16))) float col[];
-    uint32_t* cells = reinterpret_cast<uint32_t*>(col);
-    unsigned long long* sums = reinterpret_cast<unsigned long long*>(col);
-    uint32_t* slice_top = reinterpret_cast<uint32_t*>(sums + rows);
+    // win_cells 64-bit sums and behind them the bits of the slice's largest finite magnitude; no other LDS variable,
+    // so that the array starts at offset 0 (64-bit LDS atomics fault on an address that is not 8-byte aligned)
+    extern __shared__ __attribute__((aligned(16))) unsigned long long sums[];
+    uint32_t* slice_top = reinterpret_cast<uint32_t*>(sums + win_cells);
     const int h = blockIdx.y;
-    if constexpr (FIXED) {
-        for (int r = threadIdx.x; r < rows; r += kGradThreads) sums[r] = 0ull;
-    } else {
-        for (int r = threadIdx.x; r < rows; r += kGradThreads) col[r] = 0.f;
-    }
-    if (FIXED && threadIdx.x == 0) *slice_top = 0u;
+    for (int r = threadIdx.x; r < win_cells; r += kGradThreads) sums[r] = 0ull;
+    if (threadIdx.x == 0) *slice_top = 0u;
     __syncthreads();
     // slice blockIdx.x of the head's B * per_image / VEC groups of values
     const int64_t groups_per_image = per_image / VEC;
     const int64_t total = groups_per_image * B;
     const int64_t lo = (int64_t)blockIdx.x * per_slice, hi = min(total, lo + per_slice);
     int e_top = kHalfTop;
-    if constexpr (FIXED && !std::is_same<T, f16_t>::value) {
+    if constexpr (!std::is_same<T, f16_t>::value) {
         // first sweep: the largest finite magnitude of the slice names the binade the cells' unit hangs on
         uint32_t top = 0u;
         SliceWalk w;
@@ -144,47 +140,21 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
         }
 #pragma unroll
         for (int k = 0; k < kGradGroups; ++k) {
-            float x[VEC];
-            uint32_t cell[VEC];
-            uint32_t open = 0;          // bit v: the value still has to reach its cell
             if (in[k]) {
+                float x[VEC];
                 GIO::unpack(g[k], x);
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) {
-                    // the index as two 32-bit words: a row is below 2^31
+                    // the index as two 32-bit words: a row is below 2^31; entries outside the table are skipped
                     const uint32_t lo32 = raw_word(r[k][v / 2], 2 * (v % 2)), hi32 = raw_word(r[k][v / 2], 2 * (v % 2) + 1);
-                    const bool ok = hi32 == 0u && lo32 < (uint32_t)rows;
-                    cell[v] = ok ? lo32 : 0u;
-                    open |= ok ? 1u << v : 0u;
-                }
-            }
-            if constexpr (FIXED) {
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) {
-                    if ((open >> v & 1u) != 0) {
-                        if ((__float_as_uint(x[v]) & 0x7f800000u) == 0x7f800000u) {
-                            // an infinity or a NaN has no integer: it goes to the table as it is
-                            unsafeAtomicAdd(d_table + (int64_t)cell[v] * H + h, x[v]);
+                    if (hi32 == 0u && lo32 < (uint32_t)rows) {
+                        const uint32_t cell = lo32 - (uint32_t)win_lo;
+                        const bool finite = (__float_as_uint(x[v]) & 0x7f800000u) != 0x7f800000u;
+                        if (cell < (uint32_t)win_cells && finite) {
+                            atomicAdd(sums + cell, (unsigned long long)to_fixed(x[v], e_top));
                         } else {
-                            atomicAdd(sums + cell[v], (unsigned long long)to_fixed(x[v], e_top));
-                        }
-                    }
-                }
-            } else {
-                // fp32 cells: the values are added by compare-and-swap on the cells' bits (an fp32 LDS atomic add
-                // takes some 190 cycles per wave instruction here, a compare-and-swap a few): the group's cells are
-                // read, then swapped, and only the lanes that lost a race go round again.
-                uint32_t seen[VEC];
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) seen[v] = (open >> v & 1u) != 0 ? cells[cell[v]] : 0u;
-                while (open != 0) {
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) {
-                        if ((open >> v & 1u) != 0) {
-                            const uint32_t expect = seen[v];
-                            const uint32_t sum = __float_as_uint(__uint_as_float(expect) + x[v]);
-                            seen[v] = atomicCAS(cells + cell[v], expect, sum);
-                            if (seen[v] == expect) open &= ~(1u << v);
+                            // a row outside the window, or an infinity / a NaN, which has no integer: to the table as it is
+                            unsafeAtomicAdd(d_table + (int64_t)lo32 * H + h, x[v]);
                         }
                     }
                 }
@@ -192,66 +162,54 @@ __global__ __launch_bounds__(kGradThreads) void bias_table_grad_kernel(const T* 
         }
     }
     __syncthreads();
-    if constexpr (FIXED) {
-        for (int r = threadIdx.x; r < rows; r += kGradThreads) {
-            const long long v = (long long)sums[r];
-            if (v != 0) unsafeAtomicAdd(d_table + (int64_t)r * H + h, (float)ldexp((double)v, e_top - 127 - kFixedBits));
-        }
-    } else {
-        for (int r = threadIdx.x; r < rows; r += kGradThreads) {
-            const float v = col[r];
-            if (v != 0.f) unsafeAtomicAdd(d_table + (int64_t)r * H + h, v);
-        }
+    for (int r = threadIdx.x; r < win_cells; r += kGradThreads) {
+        const long long v = (long long)sums[r];
+        if (v != 0) unsafeAtomicAdd(d_table + (int64_t)(win_lo + r) * H + h, (float)ldexp((double)v, e_top - 127 - kFixedBits));
     }
-}
-
-template <typename T, bool FIXED>
-int launch_cells(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int rows, int64_t per_image,
-                 hipStream_t stream) {
-    const bool wide = per_image % 4 == 0 && aligned16(d_logit) && aligned16(pe_idx);
-    const int vec = wide ? 4 : 1;
-    // one round of workgroups: as many as fit the 256 compute units at once (4 of 512 threads each, fewer when the
-    // column takes more than a quarter of a unit's 160 KB of LDS), and no slice shorter than 16 000 values; with
-    // 64-bit cells no slice longer than 2^21 values (41 bits a value, 62 bits a sum) either
-    const size_t lds = FIXED ? (size_t)rows * sizeof(long long) + 16 : (size_t)rows * sizeof(float);
-    const int per_unit = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / max(lds, (size_t)1)));
-    const int64_t total = per_image / vec * B;
-    const int64_t want = (total * vec + 16383) / 16384;
-    const int64_t cap = max(1, 256 * per_unit / H);
-    int64_t slices = max((int64_t)1, min(want, cap));
-    if (FIXED) slices = max(slices, (total * vec + kFixedSliceMax - 1) / kFixedSliceMax);
-    const int64_t per_slice = (total + slices - 1) / slices;
-    const dim3 grid((unsigned)slices, (unsigned)H);
-    const void* fn = wide ? reinterpret_cast<const void*>(bias_table_grad_kernel<T, 4, FIXED>)
-                          : reinterpret_cast<const void*>(bias_table_grad_kernel<T, 1, FIXED>);
-    if (lds > 48 * 1024) {   // more LDS than a workgroup gets without asking
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160016) != hipSuccess) {
-            (void)hipGetLastError();
-            return CLUSTEN_ERR_LAUNCH;
-        }
-    }
-    if (wide) {
-        hipLaunchKernelGGL((bias_table_grad_kernel<T, 4, FIXED>), grid, dim3(kGradThreads), lds, stream,
-                           static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, per_image, per_slice, B);
-    } else {
-        hipLaunchKernelGGL((bias_table_grad_kernel<T, 1, FIXED>), grid, dim3(kGradThreads), lds, stream,
-                           static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, per_image, per_slice, B);
-    }
-    return CLUSTEN_OK;
 }
 
 template <typename T>
 int launch_typed(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int rows, int64_t per_image,
                  hipStream_t stream) {
-    if (rows <= kGradRowsFixed) return launch_cells<T, true>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream);
-    return launch_cells<T, false>(d_logit, pe_idx, d_table, B, H, rows, per_image, stream);
+    const bool wide = per_image % 4 == 0 && aligned16(d_logit) && aligned16(pe_idx);
+    const int vec = wide ? 4 : 1;
+    const int win_cells = min(rows, kGradWindow), win_lo = (rows - win_cells) / 2;
+    // one round of workgroups: as many as fit the 256 compute units at once (4 of 512 threads each, fewer when the
+    // copy takes more than a quarter of a unit's 160 KB of LDS), no slice shorter than 16 000 values and none longer
+    // than 2^21 (41 bits a value, 62 bits a sum)
+    const size_t lds = (size_t)win_cells * sizeof(long long) + 16;
+    const int per_unit = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / lds));
+    const int64_t total = per_image / vec * B;
+    const int64_t want = (total * vec + 16383) / 16384;
+    const int64_t cap = max(1, 256 * per_unit / H);
+    int64_t slices = max((int64_t)1, min(want, cap));
+    slices = max(slices, (total * vec + kFixedSliceMax - 1) / kFixedSliceMax);
+    const int64_t per_slice = (total + slices - 1) / slices;
+    const dim3 grid((unsigned)slices, (unsigned)H);
+    const void* fn = wide ? reinterpret_cast<const void*>(bias_table_grad_kernel<T, 4>)
+                          : reinterpret_cast<const void*>(bias_table_grad_kernel<T, 1>);
+    if (lds > 48 * 1024) {   // more LDS than a workgroup gets without asking
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kGradWindow * (int)sizeof(long long) + 16) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return CLUSTEN_ERR_LAUNCH;
+        }
+    }
+    if (wide) {
+        hipLaunchKernelGGL((bias_table_grad_kernel<T, 4>), grid, dim3(kGradThreads), lds, stream,
+                           static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, win_lo, win_cells, per_image, per_slice, B);
+    } else {
+        hipLaunchKernelGGL((bias_table_grad_kernel<T, 1>), grid, dim3(kGradThreads), lds, stream,
+                           static_cast<const T*>(d_logit), pe_idx, d_table, H, rows, win_lo, win_cells, per_image, per_slice, B);
+    }
+    return CLUSTEN_OK;
 }
 
 }  // namespace
 
 int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M, int rows,
                            int dtype, hipStream_t stream) {
-    if (rows > kGradRowsMax) return CLUSTEN_ERR_BAD_DIMS;
+    if (rows <= 0 || B <= 0 || H <= 0 || H > 65535) return CLUSTEN_ERR_BAD_DIMS;
     const int64_t per_image = (int64_t)N * M;
     int rc;
     switch (dtype) {

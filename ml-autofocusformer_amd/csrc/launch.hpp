@@ -197,7 +197,7 @@ int launch_attn_softmax_backward(const float* probs, const float* blank_prob, co
                                  const float* d_blank_prob, void* d_logit, float* d_blank_logit, int64_t rows, int M,
                                  int dtype, hipStream_t stream);
 
-// d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]; d_table (rows,H) fp32 zeroed by the caller, rows <= 40000.
+// d_table[pe_idx[b,i,j], h] += d_logit[b,h,i,j]; d_table (rows,H) fp32 zeroed by the caller.
 int launch_bias_table_grad(const void* d_logit, const int64_t* pe_idx, float* d_table, int B, int H, int N, int M, int rows,
                            int dtype, hipStream_t stream);
 

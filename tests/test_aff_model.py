@@ -568,18 +568,19 @@ def test_bias_table_grad_kernel_equals_the_scatter_add(device, dtype):
     from clusten import _native
     gen = torch.Generator().manual_seed(43)
     for b, h, n, m, rows in ((3, 2, 200, 48, 12321), (2, 8, 49, 49, 12321), (1, 1, 5, 8, 7), (4, 16, 64, 48, 16000),
-                             (2, 4, 96, 144, 36481), (1, 2, 33, 7, 40000)):
+                             (2, 4, 96, 144, 36481), (1, 2, 33, 7, 40000), (2, 3, 64, 48, 100001)):
         g = torch.randn(b, h, n, m, generator=gen).to(dtype)
-        # positions near the table's centre, as relative offsets of neighbours are, plus a few anywhere
+        # positions near the table's centre, as relative offsets of neighbours are, plus some anywhere (in a table of
+        # more than 20 000 rows those mostly fall outside the rows the kernel sums in LDS)
         idx = (rows // 2 + torch.randint(-min(60, rows // 2), min(61, rows - rows // 2), (b, n, m), generator=gen))
-        far = torch.rand(b, n, m, generator=gen) < 0.05
+        far = torch.rand(b, n, m, generator=gen) < (0.05 if rows <= 20000 else 0.3)
         idx[far] = torch.randint(rows, (int(far.sum()),), generator=gen)
         want = torch.zeros(rows, h, dtype=torch.float64)
         want.index_add_(0, idx.reshape(-1), g.double().permute(0, 2, 3, 1).reshape(-1, h))
         got = _native.bias_table_grad(g.to(device), idx.to(device), rows)
         assert got.dtype == torch.float32 and got.shape == (rows, h)
         assert oracle.rel_err(got.cpu().double(), want) <= 1e-5
-    assert not _native.bias_table_grad_supported(g.to(device), 40001)
+    assert _native.bias_table_grad_supported(g.to(device), 40001) and not _native.bias_table_grad_supported(g.to(device), 0)
     assert not _native.bias_table_grad_supported(g, 100)
     with pytest.raises(RuntimeError):
         _native.bias_table_grad(g.to(device), idx.to(device)[:, :, :3], rows)
