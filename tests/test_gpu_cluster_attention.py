@@ -92,6 +92,37 @@ def test_against_the_oracle_composition(device, kind, dtype):
             assert err <= TOL[dtype], "%s %s n=%d mask=%s rel err %.3g" % (kind, dtype, n, with_mask, err)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_on_the_lists_and_position_indices_the_benchmark_measures(device, dtype):
+    """The benchmark's attention legs take lists and position indices from `workloads.model_built_geometry` (tokens
+    on a canvas, clustered as the model clusters them, indices = offsets between positions): the same generator at a
+    small batch, through the tensors and through a plan, per-tile kernel and the one for short sequences, against the
+    oracle composition; clusters of 8 in all three types, clusters of 24 in the 16-bit ones."""
+    import workloads as wl
+    d = lambda x: None if x is None else x.to(device)
+    gen = torch.Generator().manual_seed(97)
+    for cs, b, h, n in ((8, 2, 2, 784), (8, 64, 8, 196), (8, 2, 4, 100), (24, 2, 4, 600)):   # (64 x 8 heads: the short-sequence kernel)
+        if cs == 24 and dtype == torch.float32:
+            continue
+        idx, pe_idx, rows = wl.model_built_geometry(b, n, wl.generator(41), cluster=cs, nnc=NNC)
+        cidx = (idx[:, :, ::cs] // cs).to(torch.int32).contiguous()
+        # the pad slots of a short last cluster hold row 0 in the lists; as cluster numbers they are the last cluster
+        assert torch.equal(_expand(cidx, n, cs), idx)
+        q, k, v = (torch.randn(b, h, n, C, generator=gen).to(dtype) for _ in range(3))
+        table = torch.randn(rows, h, generator=gen).to(dtype)
+        blank_k, blank_v = torch.randn(h * C, generator=gen), torch.randn(h * C, generator=gen)
+        mask = ((cidx.long().unsqueeze(3) * cs + torch.arange(cs)) < n).reshape(b, n, NNC * cs).long() if n % cs else None
+        ref = _reference(q, k, v, idx, table, pe_idx, mask, blank_k, blank_v, C ** -0.5)
+        out = _native.cluster_attention(d(q), d(k), d(v), d(cidx), d(table), d(pe_idx), d(mask), d(blank_k), d(blank_v),
+                                        scale=C ** -0.5)
+        err = oracle.rel_err(out, ref)
+        assert err <= TOL[dtype], "clusters of %d, n=%d, %s: rel err %.3g" % (cs, n, dtype, err)
+        plan = _native.cluster_attention_plan(d(cidx), d(pe_idx), d(mask))
+        planned = _native.cluster_attention(d(q), d(k), d(v), None, d(table), None, None, d(blank_k), d(blank_v),
+                                            scale=C ** -0.5, plan=plan)
+        assert torch.equal(planned, out)
+
+
 @pytest.mark.parametrize("kind", ["near", "shared", "scattered", "repeated"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_clusters_of_24_against_the_oracle_composition(device, kind, dtype):
